@@ -1,0 +1,329 @@
+"""ctypes binding of include/coalsack_moe.h.
+
+Loads the in-tree ``libcoalsack_moe.so`` and fails loudly when it is missing:
+there is no fallback path of any kind.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+OK, ERR_ARG, ERR_HIP, ERR_RANGE, ERR_ALL_EMPTY, ERR_SCALE, ERR_STATE = range(7)
+ACT_MODIFIED_SWIGLU, ACT_STANDARD_SWIGLU = 0, 1
+W_UP, W_GATE, W_DOWN = 0, 1, 2
+FWD_RMSNORM, FWD_RESIDUAL = 1, 2
+
+# name -> (restype, argtypes); every symbol include/coalsack_moe.h declares
+_P = C.c_void_p
+_F = C.POINTER(C.c_float)
+_B = C.POINTER(C.c_uint8)
+_I64 = C.c_int64
+SIGNATURES = {
+    "csk_init": (C.c_int, [C.c_int]),
+    "csk_last_error": (C.c_char_p, []),
+    "csk_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_size_t)]),
+    "csk_dev_alloc": (_P, [C.c_size_t]),
+    "csk_dev_free": (None, [_P]),
+    "csk_copy_h2d": (C.c_int, [_P, _P, C.c_size_t]),
+    "csk_copy_d2h": (C.c_int, [_P, _P, C.c_size_t]),
+    "csk_synchronize": (C.c_int, []),
+    "csk_event_create": (_P, []),
+    "csk_event_destroy": (None, [_P]),
+    "csk_event_record": (C.c_int, [_P]),
+    "csk_event_elapsed_ms": (C.c_int, [_P, _P, _F]),
+    "csk_mxfp4_upload": (C.c_int, [_P, _I64, _I64, C.POINTER(_P)]),
+    "csk_mxfp4_free": (None, [_P]),
+    "csk_mxfp4_dequant": (C.c_int, [_P, _P]),
+    "csk_mxfp4_export": (C.c_int, [_P, _P]),
+    "csk_layer_create": (C.c_int, [_I64, _I64, _I64, _I64, C.POINTER(_P)]),
+    "csk_layer_destroy": (None, [_P]),
+    "csk_layer_set_options": (C.c_int, [_P, C.c_int, C.c_int, C.c_int]),
+    "csk_layer_set_router": (C.c_int, [_P, _P, _P]),
+    "csk_layer_set_expert": (C.c_int, [_P, _I64, _P, _P, _P, _P, _P, _P]),
+    "csk_layer_set_norm": (C.c_int, [_P, _P, C.c_float]),
+    "csk_layer_fill_synthetic": (C.c_int, [_P, C.c_uint64, _I64, C.c_int, C.c_int]),
+    "csk_layer_dequant": (C.c_int, [_P, _I64, C.c_int, _P]),
+    "csk_layer_export": (C.c_int, [_P, _I64, C.c_int, _P]),
+    "csk_moe_forward": (C.c_int, [_P, _P, _I64, _P, C.c_int]),
+    "csk_moe_forward_host": (C.c_int, [_P, _P, _I64, _P, _P, C.c_int]),
+    "csk_moe_stack_forward": (C.c_int, [C.POINTER(_P), _I64, _P, _I64]),
+    "csk_layer_last_dispatch": (C.c_int, [_P, _P, _P]),
+    "csk_moe_router": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P]),
+    "csk_expert_mlp_mxfp4": (C.c_int, [C.c_int, _P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P,
+                                       _I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]),
+    "csk_expert_token_mxfp4": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, C.c_int]),
+    "csk_expert_merge": (C.c_int, [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]),
+    "csk_rmsnorm": (C.c_int, [_P, _P, _P, _I64, _I64, C.c_float]),
+    "csk_add": (C.c_int, [_P, _P, _P, _I64]),
+}
+
+
+class CskError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"[csk error {code}] {message}")
+        self.code = code
+        self.message = message
+
+
+def lib_path():
+    return os.path.join(_HERE, "libcoalsack_moe.so")
+
+
+def _ptr(a):
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"], "array must be contiguous"
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    return None if a is None else np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a):
+    return None if a is None else np.ascontiguousarray(a, dtype=np.uint8)
+
+
+class Library:
+    """Thin object wrapper; every method maps to one C entry point."""
+
+    def __init__(self, path=None):
+        path = path or lib_path()
+        if not os.path.exists(path):
+            raise FileNotFoundError(
+                f"{path} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'`")
+        self.dll = C.CDLL(path)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(self.dll, name)  # AttributeError if a declared symbol is not exported
+            fn.restype = res
+            fn.argtypes = args
+        self.initialised = False
+
+    # -- helpers
+    def check(self, rc):
+        if rc != OK:
+            raise CskError(rc, self.dll.csk_last_error().decode())
+
+    def init(self, device=0):
+        self.check(self.dll.csk_init(device))
+        self.initialised = True
+        return self
+
+    def device_info(self):
+        name = C.create_string_buffer(256)
+        cus = C.c_int()
+        mem = C.c_size_t()
+        self.check(self.dll.csk_device_info(name, 256, C.byref(cus), C.byref(mem)))
+        return name.value.decode(), cus.value, mem.value
+
+    # -- device memory
+    def dev_alloc(self, nbytes):
+        p = self.dll.csk_dev_alloc(nbytes)
+        if not p:
+            raise CskError(ERR_HIP, self.dll.csk_last_error().decode())
+        return p
+
+    def dev_free(self, p):
+        self.dll.csk_dev_free(p)
+
+    def to_device(self, arr):
+        arr = np.ascontiguousarray(arr)
+        p = self.dev_alloc(arr.nbytes)
+        self.check(self.dll.csk_copy_h2d(p, _ptr(arr), arr.nbytes))
+        return p
+
+    def to_host(self, p, shape, dtype=np.float32):
+        out = np.empty(shape, dtype=dtype)
+        self.check(self.dll.csk_copy_d2h(_ptr(out), p, out.nbytes))
+        return out
+
+    def synchronize(self):
+        self.check(self.dll.csk_synchronize())
+
+    def event(self):
+        e = self.dll.csk_event_create()
+        if not e:
+            raise CskError(ERR_HIP, "csk_event_create failed")
+        return e
+
+    def record(self, e):
+        self.check(self.dll.csk_event_record(e))
+
+    def elapsed_ms(self, a, b):
+        ms = C.c_float()
+        self.check(self.dll.csk_event_elapsed_ms(a, b, C.byref(ms)))
+        return ms.value
+
+    # -- MXFP4 matrices
+    def mxfp4_upload(self, blocks, rows, K):
+        blocks = _u8(blocks)
+        assert blocks.size == rows * (K // 32) * 17
+        h = _P()
+        self.check(self.dll.csk_mxfp4_upload(_ptr(blocks), rows, K, C.byref(h)))
+        return h
+
+    def mxfp4_free(self, h):
+        self.dll.csk_mxfp4_free(h)
+
+    def mxfp4_dequant(self, h, rows, K):
+        out = np.empty((rows, K), np.float32)
+        self.check(self.dll.csk_mxfp4_dequant(h, _ptr(out)))
+        return out
+
+    def mxfp4_export(self, h, rows, K):
+        out = np.empty(rows * (K // 32) * 17, np.uint8)
+        self.check(self.dll.csk_mxfp4_export(h, _ptr(out)))
+        return out
+
+    # -- node-level ops
+    def moe_router(self, hidden, gate_w, gate_b, k, sigmoid=False):
+        hidden, gate_w, gate_b = _f32(hidden), _f32(gate_w), _f32(gate_b)
+        T, H = hidden.shape
+        E = gate_w.shape[0]
+        out = np.empty((T, k, 2), np.float32)
+        self.check(self.dll.csk_moe_router(_ptr(hidden), T, H, _ptr(gate_w), E, _ptr(gate_b), k,
+                                           int(sigmoid), _ptr(out)))
+        return out
+
+    def expert_mlp(self, expert_id, hidden, F, h_up, h_gate, h_down, b_up, b_gate, b_down, pairs,
+                   act=ACT_MODIFIED_SWIGLU, weight_before_ffn=False):
+        hidden, pairs = _f32(hidden), _f32(pairs)
+        b_up, b_gate, b_down = _f32(b_up), _f32(b_gate), _f32(b_down)
+        T, H = hidden.shape
+        k = pairs.shape[1]
+        out = np.empty((T, H), np.float32)
+        empty = C.c_int()
+        self.check(self.dll.csk_expert_mlp_mxfp4(
+            expert_id, _ptr(hidden), T, H, F, h_up, h_gate, h_down, _ptr(b_up), _ptr(b_gate),
+            _ptr(b_down), _ptr(pairs), k, act, int(weight_before_ffn), _ptr(out), C.byref(empty)))
+        return None if empty.value else out
+
+    def expert_token(self, x, w_up, w_gate, w_down, b_up, b_gate, b_down, H, F,
+                     act=ACT_MODIFIED_SWIGLU):
+        x, w_up, w_gate, w_down = _f32(x), _u8(w_up), _u8(w_gate), _u8(w_down)
+        b_up, b_gate, b_down = _f32(b_up), _f32(b_gate), _f32(b_down)
+        out = np.empty(H, np.float32)
+        self.check(self.dll.csk_expert_token_mxfp4(_ptr(x), _ptr(w_up), _ptr(w_gate), _ptr(w_down),
+                                                   _ptr(b_up), _ptr(b_gate), _ptr(b_down),
+                                                   _ptr(out), H, F, act))
+        return out
+
+    def expert_merge(self, pairs, expert_outs, H, pre_weighted=False):
+        pairs = _f32(pairs)
+        T, k = pairs.shape[:2]
+        E = len(expert_outs)
+        keep = [_f32(a) for a in expert_outs]
+        arr = (_P * E)(*[(_ptr(a) if a is not None else None) for a in keep])
+        out = np.empty((T, H), np.float32)
+        self.check(self.dll.csk_expert_merge(_ptr(pairs), T, k, E, H, arr, int(pre_weighted),
+                                             _ptr(out)))
+        return out
+
+    def rmsnorm(self, x, w, eps):
+        x, w = _f32(x), _f32(w)
+        T, H = x.shape
+        out = np.empty((T, H), np.float32)
+        self.check(self.dll.csk_rmsnorm(_ptr(x), _ptr(w), _ptr(out), T, H, eps))
+        return out
+
+    def add(self, a, b):
+        a, b = _f32(a), _f32(b)
+        out = np.empty(a.shape, np.float32)
+        self.check(self.dll.csk_add(_ptr(a), _ptr(b), _ptr(out), a.size))
+        return out
+
+    # -- layer
+    def layer(self, E, k, H, F):
+        return Layer(self, E, k, H, F)
+
+
+class Layer:
+    """One resident MoE layer (csk_layer_*)."""
+
+    def __init__(self, lib, E, k, H, F):
+        self.lib, self.E, self.k, self.H, self.F = lib, E, k, H, F
+        self.h = _P()
+        lib.check(lib.dll.csk_layer_create(E, k, H, F, C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            self.lib.dll.csk_layer_destroy(self.h)
+            self.h = _P()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    def set_options(self, sigmoid=False, act=ACT_MODIFIED_SWIGLU, weight_before_ffn=False):
+        self.lib.check(self.lib.dll.csk_layer_set_options(self.h, int(sigmoid), act,
+                                                          int(weight_before_ffn)))
+
+    def set_router(self, gate_w, gate_b=None):
+        gate_w, gate_b = _f32(gate_w), _f32(gate_b)
+        assert gate_w.shape == (self.E, self.H)
+        self.lib.check(self.lib.dll.csk_layer_set_router(self.h, _ptr(gate_w), _ptr(gate_b)))
+
+    def set_expert(self, e, w_up, w_gate, w_down, b_up=None, b_gate=None, b_down=None):
+        w_up, w_gate, w_down = _u8(w_up), _u8(w_gate), _u8(w_down)
+        b_up, b_gate, b_down = _f32(b_up), _f32(b_gate), _f32(b_down)
+        self.lib.check(self.lib.dll.csk_layer_set_expert(
+            self.h, e, _ptr(w_up), _ptr(w_gate), _ptr(w_down), _ptr(b_up), _ptr(b_gate),
+            _ptr(b_down)))
+
+    def set_norm(self, w, eps):
+        w = _f32(w)
+        self.lib.check(self.lib.dll.csk_layer_set_norm(self.h, _ptr(w), eps))
+
+    def fill_synthetic(self, seed, layer_index, scale_lo=117, scale_span=5):
+        self.lib.check(self.lib.dll.csk_layer_fill_synthetic(self.h, seed, layer_index, scale_lo,
+                                                             scale_span))
+
+    def dequant(self, e, which):
+        rows, K = (self.H, self.F) if which == W_DOWN else (self.F, self.H)
+        out = np.empty((rows, K), np.float32)
+        self.lib.check(self.lib.dll.csk_layer_dequant(self.h, e, which, _ptr(out)))
+        return out
+
+    def export(self, e, which):
+        rows, K = (self.H, self.F) if which == W_DOWN else (self.F, self.H)
+        out = np.empty(rows * (K // 32) * 17, np.uint8)
+        self.lib.check(self.lib.dll.csk_layer_export(self.h, e, which, _ptr(out)))
+        return out
+
+    def forward_device(self, d_hidden, T, d_out, flags=0):
+        self.lib.check(self.lib.dll.csk_moe_forward(self.h, d_hidden, T, d_out, flags))
+
+    def forward(self, hidden, flags=0, want_pairs=False):
+        hidden = _f32(hidden)
+        T = hidden.shape[0]
+        out = np.empty((T, self.H), np.float32)
+        pairs = np.empty((T, self.k, 2), np.float32) if want_pairs else None
+        self.lib.check(self.lib.dll.csk_moe_forward_host(self.h, _ptr(hidden), T, _ptr(out),
+                                                         _ptr(pairs), flags))
+        return (out, pairs) if want_pairs else out
+
+    def last_dispatch(self, T):
+        counts = np.empty(self.E, np.int32)
+        toks = np.empty(T * self.k, np.int32)
+        self.lib.check(self.lib.dll.csk_layer_last_dispatch(self.h, _ptr(counts), _ptr(toks)))
+        return counts, toks
+
+
+def stack_forward(lib, layers, d_hidden, T):
+    arr = (_P * len(layers))(*[l.h for l in layers])
+    lib.check(lib.dll.csk_moe_stack_forward(arr, len(layers), d_hidden, T))
+
+
+_lib = None
+
+
+def load(device=0):
+    """Load and initialise the library once per process."""
+    global _lib
+    if _lib is None:
+        _lib = Library().init(device)
+    return _lib

@@ -1,0 +1,959 @@
+// C ABI of the gfx950 MoE path: resident weight store, workspace, kernel
+// launches.  Declarations and reference citations are in
+// include/coalsack_moe.h.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "coalsack_moe.h"
+#include "common.h"
+#include "expert_prefill_kernel.h"
+#include "expert_stream_kernel.h"
+#include "mxfp4_kernels.h"
+#include "router_kernels.h"
+
+using namespace csk;
+
+namespace {
+
+thread_local std::string g_err;
+hipStream_t g_stream = nullptr;
+bool g_ready = false;
+int g_device = -1;
+int g_cus = 0;
+
+int fail(int code, const std::string& msg) {
+  g_err = msg;
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                      \
+  do {                                                                                     \
+    hipError_t _e = (expr);                                                                \
+    if (_e != hipSuccess)                                                                  \
+      return fail(CSK_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(_e));         \
+  } while (0)
+
+#define REQUIRE_INIT()                                                          \
+  do {                                                                          \
+    if (!g_ready) return fail(CSK_ERR_STATE, "csk_init has not been called");   \
+  } while (0)
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(CSK_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+  return CSK_OK;
+}
+
+template <class T>
+int dev_alloc(T** p, size_t count) {
+  *p = nullptr;
+  if (count == 0) return CSK_OK;
+  HIP_TRY(hipMalloc(reinterpret_cast<void**>(p), count * sizeof(T)));
+  return CSK_OK;
+}
+
+inline long cdiv(long a, long b) { return (a + b - 1) / b; }
+
+// ---- workspace shared by every layer (single stream, one call at a time) --
+struct Workspace {
+  int64_t T = 0, E = 0, k = 0, H = 0, F = 0;
+  float* xn = nullptr;      // [T,H] normalised activations
+  uint16_t* xs = nullptr;   // [T][H/32][64] bf16 hi|lo
+  uint16_t* xg = nullptr;   // [P][H/32][64] gathered + pre-scaled (weight_before_ffn)
+  float* logits = nullptr;  // [T,E]
+  float* pairs = nullptr;   // [T,k,2]
+  int* ids = nullptr;       // [P]
+  int* counts = nullptr;    // [E]
+  int* offsets = nullptr;   // [E+1]
+  int* active = nullptr;    // [E]
+  int* n_active = nullptr;  // [1]
+  int* list_tok = nullptr;  // [P]
+  float* list_w = nullptr;  // [P]
+  int* pos = nullptr;       // [P]
+  uint16_t* act = nullptr;  // [P][F/32][64] bf16 hi|lo
+  float* y = nullptr;       // [P,H]
+  int* tiles = nullptr;     // prefill tile schedule
+  int* n_tiles = nullptr;
+
+  void release() {
+    void* ps[] = {xn, xs, xg, logits, pairs, ids, counts, offsets, active, n_active,
+                  list_tok, list_w, pos, act, y, tiles, n_tiles};
+    for (void* p : ps)
+      if (p) (void)hipFree(p);
+    *this = Workspace();
+  }
+  int ensure(int64_t T_, int64_t E_, int64_t k_, int64_t H_, int64_t F_, bool need_xg) {
+    if (T_ <= T && E_ <= E && k_ <= k && H_ <= H && F_ <= F && (!need_xg || xg)) return CSK_OK;
+    const int64_t nT = std::max(T, T_), nE = std::max(E, E_), nk = std::max(k, k_),
+                  nH = std::max(H, H_), nF = std::max(F, F_);
+    const bool had_xg = xg != nullptr;
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    release();
+    const size_t P = (size_t)nT * nk;
+    int rc;
+#define WS_ALLOC(ptr, cnt) \
+  if ((rc = dev_alloc(&ptr, (cnt))) != CSK_OK) return rc
+    WS_ALLOC(xn, (size_t)nT * nH);
+    WS_ALLOC(xs, (size_t)nT * nH * 2);
+    if (need_xg || had_xg) WS_ALLOC(xg, P * nH * 2);
+    WS_ALLOC(logits, (size_t)nT * nE);
+    WS_ALLOC(pairs, P * 2);
+    WS_ALLOC(ids, P);
+    WS_ALLOC(counts, (size_t)nE);
+    WS_ALLOC(offsets, (size_t)nE + 1);
+    WS_ALLOC(active, (size_t)nE);
+    WS_ALLOC(n_active, 1);
+    WS_ALLOC(list_tok, P);
+    WS_ALLOC(list_w, P);
+    WS_ALLOC(pos, P);
+    WS_ALLOC(act, P * nF * 2);
+    WS_ALLOC(y, P * nH);
+    WS_ALLOC(tiles, (size_t)4 * (P / 16 + nE + 1));
+    WS_ALLOC(n_tiles, 1);
+#undef WS_ALLOC
+    T = nT, E = nE, k = nk, H = nH, F = nF;
+    return CSK_OK;
+  }
+};
+Workspace g_ws;
+
+}  // namespace
+
+struct csk_event {
+  hipEvent_t ev;
+};
+
+struct csk_mxfp4 {
+  uint4* q = nullptr;
+  uint8_t* s = nullptr;
+  int64_t rows = 0, K = 0;
+  int64_t ntile = 0, nblk = 0;
+  bool owned = true;
+  long entries() const { return (long)(ntile * nblk * 16); }
+};
+
+struct csk_layer {
+  int64_t E = 0, k = 0, H = 0, F = 0;
+  int sigmoid = 0, act = CSK_ACT_MODIFIED_SWIGLU, wbf = 0;
+  float* gate_w = nullptr;
+  float* gate_b = nullptr;
+  bool has_gate = false, has_gate_b = false;
+  uint4* q_all = nullptr;    // [E][gate | up | down] entries
+  uint8_t* s_all = nullptr;
+  float* bias_all = nullptr;  // [E][F gate | F up | H down]
+  ExpertW* ew_dev = nullptr;
+  std::vector<ExpertW> ew_host;
+  std::vector<char> expert_set, expert_bias;
+  float* norm_w = nullptr;
+  float eps = 1e-5f;
+  bool has_norm = false;
+  int64_t last_T = 0;
+  // geometry of one expert's planes
+  int64_t nblkH = 0, nblkF = 0, ntF = 0, ntH = 0;
+  long ent_gu() const { return (long)(ntF * nblkH * 16); }  // gate or up: [F,H]
+  long ent_d() const { return (long)(ntH * nblkF * 16); }   // down: [H,F]
+  long ent_expert() const { return 2 * ent_gu() + ent_d(); }
+  csk_mxfp4 view(int64_t e, int which) const {
+    csk_mxfp4 m;
+    const long base = (long)e * ent_expert();
+    const long off = which == CSK_W_GATE ? 0 : (which == CSK_W_UP ? ent_gu() : 2 * ent_gu());
+    m.q = q_all + base + off;
+    m.s = s_all + base + off;
+    m.rows = which == CSK_W_DOWN ? H : F;
+    m.K = which == CSK_W_DOWN ? F : H;
+    m.ntile = which == CSK_W_DOWN ? ntH : ntF;
+    m.nblk = which == CSK_W_DOWN ? nblkF : nblkH;
+    m.owned = false;
+    return m;
+  }
+};
+
+namespace {
+
+int validate_scales(const uint8_t* blocks, int64_t nblocks) {
+  for (int64_t b = 0; b < nblocks; ++b) {
+    const uint8_t s = blocks[b * 17];
+    if (s < 2 || s > 254)
+      return fail(CSK_ERR_SCALE, "MXFP4 scale byte " + std::to_string((int)s) + " at block " +
+                                     std::to_string(b) +
+                                     " is outside 2..254 (denormal / reserved scales unsupported)");
+  }
+  return CSK_OK;
+}
+
+// Upload `rows x K` reference blocks and repack into (q, s).
+int pack_into(const uint8_t* host, csk_mxfp4& m) {
+  const int64_t nblocks = m.rows * m.nblk;
+  int rc = validate_scales(host, nblocks);
+  if (rc != CSK_OK) return rc;
+  uint8_t* staging = nullptr;
+  HIP_TRY(hipMalloc((void**)&staging, (size_t)nblocks * 17));
+  hipError_t e = hipMemcpyAsync(staging, host, (size_t)nblocks * 17, hipMemcpyHostToDevice, g_stream);
+  if (e == hipSuccess) {
+    const long ent = m.entries();
+    pack_mxfp4_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(
+        staging, m.q, m.s, (int)m.rows, (int)m.nblk, ent);
+    e = hipGetLastError();
+  }
+  hipError_t e2 = hipStreamSynchronize(g_stream);
+  (void)hipFree(staging);
+  if (e != hipSuccess) return fail(CSK_ERR_HIP, std::string("pack: ") + hipGetErrorString(e));
+  if (e2 != hipSuccess) return fail(CSK_ERR_HIP, std::string("pack sync: ") + hipGetErrorString(e2));
+  return CSK_OK;
+}
+
+int dequant_to_host(const csk_mxfp4& m, float* host_out) {
+  float* d = nullptr;
+  const size_t n = (size_t)m.rows * m.K;
+  HIP_TRY(hipMalloc((void**)&d, n * sizeof(float)));
+  const long ent = m.entries();
+  dequant_mxfp4_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(
+      m.q, m.s, d, (int)m.rows, (int)m.nblk, ent);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) e = hipMemcpyAsync(host_out, d, n * sizeof(float), hipMemcpyDeviceToHost, g_stream);
+  hipError_t e2 = hipStreamSynchronize(g_stream);
+  (void)hipFree(d);
+  if (e != hipSuccess) return fail(CSK_ERR_HIP, std::string("dequant: ") + hipGetErrorString(e));
+  if (e2 != hipSuccess) return fail(CSK_ERR_HIP, std::string("dequant sync: ") + hipGetErrorString(e2));
+  return CSK_OK;
+}
+
+int export_to_host(const csk_mxfp4& m, uint8_t* host_out) {
+  uint8_t* d = nullptr;
+  const size_t n = (size_t)m.rows * m.nblk * 17;
+  HIP_TRY(hipMalloc((void**)&d, n));
+  const long ent = m.entries();
+  export_mxfp4_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(
+      m.q, m.s, d, (int)m.rows, (int)m.nblk, ent);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) e = hipMemcpyAsync(host_out, d, n, hipMemcpyDeviceToHost, g_stream);
+  hipError_t e2 = hipStreamSynchronize(g_stream);
+  (void)hipFree(d);
+  if (e != hipSuccess) return fail(CSK_ERR_HIP, std::string("export: ") + hipGetErrorString(e));
+  if (e2 != hipSuccess) return fail(CSK_ERR_HIP, std::string("export sync: ") + hipGetErrorString(e2));
+  return CSK_OK;
+}
+
+int launch_prep(const float* src, const float* norm_w, float eps, float* xn, uint16_t* xs,
+                int64_t rows, int64_t H, const int* gather_tok, const float* gather_w) {
+  if (rows == 0) return CSK_OK;
+  prep_kernel<<<dim3((unsigned)rows), 256, 0, g_stream>>>(src, norm_w, eps, xn, xs, (int)H,
+                                                          gather_tok, gather_w);
+  return check_launch("prep_kernel");
+}
+
+int launch_router(const float* x, const float* gate_w, const float* gate_b, int64_t T, int64_t E,
+                  int64_t H, int64_t k, int sigmoid, float* logits, float* pairs, int* ids) {
+  if (T == 0) return CSK_OK;
+  const unsigned gx = (unsigned)cdiv(E, 4);
+  if (T <= 2) {
+    router_logits_kernel<1><<<dim3(gx, (unsigned)T), 256, 0, g_stream>>>(x, gate_w, gate_b, logits,
+                                                                         (int)T, (int)E, (int)H);
+  } else if (T <= 64) {
+    router_logits_kernel<4><<<dim3(gx, (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
+        x, gate_w, gate_b, logits, (int)T, (int)E, (int)H);
+  } else {
+    router_logits_kernel<8><<<dim3(gx, (unsigned)cdiv(T, 8)), 256, 0, g_stream>>>(
+        x, gate_w, gate_b, logits, (int)T, (int)E, (int)H);
+  }
+  int rc = check_launch("router_logits_kernel");
+  if (rc != CSK_OK) return rc;
+  router_topk_kernel<<<dim3((unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(logits, pairs, ids, (int)T,
+                                                                       (int)E, (int)k, sigmoid);
+  return check_launch("router_topk_kernel");
+}
+
+int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, int64_t E,
+                    Workspace& ws) {
+  dispatch_count_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(ids, (int)P, ws.counts);
+  int rc = check_launch("dispatch_count_kernel");
+  if (rc != CSK_OK) return rc;
+  dispatch_scatter_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(
+      ids, pairs, (int)P, (int)k, (int)E, ws.counts, ws.offsets, ws.active, ws.n_active,
+      ws.list_tok, ws.list_w, ws.pos);
+  return check_launch("dispatch_scatter_kernel");
+}
+
+template <int NMAT>
+int launch_stream(const ExpertStreamArgs& a, int64_t ntile, int64_t max_active, int64_t T) {
+  const dim3 grid((unsigned)ntile, (unsigned)max_active);
+  if (T <= 16)
+    expert_stream_kernel<NMAT, 1><<<grid, 256, 0, g_stream>>>(a);
+  else if (T <= 32)
+    expert_stream_kernel<NMAT, 2><<<grid, 256, 0, g_stream>>>(a);
+  else
+    expert_stream_kernel<NMAT, 4><<<grid, 256, 0, g_stream>>>(a);
+  return check_launch("expert_stream_kernel");
+}
+
+// Experts' MLPs over the dispatched tokens: ws.y[P,H] <- down(act(gate, up)).
+// x_split rows are indexed through list_row (token ids) or directly by packed
+// position when list_row is null.
+int run_experts(const ExpertW* ew, int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
+                int act_type, const uint16_t* x_split, const int* list_row, Workspace& ws) {
+  const int64_t P = T * k;
+  const int64_t max_active = std::min<int64_t>(E, P);
+  ExpertStreamArgs a{};
+  a.ew = ew;
+  a.active = ws.active;
+  a.n_active = ws.n_active;
+  a.counts = ws.counts;
+  a.offsets = ws.offsets;
+  a.act_type = act_type;
+  // gate/up + activation
+  a.list_row = list_row;
+  a.A = reinterpret_cast<const uint4*>(x_split);
+  a.nblk = (int)(H / 32);
+  a.N = (int)F;
+  a.act_out = ws.act;
+  a.y_out = nullptr;
+  int rc = launch_stream<2>(a, cdiv(F, 16), max_active, T);
+  if (rc != CSK_OK) return rc;
+  // down
+  a.list_row = nullptr;
+  a.A = reinterpret_cast<const uint4*>(ws.act);
+  a.nblk = (int)(F / 32);
+  a.N = (int)H;
+  a.act_out = nullptr;
+  a.y_out = ws.y;
+  return launch_stream<1>(a, cdiv(H, 16), max_active, T);
+}
+
+int launch_combine(const float* y, const float* pairs, const int* pos, const float* residual,
+                   float* out, int64_t T, int64_t k, int64_t H, int pre_weighted) {
+  if (T == 0) return CSK_OK;
+  combine_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)T), 256, 0, g_stream>>>(
+      y, pairs, pos, residual, out, (int)T, (int)k, (int)H, pre_weighted);
+  return check_launch("combine_kernel");
+}
+
+int check_dims(int64_t E, int64_t k, int64_t H, int64_t F) {
+  if (E <= 0 || E > kMaxExperts) return fail(CSK_ERR_ARG, "num_experts must be in 1..256");
+  if (k <= 0 || k > kMaxTopK || k > E) return fail(CSK_ERR_ARG, "top_k must be in 1..min(16, E)");
+  if (H <= 0 || H % 32) return fail(CSK_ERR_ARG, "hidden_dim must be a positive multiple of 32");
+  if (F <= 0 || F % 32) return fail(CSK_ERR_ARG, "expert_ffn_dim must be a positive multiple of 32");
+  return CSK_OK;
+}
+
+}  // namespace
+
+// ============================================================ process-wide
+
+extern "C" int csk_init(int device) {
+  int n = 0;
+  HIP_TRY(hipGetDeviceCount(&n));
+  if (device < 0 || device >= n) return fail(CSK_ERR_HIP, "no such GPU device");
+  HIP_TRY(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0)
+    return fail(CSK_ERR_HIP, std::string("device is ") + prop.gcnArchName + ", this library is built for gfx950 only");
+  if (!g_stream) HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  g_device = device;
+  g_cus = prop.multiProcessorCount;
+  g_ready = true;
+  return CSK_OK;
+}
+
+extern "C" const char* csk_last_error(void) { return g_err.c_str(); }
+
+extern "C" int csk_device_info(char* name, size_t cap, int* compute_units, size_t* hbm_bytes) {
+  REQUIRE_INIT();
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, g_device));
+  if (name && cap) {
+    std::snprintf(name, cap, "%s (%s)", prop.name, prop.gcnArchName);
+  }
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  if (hbm_bytes) *hbm_bytes = prop.totalGlobalMem;
+  return CSK_OK;
+}
+
+extern "C" void* csk_dev_alloc(size_t bytes) {
+  if (!g_ready) {
+    g_err = "csk_init has not been called";
+    return nullptr;
+  }
+  void* p = nullptr;
+  hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+  if (e != hipSuccess) {
+    g_err = std::string("hipMalloc: ") + hipGetErrorString(e);
+    return nullptr;
+  }
+  return p;
+}
+extern "C" void csk_dev_free(void* p) {
+  if (p) (void)hipFree(p);
+}
+extern "C" int csk_copy_h2d(void* dst, const void* src, size_t bytes) {
+  REQUIRE_INIT();
+  HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+extern "C" int csk_copy_d2h(void* dst, const void* src, size_t bytes) {
+  REQUIRE_INIT();
+  HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+extern "C" int csk_synchronize(void) {
+  REQUIRE_INIT();
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+extern "C" csk_event* csk_event_create(void) {
+  if (!g_ready) return nullptr;
+  csk_event* e = new csk_event;
+  if (hipEventCreate(&e->ev) != hipSuccess) {
+    delete e;
+    return nullptr;
+  }
+  return e;
+}
+extern "C" void csk_event_destroy(csk_event* e) {
+  if (!e) return;
+  (void)hipEventDestroy(e->ev);
+  delete e;
+}
+extern "C" int csk_event_record(csk_event* e) {
+  REQUIRE_INIT();
+  if (!e) return fail(CSK_ERR_ARG, "null event");
+  HIP_TRY(hipEventRecord(e->ev, g_stream));
+  return CSK_OK;
+}
+extern "C" int csk_event_elapsed_ms(csk_event* a, csk_event* b, float* ms) {
+  REQUIRE_INIT();
+  if (!a || !b || !ms) return fail(CSK_ERR_ARG, "null event");
+  HIP_TRY(hipEventSynchronize(b->ev));
+  HIP_TRY(hipEventElapsedTime(ms, a->ev, b->ev));
+  return CSK_OK;
+}
+
+// ============================================================ MXFP4 matrices
+
+extern "C" int csk_mxfp4_upload(const uint8_t* blocks, int64_t rows, int64_t K, csk_mxfp4** out) {
+  REQUIRE_INIT();
+  if (!blocks || !out || rows <= 0 || K <= 0 || K % 32)
+    return fail(CSK_ERR_ARG, "csk_mxfp4_upload: need rows > 0 and K a positive multiple of 32");
+  csk_mxfp4* m = new csk_mxfp4;
+  m->rows = rows;
+  m->K = K;
+  m->nblk = K / 32;
+  m->ntile = cdiv(rows, 16);
+  int rc = dev_alloc(&m->q, (size_t)m->entries());
+  if (rc == CSK_OK) rc = dev_alloc(&m->s, (size_t)m->entries());
+  if (rc == CSK_OK) rc = pack_into(blocks, *m);
+  if (rc != CSK_OK) {
+    csk_mxfp4_free(m);
+    return rc;
+  }
+  *out = m;
+  return CSK_OK;
+}
+extern "C" void csk_mxfp4_free(csk_mxfp4* m) {
+  if (!m) return;
+  if (m->owned) {
+    if (m->q) (void)hipFree(m->q);
+    if (m->s) (void)hipFree(m->s);
+  }
+  delete m;
+}
+extern "C" int csk_mxfp4_dequant(const csk_mxfp4* m, float* host_out) {
+  REQUIRE_INIT();
+  if (!m || !host_out) return fail(CSK_ERR_ARG, "csk_mxfp4_dequant: null argument");
+  return dequant_to_host(*m, host_out);
+}
+extern "C" int csk_mxfp4_export(const csk_mxfp4* m, uint8_t* host_out) {
+  REQUIRE_INIT();
+  if (!m || !host_out) return fail(CSK_ERR_ARG, "csk_mxfp4_export: null argument");
+  return export_to_host(*m, host_out);
+}
+
+// ============================================================ layer
+
+extern "C" int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_layer** out) {
+  REQUIRE_INIT();
+  if (!out) return fail(CSK_ERR_ARG, "csk_layer_create: null out");
+  int rc = check_dims(E, k, H, F);
+  if (rc != CSK_OK) return rc;
+  csk_layer* L = new csk_layer;
+  L->E = E, L->k = k, L->H = H, L->F = F;
+  L->nblkH = H / 32, L->nblkF = F / 32, L->ntF = cdiv(F, 16), L->ntH = cdiv(H, 16);
+  L->expert_set.assign((size_t)E, 0);
+  L->expert_bias.assign((size_t)E, 0);
+  L->ew_host.assign((size_t)E, ExpertW{});
+  rc = dev_alloc(&L->gate_w, (size_t)E * H);
+  if (rc == CSK_OK) rc = dev_alloc(&L->gate_b, (size_t)E);
+  if (rc == CSK_OK) rc = dev_alloc(&L->q_all, (size_t)E * L->ent_expert());
+  if (rc == CSK_OK) rc = dev_alloc(&L->s_all, (size_t)E * L->ent_expert());
+  if (rc == CSK_OK) rc = dev_alloc(&L->bias_all, (size_t)E * (2 * F + H));
+  if (rc == CSK_OK) rc = dev_alloc(&L->ew_dev, (size_t)E);
+  if (rc == CSK_OK) rc = dev_alloc(&L->norm_w, (size_t)H);
+  if (rc != CSK_OK) {
+    csk_layer_destroy(L);
+    return rc;
+  }
+  for (int64_t e = 0; e < E; ++e) {
+    ExpertW& w = L->ew_host[(size_t)e];
+    const csk_mxfp4 g = L->view(e, CSK_W_GATE), u = L->view(e, CSK_W_UP), d = L->view(e, CSK_W_DOWN);
+    w.q_gate = g.q, w.s_gate = g.s, w.q_up = u.q, w.s_up = u.s, w.q_down = d.q, w.s_down = d.s;
+    w.b_gate = w.b_up = w.b_down = nullptr;
+  }
+  hipError_t e1 = hipMemcpy(L->ew_dev, L->ew_host.data(), (size_t)E * sizeof(ExpertW), hipMemcpyHostToDevice);
+  if (e1 != hipSuccess) {
+    csk_layer_destroy(L);
+    return fail(CSK_ERR_HIP, std::string("upload expert table: ") + hipGetErrorString(e1));
+  }
+  *out = L;
+  return CSK_OK;
+}
+
+extern "C" void csk_layer_destroy(csk_layer* L) {
+  if (!L) return;
+  if (g_stream) (void)hipStreamSynchronize(g_stream);
+  void* ps[] = {L->gate_w, L->gate_b, L->q_all, L->s_all, L->bias_all, L->ew_dev, L->norm_w};
+  for (void* p : ps)
+    if (p) (void)hipFree(p);
+  delete L;
+}
+
+extern "C" int csk_layer_set_options(csk_layer* L, int sigmoid_gating, int activation,
+                                     int weight_before_ffn) {
+  if (!L) return fail(CSK_ERR_ARG, "null layer");
+  if (activation != CSK_ACT_MODIFIED_SWIGLU && activation != CSK_ACT_STANDARD_SWIGLU)
+    return fail(CSK_ERR_ARG, "unknown activation type");
+  L->sigmoid = sigmoid_gating != 0;
+  L->act = activation;
+  L->wbf = weight_before_ffn != 0;
+  return CSK_OK;
+}
+
+extern "C" int csk_layer_set_router(csk_layer* L, const float* gate_w, const float* gate_b) {
+  REQUIRE_INIT();
+  if (!L || !gate_w) return fail(CSK_ERR_ARG, "csk_layer_set_router: null argument");
+  HIP_TRY(hipMemcpyAsync(L->gate_w, gate_w, (size_t)L->E * L->H * sizeof(float), hipMemcpyHostToDevice, g_stream));
+  if (gate_b)
+    HIP_TRY(hipMemcpyAsync(L->gate_b, gate_b, (size_t)L->E * sizeof(float), hipMemcpyHostToDevice, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  L->has_gate = true;
+  L->has_gate_b = gate_b != nullptr;
+  return CSK_OK;
+}
+
+static int upload_biases(csk_layer* L, int64_t e, const float* b_up, const float* b_gate,
+                         const float* b_down) {
+  const int nb = (b_up != nullptr) + (b_gate != nullptr) + (b_down != nullptr);
+  if (nb != 0 && nb != 3) return fail(CSK_ERR_ARG, "biases must be all present or all absent");
+  ExpertW& w = L->ew_host[(size_t)e];
+  if (nb == 3) {
+    float* base = L->bias_all + (size_t)e * (2 * L->F + L->H);
+    HIP_TRY(hipMemcpyAsync(base, b_gate, (size_t)L->F * sizeof(float), hipMemcpyHostToDevice, g_stream));
+    HIP_TRY(hipMemcpyAsync(base + L->F, b_up, (size_t)L->F * sizeof(float), hipMemcpyHostToDevice, g_stream));
+    HIP_TRY(hipMemcpyAsync(base + 2 * L->F, b_down, (size_t)L->H * sizeof(float), hipMemcpyHostToDevice, g_stream));
+    w.b_gate = base, w.b_up = base + L->F, w.b_down = base + 2 * L->F;
+  } else {
+    w.b_gate = w.b_up = w.b_down = nullptr;
+  }
+  HIP_TRY(hipMemcpyAsync(L->ew_dev + e, &w, sizeof(ExpertW), hipMemcpyHostToDevice, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  L->expert_bias[(size_t)e] = nb == 3;
+  return CSK_OK;
+}
+
+extern "C" int csk_layer_set_expert(csk_layer* L, int64_t e, const uint8_t* w_up,
+                                    const uint8_t* w_gate, const uint8_t* w_down,
+                                    const float* b_up, const float* b_gate, const float* b_down) {
+  REQUIRE_INIT();
+  if (!L || e < 0 || e >= L->E) return fail(CSK_ERR_RANGE, "csk_layer_set_expert: expert index out of range");
+  if ((w_up == nullptr) != (w_gate == nullptr) || (w_up == nullptr) != (w_down == nullptr))
+    return fail(CSK_ERR_ARG, "weights must be all present or all absent");
+  if (w_up) {
+    const uint8_t* src[3] = {w_up, w_gate, w_down};
+    const int which[3] = {CSK_W_UP, CSK_W_GATE, CSK_W_DOWN};
+    for (int i = 0; i < 3; ++i) {
+      csk_mxfp4 m = L->view(e, which[i]);
+      int rc = pack_into(src[i], m);
+      if (rc != CSK_OK) return rc;
+    }
+    L->expert_set[(size_t)e] = 1;
+  }
+  return upload_biases(L, e, b_up, b_gate, b_down);
+}
+
+extern "C" int csk_layer_set_norm(csk_layer* L, const float* weight, float eps) {
+  REQUIRE_INIT();
+  if (!L || !weight) return fail(CSK_ERR_ARG, "csk_layer_set_norm: null argument");
+  HIP_TRY(hipMemcpyAsync(L->norm_w, weight, (size_t)L->H * sizeof(float), hipMemcpyHostToDevice, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  L->eps = eps;
+  L->has_norm = true;
+  return CSK_OK;
+}
+
+extern "C" int csk_layer_fill_synthetic(csk_layer* L, uint64_t seed, int64_t layer_index,
+                                        int scale_lo, int scale_span) {
+  REQUIRE_INIT();
+  if (!L) return fail(CSK_ERR_ARG, "null layer");
+  if (scale_lo < 2 || scale_span < 1 || scale_lo + scale_span - 1 > 254)
+    return fail(CSK_ERR_SCALE, "synthetic scale bytes must stay within 2..254");
+  for (int64_t e = 0; e < L->E; ++e) {
+    for (int which = 0; which < 3; ++which) {
+      const csk_mxfp4 m = L->view(e, which);
+      // host twin of mix64 (same constants as the device function)
+      auto mix = [](uint64_t z) {
+        z += 0x9E3779B97F4A7C15ull;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+      };
+      const uint64_t key = mix(seed ^ mix((uint64_t)layer_index * 1000003ull + (uint64_t)e * 16ull + (uint64_t)which));
+      const long ent = m.entries();
+      synth_mxfp4_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(
+          m.q, m.s, (int)m.rows, (int)m.nblk, ent, key, scale_lo, scale_span);
+    }
+    L->expert_set[(size_t)e] = 1;
+  }
+  int rc = check_launch("synth_mxfp4_kernel");
+  if (rc != CSK_OK) return rc;
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+extern "C" int csk_layer_dequant(const csk_layer* L, int64_t e, int which, float* host_out) {
+  REQUIRE_INIT();
+  if (!L || !host_out || e < 0 || e >= L->E || which < 0 || which > 2)
+    return fail(CSK_ERR_ARG, "csk_layer_dequant: bad argument");
+  return dequant_to_host(L->view(e, which), host_out);
+}
+extern "C" int csk_layer_export(const csk_layer* L, int64_t e, int which, uint8_t* host_out) {
+  REQUIRE_INIT();
+  if (!L || !host_out || e < 0 || e >= L->E || which < 0 || which > 2)
+    return fail(CSK_ERR_ARG, "csk_layer_export: bad argument");
+  return export_to_host(L->view(e, which), host_out);
+}
+
+static int layer_ready(const csk_layer* L, int flags) {
+  if (!L->has_gate) return fail(CSK_ERR_STATE, "router weights not set");
+  for (char c : L->expert_set)
+    if (!c) return fail(CSK_ERR_STATE, "not every expert has weights");
+  if ((flags & CSK_FWD_RMSNORM) && !L->has_norm) return fail(CSK_ERR_STATE, "RMSNorm weight not set");
+  return CSK_OK;
+}
+
+extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, float* out, int flags) {
+  REQUIRE_INIT();
+  if (!L || !hidden || !out || T < 0) return fail(CSK_ERR_ARG, "csk_moe_forward: bad argument");
+  int rc = layer_ready(L, flags);
+  if (rc != CSK_OK) return rc;
+  L->last_T = T;
+  if (T == 0) return CSK_OK;
+  if (T * L->k > (int64_t)1 << 24) return fail(CSK_ERR_ARG, "T * top_k exceeds 2^24");
+  Workspace& ws = g_ws;
+  rc = ws.ensure(T, L->E, L->k, L->H, L->F, L->wbf);
+  if (rc != CSK_OK) return rc;
+  const int64_t P = T * L->k;
+  const bool norm = (flags & CSK_FWD_RMSNORM) != 0;
+  rc = launch_prep(hidden, norm ? L->norm_w : nullptr, L->eps, norm ? ws.xn : nullptr, ws.xs, T,
+                   L->H, nullptr, nullptr);
+  if (rc != CSK_OK) return rc;
+  const float* xr = norm ? ws.xn : hidden;
+  rc = launch_router(xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, T, L->E, L->H, L->k,
+                     L->sigmoid, ws.logits, ws.pairs, ws.ids);
+  if (rc != CSK_OK) return rc;
+  rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, ws);
+  if (rc != CSK_OK) return rc;
+  const uint16_t* xa = ws.xs;
+  const int* list_row = ws.list_tok;
+  if (L->wbf) {
+    rc = launch_prep(xr, nullptr, 0.f, nullptr, ws.xg, P, L->H, ws.list_tok, ws.list_w);
+    if (rc != CSK_OK) return rc;
+    xa = ws.xg;
+    list_row = nullptr;
+  }
+  rc = run_experts(L->ew_dev, L->E, T, L->k, L->H, L->F, L->act, xa, list_row, ws);
+  if (rc != CSK_OK) return rc;
+  return launch_combine(ws.y, ws.pairs, ws.pos, (flags & CSK_FWD_RESIDUAL) ? hidden : nullptr, out,
+                        T, L->k, L->H, L->wbf);
+}
+
+extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T, float* out,
+                                    float* pairs_out, int flags) {
+  REQUIRE_INIT();
+  if (!L || !hidden || !out || T < 0) return fail(CSK_ERR_ARG, "csk_moe_forward_host: bad argument");
+  if (T == 0) return CSK_OK;
+  float *dh = nullptr, *dout = nullptr;
+  const size_t n = (size_t)T * L->H;
+  HIP_TRY(hipMalloc((void**)&dh, n * sizeof(float)));
+  hipError_t e = hipMalloc((void**)&dout, n * sizeof(float));
+  int rc = CSK_OK;
+  if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("hipMalloc: ") + hipGetErrorString(e));
+  if (rc == CSK_OK) rc = csk_copy_h2d(dh, hidden, n * sizeof(float));
+  if (rc == CSK_OK) rc = csk_moe_forward(L, dh, T, dout, flags);
+  if (rc == CSK_OK) rc = csk_copy_d2h(out, dout, n * sizeof(float));
+  if (rc == CSK_OK && pairs_out)
+    rc = csk_copy_d2h(pairs_out, g_ws.pairs, (size_t)T * L->k * 2 * sizeof(float));
+  (void)hipStreamSynchronize(g_stream);
+  (void)hipFree(dh);
+  if (dout) (void)hipFree(dout);
+  return rc;
+}
+
+extern "C" int csk_moe_stack_forward(csk_layer* const* layers, int64_t n_layers, float* hidden,
+                                     int64_t T) {
+  REQUIRE_INIT();
+  if (!layers || n_layers < 0 || !hidden) return fail(CSK_ERR_ARG, "csk_moe_stack_forward: bad argument");
+  for (int64_t i = 0; i < n_layers; ++i) {
+    int rc = csk_moe_forward(layers[i], hidden, T, hidden, CSK_FWD_RMSNORM | CSK_FWD_RESIDUAL);
+    if (rc != CSK_OK) return rc;
+  }
+  return CSK_OK;
+}
+
+extern "C" int csk_layer_last_dispatch(csk_layer* L, int32_t* counts_host, int32_t* tokens_host) {
+  REQUIRE_INIT();
+  if (!L) return fail(CSK_ERR_ARG, "null layer");
+  if (L->last_T <= 0) return fail(CSK_ERR_STATE, "no forward has run on this layer");
+  if (counts_host) {
+    int rc = csk_copy_d2h(counts_host, g_ws.counts, (size_t)L->E * sizeof(int));
+    if (rc != CSK_OK) return rc;
+  }
+  if (tokens_host) return csk_copy_d2h(tokens_host, g_ws.list_tok, (size_t)L->last_T * L->k * sizeof(int));
+  return CSK_OK;
+}
+
+// ============================================================ node-level ops
+
+namespace {
+// Scoped device buffer for the host-pointer entry points.
+struct DevBuf {
+  void* p = nullptr;
+  ~DevBuf() {
+    if (p) (void)hipFree(p);
+  }
+  int alloc(size_t bytes) {
+    HIP_TRY(hipMalloc(&p, bytes ? bytes : 1));
+    return CSK_OK;
+  }
+  int upload(const void* host, size_t bytes) {
+    int rc = alloc(bytes);
+    if (rc != CSK_OK) return rc;
+    HIP_TRY(hipMemcpyAsync(p, host, bytes, hipMemcpyHostToDevice, g_stream));
+    return CSK_OK;
+  }
+  template <class T>
+  T* as() {
+    return reinterpret_cast<T*>(p);
+  }
+};
+}  // namespace
+
+extern "C" int csk_moe_router(const float* hidden, int64_t T, int64_t H, const float* gate_w,
+                              int64_t E, const float* gate_b, int64_t k, int sigmoid,
+                              float* out_pairs) {
+  REQUIRE_INIT();
+  if (!hidden || !gate_w || !out_pairs || T < 0) return fail(CSK_ERR_ARG, "csk_moe_router: null argument");
+  if (E <= 0 || E > kMaxExperts || k <= 0 || k > kMaxTopK || k > E || H <= 0 || H % 4)
+    return fail(CSK_ERR_ARG, "csk_moe_router: need 1 <= top_k <= min(16, E), E <= 256, H a multiple of 4");
+  if (T == 0) return CSK_OK;
+  DevBuf dx, dg, db, dl, dp, di;
+  int rc;
+  if ((rc = dx.upload(hidden, (size_t)T * H * 4)) != CSK_OK) return rc;
+  if ((rc = dg.upload(gate_w, (size_t)E * H * 4)) != CSK_OK) return rc;
+  if (gate_b && (rc = db.upload(gate_b, (size_t)E * 4)) != CSK_OK) return rc;
+  if ((rc = dl.alloc((size_t)T * E * 4)) != CSK_OK) return rc;
+  if ((rc = dp.alloc((size_t)T * k * 8)) != CSK_OK) return rc;
+  if ((rc = di.alloc((size_t)T * k * 4)) != CSK_OK) return rc;
+  rc = launch_router(dx.as<float>(), dg.as<float>(), gate_b ? db.as<float>() : nullptr, T, E, H, k,
+                     sigmoid, dl.as<float>(), dp.as<float>(), di.as<int>());
+  if (rc != CSK_OK) return rc;
+  HIP_TRY(hipMemcpyAsync(out_pairs, dp.p, (size_t)T * k * 8, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+namespace {
+__global__ void select_expert_ids_kernel(const float* __restrict__ pairs, int* __restrict__ ids,
+                                         int P, int expert_id) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p < P) ids[p] = ((int)pairs[2 * (size_t)p] == expert_id) ? 0 : -1;
+}
+}  // namespace
+
+extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t T, int64_t H,
+                                    int64_t F, const csk_mxfp4* w_up, const csk_mxfp4* w_gate,
+                                    const csk_mxfp4* w_down, const float* b_up,
+                                    const float* b_gate, const float* b_down, const float* pairs,
+                                    int64_t k, int activation, int weight_before_ffn, float* out,
+                                    int* is_empty) {
+  REQUIRE_INIT();
+  if (!hidden || !w_up || !w_gate || !w_down || !pairs || !out || !is_empty || T < 0)
+    return fail(CSK_ERR_ARG, "csk_expert_mlp_mxfp4: null argument");
+  // router scan happens before the shape checks (expert_mlp_node.h:441-443)
+  bool any = false;
+  for (int64_t p = 0; p < T * k && !any; ++p) any = (int)pairs[2 * p] == expert_id;
+  *is_empty = !any;
+  if (!any) return CSK_OK;
+  if (w_up->rows != F || w_up->K != H || w_gate->rows != F || w_gate->K != H || w_down->rows != H ||
+      w_down->K != F)
+    return fail(CSK_ERR_ARG, "expert_mlp: weight dimension mismatch");
+  if (H % 32) return fail(CSK_ERR_ARG, "expert_mlp: hidden_dim must be a multiple of 32 for MXFP4, got " + std::to_string(H));
+  if (F % 32) return fail(CSK_ERR_ARG, "expert_mlp: expert_ffn_dim must be a multiple of 32 for MXFP4, got " + std::to_string(F));
+  if (k <= 0 || k > kMaxTopK) return fail(CSK_ERR_ARG, "expert_mlp: top_k must be in 1..16");
+  const int nb = (b_up != nullptr) + (b_gate != nullptr) + (b_down != nullptr);
+  if (nb != 0 && nb != 3) return fail(CSK_ERR_ARG, "expert_mlp: biases must be all present or all absent");
+  Workspace& ws = g_ws;
+  int rc = ws.ensure(T, 1, k, H, F, weight_before_ffn != 0);
+  if (rc != CSK_OK) return rc;
+  const int64_t P = T * k;
+  DevBuf dx, dpairs, dbu, dbg, dbd, dew, dout;
+  if ((rc = dx.upload(hidden, (size_t)T * H * 4)) != CSK_OK) return rc;
+  if ((rc = dpairs.upload(pairs, (size_t)P * 8)) != CSK_OK) return rc;
+  if (nb == 3) {
+    if ((rc = dbu.upload(b_up, (size_t)F * 4)) != CSK_OK) return rc;
+    if ((rc = dbg.upload(b_gate, (size_t)F * 4)) != CSK_OK) return rc;
+    if ((rc = dbd.upload(b_down, (size_t)H * 4)) != CSK_OK) return rc;
+  }
+  ExpertW w{};
+  w.q_gate = w_gate->q, w.s_gate = w_gate->s, w.q_up = w_up->q, w.s_up = w_up->s;
+  w.q_down = w_down->q, w.s_down = w_down->s;
+  w.b_gate = nb ? dbg.as<float>() : nullptr;
+  w.b_up = nb ? dbu.as<float>() : nullptr;
+  w.b_down = nb ? dbd.as<float>() : nullptr;
+  if ((rc = dew.upload(&w, sizeof w)) != CSK_OK) return rc;
+  if ((rc = dout.alloc((size_t)T * H * 4)) != CSK_OK) return rc;
+  select_expert_ids_kernel<<<dim3((unsigned)cdiv(P, 256)), 256, 0, g_stream>>>(
+      dpairs.as<float>(), ws.ids, (int)P, expert_id);
+  if ((rc = check_launch("select_expert_ids_kernel")) != CSK_OK) return rc;
+  HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
+  HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
+  if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, ws)) != CSK_OK) return rc;
+  const uint16_t* xa;
+  const int* list_row;
+  if (weight_before_ffn) {
+    // The expert's token count is only known on the device, and at most T
+    // tokens can select it: gather T rows.  Positions past the count read the
+    // zeroed tail of the lists (token 0, weight 0) and are never consumed.
+    rc = launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xg, T, H, ws.list_tok, ws.list_w);
+    if (rc != CSK_OK) return rc;
+    xa = ws.xg;
+    list_row = nullptr;
+  } else {
+    rc = launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xs, T, H, nullptr, nullptr);
+    if (rc != CSK_OK) return rc;
+    xa = ws.xs;
+    list_row = ws.list_tok;
+  }
+  rc = run_experts(dew.as<ExpertW>(), 1, T, k, H, F, activation, xa, list_row, ws);
+  if (rc != CSK_OK) return rc;
+  expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)T), 256, 0, g_stream>>>(
+      ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
+  if ((rc = check_launch("expand_expert_rows_kernel")) != CSK_OK) return rc;
+  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+extern "C" int csk_expert_token_mxfp4(const float* x, const uint8_t* w_up, const uint8_t* w_gate,
+                                      const uint8_t* w_down, const float* b_up,
+                                      const float* b_gate, const float* b_down, float* out,
+                                      int64_t H, int64_t F, int activation) {
+  REQUIRE_INIT();
+  if (!x || !w_up || !w_gate || !w_down || !out) return fail(CSK_ERR_ARG, "csk_expert_token_mxfp4: null argument");
+  if (H <= 0 || F <= 0 || H % 32 || F % 32)
+    return fail(CSK_ERR_ARG, "compute_token_mxfp4: hidden_dim and expert_ffn_dim must be multiples of 32");
+  csk_mxfp4 *mu = nullptr, *mg = nullptr, *md = nullptr;
+  int rc = csk_mxfp4_upload(w_up, F, H, &mu);
+  if (rc == CSK_OK) rc = csk_mxfp4_upload(w_gate, F, H, &mg);
+  if (rc == CSK_OK) rc = csk_mxfp4_upload(w_down, H, F, &md);
+  if (rc == CSK_OK) {
+    const float pairs[2] = {0.0f, 1.0f};
+    int empty = 0;
+    rc = csk_expert_mlp_mxfp4(0, x, 1, H, F, mu, mg, md, b_up, b_gate, b_down, pairs, 1, activation,
+                              0, out, &empty);
+  }
+  csk_mxfp4_free(mu);
+  csk_mxfp4_free(mg);
+  csk_mxfp4_free(md);
+  return rc;
+}
+
+extern "C" int csk_expert_merge(const float* pairs, int64_t T, int64_t k, int64_t E, int64_t H,
+                                const float* const* expert_outs, int pre_weighted, float* out) {
+  REQUIRE_INIT();
+  if (!pairs || !expert_outs || !out || T < 0 || k <= 0 || E <= 0 || H <= 0)
+    return fail(CSK_ERR_ARG, "csk_expert_merge: bad argument");
+  bool any = false;
+  for (int64_t e = 0; e < E; ++e) any |= expert_outs[e] != nullptr;
+  if (!any) return fail(CSK_ERR_ALL_EMPTY, "expert_merge: no non-empty expert outputs found");
+  if (T == 0) return CSK_OK;
+  const int64_t P = T * k;
+  // Gather the k rows each token needs; an empty expert contributes nothing.
+  std::vector<float> rows((size_t)P * H, 0.0f);
+  std::vector<int> pos((size_t)P);
+  for (int64_t p = 0; p < P; ++p) {
+    const int e = (int)pairs[2 * p];
+    if (e < 0 || e >= E) return fail(CSK_ERR_RANGE, "expert_merge: expert_idx out of range: " + std::to_string(e));
+    const float* src = expert_outs[e];
+    pos[(size_t)p] = src ? (int)p : -1;
+    if (src) std::memcpy(&rows[(size_t)p * H], src + (p / k) * H, (size_t)H * sizeof(float));
+  }
+  DevBuf dy, dpairs, dpos, dout;
+  int rc;
+  if ((rc = dy.upload(rows.data(), rows.size() * 4)) != CSK_OK) return rc;
+  if ((rc = dpairs.upload(pairs, (size_t)P * 8)) != CSK_OK) return rc;
+  if ((rc = dpos.upload(pos.data(), pos.size() * 4)) != CSK_OK) return rc;
+  if ((rc = dout.alloc((size_t)T * H * 4)) != CSK_OK) return rc;
+  rc = launch_combine(dy.as<float>(), dpairs.as<float>(), dpos.as<int>(), nullptr, dout.as<float>(),
+                      T, k, H, pre_weighted);
+  if (rc != CSK_OK) return rc;
+  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+namespace {
+__global__ void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                           float* __restrict__ o, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) o[i] = a[i] + b[i];
+}
+}  // namespace
+
+extern "C" int csk_rmsnorm(const float* x, const float* weight, float* out, int64_t T, int64_t H,
+                           float eps) {
+  REQUIRE_INIT();
+  if (!x || !weight || !out || T < 0 || H <= 0) return fail(CSK_ERR_ARG, "csk_rmsnorm: bad argument");
+  if (T == 0) return CSK_OK;
+  DevBuf dx, dw, dout;
+  int rc;
+  if ((rc = dx.upload(x, (size_t)T * H * 4)) != CSK_OK) return rc;
+  if ((rc = dw.upload(weight, (size_t)H * 4)) != CSK_OK) return rc;
+  if ((rc = dout.alloc((size_t)T * H * 4)) != CSK_OK) return rc;
+  rc = launch_prep(dx.as<float>(), dw.as<float>(), eps, dout.as<float>(), nullptr, T, H, nullptr, nullptr);
+  if (rc != CSK_OK) return rc;
+  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+extern "C" int csk_add(const float* a, const float* b, float* out, int64_t n) {
+  REQUIRE_INIT();
+  if (!a || !b || !out || n < 0) return fail(CSK_ERR_ARG, "csk_add: bad argument");
+  if (n == 0) return CSK_OK;
+  DevBuf da, db, dout;
+  int rc;
+  if ((rc = da.upload(a, (size_t)n * 4)) != CSK_OK) return rc;
+  if ((rc = db.upload(b, (size_t)n * 4)) != CSK_OK) return rc;
+  if ((rc = dout.alloc((size_t)n * 4)) != CSK_OK) return rc;
+  add_kernel<<<dim3((unsigned)cdiv(n, 256)), 256, 0, g_stream>>>(da.as<float>(), db.as<float>(), dout.as<float>(), n);
+  if ((rc = check_launch("add_kernel")) != CSK_OK) return rc;
+  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)n * 4, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}

@@ -1,0 +1,70 @@
+// Shared device/host declarations for the gfx950 MoE kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace csk {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+
+constexpr int kWave = 64;
+constexpr int kTileRows = 16;   // weight rows per packed tile (= MFMA N)
+constexpr int kBlk = 32;        // MXFP4 block length along K
+constexpr int kMaxTopK = 16;
+constexpr int kMaxExperts = 256;
+
+// Resident weights of one expert.  Each matrix [rows, K] is stored as
+//   q: [rows/16][K/32][16] x 16 bytes -- byte b of an entry holds elements
+//      2b (low nibble) and 2b+1 (high nibble) of one 32-element block, which
+//      is the order v_cvt_scalef32_pk_*_fp4 consumes;
+//   s: [rows/16][K/32][16] scale bytes (E8M0).
+// A wave reading entries [kb..kb+3][0..15] of one tile fetches 1 KiB of
+// contiguous nibbles; lane (g = lane/16, n = lane%16) owns block kb+g of row n.
+struct ExpertW {
+  const uint4* q_gate;
+  const uint8_t* s_gate;
+  const uint4* q_up;
+  const uint8_t* s_up;
+  const uint4* q_down;
+  const uint8_t* s_down;
+  const float* b_gate;  // may be null
+  const float* b_up;
+  const float* b_down;
+};
+
+// E8M0 byte -> scale of true E2M1 values, 2^(b-127); exact for b in 1..254.
+__device__ __forceinline__ float e8m0_scale(uint32_t b) { return __uint_as_float(b << 23); }
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t h) { return __uint_as_float(h << 16); }
+
+// Round-to-nearest-even fp32 -> bf16 bit pattern (finite inputs).
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float x) {
+  uint32_t u = __float_as_uint(x);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+// x = hi + lo + O(2^-17 |x|): two bf16 terms carry 16 mantissa bits.
+__device__ __forceinline__ void split_bf16(float x, uint16_t& hi, uint16_t& lo) {
+  const uint32_t h = float_to_bf16_bits(x);
+  hi = (uint16_t)h;
+  lo = (uint16_t)float_to_bf16_bits(x - bf16_bits_to_float(h));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+}  // namespace csk

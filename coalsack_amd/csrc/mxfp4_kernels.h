@@ -1,0 +1,145 @@
+// MXFP4 storage kernels: repack the reference's 17-byte blocks into the tiled
+// device layout, the inverse, device-side dequantisation, and the synthetic
+// weight generator.  All are one thread per (tile, block, row-in-tile) entry of
+// the packed layout, so packed-side accesses are fully coalesced.
+#pragma once
+#include "common.h"
+
+namespace csk {
+
+// Reference block (include/coalsack/gguf/gguf_dequant.h:437-455): byte 0 scale,
+// byte 1+j = element j (low nibble) | element j+16 (high nibble).
+// Packed entry: byte b = element 2b (low) | element 2b+1 (high).
+__device__ __forceinline__ uint4 ref_block_to_entry(const uint8_t* blk) {
+  uint32_t w[4];
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    uint32_t v = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int b = d * 4 + c;  // packed byte index, elements 2b and 2b+1
+      uint32_t lo, hi;
+      if (b < 8) {
+        lo = blk[1 + 2 * b] & 15u;
+        hi = blk[2 + 2 * b] & 15u;
+      } else {
+        lo = blk[1 + 2 * b - 16] >> 4;
+        hi = blk[2 + 2 * b - 16] >> 4;
+      }
+      v |= (lo | (hi << 4)) << (8 * c);
+    }
+    w[d] = v;
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+__device__ __forceinline__ void entry_to_ref_block(uint4 q, uint8_t scale, uint8_t* blk) {
+  const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+  uint8_t code[32];
+#pragma unroll
+  for (int b = 0; b < 16; ++b) {
+    const uint32_t byte = (w[b >> 2] >> (8 * (b & 3))) & 0xFFu;
+    code[2 * b] = byte & 15u;
+    code[2 * b + 1] = byte >> 4;
+  }
+  blk[0] = scale;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) blk[1 + j] = (uint8_t)(code[j] | (code[j + 16] << 4));
+}
+
+// entries = ntile * nblk * 16
+__global__ void pack_mxfp4_kernel(const uint8_t* __restrict__ src, uint4* __restrict__ q,
+                                  uint8_t* __restrict__ s, int rows, int nblk, long entries) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= entries) return;
+  const int n = (int)(i & 15);
+  const long tk = i >> 4;
+  const int kb = (int)(tk % nblk);
+  const long row = (tk / nblk) * 16 + n;
+  if (row >= rows) {
+    q[i] = make_uint4(0, 0, 0, 0);
+    s[i] = 127;
+    return;
+  }
+  const uint8_t* blk = src + (row * nblk + kb) * 17;
+  q[i] = ref_block_to_entry(blk);
+  s[i] = blk[0];
+}
+
+__global__ void export_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t* __restrict__ s,
+                                    uint8_t* __restrict__ dst, int rows, int nblk, long entries) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= entries) return;
+  const int n = (int)(i & 15);
+  const long tk = i >> 4;
+  const int kb = (int)(tk % nblk);
+  const long row = (tk / nblk) * 16 + n;
+  if (row >= rows) return;
+  entry_to_ref_block(q[i], s[i], dst + (row * nblk + kb) * 17);
+}
+
+// Dequantise through the same conversion instruction the expert kernels use
+// (v_cvt_scalef32_pk_bf16_fp4), then widen bf16 -> f32, which is exact.
+__global__ void dequant_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t* __restrict__ s,
+                                     float* __restrict__ dst, int rows, int nblk, long entries) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= entries) return;
+  const int n = (int)(i & 15);
+  const long tk = i >> 4;
+  const int kb = (int)(tk % nblk);
+  const long row = (tk / nblk) * 16 + n;
+  if (row >= rows) return;
+  const uint4 e = q[i];
+  const float sc = e8m0_scale(s[i]);
+  const uint32_t w[4] = {e.x, e.y, e.z, e.w};
+  float* o = dst + (row * nblk + kb) * 32;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    bf16x2 r0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], sc, 0);
+    bf16x2 r1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], sc, 1);
+    bf16x2 r2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], sc, 2);
+    bf16x2 r3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], sc, 3);
+    o[d * 8 + 0] = (float)r0[0];
+    o[d * 8 + 1] = (float)r0[1];
+    o[d * 8 + 2] = (float)r1[0];
+    o[d * 8 + 3] = (float)r1[1];
+    o[d * 8 + 4] = (float)r2[0];
+    o[d * 8 + 5] = (float)r2[1];
+    o[d * 8 + 6] = (float)r3[0];
+    o[d * 8 + 7] = (float)r3[1];
+  }
+}
+
+// Synthetic weights, generated straight into the packed layout.  Block b =
+// row * nblk + kb of the stream with key `key` is, in the reference's format,
+//   scale byte = scale_lo + (h0 >> 33) % scale_span,
+//   quant bytes 1..8 = little-endian bytes of h1, 9..16 = those of h2,
+// with h_i = mix64(key + 3 b + i).
+__global__ void synth_mxfp4_kernel(uint4* __restrict__ q, uint8_t* __restrict__ s, int rows,
+                                   int nblk, long entries, uint64_t key, int scale_lo,
+                                   int scale_span) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= entries) return;
+  const int n = (int)(i & 15);
+  const long tk = i >> 4;
+  const int kb = (int)(tk % nblk);
+  const long row = (tk / nblk) * 16 + n;
+  if (row >= rows) {
+    q[i] = make_uint4(0, 0, 0, 0);
+    s[i] = 127;
+    return;
+  }
+  const uint64_t b = (uint64_t)(row * nblk + kb);
+  const uint64_t h0 = mix64(key + 3 * b), h1 = mix64(key + 3 * b + 1), h2 = mix64(key + 3 * b + 2);
+  uint8_t blk[17];
+  blk[0] = (uint8_t)(scale_lo + (int)((h0 >> 33) % (uint64_t)scale_span));
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    blk[1 + j] = (uint8_t)(h1 >> (8 * j));
+    blk[9 + j] = (uint8_t)(h2 >> (8 * j));
+  }
+  q[i] = ref_block_to_entry(blk);
+  s[i] = blk[0];
+}
+
+}  // namespace csk

@@ -1,0 +1,283 @@
+// Prologue (optional RMSNorm + bf16 hi/lo split of the activations), router
+// (gate GEMV, wavefront top-k, softmax over the selected k), dispatch
+// (histogram -> prefix scan -> ordered scatter) and the weighted combine.
+#pragma once
+#include "common.h"
+
+namespace csk {
+
+// ---------------------------------------------------------------- prologue
+// One workgroup per row.  Optionally applies RMSNorm
+// (include/coalsack/nn/nn_ops/rmsnorm_node.h:62-83: rms = sqrt(sum x^2 / H +
+// eps), out = (x / rms) * w) and writes the result as f32 (xn, may be null)
+// and as two bf16 terms in the layout the expert kernels read:
+//   xs[row][kb][0..31] = hi, xs[row][kb][32..63] = lo   (kb = 32-element block)
+// With gather != null the rows are gathered and pre-scaled per packed dispatch
+// position (weight_before_ffn, expert_mlp_node.h:515-522):
+//   row p <- src[gather_tok[p]] * gather_w[p].
+__global__ __launch_bounds__(256) void prep_kernel(const float* __restrict__ src,
+                                                   const float* __restrict__ norm_w, float eps,
+                                                   float* __restrict__ xn,
+                                                   uint16_t* __restrict__ xs, int H,
+                                                   const int* __restrict__ gather_tok,
+                                                   const float* __restrict__ gather_w) {
+  const int row = blockIdx.x;
+  const int srow = gather_tok ? gather_tok[row] : row;
+  const float* x = src + (size_t)srow * H;
+  const float gw = gather_w ? gather_w[row] : 1.0f;
+  float inv_den = 0.0f;
+  if (norm_w) {
+    float ss = 0.0f;
+    for (int d = threadIdx.x; d < H; d += 256) ss += x[d] * x[d];
+    ss = wave_sum(ss);
+    __shared__ float part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = (part[0] + part[1]) + (part[2] + part[3]);
+    inv_den = sqrtf(ss / (float)H + eps);
+  }
+  for (int d = threadIdx.x; d < H; d += 256) {
+    float v = x[d];
+    if (norm_w) v = (v / inv_den) * norm_w[d];
+    if (xn) xn[(size_t)row * H + d] = v;
+    if (gather_w) v = v * gw;
+    uint16_t hi, lo;
+    split_bf16(v, hi, lo);
+    uint16_t* o = xs + ((size_t)row * (H / 32) + (d >> 5)) * 64 + (d & 31);
+    o[0] = hi;
+    o[32] = lo;
+  }
+}
+
+// ------------------------------------------------------------ router logits
+// logits[t][e] = sum_d x[t][d] * g[e][d] + b[e]
+// (include/coalsack/nn/nn_ops/moe_router_node.h:161-167).  One wave per
+// (TT tokens, one expert): the gate row is read once per wave with 128-bit
+// loads and reused for TT tokens; lanes own strided float4 chunks and the
+// partial sums meet in a butterfly reduction.
+template <int TT>
+__global__ __launch_bounds__(256) void router_logits_kernel(const float* __restrict__ x,
+                                                            const float* __restrict__ g,
+                                                            const float* __restrict__ b,
+                                                            float* __restrict__ logits, int T,
+                                                            int E, int H) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int t0 = blockIdx.y * TT;
+  if (e >= E) return;
+  const int H4 = H >> 2;
+  const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)e * H);
+  float acc[TT];
+#pragma unroll
+  for (int i = 0; i < TT; ++i) acc[i] = 0.0f;
+  for (int c = lane; c < H4; c += 64) {
+    const float4 gv = g4[c];
+#pragma unroll
+    for (int i = 0; i < TT; ++i) {
+      if (t0 + i < T) {
+        const float4 xv = reinterpret_cast<const float4*>(x + (size_t)(t0 + i) * H)[c];
+        acc[i] += xv.x * gv.x + xv.y * gv.y + xv.z * gv.z + xv.w * gv.w;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TT; ++i) {
+    const float s = wave_sum(acc[i]);
+    if (lane == 0 && t0 + i < T) logits[(size_t)(t0 + i) * E + e] = s + (b ? b[e] : 0.0f);
+  }
+}
+
+// ------------------------------------------------------------------- top-k
+// One wave per token.  Lane l holds the logits of experts l, l+64, l+128,
+// l+192; each of the k rounds finds the wave-wide maximum (ties -> lowest
+// expert index) with a butterfly over (value, index) and retires it.  Weights
+// follow moe_router_node.h:180-202: sigmoid of the raw logit, or softmax over
+// the selected k with max subtraction, sum in slot order, multiply by 1/sum.
+__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits,
+                                                          float* __restrict__ pairs,
+                                                          int* __restrict__ ids, int T, int E,
+                                                          int k, int sigmoid) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  const float NEG = -__builtin_inff();
+  float v[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = lane + 64 * j;
+    v[j] = (e < E) ? logits[(size_t)t * E + e] : NEG;
+  }
+  float my_val = 0.0f;  // lane s keeps slot s
+  int my_idx = 0;
+  float vmax = 0.0f;
+  for (int s = 0; s < k; ++s) {
+    float bv = v[0];
+    int bi = lane;
+#pragma unroll
+    for (int j = 1; j < 4; ++j) {
+      if (v[j] > bv) {
+        bv = v[j];
+        bi = lane + 64 * j;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    if (s == 0) vmax = bv;
+    if (lane == s) {
+      my_val = bv;
+      my_idx = bi;
+    }
+    if ((bi & 63) == lane) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if ((bi >> 6) == j) v[j] = NEG;
+    }
+  }
+  float w;
+  if (sigmoid) {
+    w = 1.0f / (1.0f + expf(-my_val));
+  } else {
+    w = (lane < k) ? expf(my_val - vmax) : 0.0f;
+    float sum = 0.0f;
+    for (int s = 0; s < k; ++s) sum += __shfl(w, s, 64);  // slot order
+    const float inv = (sum > 0.0f) ? (1.0f / sum) : 0.0f;
+    w *= inv;
+  }
+  if (lane < k) {
+    float2* o = reinterpret_cast<float2*>(pairs) + (size_t)t * k + lane;
+    *o = make_float2((float)my_idx, w);
+    ids[(size_t)t * k + lane] = my_idx;
+  }
+}
+
+// Expert ids from an existing router output (node-level expert / merge calls):
+// static_cast<int>(float) as expert_mlp_node.h:788 does.
+__global__ void pairs_to_ids_kernel(const float* __restrict__ pairs, int* __restrict__ ids, int P) {
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p < P) ids[p] = (int)pairs[2 * (size_t)p];
+}
+
+// ----------------------------------------------------------------- dispatch
+// Step 1, histogram: workgroup e counts the assignments that name expert e.
+__global__ __launch_bounds__(256) void dispatch_count_kernel(const int* __restrict__ ids, int P,
+                                                             int* __restrict__ counts) {
+  const int e = blockIdx.x;
+  int c = 0;
+  for (int p = threadIdx.x; p < P; p += 256) c += (ids[p] == e);
+  c = (int)wave_sum((float)c);  // exact below 2^24
+  __shared__ int part[4];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) counts[e] = part[0] + part[1] + part[2] + part[3];
+}
+
+// Steps 2+3, exclusive scan and ordered scatter: workgroup e derives its
+// offset from the histogram, then walks the assignments in order and writes
+// the ones naming e at offset + rank, so each expert's list is ascending in
+// token index -- the order the reference's per-expert token loop visits them
+// (expert_mlp_node.h:503-529).  Workgroup 0 also publishes offsets[0..E] and
+// the compact list of experts with at least one token
+// (moe_weight_fetch_node.h:31-60).
+__global__ __launch_bounds__(256) void dispatch_scatter_kernel(
+    const int* __restrict__ ids, const float* __restrict__ pairs, int P, int k, int E,
+    const int* __restrict__ counts, int* __restrict__ offsets, int* __restrict__ active,
+    int* __restrict__ n_active, int* __restrict__ list_tok, float* __restrict__ list_w,
+    int* __restrict__ pos_of_slot) {
+  const int e = blockIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  __shared__ int sh[8];
+  int c = (threadIdx.x < e) ? counts[threadIdx.x] : 0;  // E <= 256 = blockDim
+  c = (int)wave_sum((float)c);
+  if (lane == 0) sh[wv] = c;
+  __syncthreads();
+  const int off = sh[0] + sh[1] + sh[2] + sh[3];
+  if (e == 0 && threadIdx.x == 0) {
+    int run = 0, na = 0;
+    for (int i = 0; i < E; ++i) {
+      offsets[i] = run;
+      if (counts[i] > 0) active[na++] = i;
+      run += counts[i];
+    }
+    offsets[E] = run;
+    *n_active = na;
+  }
+  int base = off;
+  for (int p0 = 0; p0 < P; p0 += 256) {
+    const int p = p0 + threadIdx.x;
+    const bool hit = (p < P) && (ids[p] == e);
+    const unsigned long long m = __ballot(hit);
+    const int below = __popcll(m & ((1ull << lane) - 1ull));
+    __syncthreads();
+    if (lane == 0) sh[4 + wv] = __popcll(m);
+    __syncthreads();
+    int woff = 0;
+    for (int i = 0; i < wv; ++i) woff += sh[4 + i];
+    if (hit) {
+      const int pos = base + woff + below;
+      list_tok[pos] = p / k;
+      list_w[pos] = pairs[2 * (size_t)p + 1];
+      pos_of_slot[p] = pos;
+    }
+    base += sh[4] + sh[5] + sh[6] + sh[7];
+  }
+}
+
+// ------------------------------------------------------------------ combine
+// out[t] = sum over slots in router order of w * y[pos(t, slot)]
+// (include/coalsack/nn/nn_ops/expert_merge_node.h:97-128), multiply and add
+// rounded separately as the reference's scalar loop does; no atomics, one
+// thread owns one output element.  residual != null adds the layer input
+// (add_node.h:8-55).
+__global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ y,
+                                                      const float* __restrict__ pairs,
+                                                      const int* __restrict__ pos_of_slot,
+                                                      const float* __restrict__ residual,
+                                                      float* __restrict__ out, int T, int k, int H,
+                                                      int pre_weighted) {
+  const int t = blockIdx.y;
+  const int d = blockIdx.x * 256 + threadIdx.x;
+  if (d >= H) return;
+  float acc = 0.0f;
+  for (int s = 0; s < k; ++s) {
+    const int pos = pos_of_slot[(size_t)t * k + s];
+    if (pos < 0) continue;  // empty expert tensor: skipped (expert_merge_node.h:111-113)
+    const float v = y[(size_t)pos * H + d];
+    if (pre_weighted) {
+      acc = __fadd_rn(acc, v);
+    } else {
+      const float w = pairs[2 * ((size_t)t * k + s) + 1];
+      acc = __fadd_rn(acc, __fmul_rn(w, v));
+    }
+  }
+  if (residual) acc = __fadd_rn(residual[(size_t)t * H + d], acc);
+  out[(size_t)t * H + d] = acc;
+}
+
+// Dense per-expert output of the node-level call (expert_mlp_node.h:503-529):
+// row t = y[pos] if token t selected the expert, else zeros.
+__global__ __launch_bounds__(256) void expand_expert_rows_kernel(const float* __restrict__ y,
+                                                                 const int* __restrict__ ids,
+                                                                 const int* __restrict__ pos_of_slot,
+                                                                 float* __restrict__ out, int k,
+                                                                 int H, int expert_id) {
+  const int t = blockIdx.y;
+  const int d = blockIdx.x * 256 + threadIdx.x;
+  if (d >= H) return;
+  int pos = -1;
+  for (int s = 0; s < k; ++s) {
+    if (ids[(size_t)t * k + s] == expert_id) {
+      pos = pos_of_slot[(size_t)t * k + s];
+      break;  // first matching slot, as is_token_selecting_expert / get_router_weight
+    }
+  }
+  out[(size_t)t * H + d] = (pos >= 0) ? y[(size_t)pos * H + d] : 0.0f;
+}
+
+}  // namespace csk

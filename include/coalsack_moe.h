@@ -1,0 +1,169 @@
+/*
+ * coalsack_moe.h -- C ABI of the MI355X (gfx950) implementation of coalsack's
+ * mixture-of-experts path: router -> dispatch -> MXFP4 expert MLP -> merge.
+ *
+ * Plain C, plain pointers and sizes.  Every function returns CSK_OK or an
+ * error code; csk_last_error() gives the text for the calling thread.  No
+ * exception crosses this boundary.  Citations name the reference interface
+ * each entry point stands in for (paths relative to the reference root).
+ *
+ * Pointer conventions: "host" pointers are ordinary process memory, "device"
+ * pointers come from csk_dev_alloc (or any hipMalloc).  All tensors are
+ * row-major and contiguous, as dynamic_tensor is
+ * (include/coalsack/tensor/dynamic_tensor.h:114-161).
+ */
+#ifndef COALSACK_MOE_H
+#define COALSACK_MOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CSK_OK 0
+#define CSK_ERR_ARG 1          /* bad shape / null pointer / unsupported size   */
+#define CSK_ERR_HIP 2          /* a HIP runtime call failed                      */
+#define CSK_ERR_RANGE 3        /* expert index outside [0, E)                    */
+#define CSK_ERR_ALL_EMPTY 4    /* merge: every expert tensor is empty            */
+#define CSK_ERR_SCALE 5        /* MXFP4 scale byte outside the exact range 2..254 */
+#define CSK_ERR_STATE 6        /* layer not fully populated                      */
+
+/* expert_mlp_node::activation_type (include/coalsack/nn/nn_ops/expert_mlp_node.h:27-30) */
+#define CSK_ACT_MODIFIED_SWIGLU 0
+#define CSK_ACT_STANDARD_SWIGLU 1
+
+/* which matrix of an expert */
+#define CSK_W_UP 0
+#define CSK_W_GATE 1
+#define CSK_W_DOWN 2
+
+/* csk_moe_forward flags */
+#define CSK_FWD_RMSNORM 1  /* RMSNorm (csk_layer_set_norm) in front of router and experts */
+#define CSK_FWD_RESIDUAL 2 /* out = hidden + moe(...)                                      */
+
+typedef struct csk_layer csk_layer;   /* resident weights of one MoE layer */
+typedef struct csk_mxfp4 csk_mxfp4;   /* one resident MXFP4 matrix         */
+
+/* ---- process-wide ------------------------------------------------------ */
+
+/* Select the GPU and create the library's stream.  Must precede everything
+ * else; fails (CSK_ERR_HIP) when no gfx950 device is usable. */
+int csk_init(int device);
+const char* csk_last_error(void);
+/* name (NUL-terminated, cap bytes), compute-unit count, total device memory */
+int csk_device_info(char* name, size_t cap, int* compute_units, size_t* hbm_bytes);
+
+/* Device memory and timing for hosts with no HIP binding of their own. */
+void* csk_dev_alloc(size_t bytes);
+void csk_dev_free(void* p);
+int csk_copy_h2d(void* dst_device, const void* src_host, size_t bytes);
+int csk_copy_d2h(void* dst_host, const void* src_device, size_t bytes);
+int csk_synchronize(void);
+typedef struct csk_event csk_event;
+csk_event* csk_event_create(void);
+void csk_event_destroy(csk_event* e);
+int csk_event_record(csk_event* e);                 /* on the library's stream */
+int csk_event_elapsed_ms(csk_event* a, csk_event* b, float* ms); /* waits for b */
+
+/* ---- resident MXFP4 matrices ------------------------------------------- */
+
+/* Take a [rows, K] matrix in the reference's storage format -- rows of K/32
+ * consecutive 17-byte blocks, scale byte first, byte j carrying element j in
+ * the low nibble and element j+16 in the high nibble
+ * (include/coalsack/tensor/dynamic_mx_tensor.h:19-45,
+ *  include/coalsack/gguf/gguf_dequant.h:437-455) -- and keep a repacked copy in
+ * HBM.  Replaces what moe_weight_provider::get returns for one expert tensor
+ * (src/llm/moe_weight_provider.cpp:160-188).  K % 32 == 0. */
+int csk_mxfp4_upload(const uint8_t* blocks17_host, int64_t rows, int64_t K, csk_mxfp4** out);
+void csk_mxfp4_free(csk_mxfp4* m);
+/* Dequantise the resident copy on the GPU into host_out[rows*K]; bit-identical
+ * to dequantize_block_mxfp4 (gguf_dequant.h:437-455) for scale bytes 2..254. */
+int csk_mxfp4_dequant(const csk_mxfp4* m, float* host_out);
+/* Recover the 17-byte blocks from the resident copy (round-trip check). */
+int csk_mxfp4_export(const csk_mxfp4* m, uint8_t* blocks17_host);
+
+/* ---- one MoE layer, weights resident ------------------------------------ */
+
+/* E experts, top-k, hidden size H, expert intermediate size F.  H and F must
+ * be multiples of 32 (expert_mlp_node.h:463-472). */
+int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_layer** out);
+void csk_layer_destroy(csk_layer* L);
+/* moe_router_node::set_sigmoid_gating (moe_router_node.h:34),
+ * expert_mlp_node::set_activation_type / set_weight_before_ffn
+ * (expert_mlp_node.h:47-52), expert_merge_node::set_weight_before_ffn
+ * (expert_merge_node.h:24). */
+int csk_layer_set_options(csk_layer* L, int sigmoid_gating, int activation, int weight_before_ffn);
+/* gate_w [E,H] f32, gate_b [E] f32 or NULL (moe_router_node.h:51-124 inputs 1,2) */
+int csk_layer_set_router(csk_layer* L, const float* gate_w_host, const float* gate_b_host);
+/* One expert's tensors as moe_weight_fetch_node hands them to expert e
+ * (moe_weight_fetch_node.h:189-206): w_up/w_gate [F,H], w_down [H,F] in
+ * 17-byte blocks; biases f32 [F],[F],[H] or all NULL. */
+int csk_layer_set_expert(csk_layer* L, int64_t e, const uint8_t* w_up, const uint8_t* w_gate,
+                         const uint8_t* w_down, const float* b_up, const float* b_gate,
+                         const float* b_down);
+/* rmsnorm_node weight [H] and epsilon (rmsnorm_node.h:62-83) */
+int csk_layer_set_norm(csk_layer* L, const float* weight_host, float eps);
+/* Fill every expert's three matrices on the GPU from a counter-based
+ * generator (no host copy): block b of stream (seed, layer_index, expert,
+ * matrix) gets scale byte scale_lo + h0 % scale_span and 16 quant bytes from
+ * h1, h2, with h_i = splitmix64 finaliser of (stream_key + 3 b + i).  A host
+ * can replay any slice.  Biases are left as set (or absent). */
+int csk_layer_fill_synthetic(csk_layer* L, uint64_t seed, int64_t layer_index, int scale_lo,
+                             int scale_span);
+int csk_layer_dequant(const csk_layer* L, int64_t e, int which, float* host_out);
+int csk_layer_export(const csk_layer* L, int64_t e, int which, uint8_t* blocks17_host);
+
+/* Router -> dispatch -> expert MLPs -> merge for T tokens, everything on the
+ * GPU: hidden and out are device pointers [T,H] f32 (out may not alias
+ * hidden).  Stands in for the node chain llm_engine wires per layer
+ * (src/llm/llm_engine.cpp:714-777).  Asynchronous on the library's stream. */
+int csk_moe_forward(csk_layer* L, const float* hidden_device, int64_t T, float* out_device,
+                    int flags);
+/* Same through host buffers; also returns the router output [T,k,2] when
+ * pairs_out is not NULL.  Synchronous. */
+int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T, float* out, float* pairs_out,
+                         int flags);
+/* n layers in sequence, each h <- h + moe(rmsnorm(h)); hidden_device [T,H] is
+ * updated in place. */
+int csk_moe_stack_forward(csk_layer* const* layers, int64_t n_layers, float* hidden_device,
+                          int64_t T);
+/* Intermediate results of the last csk_moe_forward on L, for tests:
+ * per-expert token counts [E] and the packed token list (token ids grouped by
+ * expert, ascending within an expert) [T*k]. */
+int csk_layer_last_dispatch(csk_layer* L, int32_t* counts_host, int32_t* tokens_host);
+
+/* ---- node-level operations through host buffers -------------------------- */
+
+/* moe_router_node::compute (moe_router_node.h:51-214): hidden [T,H], gate_w
+ * [E,H], gate_b [E] or NULL -> out_pairs [T,k,2] = (expert index as float,
+ * weight). */
+int csk_moe_router(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
+                   const float* gate_b, int64_t k, int sigmoid_gating, float* out_pairs);
+/* expert_mlp_node::compute_with_mxfp4 for one expert (expert_mlp_node.h:392-530):
+ * out [T,H]; *is_empty = 1 and out untouched when no token selected expert_id
+ * (:441-443); rows of unselected tokens are zero (:509-512). */
+int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t T, int64_t H, int64_t F,
+                         const csk_mxfp4* w_up, const csk_mxfp4* w_gate, const csk_mxfp4* w_down,
+                         const float* b_up, const float* b_gate, const float* b_down,
+                         const float* router_pairs, int64_t k, int activation,
+                         int weight_before_ffn, float* out, int* is_empty);
+/* expert_mlp_node::compute_test_mxfp4 (expert_mlp_node.h:63-70): one token,
+ * raw 17-byte-block weights in host memory. */
+int csk_expert_token_mxfp4(const float* hidden_vec, const uint8_t* w_up, const uint8_t* w_gate,
+                           const uint8_t* w_down, const float* b_up, const float* b_gate,
+                           const float* b_down, float* out_vec, int64_t H, int64_t F,
+                           int activation);
+/* expert_merge_node::compute (expert_merge_node.h:30-134): expert_outs[e] is a
+ * host [T,H] tensor or NULL for an empty one. */
+int csk_expert_merge(const float* router_pairs, int64_t T, int64_t k, int64_t E, int64_t H,
+                     const float* const* expert_outs, int pre_weighted, float* out);
+/* rmsnorm_node::compute (rmsnorm_node.h:62-83) and add_node (add_node.h:8-55) */
+int csk_rmsnorm(const float* x, const float* weight, float* out, int64_t T, int64_t H, float eps);
+int csk_add(const float* a, const float* b, float* out, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COALSACK_MOE_H */

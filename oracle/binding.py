@@ -1,0 +1,186 @@
+"""ctypes binding of oracle/liboracle.so (and oracle/_ref/libref_mxfp4.so).
+
+TEST INFRASTRUCTURE: imported only by tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+ACT_MODIFIED_SWIGLU, ACT_STANDARD_SWIGLU = 0, 1
+OK, ERR_ARG, ERR_RANGE, ERR_ALL_EMPTY = 0, 1, 2, 3
+_P = C.c_void_p
+_I64 = C.c_int64
+
+
+def build():
+    subprocess.check_call(["make", "-C", _HERE, "all"], stdout=subprocess.DEVNULL)
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    return None if a is None else np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a):
+    return None if a is None else np.ascontiguousarray(a, dtype=np.uint8)
+
+
+class _LayerStruct(C.Structure):
+    _fields_ = [("E", _I64), ("k", _I64), ("H", _I64), ("F", _I64),
+                ("gate_w", _P), ("gate_b", _P), ("w_up", _P), ("w_gate", _P), ("w_down", _P),
+                ("b_up", _P), ("b_gate", _P), ("b_down", _P), ("norm_w", _P),
+                ("norm_eps", C.c_float), ("residual", C.c_int), ("sigmoid", C.c_int),
+                ("act", C.c_int), ("weight_before_ffn", C.c_int)]
+
+
+class Oracle:
+    def __init__(self):
+        path = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(path):
+            build()
+        d = self.dll = C.CDLL(path)
+        d.orc_e8m0_to_fp32_half.restype = C.c_float
+        d.orc_e8m0_to_fp32_half.argtypes = [C.c_uint8]
+        d.orc_dequant_mxfp4.restype = None
+        d.orc_dequant_mxfp4.argtypes = [_P, _P, _I64]
+        d.orc_router.restype = C.c_int
+        d.orc_router.argtypes = [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P]
+        d.orc_router_logits.restype = None
+        d.orc_router_logits.argtypes = [_P, _I64, _I64, _P, _I64, _P, _P]
+        d.orc_expert_token_mxfp4.restype = C.c_int
+        d.orc_expert_token_mxfp4.argtypes = [_P] * 8 + [_I64, _I64, C.c_int]
+        d.orc_expert_mlp_mxfp4.restype = C.c_int
+        d.orc_expert_mlp_mxfp4.argtypes = [C.c_int, _P, _I64, _I64, _I64] + [_P] * 7 + \
+            [_I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]
+        d.orc_expert_merge.restype = C.c_int
+        d.orc_expert_merge.argtypes = [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]
+        d.orc_rmsnorm.restype = None
+        d.orc_rmsnorm.argtypes = [_P, _P, _P, _I64, _I64, C.c_float]
+        d.orc_add.restype = None
+        d.orc_add.argtypes = [_P, _P, _P, _I64]
+        d.orc_moe_layer.restype = C.c_int
+        d.orc_moe_layer.argtypes = [C.POINTER(_LayerStruct), _P, _I64, _P, _P, _I64]
+
+    def e8m0(self, x):
+        return self.dll.orc_e8m0_to_fp32_half(int(x))
+
+    def dequant(self, blocks, k):
+        blocks = _u8(blocks)
+        out = np.empty(k, np.float32)
+        self.dll.orc_dequant_mxfp4(_p(blocks), _p(out), k)
+        return out
+
+    def router(self, hidden, gate_w, gate_b, k, sigmoid=False):
+        hidden, gate_w, gate_b = _f32(hidden), _f32(gate_w), _f32(gate_b)
+        T, H = hidden.shape
+        E = gate_w.shape[0]
+        out = np.empty((T, k, 2), np.float32)
+        rc = self.dll.orc_router(_p(hidden), T, H, _p(gate_w), E, _p(gate_b), k, int(sigmoid), _p(out))
+        if rc:
+            raise ValueError(f"orc_router rc={rc}")
+        return out
+
+    def router_logits(self, hidden, gate_w, gate_b):
+        hidden, gate_w, gate_b = _f32(hidden), _f32(gate_w), _f32(gate_b)
+        T, H = hidden.shape
+        E = gate_w.shape[0]
+        out = np.empty((T, E), np.float32)
+        self.dll.orc_router_logits(_p(hidden), T, H, _p(gate_w), E, _p(gate_b), _p(out))
+        return out
+
+    def expert_token(self, x, w_up, w_gate, w_down, b_up, b_gate, b_down, H, F, act=0):
+        x = _f32(x)
+        w_up, w_gate, w_down = _u8(w_up), _u8(w_gate), _u8(w_down)
+        b_up, b_gate, b_down = _f32(b_up), _f32(b_gate), _f32(b_down)
+        out = np.empty(H, np.float32)
+        rc = self.dll.orc_expert_token_mxfp4(_p(x), _p(w_up), _p(w_gate), _p(w_down), _p(b_up),
+                                             _p(b_gate), _p(b_down), _p(out), H, F, act)
+        if rc:
+            raise ValueError(f"orc_expert_token_mxfp4 rc={rc}")
+        return out
+
+    def expert_mlp(self, expert_id, hidden, F, w_up, w_gate, w_down, b_up, b_gate, b_down, pairs,
+                   act=0, weight_before_ffn=False):
+        hidden, pairs = _f32(hidden), _f32(pairs)
+        w_up, w_gate, w_down = _u8(w_up), _u8(w_gate), _u8(w_down)
+        b_up, b_gate, b_down = _f32(b_up), _f32(b_gate), _f32(b_down)
+        T, H = hidden.shape
+        k = pairs.shape[1]
+        out = np.empty((T, H), np.float32)
+        empty = C.c_int()
+        rc = self.dll.orc_expert_mlp_mxfp4(expert_id, _p(hidden), T, H, F, _p(w_up), _p(w_gate),
+                                           _p(w_down), _p(b_up), _p(b_gate), _p(b_down), _p(pairs),
+                                           k, act, int(weight_before_ffn), _p(out), C.byref(empty))
+        if rc:
+            raise ValueError(f"orc_expert_mlp_mxfp4 rc={rc}")
+        return None if empty.value else out
+
+    def expert_merge(self, pairs, expert_outs, H, pre_weighted=False):
+        pairs = _f32(pairs)
+        T, k = pairs.shape[:2]
+        E = len(expert_outs)
+        keep = [_f32(a) for a in expert_outs]
+        arr = (_P * E)(*[_p(a) for a in keep])
+        out = np.empty((T, H), np.float32)
+        rc = self.dll.orc_expert_merge(_p(pairs), T, k, E, H, arr, int(pre_weighted), _p(out))
+        return rc, out
+
+    def rmsnorm(self, x, w, eps):
+        x, w = _f32(x), _f32(w)
+        T, H = x.shape
+        out = np.empty((T, H), np.float32)
+        self.dll.orc_rmsnorm(_p(x), _p(w), _p(out), T, H, eps)
+        return out
+
+    def add(self, a, b):
+        a, b = _f32(a), _f32(b)
+        out = np.empty(a.shape, np.float32)
+        self.dll.orc_add(_p(a), _p(b), _p(out), a.size)
+        return out
+
+    def moe_layer(self, hidden, E, k, H, F, gate_w, gate_b, w_up, w_gate, w_down, b_up, b_gate,
+                  b_down, norm_w=None, norm_eps=1e-5, residual=False, sigmoid=False, act=0,
+                  weight_before_ffn=False, max_tokens=-1):
+        """w_up/w_gate/w_down: uint8 arrays holding all E experts back to back."""
+        hidden = _f32(hidden)
+        keep = [_f32(gate_w), _f32(gate_b), _u8(w_up), _u8(w_gate), _u8(w_down), _f32(b_up),
+                _f32(b_gate), _f32(b_down), _f32(norm_w)]
+        L = _LayerStruct(E, k, H, F, *[_p(a) for a in keep], norm_eps, int(residual), int(sigmoid),
+                         act, int(weight_before_ffn))
+        T = hidden.shape[0]
+        out = np.zeros((T, H), np.float32)
+        pairs = np.empty((T, k, 2), np.float32)
+        rc = self.dll.orc_moe_layer(C.byref(L), _p(hidden), T, _p(out), _p(pairs), max_tokens)
+        if rc:
+            raise ValueError(f"orc_moe_layer rc={rc}")
+        return out, pairs
+
+
+class RefCodec:
+    """The reference's own MXFP4 codec, when oracle/_ref was built."""
+
+    def __init__(self):
+        path = os.path.join(_HERE, "_ref", "libref_mxfp4.so")
+        if not os.path.exists(path):
+            raise FileNotFoundError(path)
+        d = self.dll = C.CDLL(path)
+        d.ref_e8m0_to_fp32_half.restype = C.c_float
+        d.ref_e8m0_to_fp32_half.argtypes = [C.c_uint8]
+        d.ref_dequantize_block_mxfp4.restype = None
+        d.ref_dequantize_block_mxfp4.argtypes = [_P, _P, _I64]
+
+    def e8m0(self, x):
+        return self.dll.ref_e8m0_to_fp32_half(int(x))
+
+    def dequant(self, blocks, k):
+        blocks = _u8(blocks)
+        out = np.empty(k, np.float32)
+        self.dll.ref_dequantize_block_mxfp4(_p(blocks), _p(out), k)
+        return out

@@ -1,0 +1,490 @@
+/*
+ * CPU restatement of coalsack's mixture-of-experts path (router -> per-expert
+ * MXFP4 MLP -> merge, plus the RMSNorm / residual add that bracket it).
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE.  It is the checker the HIP path is compared
+ * against and the CPU baseline that the benchmark times; nothing the library
+ * ships may call it.
+ *
+ * Every function cites the reference lines it restates (paths relative to the
+ * reference root).  The code is an independent restatement in C, not a copy:
+ * the reference is C++ templates over dynamic_tensor.
+ *
+ * What pins each function (see tests/test_oracle_*.py):
+ *   orc_e8m0_to_fp32_half / orc_dequant_mxfp4
+ *        - the reference's own header compiled as oracle/_ref (bit-exact, all
+ *          256 scale bytes x 16 codes), the reference's known answers
+ *          (test/test_gguf_dequant.cpp:244-279) and the closed form
+ *          lut[c] * 2^(e-128) via ldexp.
+ *   orc_router
+ *        - known answer {5,4,3} (test/test_moe_router.cpp:82-138), invariants
+ *          (:62-78,:178-201), brute-force argsort + float64 softmax on random
+ *          inputs, and the libstdc++ tie order 1,3,0,2 for all-equal logits.
+ *   orc_expert_token_mxfp4 / orc_expert_mlp_mxfp4
+ *        - float64 GEMV over weights dequantised with the pinned codec, the
+ *          activation known answer gate=1, up=1.5
+ *          (test/test_expert_mlp.cpp:37-46,118-200), zero rows / empty result
+ *          for unselected tokens / experts.
+ *          PARITY UNPINNED at the last ulp: the exact fp32 accumulation order
+ *          (lane striding + horizontal-sum tree) can only be pinned by running
+ *          the reference, which cannot be built here without stand-in
+ *          headers.  It does not gate the 1e-3 acceptance bar.
+ *   orc_expert_merge
+ *        - definition sum_k w_k * y_{e_k}; one-hot weights reduce to a copy;
+ *          linearity; error cases.
+ *   orc_rmsnorm / orc_add
+ *        - known answers test/test_rmsnorm.cpp:74-142 and closed form.
+ *
+ * Build: gcc -O2 -shared -fPIC (the reference's Release flags are plain -O2,
+ * CMakeLists.txt:19-21).  No -march: scalar code must not be contracted into
+ * FMAs; only the function carrying target("avx2,fma") uses them, as in the
+ * reference (expert_mlp_node.h:651).
+ */
+#include <immintrin.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_OK 0
+#define ORC_ERR_ARG 1
+#define ORC_ERR_RANGE 2
+#define ORC_ERR_ALL_EMPTY 3
+
+#define ORC_ACT_MODIFIED_SWIGLU 0
+#define ORC_ACT_STANDARD_SWIGLU 1
+
+/* ------------------------------------------------------------------ codec */
+
+/* gguf_dequant.h:413-415 */
+static const int8_t k_lut[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+
+/* gguf_dequant.h:419-433: scale byte -> 2^(x-128); x<2 gives the two fp32
+ * denormals 2^-128, 2^-127. */
+float orc_e8m0_to_fp32_half(uint8_t x) {
+  uint32_t bits;
+  if (x < 2) {
+    bits = 0x00200000u << x;
+  } else {
+    bits = (uint32_t)(x - 1) << 23;
+  }
+  float r;
+  memcpy(&r, &bits, sizeof r);
+  return r;
+}
+
+/* gguf_dequant.h:437-455: block = [scale byte][16 bytes]; byte j carries
+ * element j in its low nibble and element j+16 in its high nibble. */
+void orc_dequant_mxfp4(const uint8_t* src, float* dst, int64_t k) {
+  const int64_t nb = k / 32;
+  for (int64_t i = 0; i < nb; ++i) {
+    const uint8_t* blk = src + i * 17;
+    const float scale = orc_e8m0_to_fp32_half(blk[0]);
+    for (int j = 0; j < 16; ++j) {
+      dst[i * 32 + j] = (float)k_lut[blk[1 + j] & 0x0F] * scale;
+      dst[i * 32 + j + 16] = (float)k_lut[blk[1 + j] >> 4] * scale;
+    }
+  }
+}
+
+/* ----------------------------------------------------------------- router */
+
+typedef struct {
+  float score;
+  int64_t idx;
+} scored_t;
+
+/* comparator of moe_router_node.h:177: a before b iff a.score > b.score */
+static inline int cmp_gt(const scored_t* a, const scored_t* b) { return a->score > b->score; }
+
+/* libstdc++ (GCC 11.4, bits/stl_heap.h) __push_heap / __adjust_heap restated,
+ * so that exact ties come out in the order std::partial_sort leaves them. */
+static void heap_push(scored_t* first, int64_t hole, int64_t top, scored_t value) {
+  int64_t parent = (hole - 1) / 2;
+  while (hole > top && cmp_gt(&first[parent], &value)) {
+    first[hole] = first[parent];
+    hole = parent;
+    parent = (hole - 1) / 2;
+  }
+  first[hole] = value;
+}
+
+static void heap_adjust(scored_t* first, int64_t hole, int64_t len, scored_t value) {
+  const int64_t top = hole;
+  int64_t child = hole;
+  while (child < (len - 1) / 2) {
+    child = 2 * (child + 1);
+    if (cmp_gt(&first[child], &first[child - 1])) child--;
+    first[hole] = first[child];
+    hole = child;
+  }
+  if ((len & 1) == 0 && child == (len - 2) / 2) {
+    child = 2 * (child + 1);
+    first[hole] = first[child - 1];
+    hole = child - 1;
+  }
+  heap_push(first, hole, top, value);
+}
+
+/* std::partial_sort(first, first+mid, first+n, cmp_gt) as libstdc++ does it
+ * (bits/stl_algo.h __heap_select + __sort_heap). */
+static void partial_sort_desc(scored_t* first, int64_t mid, int64_t n) {
+  if (mid >= 2) {
+    int64_t parent = (mid - 2) / 2;
+    for (;;) {
+      scored_t v = first[parent];
+      heap_adjust(first, parent, mid, v);
+      if (parent == 0) break;
+      parent--;
+    }
+  }
+  for (int64_t i = mid; i < n; ++i) {
+    if (mid > 0 && cmp_gt(&first[i], &first[0])) {
+      scored_t v = first[i];
+      first[i] = first[0];
+      heap_adjust(first, 0, mid, v);
+    }
+  }
+  int64_t last = mid;
+  while (last > 1) {
+    --last;
+    scored_t v = first[last];
+    first[last] = first[0];
+    heap_adjust(first, 0, last, v);
+  }
+}
+
+/* moe_router_node.h:141-214.  hidden [T,H] f32, gate_w [E,H] f32, gate_b [E]
+ * or NULL, out [T,k,2] f32 = (expert index as float, weight). */
+int orc_router(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
+               const float* gate_b, int64_t k, int sigmoid, float* out) {
+  if (T < 0 || H <= 0 || E <= 0 || k <= 0 || k > E) return ORC_ERR_ARG;
+  scored_t* sc = (scored_t*)malloc((size_t)E * sizeof(scored_t));
+  float* w = (float*)malloc((size_t)k * sizeof(float));
+  if (!sc || !w) {
+    free(sc);
+    free(w);
+    return ORC_ERR_ARG;
+  }
+  for (int64_t t = 0; t < T; ++t) {
+    const float* x = hidden + t * H;
+    for (int64_t e = 0; e < E; ++e) {
+      /* :161-167 sequential fp32 sum, multiply then add, bias afterwards */
+      float sum = 0.0f;
+      const float* g = gate_w + e * H;
+      for (int64_t d = 0; d < H; ++d) sum += x[d] * g[d];
+      sc[e].score = sum + (gate_b ? gate_b[e] : 0.0f);
+      sc[e].idx = e;
+    }
+    partial_sort_desc(sc, k, E); /* :175-177 */
+    if (sigmoid) {               /* :180-185 */
+      for (int64_t j = 0; j < k; ++j) w[j] = 1.0f / (1.0f + expf(-sc[j].score));
+    } else { /* :186-202 */
+      float mx = sc[0].score;
+      for (int64_t j = 1; j < k; ++j)
+        if (sc[j].score > mx) mx = sc[j].score;
+      float sum = 0.0f;
+      for (int64_t j = 0; j < k; ++j) {
+        w[j] = expf(sc[j].score - mx);
+        sum += w[j];
+      }
+      const float inv = (sum > 0.0f) ? (1.0f / sum) : 0.0f;
+      for (int64_t j = 0; j < k; ++j) w[j] *= inv;
+    }
+    float* o = out + t * k * 2; /* :205-211 */
+    for (int64_t j = 0; j < k; ++j) {
+      o[2 * j + 0] = (float)sc[j].idx;
+      o[2 * j + 1] = w[j];
+    }
+  }
+  free(sc);
+  free(w);
+  return ORC_OK;
+}
+
+/* Raw logits only (:161-167), for tests that classify near-ties. */
+void orc_router_logits(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
+                       const float* gate_b, float* logits) {
+  for (int64_t t = 0; t < T; ++t)
+    for (int64_t e = 0; e < E; ++e) {
+      float sum = 0.0f;
+      for (int64_t d = 0; d < H; ++d) sum += hidden[t * H + d] * gate_w[e * H + d];
+      logits[t * E + e] = sum + (gate_b ? gate_b[e] : 0.0f);
+    }
+}
+
+/* ------------------------------------------------------------- expert MLP */
+
+typedef struct {
+  __m256 v0, v1, v2, v3;
+} blk32_t;
+
+/* expert_mlp_node.h:211-245: one block -> four 8-lane vectors holding
+ * elements 0-7, 8-15, 16-23, 24-31, each multiplied by the block scale. */
+__attribute__((target("avx2"))) static inline blk32_t dequant_block_avx2(const uint8_t* blk) {
+  const __m256 scale = _mm256_set1_ps(orc_e8m0_to_fp32_half(blk[0]));
+  const __m128i lut = _mm_setr_epi8(0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12);
+  const __m128i raw = _mm_loadu_si128((const __m128i*)(blk + 1));
+  const __m128i m = _mm_set1_epi8(0x0F);
+  const __m128i lo = _mm_shuffle_epi8(lut, _mm_and_si128(raw, m));
+  const __m128i hi = _mm_shuffle_epi8(lut, _mm_and_si128(_mm_srli_epi16(raw, 4), m));
+  blk32_t r;
+  r.v0 = _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi8_epi32(lo)), scale);
+  r.v1 = _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi8_epi32(_mm_srli_si128(lo, 8))), scale);
+  r.v2 = _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi8_epi32(hi)), scale);
+  r.v3 = _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi8_epi32(_mm_srli_si128(hi, 8))), scale);
+  return r;
+}
+
+/* expert_mlp_node.h:194-206: ((l0+l4)+(l1+l5)) + ((l2+l6)+(l3+l7)) */
+__attribute__((target("avx2"))) static inline float hsum_avx2(__m256 v) {
+  __m128 s = _mm_add_ps(_mm256_castps256_ps128(v), _mm256_extractf128_ps(v, 1));
+  __m128 sh = _mm_movehdup_ps(s);
+  __m128 t = _mm_add_ps(s, sh);
+  sh = _mm_movehl_ps(sh, t);
+  t = _mm_add_ss(t, sh);
+  return _mm_cvtss_f32(t);
+}
+
+/* expert_mlp_node.h:259-266: four FMAs in order v0..v3 into one accumulator */
+__attribute__((target("avx2,fma"))) static inline __m256 fma_block(__m256 acc, const float* x,
+                                                                   blk32_t w) {
+  acc = _mm256_fmadd_ps(_mm256_loadu_ps(x + 0), w.v0, acc);
+  acc = _mm256_fmadd_ps(_mm256_loadu_ps(x + 8), w.v1, acc);
+  acc = _mm256_fmadd_ps(_mm256_loadu_ps(x + 16), w.v2, acc);
+  acc = _mm256_fmadd_ps(_mm256_loadu_ps(x + 24), w.v3, acc);
+  return acc;
+}
+
+/* expert_mlp_node.h:699-706 */
+static inline float activation(float gate_v, float up_v, int act) {
+  if (act == ORC_ACT_MODIFIED_SWIGLU) {
+    const float limit = 7.0f, alpha = 1.702f;
+    const float x = gate_v < limit ? gate_v : limit;
+    const float y = up_v < -limit ? -limit : (up_v > limit ? limit : up_v);
+    const float glu = x / (1.0f + expf(alpha * (-x)));
+    return glu * (y + 1.0f);
+  }
+  const float silu = gate_v / (1.0f + expf(-gate_v));
+  return silu * up_v;
+}
+
+/* expert_mlp_node.h:651-732: one token through one expert.  Weight rows are
+ * K/32 consecutive 17-byte blocks; w_up/w_gate are [F,H], w_down is [H,F].
+ * scratch holds F floats. */
+__attribute__((target("avx2,fma"))) static int expert_token(
+    const float* x, const uint8_t* w_up, const uint8_t* w_gate, const uint8_t* w_down,
+    const float* b_up, const float* b_gate, const float* b_down, float* out, int64_t H, int64_t F,
+    int act, float* scratch) {
+  if (H % 32 || F % 32 || H <= 0 || F <= 0) return ORC_ERR_ARG;
+  const int64_t nbh = H / 32, nbf = F / 32;
+  for (int64_t r = 0; r < F; ++r) { /* :677-709 (row pairs there; rows are independent) */
+    __m256 au = _mm256_setzero_ps(), ag = _mm256_setzero_ps();
+    for (int64_t b = 0; b < nbh; ++b) {
+      const int64_t off = (r * nbh + b) * 17;
+      au = fma_block(au, x + b * 32, dequant_block_avx2(w_up + off));
+      ag = fma_block(ag, x + b * 32, dequant_block_avx2(w_gate + off));
+    }
+    const float up_v = hsum_avx2(au) + (b_up ? b_up[r] : 0.0f);
+    const float gate_v = hsum_avx2(ag) + (b_gate ? b_gate[r] : 0.0f);
+    scratch[r] = activation(gate_v, up_v, act);
+  }
+  for (int64_t r = 0; r < H; ++r) { /* :712-731 */
+    __m256 a = _mm256_setzero_ps();
+    for (int64_t b = 0; b < nbf; ++b) {
+      a = fma_block(a, scratch + b * 32, dequant_block_avx2(w_down + (r * nbf + b) * 17));
+    }
+    out[r] = hsum_avx2(a) + (b_down ? b_down[r] : 0.0f);
+  }
+  return ORC_OK;
+}
+
+/* expert_mlp_node.h:63-70 (compute_test_mxfp4) */
+int orc_expert_token_mxfp4(const float* x, const uint8_t* w_up, const uint8_t* w_gate,
+                           const uint8_t* w_down, const float* b_up, const float* b_gate,
+                           const float* b_down, float* out, int64_t H, int64_t F, int act) {
+  if (F <= 0) return ORC_ERR_ARG;
+  float* scratch = (float*)malloc((size_t)F * sizeof(float));
+  if (!scratch) return ORC_ERR_ARG;
+  int rc = expert_token(x, w_up, w_gate, w_down, b_up, b_gate, b_down, out, H, F, act, scratch);
+  free(scratch);
+  return rc;
+}
+
+/* expert_mlp_node.h:784-805 */
+static int slot_of_expert(const float* pairs, int64_t t, int64_t k, int expert_id) {
+  for (int64_t j = 0; j < k; ++j)
+    if ((int)pairs[(t * k + j) * 2] == expert_id) return (int)j;
+  return -1;
+}
+
+/* expert_mlp_node.h:392-530: the node body for one expert over T tokens.
+ * out is [T,H]; *is_empty = 1 (and out untouched) when no token selected the
+ * expert (:441-443).  Rows of unselected tokens are zero (:509-512). */
+int orc_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t T, int64_t H, int64_t F,
+                         const uint8_t* w_up, const uint8_t* w_gate, const uint8_t* w_down,
+                         const float* b_up, const float* b_gate, const float* b_down,
+                         const float* pairs, int64_t k, int act, int weight_before_ffn, float* out,
+                         int* is_empty) {
+  int any = 0;
+  for (int64_t t = 0; t < T && !any; ++t) any = slot_of_expert(pairs, t, k, expert_id) >= 0;
+  *is_empty = !any;
+  if (!any) return ORC_OK;
+  if (H % 32 || F % 32) return ORC_ERR_ARG; /* :463-472 */
+  float* scratch = (float*)malloc((size_t)(F + H) * sizeof(float));
+  if (!scratch) return ORC_ERR_ARG;
+  float* scaled = scratch + F;
+  int rc = ORC_OK;
+  for (int64_t t = 0; t < T && rc == ORC_OK; ++t) {
+    const int s = slot_of_expert(pairs, t, k, expert_id);
+    float* o = out + t * H;
+    if (s < 0) {
+      memset(o, 0, (size_t)H * sizeof(float));
+      continue;
+    }
+    const float* x = hidden + t * H;
+    if (weight_before_ffn) { /* :515-522 */
+      const float wt = pairs[(t * k + s) * 2 + 1];
+      for (int64_t d = 0; d < H; ++d) scaled[d] = x[d] * wt;
+      x = scaled;
+    }
+    rc = expert_token(x, w_up, w_gate, w_down, b_up, b_gate, b_down, o, H, F, act, scratch);
+  }
+  free(scratch);
+  return rc;
+}
+
+/* ------------------------------------------------------------------ merge */
+
+/* expert_merge_node.h:30-134.  expert_outs[e] is [T,H] or NULL for an empty
+ * ({0}-shaped) tensor. */
+int orc_expert_merge(const float* pairs, int64_t T, int64_t k, int64_t E, int64_t H,
+                     const float* const* expert_outs, int pre_weighted, float* out) {
+  int any = 0;
+  for (int64_t e = 0; e < E; ++e) any |= expert_outs[e] != NULL;
+  if (!any) return ORC_ERR_ALL_EMPTY; /* :60-62 */
+  memset(out, 0, (size_t)(T * H) * sizeof(float));
+  for (int64_t t = 0; t < T; ++t) {
+    for (int64_t j = 0; j < k; ++j) {
+      const int e = (int)pairs[(t * k + j) * 2];
+      const float w = pairs[(t * k + j) * 2 + 1];
+      if (e < 0 || e >= E) return ORC_ERR_RANGE; /* :102-105 */
+      const float* y = expert_outs[e];
+      if (!y) continue; /* :111-113 */
+      y += t * H;
+      float* o = out + t * H;
+      if (pre_weighted) {
+        for (int64_t d = 0; d < H; ++d) o[d] += y[d];
+      } else {
+        for (int64_t d = 0; d < H; ++d) o[d] += w * y[d];
+      }
+    }
+  }
+  return ORC_OK;
+}
+
+/* ------------------------------------------------------ rmsnorm / add */
+
+/* rmsnorm_node.h:62-83 */
+void orc_rmsnorm(const float* x, const float* w, float* out, int64_t T, int64_t H, float eps) {
+  for (int64_t i = 0; i < T; ++i) {
+    float ss = 0.0f;
+    for (int64_t j = 0; j < H; ++j) {
+      const float v = x[i * H + j];
+      ss += v * v;
+    }
+    const float rms = sqrtf(ss / (float)H + eps);
+    for (int64_t j = 0; j < H; ++j) out[i * H + j] = (x[i * H + j] / rms) * w[j];
+  }
+}
+
+/* add_node.h:8-55 on equal shapes */
+void orc_add(const float* a, const float* b, float* out, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) out[i] = a[i] + b[i];
+}
+
+/* -------------------------------------------------------- composed layer */
+
+/* Weights of one layer in the provider's layout (moe_weight_provider.cpp:
+ * 160-188): per tensor, expert e starts at e * rows * (K/32) * 17 bytes;
+ * biases are [E, rows] f32. */
+typedef struct {
+  int64_t E, k, H, F;
+  const float* gate_w; /* [E,H] */
+  const float* gate_b; /* [E] or NULL */
+  const uint8_t* w_up; /* [E][F][H/32][17] */
+  const uint8_t* w_gate;
+  const uint8_t* w_down; /* [E][H][F/32][17] */
+  const float* b_up;     /* [E,F] or NULL */
+  const float* b_gate;
+  const float* b_down;   /* [E,H] or NULL */
+  const float* norm_w;   /* [H] or NULL: RMSNorm before router and experts */
+  float norm_eps;
+  int residual; /* out = hidden + moe(norm(hidden)) */
+  int sigmoid, act, weight_before_ffn;
+} orc_layer_t;
+
+/* Router -> experts -> merge for one layer (llm_engine.cpp:714-777).  The
+ * reference materialises one dense [T,H] tensor per active expert and sums
+ * them per token in router-slot order; evaluating token by token, slot by
+ * slot, performs the same fp32 operations in the same order without the E
+ * dense tensors.  pairs_out ([T,k,2]) may be NULL.  max_tokens < T limits the
+ * expert work to the first max_tokens tokens (used to time a bounded sample);
+ * the router still runs on all T. */
+int orc_moe_layer(const orc_layer_t* L, const float* hidden, int64_t T, float* out,
+                  float* pairs_out, int64_t max_tokens) {
+  const int64_t H = L->H, F = L->F, k = L->k, E = L->E;
+  float* pairs = (float*)malloc((size_t)(T * k * 2 + 1) * sizeof(float));
+  float* tmp = (float*)malloc((size_t)(2 * H + F) * sizeof(float));
+  float* normed = NULL;
+  if (!pairs || !tmp) return ORC_ERR_ARG;
+  const float* xin = hidden;
+  if (L->norm_w) {
+    normed = (float*)malloc((size_t)(T * H) * sizeof(float));
+    if (!normed) return ORC_ERR_ARG;
+    orc_rmsnorm(hidden, L->norm_w, normed, T, H, L->norm_eps);
+    xin = normed;
+  }
+  int rc = orc_router(xin, T, H, L->gate_w, E, L->gate_b, k, L->sigmoid, pairs);
+  if (pairs_out && rc == ORC_OK) memcpy(pairs_out, pairs, (size_t)(T * k * 2) * sizeof(float));
+  const int64_t nbh = H / 32, nbf = F / 32;
+  float* y = tmp;
+  float* scaled = tmp + H;
+  float* scratch = tmp + 2 * H;
+  const int64_t Tm = (max_tokens >= 0 && max_tokens < T) ? max_tokens : T;
+  for (int64_t t = 0; t < Tm && rc == ORC_OK; ++t) {
+    float* o = out + t * H;
+    memset(o, 0, (size_t)H * sizeof(float));
+    for (int64_t j = 0; j < k && rc == ORC_OK; ++j) {
+      const int e = (int)pairs[(t * k + j) * 2];
+      const float w = pairs[(t * k + j) * 2 + 1];
+      if (e < 0 || e >= E) {
+        rc = ORC_ERR_RANGE;
+        break;
+      }
+      /* a token whose slots name the same expert twice is served by the first
+       * matching slot inside the expert node (:796-805); cannot happen with
+       * top-k over distinct experts */
+      const float* x = xin + t * H;
+      if (L->weight_before_ffn) {
+        for (int64_t d = 0; d < H; ++d) scaled[d] = x[d] * w;
+        x = scaled;
+      }
+      rc = expert_token(x, L->w_up + (size_t)e * F * nbh * 17, L->w_gate + (size_t)e * F * nbh * 17,
+                        L->w_down + (size_t)e * H * nbf * 17, L->b_up ? L->b_up + e * F : NULL,
+                        L->b_gate ? L->b_gate + e * F : NULL, L->b_down ? L->b_down + e * H : NULL,
+                        y, H, F, L->act, scratch);
+      if (L->weight_before_ffn) {
+        for (int64_t d = 0; d < H; ++d) o[d] += y[d];
+      } else {
+        for (int64_t d = 0; d < H; ++d) o[d] += w * y[d];
+      }
+    }
+    if (L->residual)
+      for (int64_t d = 0; d < H; ++d) o[d] = hidden[t * H + d] + o[d];
+  }
+  free(pairs);
+  free(tmp);
+  free(normed);
+  return rc;
+}

@@ -1,0 +1,68 @@
+"""Shared helpers of the GPU parity tests."""
+import numpy as np
+
+from coalsack_amd import synth
+
+
+def all_blocks(L, which):
+    return np.concatenate([L.blocks(e, which) for e in range(L.E)])
+
+
+def build_layer(lib, L, bias=True, norm=False, device_weights=False, **opts):
+    """Populate a resident layer from LayerInputs; weights either uploaded from
+    the host replay of the generator or generated on the device."""
+    layer = lib.layer(L.E, L.k, L.H, L.F)
+    layer.set_router(L.gate_w, L.gate_b)
+    if device_weights:
+        layer.fill_synthetic(L.seed, L.layer)
+        for e in range(L.E):
+            if bias:
+                layer.set_expert(e, None, None, None, L.b_up[e], L.b_gate[e], L.b_down[e])
+    else:
+        for e in range(L.E):
+            b = (L.b_up[e], L.b_gate[e], L.b_down[e]) if bias else (None, None, None)
+            layer.set_expert(e, L.blocks(e, 0), L.blocks(e, 1), L.blocks(e, 2), *b)
+    if norm:
+        layer.set_norm(L.norm_w, 1e-5)
+    if opts:
+        layer.set_options(**opts)
+    return layer
+
+
+def oracle_layer(oracle, L, hidden, bias=True, norm=False, residual=False, max_tokens=-1, **opts):
+    return oracle.moe_layer(
+        hidden, L.E, L.k, L.H, L.F, L.gate_w, L.gate_b, all_blocks(L, 0), all_blocks(L, 1),
+        all_blocks(L, 2), L.b_up if bias else None, L.b_gate if bias else None,
+        L.b_down if bias else None, norm_w=L.norm_w if norm else None, norm_eps=1e-5,
+        residual=residual, max_tokens=max_tokens, **opts)
+
+
+def classify_index_mismatches(oracle, hidden, L, got_pairs, want_pairs):
+    """Returns (real, near_tie): tokens whose expert indices differ from the
+    oracle's, split by whether float64 logits show a rank boundary closer than
+    fp32 summation noise (gap < 1e-5 * |logit| + 1e-6)."""
+    gi, wi = got_pairs[..., 0].astype(int), want_pairs[..., 0].astype(int)
+    bad = np.nonzero(np.any(gi != wi, axis=1))[0]
+    if bad.size == 0:
+        return 0, 0
+    logits = hidden[bad].astype(np.float64) @ L.gate_w.astype(np.float64).T + L.gate_b
+    real = near = 0
+    k = L.k
+    for r in range(bad.size):
+        srt = np.sort(logits[r])[::-1][:k + 1]
+        gaps = np.abs(np.diff(srt))
+        tol = 1e-5 * np.abs(srt[:-1]) + 1e-6
+        if np.any(gaps < tol):
+            near += 1
+        else:
+            real += 1
+    return real, near
+
+
+def assert_layer_close(got, want, tol=1e-3):
+    """max|d| / max(1e-6, max|want|) <= tol and |d| <= tol * max(1, |want|) per element."""
+    d = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert np.all(np.isfinite(got))
+    assert d.max() / max(1e-6, np.abs(want).max()) <= tol, d.max()
+    assert np.all(d <= tol * np.maximum(1.0, np.abs(want))), d.max()
+    return d.max()
