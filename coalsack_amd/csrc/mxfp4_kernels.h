@@ -80,6 +80,9 @@ __global__ void export_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t* 
 
 // Dequantise through the same conversion instruction the expert kernels use
 // (v_cvt_scalef32_pk_bf16_fp4), then widen bf16 -> f32, which is exact.
+// Code 8 (sign set, magnitude 0) converts to -0.0 in hardware where the
+// reference's integer table gives +0.0 (gguf_dequant.h:413-415); adding +0.0
+// canonicalises it.  Inside a contraction the two zeros are interchangeable.
 __global__ void dequant_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t* __restrict__ s,
                                      float* __restrict__ dst, int rows, int nblk, long entries) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -99,14 +102,14 @@ __global__ void dequant_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t*
     bf16x2 r1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], sc, 1);
     bf16x2 r2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], sc, 2);
     bf16x2 r3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], sc, 3);
-    o[d * 8 + 0] = (float)r0[0];
-    o[d * 8 + 1] = (float)r0[1];
-    o[d * 8 + 2] = (float)r1[0];
-    o[d * 8 + 3] = (float)r1[1];
-    o[d * 8 + 4] = (float)r2[0];
-    o[d * 8 + 5] = (float)r2[1];
-    o[d * 8 + 6] = (float)r3[0];
-    o[d * 8 + 7] = (float)r3[1];
+    o[d * 8 + 0] = (float)r0[0] + 0.0f;
+    o[d * 8 + 1] = (float)r0[1] + 0.0f;
+    o[d * 8 + 2] = (float)r1[0] + 0.0f;
+    o[d * 8 + 3] = (float)r1[1] + 0.0f;
+    o[d * 8 + 4] = (float)r2[0] + 0.0f;
+    o[d * 8 + 5] = (float)r2[1] + 0.0f;
+    o[d * 8 + 6] = (float)r3[0] + 0.0f;
+    o[d * 8 + 7] = (float)r3[1] + 0.0f;
   }
 }
 

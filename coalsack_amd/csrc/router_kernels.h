@@ -40,6 +40,7 @@ __global__ __launch_bounds__(256) void prep_kernel(const float* __restrict__ src
     float v = x[d];
     if (norm_w) v = (v / inv_den) * norm_w[d];
     if (xn) xn[(size_t)row * H + d] = v;
+    if (!xs) continue;
     if (gather_w) v = v * gw;
     uint16_t hi, lo;
     split_bf16(v, hi, lo);
@@ -241,6 +242,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
                                                       const float* __restrict__ residual,
                                                       float* __restrict__ out, int T, int k, int H,
                                                       int pre_weighted) {
+#pragma clang fp contract(off)  // w * y and the add round separately, as in the reference
   const int t = blockIdx.y;
   const int d = blockIdx.x * 256 + threadIdx.x;
   if (d >= H) return;
@@ -250,13 +252,14 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
     if (pos < 0) continue;  // empty expert tensor: skipped (expert_merge_node.h:111-113)
     const float v = y[(size_t)pos * H + d];
     if (pre_weighted) {
-      acc = __fadd_rn(acc, v);
+      acc = acc + v;
     } else {
       const float w = pairs[2 * ((size_t)t * k + s) + 1];
-      acc = __fadd_rn(acc, __fmul_rn(w, v));
+      const float wv = w * v;
+      acc = acc + wv;
     }
   }
-  if (residual) acc = __fadd_rn(residual[(size_t)t * H + d], acc);
+  if (residual) acc = residual[(size_t)t * H + d] + acc;
   out[(size_t)t * H + d] = acc;
 }
 

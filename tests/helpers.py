@@ -66,3 +66,10 @@ def assert_layer_close(got, want, tol=1e-3):
     assert d.max() / max(1e-6, np.abs(want).max()) <= tol, d.max()
     assert np.all(d <= tol * np.maximum(1.0, np.abs(want))), d.max()
     return d.max()
+
+
+def nbits_differ(a, b):
+    """Number of elements whose fp32 bit patterns differ."""
+    a = np.ascontiguousarray(a, np.float32).reshape(-1).view(np.uint32)
+    b = np.ascontiguousarray(b, np.float32).reshape(-1).view(np.uint32)
+    return int(np.count_nonzero(a != b))
