@@ -1,0 +1,264 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE layer (router -> dispatch -> MXFP4 expert MLP -> combine)
+on one MI355X through the C ABI.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--tokens T]
+
+Prints ONE JSON line.  A step is one forward of the layer over one batch of T
+synthetic tokens with weights, input and output resident in HBM.  `value` is
+tokens/s of the whole layer; `roofline` describes the dominant kernel (gate/up
+projections), timed live with HIP events on the library's stream;
+`cpu_baseline` is the CPU checker (a restatement of the reference's
+single-threaded path) timed on this host on a bounded sample.
+
+Workloads (BASELINE.json configs):
+  c2_20b_decode   32 experts, top-4, H = F = 2880, T in {1,2,4,8,16,32} (default, T=16)
+  c3_20b_prefill  same layer, T = 2048
+  c4_120b         128 experts, 8 hot experts (+2.0 router bias), T in {1,16,4096}
+  c5_stack        36 layers of the 120b shape with RMSNorm + residual, T in {1,8,64}
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_FP4_PEAK_TFLOPS = 10100.0  # dense MXFP4, published
+MAT_BYTES = 2880 * 90 * 17      # one [2880, 2880] MXFP4 matrix in 17-byte blocks
+
+SHAPES = {
+    "c2_20b_decode": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=16, sweep=[1, 2, 4, 8, 16, 32]),
+    "c3_20b_prefill": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=2048, sweep=[]),
+    "c4_120b": dict(E=128, k=4, H=2880, F=2880, hot=8, default_T=16, sweep=[1, 16]),
+    "c5_stack": dict(E=128, k=4, H=2880, F=2880, hot=8, default_T=8, sweep=[1, 8, 64], layers=36),
+}
+
+
+def layer_bytes(E, k, H, F, T, U):
+    """Algorithmic HBM bytes of one layer forward: every distinct expert's three
+    matrices and biases once, the router weights, activations in and out, router
+    output."""
+    mat_gu = F * (H // 32) * 17
+    mat_d = H * (F // 32) * 17
+    return U * (2 * mat_gu + mat_d + (2 * F + H) * 4) + E * H * 4 + E * 4 + 2 * T * H * 4 + T * k * 8
+
+
+def gateup_bytes(H, F, T, k, U):
+    """Algorithmic bytes of the gate/up kernel: both matrices and biases of every
+    distinct expert once, the fp32 activations in, the fp32 activations out."""
+    return U * (2 * F * (H // 32) * 17 + 2 * F * 4) + T * H * 4 + T * k * F * 4
+
+
+def layer_flops(E, k, H, F, T):
+    return T * (k * 6 * H * F + 2 * E * H)
+
+
+def make_layer(lib, synth, shape, seed, layer_index=0, norm=False):
+    L = synth.LayerInputs(shape["E"], shape["k"], shape["H"], shape["F"], seed=seed, layer=layer_index,
+                          hot_experts=shape["hot"], with_norm=norm)
+    layer = lib.layer(L.E, L.k, L.H, L.F)
+    layer.set_router(L.gate_w, L.gate_b)
+    layer.fill_synthetic(L.seed, L.layer)
+    for e in range(L.E):
+        layer.set_expert(e, None, None, None, L.b_up[e], L.b_gate[e], L.b_down[e])
+    if norm:
+        layer.set_norm(L.norm_w, 1e-5)
+    return L, layer
+
+
+def time_forward(lib, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    lib.synchronize()
+    e0, e1 = lib.event(), lib.event()
+    lib.record(e0)
+    for _ in range(steps):
+        fn()
+    lib.record(e1)
+    ms = lib.elapsed_ms(e0, e1)
+    lib.synchronize()
+    lib.dll.csk_event_destroy(e0)
+    lib.dll.csk_event_destroy(e1)
+    return ms / steps
+
+
+def stage_profile(lib, fn, steps):
+    lib.stage_timing(True)
+    acc = {}
+    for _ in range(steps):
+        fn()
+        for kk, v in lib.stage_times().items():
+            acc[kk] = acc.get(kk, 0.0) + v
+    lib.stage_timing(False)
+    return {kk: v / steps for kk, v in acc.items()}
+
+
+def bench_layer(lib, synth, shape, T, steps, warmup, seed=1234):
+    L, layer = make_layer(lib, synth, shape, seed)
+    hidden = synth.hidden_states(T, L.H, seed=T)
+    d_in = lib.to_device(hidden)
+    d_out = lib.dev_alloc(hidden.nbytes)
+    fn = lambda: layer.forward_device(d_in, T, d_out)  # noqa: E731
+    ms = time_forward(lib, fn, steps, warmup)
+    stages = stage_profile(lib, fn, max(5, min(steps, 50)))
+    counts, _ = layer.last_dispatch(T)
+    U = int(np.count_nonzero(counts))
+    out = lib.to_host(d_out, (T, L.H))
+    lib.dev_free(d_in)
+    lib.dev_free(d_out)
+    layer.close()
+    res = dict(T=T, ms_per_step=ms, tokens_per_s=T / (ms * 1e-3), distinct_experts=U,
+               stage_ms=stages, finite=bool(np.all(np.isfinite(out))),
+               max_tokens_per_expert=int(counts.max()))
+    res["layer_bytes"] = layer_bytes(L.E, L.k, L.H, L.F, T, U)
+    res["layer_hbm_frac"] = res["layer_bytes"] / (ms * 1e-3) / (HBM_PEAK_GBS * 1e9)
+    res["layer_flops"] = layer_flops(L.E, L.k, L.H, L.F, T)
+    res["layer_fp4_frac"] = res["layer_flops"] / (ms * 1e-3) / (MFMA_FP4_PEAK_TFLOPS * 1e12)
+    gu = gateup_bytes(L.H, L.F, T, L.k, U)
+    res["gateup_bytes"] = gu
+    res["gateup_gbs"] = gu / (stages["gateup"] * 1e-3) / 1e9
+    return res, (L, hidden, out)
+
+
+def bench_stack(lib, synth, shape, T, steps, warmup, n_layers, seed=1234):
+    layers = []
+    for i in range(n_layers):
+        _, layer = make_layer(lib, synth, shape, seed, layer_index=i, norm=True)
+        layers.append(layer)
+    from coalsack_amd.capi import stack_forward
+    hidden = synth.hidden_states(T, shape["H"], seed=T)
+    d_h = lib.to_device(hidden)
+
+    def fn():
+        # hidden states grow by the residual each pass; reload so every step sees N(0,1)
+        lib.check(lib.dll.csk_copy_h2d(d_h, hidden.ctypes.data, hidden.nbytes))
+        stack_forward(lib, layers, d_h, T)
+    ms = time_forward(lib, fn, steps, warmup)
+    out = lib.to_host(d_h, hidden.shape)
+    lib.dev_free(d_h)
+    for layer in layers:
+        layer.close()
+    return dict(T=T, layers=n_layers, ms_per_step=ms, tokens_per_s=T / (ms * 1e-3),
+                finite=bool(np.all(np.isfinite(out))))
+
+
+def cpu_baseline(L, hidden, gpu_out, budget_s=12.0):
+    """Times the CPU checker (single thread, as the reference's layer runs) on
+    the same layer and tokens; repeats the forward until about budget_s of CPU
+    work.  Host weights are replayed only for the experts the batch selects."""
+    from oracle.binding import Oracle
+    orc = Oracle()
+    T = hidden.shape[0]
+    pairs = orc.router(hidden, L.gate_w, L.gate_b, L.k)
+    used = sorted(set(pairs[..., 0].astype(int).ravel().tolist()))
+    per_gu, per_d = L.F * (L.H // 32) * 17, L.H * (L.F // 32) * 17
+    wu = np.zeros(L.E * per_gu, np.uint8)
+    wg = np.zeros(L.E * per_gu, np.uint8)
+    wd = np.zeros(L.E * per_d, np.uint8)
+    for e in used:
+        wu[e * per_gu:(e + 1) * per_gu] = L.blocks(e, 0)
+        wg[e * per_gu:(e + 1) * per_gu] = L.blocks(e, 1)
+        wd[e * per_d:(e + 1) * per_d] = L.blocks(e, 2)
+    args = (hidden, L.E, L.k, L.H, L.F, L.gate_w, L.gate_b, wu, wg, wd, L.b_up, L.b_gate, L.b_down)
+    # bounded sample: at most Tm tokens of the batch, repeated
+    t0 = time.perf_counter()
+    Tm = min(T, 4)
+    ref, _ = orc.moe_layer(*args, max_tokens=Tm)
+    first = time.perf_counter() - t0
+    per_tok = first / Tm
+    Tm = int(max(1, min(T, budget_s / max(per_tok, 1e-6))))
+    reps = int(max(1, min(50, budget_s / (per_tok * Tm))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        ref, _ = orc.moe_layer(*args, max_tokens=Tm)
+    dt = time.perf_counter() - t0
+    err = float(np.max(np.abs(gpu_out[:Tm] - ref[:Tm])) / max(1e-6, np.max(np.abs(ref[:Tm]))))
+    return dict(value=Tm * reps / dt, unit="tokens/s", cores=1, kind="port",
+                sample=f"first {Tm} of {T} tokens x {reps} repeats, {dt:.1f} s on one host core "
+                       f"(CPU cost is linear in tokens x top_k)",
+                gpu_vs_cpu_max_rel_err=err)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2_20b_decode", choices=sorted(SHAPES))
+    ap.add_argument("--tokens", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sweep", action="store_true", help="only the headline batch size")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
+              "(no collectives, sharding or rank code are part of it).", file=sys.stderr)
+        sys.exit(2)
+
+    from coalsack_amd import load, synth
+    lib = load(0)
+    dev_name, cus, mem = lib.device_info()
+    shape = SHAPES[a.workload]
+    T = a.tokens or shape["default_T"]
+
+    if a.workload == "c5_stack":
+        res = bench_stack(lib, synth, shape, T, a.steps, a.warmup, shape["layers"])
+        line = dict(metric="MoE stack tokens/s", value=res["tokens_per_s"], unit="tokens/s", n_gpus=1,
+                    steps=a.steps, warmup=a.warmup, ms_per_step=res["ms_per_step"],
+                    higher_is_better=True, scaling="weak", vs_baseline=None, dtype="mxfp4 x bf16(2-term) -> f32",
+                    data="synthetic",
+                    config=dict(workload=f"c5_stack: 36 x 120b-shaped MoE layer (RMSNorm + residual), T={T}",
+                                tokens=T, device=dev_name),
+                    roofline=None, cpu_baseline=None, finite=res["finite"])
+        print(json.dumps(line))
+        return
+
+    res, (L, hidden, out) = bench_layer(lib, synth, shape, T, a.steps, a.warmup)
+    prefill = T >= 512
+    if prefill:
+        st = res["stage_ms"]
+        fl = T * shape["k"] * 4 * shape["H"] * shape["F"]  # gate + up flops
+        roof = dict(bound="mfma", kernel="gate/up grouped GEMM", achieved=fl / (st["gateup"] * 1e-3) / 1e12,
+                    peak=MFMA_FP4_PEAK_TFLOPS, unit="TFLOP/s", traffic=None)
+    else:
+        roof = dict(bound="hbm", kernel="expert_stream_kernel<2,*> (gate/up + SwiGLU)",
+                    achieved=res["gateup_gbs"], peak=HBM_PEAK_GBS, unit="GB/s", traffic=None)
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["kernel_ms"] = res["stage_ms"]["gateup"]
+    roof["algorithmic_bytes"] = res["gateup_bytes"]
+
+    sweep = []
+    if not a.no_sweep:
+        for Ts in shape["sweep"]:
+            if Ts == T:
+                r = res
+            else:
+                r, _ = bench_layer(lib, synth, shape, Ts, max(20, a.steps // 2), a.warmup)
+            sweep.append(dict(T=Ts, tokens_per_s=round(r["tokens_per_s"], 1), ms_per_step=round(r["ms_per_step"], 5),
+                              distinct_experts=r["distinct_experts"], layer_hbm_frac=round(r["layer_hbm_frac"], 4),
+                              gateup_hbm_frac=round(r["gateup_gbs"] / HBM_PEAK_GBS, 4),
+                              stage_ms={kk: round(v, 5) for kk, v in r["stage_ms"].items()}))
+
+    cpu = None if a.no_cpu else cpu_baseline(L, hidden, out)
+    line = dict(
+        metric="MoE layer tokens/s", value=res["tokens_per_s"], unit="tokens/s", n_gpus=1, steps=a.steps,
+        warmup=a.warmup, ms_per_step=res["ms_per_step"], higher_is_better=True, scaling="weak",
+        vs_baseline=None, dtype="mxfp4 x bf16(2-term) -> f32", data="synthetic",
+        config=dict(workload=f"{a.workload}: E={shape['E']} top-{shape['k']} H={shape['H']} F={shape['F']} "
+                             f"MXFP4, T={T}" + (", 8 hot experts" if shape["hot"] else ""),
+                    tokens=T, distinct_experts=res["distinct_experts"], device=dev_name, compute_units=cus),
+        roofline=roof, cpu_baseline=cpu,
+        layer=dict(hbm_frac=res["layer_hbm_frac"], fp4_mfma_frac=res["layer_fp4_frac"],
+                   algorithmic_bytes=res["layer_bytes"], algorithmic_flops=res["layer_flops"],
+                   stage_ms=res["stage_ms"], finite=res["finite"]),
+        sweep=sweep)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -33,6 +33,8 @@ SIGNATURES = {
     "csk_event_destroy": (None, [_P]),
     "csk_event_record": (C.c_int, [_P]),
     "csk_event_elapsed_ms": (C.c_int, [_P, _P, _F]),
+    "csk_stage_timing": (C.c_int, [C.c_int]),
+    "csk_stage_times": (C.c_int, [_F]),
     "csk_mxfp4_upload": (C.c_int, [_P, _I64, _I64, C.POINTER(_P)]),
     "csk_mxfp4_free": (None, [_P]),
     "csk_mxfp4_dequant": (C.c_int, [_P, _P]),
@@ -155,6 +157,16 @@ class Library:
         ms = C.c_float()
         self.check(self.dll.csk_event_elapsed_ms(a, b, C.byref(ms)))
         return ms.value
+
+    STAGES = ("prep", "router", "dispatch", "gateup", "down", "combine")
+
+    def stage_timing(self, on):
+        self.check(self.dll.csk_stage_timing(int(on)))
+
+    def stage_times(self):
+        ms = (C.c_float * len(self.STAGES))()
+        self.check(self.dll.csk_stage_times(ms))
+        return dict(zip(self.STAGES, list(ms)))
 
     # -- MXFP4 matrices
     def mxfp4_upload(self, blocks, rows, K):

@@ -122,6 +122,14 @@ struct Workspace {
 };
 Workspace g_ws;
 
+// optional per-stage events of the last forward
+bool g_timing = false;
+hipEvent_t g_stage_ev[CSK_N_STAGES + 1] = {};
+bool g_stage_valid = false;
+inline void mark(int i) {
+  if (g_timing) (void)hipEventRecord(g_stage_ev[i], g_stream);
+}
+
 }  // namespace
 
 struct csk_event {
@@ -295,7 +303,8 @@ int launch_stream(const ExpertStreamArgs& a, int64_t ntile, int64_t max_active, 
 // x_split rows are indexed through list_row (token ids) or directly by packed
 // position when list_row is null.
 int run_experts(const ExpertW* ew, int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
-                int act_type, const uint16_t* x_split, const int* list_row, Workspace& ws) {
+                int act_type, const uint16_t* x_split, const int* list_row, Workspace& ws,
+                bool timed = false) {
   const int64_t P = T * k;
   const int64_t max_active = std::min<int64_t>(E, P);
   ExpertStreamArgs a{};
@@ -312,8 +321,10 @@ int run_experts(const ExpertW* ew, int64_t E, int64_t T, int64_t k, int64_t H, i
   a.N = (int)F;
   a.act_out = ws.act;
   a.y_out = nullptr;
+  if (timed) mark(CSK_STAGE_GATEUP);
   int rc = launch_stream<2>(a, cdiv(F, 16), max_active, T);
   if (rc != CSK_OK) return rc;
+  if (timed) mark(CSK_STAGE_DOWN);
   // down
   a.list_row = nullptr;
   a.A = reinterpret_cast<const uint4*>(ws.act);
@@ -371,6 +382,23 @@ extern "C" int csk_device_info(char* name, size_t cap, int* compute_units, size_
   }
   if (compute_units) *compute_units = prop.multiProcessorCount;
   if (hbm_bytes) *hbm_bytes = prop.totalGlobalMem;
+  return CSK_OK;
+}
+
+extern "C" int csk_stage_timing(int enable) {
+  REQUIRE_INIT();
+  if (enable && !g_stage_ev[0])
+    for (auto& e : g_stage_ev) HIP_TRY(hipEventCreate(&e));
+  g_timing = enable != 0;
+  g_stage_valid = false;
+  return CSK_OK;
+}
+extern "C" int csk_stage_times(float* ms_out) {
+  REQUIRE_INIT();
+  if (!ms_out) return fail(CSK_ERR_ARG, "csk_stage_times: null output");
+  if (!g_stage_valid) return fail(CSK_ERR_STATE, "no forward has run with stage timing enabled");
+  HIP_TRY(hipEventSynchronize(g_stage_ev[CSK_N_STAGES]));
+  for (int i = 0; i < CSK_N_STAGES; ++i) HIP_TRY(hipEventElapsedTime(&ms_out[i], g_stage_ev[i], g_stage_ev[i + 1]));
   return CSK_OK;
 }
 
@@ -659,13 +687,16 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
   if (rc != CSK_OK) return rc;
   const int64_t P = T * L->k;
   const bool norm = (flags & CSK_FWD_RMSNORM) != 0;
+  mark(CSK_STAGE_PREP);
   rc = launch_prep(hidden, norm ? L->norm_w : nullptr, L->eps, norm ? ws.xn : nullptr, ws.xs, T,
                    L->H, nullptr, nullptr);
   if (rc != CSK_OK) return rc;
   const float* xr = norm ? ws.xn : hidden;
+  mark(CSK_STAGE_ROUTER);
   rc = launch_router(xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, T, L->E, L->H, L->k,
                      L->sigmoid, ws.logits, ws.pairs, ws.ids);
   if (rc != CSK_OK) return rc;
+  mark(CSK_STAGE_DISPATCH);
   rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, ws);
   if (rc != CSK_OK) return rc;
   const uint16_t* xa = ws.xs;
@@ -676,10 +707,14 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
     xa = ws.xg;
     list_row = nullptr;
   }
-  rc = run_experts(L->ew_dev, L->E, T, L->k, L->H, L->F, L->act, xa, list_row, ws);
+  rc = run_experts(L->ew_dev, L->E, T, L->k, L->H, L->F, L->act, xa, list_row, ws, true);
   if (rc != CSK_OK) return rc;
-  return launch_combine(ws.y, ws.pairs, ws.pos, (flags & CSK_FWD_RESIDUAL) ? hidden : nullptr, out,
-                        T, L->k, L->H, L->wbf);
+  mark(CSK_STAGE_COMBINE);
+  rc = launch_combine(ws.y, ws.pairs, ws.pos, (flags & CSK_FWD_RESIDUAL) ? hidden : nullptr, out, T,
+                      L->k, L->H, L->wbf);
+  mark(CSK_N_STAGES);
+  g_stage_valid = g_timing;
+  return rc;
 }
 
 extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T, float* out,

@@ -67,6 +67,20 @@ void csk_event_destroy(csk_event* e);
 int csk_event_record(csk_event* e);                 /* on the library's stream */
 int csk_event_elapsed_ms(csk_event* a, csk_event* b, float* ms); /* waits for b */
 
+/* Per-kernel timing of csk_moe_forward, for benchmarks: when enabled every
+ * forward brackets its stages with events on the library's stream (a small
+ * overhead, so throughput is measured with it off).  csk_stage_times waits for
+ * the last forward and returns milliseconds per stage. */
+#define CSK_STAGE_PREP 0     /* RMSNorm + activation split            */
+#define CSK_STAGE_ROUTER 1   /* gate GEMV + top-k + softmax           */
+#define CSK_STAGE_DISPATCH 2 /* histogram + scan + scatter            */
+#define CSK_STAGE_GATEUP 3   /* gate/up projections + activation      */
+#define CSK_STAGE_DOWN 4     /* down projection                       */
+#define CSK_STAGE_COMBINE 5  /* weighted combine (+ residual)         */
+#define CSK_N_STAGES 6
+int csk_stage_timing(int enable);
+int csk_stage_times(float* ms_out);
+
 /* ---- resident MXFP4 matrices ------------------------------------------- */
 
 /* Take a [rows, K] matrix in the reference's storage format -- rows of K/32
