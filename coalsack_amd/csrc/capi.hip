@@ -11,8 +11,8 @@
 
 #include "coalsack_moe.h"
 #include "common.h"
-#include "expert_prefill_kernel.h"
 #include "expert_stream_kernel.h"
+#include "expert_prefill_kernel.h"
 #include "mxfp4_kernels.h"
 #include "router_kernels.h"
 
@@ -70,8 +70,7 @@ struct Workspace {
   int* ids = nullptr;       // [P]
   int* counts = nullptr;    // [E]
   int* offsets = nullptr;   // [E+1]
-  int* active = nullptr;    // [E]
-  int* n_active = nullptr;  // [1]
+  WorkDesc* desc = nullptr; // [E] work descriptors of the active experts
   int* list_tok = nullptr;  // [P]
   float* list_w = nullptr;  // [P]
   int* pos = nullptr;       // [P]
@@ -81,7 +80,7 @@ struct Workspace {
   int* n_tiles = nullptr;
 
   void release() {
-    void* ps[] = {xn, xs, xg, logits, pairs, ids, counts, offsets, active, n_active,
+    void* ps[] = {xn, xs, xg, logits, pairs, ids, counts, offsets, desc,
                   list_tok, list_w, pos, act, y, tiles, n_tiles};
     for (void* p : ps)
       if (p) (void)hipFree(p);
@@ -106,8 +105,7 @@ struct Workspace {
     WS_ALLOC(ids, P);
     WS_ALLOC(counts, (size_t)nE);
     WS_ALLOC(offsets, (size_t)nE + 1);
-    WS_ALLOC(active, (size_t)nE);
-    WS_ALLOC(n_active, 1);
+    WS_ALLOC(desc, (size_t)nE);
     WS_ALLOC(list_tok, P);
     WS_ALLOC(list_w, P);
     WS_ALLOC(pos, P);
@@ -121,6 +119,8 @@ struct Workspace {
   }
 };
 Workspace g_ws;
+float* g_zero = nullptr;  // zero vector standing in for absent biases
+constexpr size_t kZeroLen = 1 << 16;
 
 // optional per-stage events of the last forward
 bool g_timing = false;
@@ -277,52 +277,55 @@ int launch_router(const float* x, const float* gate_w, const float* gate_b, int6
 }
 
 int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, int64_t E,
-                    Workspace& ws) {
+                    const ExpertW* ew, Workspace& ws) {
   dispatch_count_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(ids, (int)P, ws.counts);
   int rc = check_launch("dispatch_count_kernel");
   if (rc != CSK_OK) return rc;
   dispatch_scatter_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(
-      ids, pairs, (int)P, (int)k, (int)E, ws.counts, ws.offsets, ws.active, ws.n_active,
-      ws.list_tok, ws.list_w, ws.pos);
+      ids, pairs, (int)P, (int)k, (int)E, ws.counts, ew, ws.offsets, ws.desc, ws.list_tok,
+      ws.list_w, ws.pos);
   return check_launch("dispatch_scatter_kernel");
 }
 
 template <int NMAT>
-int launch_stream(const ExpertStreamArgs& a, int64_t ntile, int64_t max_active, int64_t T) {
-  const dim3 grid((unsigned)ntile, (unsigned)max_active);
-  if (T <= 16)
-    expert_stream_kernel<NMAT, 1><<<grid, 256, 0, g_stream>>>(a);
-  else if (T <= 32)
-    expert_stream_kernel<NMAT, 2><<<grid, 256, 0, g_stream>>>(a);
-  else
-    expert_stream_kernel<NMAT, 4><<<grid, 256, 0, g_stream>>>(a);
+int launch_stream(ExpertStreamArgs a, int64_t max_active, int64_t T) {
+  if (a.nblk > 96) {  // contraction length above 3072
+    expert_generic_kernel<NMAT><<<dim3((unsigned)a.ntile, (unsigned)max_active), 256, 0, g_stream>>>(a);
+    return check_launch("expert_generic_kernel");
+  }
+  constexpr int G = 4;
+  // enough workgroups for two per compute unit, each walking through consecutive tiles
+  const int64_t want = 2 * (int64_t)std::max(g_cus, 1);
+  int64_t chunks = std::min<int64_t>(a.ntile, std::max<int64_t>(1, cdiv(want, max_active)));
+  a.tiles_per_wg = (int)cdiv(a.ntile, chunks);
+  chunks = cdiv(a.ntile, a.tiles_per_wg);
+  const dim3 grid((unsigned)chunks, (unsigned)max_active, (unsigned)cdiv(T, G));
+  const size_t lds = (size_t)G * a.nblk * 128 + 2 * 4 * NMAT * 4 * 64 * sizeof(float);
+  expert_stream_kernel<NMAT, G><<<grid, 256, lds, g_stream>>>(a);
   return check_launch("expert_stream_kernel");
 }
 
 // Experts' MLPs over the dispatched tokens: ws.y[P,H] <- down(act(gate, up)).
 // x_split rows are indexed through list_row (token ids) or directly by packed
 // position when list_row is null.
-int run_experts(const ExpertW* ew, int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
+int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
                 int act_type, const uint16_t* x_split, const int* list_row, Workspace& ws,
                 bool timed = false) {
   const int64_t P = T * k;
   const int64_t max_active = std::min<int64_t>(E, P);
   ExpertStreamArgs a{};
-  a.ew = ew;
-  a.active = ws.active;
-  a.n_active = ws.n_active;
-  a.counts = ws.counts;
-  a.offsets = ws.offsets;
+  a.desc = ws.desc;
   a.act_type = act_type;
   // gate/up + activation
   a.list_row = list_row;
   a.A = reinterpret_cast<const uint4*>(x_split);
   a.nblk = (int)(H / 32);
   a.N = (int)F;
+  a.ntile = (int)cdiv(F, 16);
   a.act_out = ws.act;
   a.y_out = nullptr;
   if (timed) mark(CSK_STAGE_GATEUP);
-  int rc = launch_stream<2>(a, cdiv(F, 16), max_active, T);
+  int rc = launch_stream<2>(a, max_active, T);
   if (rc != CSK_OK) return rc;
   if (timed) mark(CSK_STAGE_DOWN);
   // down
@@ -330,9 +333,10 @@ int run_experts(const ExpertW* ew, int64_t E, int64_t T, int64_t k, int64_t H, i
   a.A = reinterpret_cast<const uint4*>(ws.act);
   a.nblk = (int)(F / 32);
   a.N = (int)H;
+  a.ntile = (int)cdiv(H, 16);
   a.act_out = nullptr;
   a.y_out = ws.y;
-  return launch_stream<1>(a, cdiv(H, 16), max_active, T);
+  return launch_stream<1>(a, max_active, T);
 }
 
 int launch_combine(const float* y, const float* pairs, const int* pos, const float* residual,
@@ -346,8 +350,8 @@ int launch_combine(const float* y, const float* pairs, const int* pos, const flo
 int check_dims(int64_t E, int64_t k, int64_t H, int64_t F) {
   if (E <= 0 || E > kMaxExperts) return fail(CSK_ERR_ARG, "num_experts must be in 1..256");
   if (k <= 0 || k > kMaxTopK || k > E) return fail(CSK_ERR_ARG, "top_k must be in 1..min(16, E)");
-  if (H <= 0 || H % 32) return fail(CSK_ERR_ARG, "hidden_dim must be a positive multiple of 32");
-  if (F <= 0 || F % 32) return fail(CSK_ERR_ARG, "expert_ffn_dim must be a positive multiple of 32");
+  if (H <= 0 || H % 32 || H > (int64_t)kZeroLen) return fail(CSK_ERR_ARG, "hidden_dim must be a positive multiple of 32, at most 65536");
+  if (F <= 0 || F % 32 || F > (int64_t)kZeroLen) return fail(CSK_ERR_ARG, "expert_ffn_dim must be a positive multiple of 32, at most 65536");
   return CSK_OK;
 }
 
@@ -365,6 +369,10 @@ extern "C" int csk_init(int device) {
   if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0)
     return fail(CSK_ERR_HIP, std::string("device is ") + prop.gcnArchName + ", this library is built for gfx950 only");
   if (!g_stream) HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  if (!g_zero) {
+    HIP_TRY(hipMalloc((void**)&g_zero, kZeroLen * sizeof(float)));
+    HIP_TRY(hipMemset(g_zero, 0, kZeroLen * sizeof(float)));
+  }
   g_device = device;
   g_cus = prop.multiProcessorCount;
   g_ready = true;
@@ -531,7 +539,7 @@ extern "C" int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_
     ExpertW& w = L->ew_host[(size_t)e];
     const csk_mxfp4 g = L->view(e, CSK_W_GATE), u = L->view(e, CSK_W_UP), d = L->view(e, CSK_W_DOWN);
     w.q_gate = g.q, w.s_gate = g.s, w.q_up = u.q, w.s_up = u.s, w.q_down = d.q, w.s_down = d.s;
-    w.b_gate = w.b_up = w.b_down = nullptr;
+    w.b_gate = w.b_up = w.b_down = g_zero;
   }
   hipError_t e1 = hipMemcpy(L->ew_dev, L->ew_host.data(), (size_t)E * sizeof(ExpertW), hipMemcpyHostToDevice);
   if (e1 != hipSuccess) {
@@ -586,7 +594,7 @@ static int upload_biases(csk_layer* L, int64_t e, const float* b_up, const float
     HIP_TRY(hipMemcpyAsync(base + 2 * L->F, b_down, (size_t)L->H * sizeof(float), hipMemcpyHostToDevice, g_stream));
     w.b_gate = base, w.b_up = base + L->F, w.b_down = base + 2 * L->F;
   } else {
-    w.b_gate = w.b_up = w.b_down = nullptr;
+    w.b_gate = w.b_up = w.b_down = g_zero;
   }
   HIP_TRY(hipMemcpyAsync(L->ew_dev + e, &w, sizeof(ExpertW), hipMemcpyHostToDevice, g_stream));
   HIP_TRY(hipStreamSynchronize(g_stream));
@@ -697,7 +705,7 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
                      L->sigmoid, ws.logits, ws.pairs, ws.ids);
   if (rc != CSK_OK) return rc;
   mark(CSK_STAGE_DISPATCH);
-  rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, ws);
+  rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, L->ew_dev, ws);
   if (rc != CSK_OK) return rc;
   const uint16_t* xa = ws.xs;
   const int* list_row = ws.list_tok;
@@ -707,7 +715,7 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
     xa = ws.xg;
     list_row = nullptr;
   }
-  rc = run_experts(L->ew_dev, L->E, T, L->k, L->H, L->F, L->act, xa, list_row, ws, true);
+  rc = run_experts(L->E, T, L->k, L->H, L->F, L->act, xa, list_row, ws, true);
   if (rc != CSK_OK) return rc;
   mark(CSK_STAGE_COMBINE);
   rc = launch_combine(ws.y, ws.pairs, ws.pos, (flags & CSK_FWD_RESIDUAL) ? hidden : nullptr, out, T,
@@ -840,6 +848,7 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
   if (H % 32) return fail(CSK_ERR_ARG, "expert_mlp: hidden_dim must be a multiple of 32 for MXFP4, got " + std::to_string(H));
   if (F % 32) return fail(CSK_ERR_ARG, "expert_mlp: expert_ffn_dim must be a multiple of 32 for MXFP4, got " + std::to_string(F));
   if (k <= 0 || k > kMaxTopK) return fail(CSK_ERR_ARG, "expert_mlp: top_k must be in 1..16");
+  if (H > (int64_t)kZeroLen || F > (int64_t)kZeroLen) return fail(CSK_ERR_ARG, "expert_mlp: dimensions above 65536 are not supported");
   const int nb = (b_up != nullptr) + (b_gate != nullptr) + (b_down != nullptr);
   if (nb != 0 && nb != 3) return fail(CSK_ERR_ARG, "expert_mlp: biases must be all present or all absent");
   Workspace& ws = g_ws;
@@ -857,9 +866,9 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
   ExpertW w{};
   w.q_gate = w_gate->q, w.s_gate = w_gate->s, w.q_up = w_up->q, w.s_up = w_up->s;
   w.q_down = w_down->q, w.s_down = w_down->s;
-  w.b_gate = nb ? dbg.as<float>() : nullptr;
-  w.b_up = nb ? dbu.as<float>() : nullptr;
-  w.b_down = nb ? dbd.as<float>() : nullptr;
+  w.b_gate = nb ? dbg.as<float>() : g_zero;
+  w.b_up = nb ? dbu.as<float>() : g_zero;
+  w.b_down = nb ? dbd.as<float>() : g_zero;
   if ((rc = dew.upload(&w, sizeof w)) != CSK_OK) return rc;
   if ((rc = dout.alloc((size_t)T * H * 4)) != CSK_OK) return rc;
   select_expert_ids_kernel<<<dim3((unsigned)cdiv(P, 256)), 256, 0, g_stream>>>(
@@ -867,7 +876,7 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
   if ((rc = check_launch("select_expert_ids_kernel")) != CSK_OK) return rc;
   HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
   HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
-  if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, ws)) != CSK_OK) return rc;
+  if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
   const uint16_t* xa;
   const int* list_row;
   if (weight_before_ffn) {
@@ -884,7 +893,7 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
     xa = ws.xs;
     list_row = ws.list_tok;
   }
-  rc = run_experts(dew.as<ExpertW>(), 1, T, k, H, F, activation, xa, list_row, ws);
+  rc = run_experts(1, T, k, H, F, activation, xa, list_row, ws);
   if (rc != CSK_OK) return rc;
   expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)T), 256, 0, g_stream>>>(
       ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);

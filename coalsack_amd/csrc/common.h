@@ -9,6 +9,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes, address-space friendly
 
 constexpr int kWave = 64;
 constexpr int kTileRows = 16;   // weight rows per packed tile (= MFMA N)
@@ -34,6 +35,15 @@ struct ExpertW {
   const float* b_up;
   const float* b_down;
 };
+
+// Pointers read out of device structures are generic to the compiler, which
+// would then use FLAT loads (tracked by both memory counters and therefore
+// always waited for in full).  These casts pin them to global memory.
+#define CSK_GLOBAL __attribute__((address_space(1)))
+template <class T>
+__device__ __forceinline__ const CSK_GLOBAL T* as_global(const T* p) {
+  return (const CSK_GLOBAL T*)p;
+}
 
 // E8M0 byte -> scale of true E2M1 values, 2^(b-127); exact for b in 1..254.
 __device__ __forceinline__ float e8m0_scale(uint32_t b) { return __uint_as_float(b << 23); }

@@ -1,14 +1,17 @@
 // Expert MLP for the weight-streaming (decode) regime.
 //
-// Each workgroup owns one 16-row tile of one active expert's matrix (gate and
-// up together, or down) and streams it from HBM exactly once: 64 lanes x 16
-// bytes = 1 KiB of contiguous nibbles per matrix per step, the four waves
-// taking interleaved K steps.  MXFP4 is expanded in registers by
-// v_cvt_scalef32_pk_bf16_fp4 (exact: an E2M1 value times a power of two always
-// fits bf16) and contracted on the matrix cores against up to 16*MT tokens of
-// that expert.  Activations arrive as two bf16 terms (hi + lo, 16 mantissa
-// bits) so the products are those of the reference's fp32 x exactly-dequantised
-// weight to within 2^-17; accumulation is fp32.
+// A workgroup owns TPW consecutive 16-row tiles of one active expert's matrix
+// (gate and up together, or down) and streams them from HBM exactly once:
+// 64 lanes x 16 bytes = 1 KiB of contiguous nibbles per matrix per tile per
+// step.  The four waves take interleaved K steps (128 elements each); a wave
+// loads its slice of the activations once per step and reuses it for all TPW
+// tiles.  MXFP4 is expanded in registers by v_cvt_scalef32_pk_bf16_fp4 (exact:
+// an E2M1 value times a power of two always fits bf16) and contracted on the
+// matrix cores against up to 16*MT tokens of that expert.  Activations arrive
+// as two bf16 terms (hi + lo, 16 mantissa bits), so each product is that of the
+// reference's fp32 activation and exactly dequantised weight to within 2^-17;
+// accumulation is fp32.  The K slices of the four waves meet in LDS in a fixed
+// order.
 //
 // Restates include/coalsack/nn/nn_ops/expert_mlp_node.h:651-732
 // (compute_token_mxfp4): gate/up projections + bias, activation (:699-706),
@@ -18,17 +21,25 @@
 
 namespace csk {
 
+// One entry per active expert, written by the dispatch kernel; entries past
+// the active count have Te == 0.
+struct WorkDesc {
+  int e, Te, base, pad;
+  ExpertW w;
+};
+
+// Bias pointers inside desc[].w must not be null for expert_stream_kernel: the
+// host substitutes a zero vector for an absent bias, so that the loads are
+// unconditional.
 struct ExpertStreamArgs {
-  const ExpertW* ew;
-  const int* active;     // compact list of experts with tokens
-  const int* n_active;
-  const int* counts;     // [E]
-  const int* offsets;    // [E+1] packed position of each expert's first token
+  const WorkDesc* desc;
   const int* list_row;   // packed position -> row of A; null: row = packed position
   const uint4* A;        // [rows][nblk][8] x 16 B: 32 bf16 hi then 32 bf16 lo per block
   int nblk;              // K / 32
+  int ntile;             // ceil(N / 16)
   int N;                 // output features (F for gate/up, H for down)
   int act_type;
+  int tiles_per_wg;      // consecutive row tiles one workgroup walks through
   uint16_t* act_out;     // gate/up: [P][N/32][64] bf16 hi|lo
   float* y_out;          // down: [P][N] f32
 };
@@ -66,138 +77,276 @@ union U4B8 {
   bf16x8 b;
 };
 
+__device__ __forceinline__ uint32_t u4_word(const uint4& v, int i) {
+  return i == 0 ? v.x : (i == 1 ? v.y : (i == 2 ? v.z : v.w));
+}
+
+// ---------------------------------------------------------------------------
+// Persistent, software-pipelined kernel (K <= 3072).
+//
 // NMAT = 2: gate and up tiles together, SwiGLU epilogue.  NMAT = 1: down.
-// MT = number of 16-token M tiles kept live per pass over the weights.
-template <int NMAT, int MT>
+// G = tokens contracted per workgroup (rows 0..G-1 of the 16-row MFMA tile);
+// token group blockIdx.z of expert slot blockIdx.y, tiles
+// [blockIdx.x * tiles_per_wg, ...).
+//
+// Memory-level parallelism bounds this kernel, so it never lets the memory
+// queue drain: the group's activation rows are copied once into LDS
+// (global_load_lds, no registers), and while the matrix cores work on tile t
+// from one register set the 24 weight loads of tile t+1 -- all of a wave's K
+// steps, issued back to back from clamped addresses so that no wait separates
+// them -- are already in flight into the other set.  The four waves split K;
+// their partial sums meet in double-buffered LDS (one barrier per tile) in the
+// fixed order w0 + w1 + w2 + w3, and wave t mod 4 finishes tile t.
+template <int NMAT, int G>
 __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) {
-  const int u = blockIdx.y;
-  if (u >= *a.n_active) return;
-  const int e = a.active[u];
-  const int Te = a.counts[e];
-  const int base = a.offsets[e];
-  const ExpertW w = a.ew[e];
+  constexpr int NS = 6;  // K steps per wave: 4 waves x 6 x 128 = 3072 elements
+  constexpr int NV = NMAT * 4;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int nblk = a.nblk;
+  const int row_u4 = nblk * 8;                   // uint4 per activation row
+  uint4* As = reinterpret_cast<uint4*>(smem);    // [G][row_u4]
+  float* red = reinterpret_cast<float*>(smem + (size_t)G * row_u4 * 16);  // [2][4][NV][64]
+
+  const WorkDesc* wd = a.desc + blockIdx.y;
+  const int Te = wd->Te;
+  const int gbase = blockIdx.z * G;
+  if (gbase >= Te) return;
+  const int gcount = min(G, Te - gbase);
+  const int t_begin = blockIdx.x * a.tiles_per_wg;
+  const int t_end = min(a.ntile, t_begin + a.tiles_per_wg);
+  if (t_begin >= t_end) return;
+  const int base = wd->base + gbase;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int n = lane & 15, g = lane >> 4;
+  const CSK_GLOBAL u32x4* q0 = as_global(reinterpret_cast<const u32x4*>(NMAT == 2 ? wd->w.q_gate : wd->w.q_down)) + n;
+  const CSK_GLOBAL uint8_t* s0 = as_global(NMAT == 2 ? wd->w.s_gate : wd->w.s_down) + n;
+  const CSK_GLOBAL u32x4* q1 = as_global(reinterpret_cast<const u32x4*>(wd->w.q_up)) + n;
+  const CSK_GLOBAL uint8_t* s1 = as_global(wd->w.s_up) + n;
+  const CSK_GLOBAL float* bp0 = as_global(NMAT == 2 ? wd->w.b_gate : wd->w.b_down);
+  const CSK_GLOBAL float* bp1 = as_global(wd->w.b_up);
+
+  // activation rows of this token group -> LDS
+#pragma unroll
+  for (int rr = 0; rr < G; ++rr) {
+    if (rr < gcount) {
+      const int row = a.list_row ? a.list_row[base + rr] : base + rr;
+      const uint4* src = a.A + (size_t)row * row_u4;
+      for (int c0 = wv * 64; c0 < row_u4; c0 += 256) {
+        if (c0 + lane < row_u4)
+          __builtin_amdgcn_global_load_lds(
+              src + c0 + lane,
+              reinterpret_cast<__attribute__((address_space(3))) uint4*>(
+                  reinterpret_cast<uintptr_t>(As + rr * row_u4 + c0)),
+              16, 0, 0);
+      }
+    }
+  }
+
+  struct WSet {
+    u32x4 q[NS][NMAT];
+    uint32_t sb[NS][NMAT];
+    float b0, b1;
+  };
+  auto load_tile = [&](WSet& ws, int tile) {
+    const size_t te = (size_t)tile * nblk * 16;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const int kb = min(4 * (wv + 4 * s) + g, nblk - 1);
+      ws.q[s][0] = q0[te + kb * 16];
+      ws.sb[s][0] = s0[te + kb * 16];
+      if (NMAT == 2) {
+        ws.q[s][1] = q1[te + kb * 16];
+        ws.sb[s][1] = s1[te + kb * 16];
+      }
+    }
+    const int r = min(tile * 16 + n, a.N - 1);
+    ws.b0 = bp0[r];  // bias pointers are never null here (an absent bias is a zero vector)
+    if (NMAT == 2) ws.b1 = bp1[r];
+  };
+
+  const int arow = min(n, G - 1) * row_u4;  // lanes past G re-read a live row; their outputs are unused
+  const bool live = g * 4 < gcount;         // this lane's accumulator rows belong to live tokens
+
+  auto compute_tile = [&](const WSet& ws, int tile, int par) {
+    floatx4 acc[NMAT][2];  // [matrix][hi, lo term]: independent accumulation chains
+#pragma unroll
+    for (int m = 0; m < NMAT; ++m) acc[m][0] = acc[m][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    U4B8 ahi[2], alo[2];  // activation fragments run one quarter-step ahead of the matrix cores
+    {
+      const int kb0 = min(4 * wv + g, nblk - 1);
+      ahi[0].u = As[arow + kb0 * 8];
+      alo[0].u = As[arow + kb0 * 8 + 4];
+    }
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      const int kb = 4 * (wv + 4 * s) + g;
+      const bool kvs = kb < nblk;
+      const float sc0 = kvs ? e8m0_scale(ws.sb[s][0]) : 0.0f;
+      const float sc1 = (NMAT == 2 && kvs) ? e8m0_scale(ws.sb[s][1]) : 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int cur = (s * 4 + i) & 1, nxt = cur ^ 1;
+        if (s * 4 + i + 1 < NS * 4) {
+          const int s2 = (s * 4 + i + 1) >> 2, i2 = (s * 4 + i + 1) & 3;
+          const int kb2 = min(4 * (wv + 4 * s2) + g, nblk - 1);
+          ahi[nxt].u = As[arow + kb2 * 8 + i2];
+          alo[nxt].u = As[arow + kb2 * 8 + 4 + i2];
+        }
+        const bf16x8 b0 = cvt_fp4x8(ws.q[s][0][i], sc0);
+        acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[cur].b, b0, acc[0][0], 0, 0, 0);
+        acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[cur].b, b0, acc[0][1], 0, 0, 0);
+        if (NMAT == 2) {
+          const bf16x8 b1 = cvt_fp4x8(ws.q[s][1][i], sc1);
+          acc[NMAT - 1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[cur].b, b1, acc[NMAT - 1][0], 0, 0, 0);
+          acc[NMAT - 1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[cur].b, b1, acc[NMAT - 1][1], 0, 0, 0);
+        }
+      }
+    }
+    float* rbuf = red + (size_t)par * 4 * NV * 64;
+    if (live) {
+#pragma unroll
+      for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rbuf[(wv * NV + m * 4 + i) * 64 + lane] = acc[m][0][i] + acc[m][1][i];
+    }
+    __syncthreads();
+    if (wv == (tile & 3) && live) {
+      const int r = tile * 16 + n;  // output feature
+      float v[NMAT][4];
+#pragma unroll
+      for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int o = m * 4 + i;
+          v[m][i] = ((rbuf[(0 * NV + o) * 64 + lane] + rbuf[(1 * NV + o) * 64 + lane]) +
+                     rbuf[(2 * NV + o) * 64 + lane]) + rbuf[(3 * NV + o) * 64 + lane];
+        }
+      if (r < a.N) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int t = g * 4 + i;  // token slot within the group
+          if (t < gcount) {
+            const size_t p = (size_t)(base + t);
+            if (NMAT == 2) {
+              uint16_t hi, lo;
+              split_bf16(moe_activation(v[0][i] + ws.b0, v[NMAT - 1][i] + ws.b1, a.act_type), hi, lo);
+              uint16_t* o = a.act_out + (p * (size_t)(a.N >> 5) + (r >> 5)) * 64 + (r & 31);
+              o[0] = hi;
+              o[32] = lo;
+            } else {
+              a.y_out[p * (size_t)a.N + r] = v[0][i] + ws.b0;
+            }
+          }
+        }
+      }
+    }
+  };
+
+  // Prefetches are unconditional (past the last tile they re-read it), so that the
+  // number of loads in flight behind a register set is the same on every path and
+  // the waits in front of the matrix cores stay partial.
+  WSet wa, wb;
+  load_tile(wa, t_begin);
+  __syncthreads();  // (the compiler waits for the LDS copies before the barrier)
+  int par = 0;
+  for (int t = t_begin; t < t_end; t += 2) {
+    load_tile(wb, min(t + 1, t_end - 1));
+    compute_tile(wa, t, par);
+    load_tile(wa, min(t + 2, t_end - 1));
+    if (t + 1 < t_end) compute_tile(wb, t + 1, par ^ 1);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Generic fallback for contraction lengths above 3072: one 16-row tile per
+// workgroup, the four waves striding over K steps, activation fragments read
+// straight from global memory (L2), 16 tokens per pass.
+template <int NMAT>
+__global__ __launch_bounds__(256) void expert_generic_kernel(ExpertStreamArgs a) {
+  const WorkDesc* wd = a.desc + blockIdx.y;
+  const int Te = wd->Te;
+  if (Te == 0) return;
+  const int base = wd->base;
   const int R = blockIdx.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
   const int nblk = a.nblk;
-  const size_t tile0 = (size_t)R * nblk * 16;
-  const uint4* q0 = (NMAT == 2 ? w.q_gate : w.q_down) + tile0;
-  const uint8_t* s0 = (NMAT == 2 ? w.s_gate : w.s_down) + tile0;
-  const uint4* q1 = w.q_up + tile0;
-  const uint8_t* s1 = w.s_up + tile0;
+  const size_t tile0 = (size_t)R * nblk * 16 + n;
+  const uint4* q0 = (NMAT == 2 ? wd->w.q_gate : wd->w.q_down) + tile0;
+  const uint8_t* s0 = (NMAT == 2 ? wd->w.s_gate : wd->w.s_down) + tile0;
+  const uint4* q1 = wd->w.q_up + tile0;
+  const uint8_t* s1 = wd->w.s_up + tile0;
   const int nsteps = (nblk + 3) >> 2;
+  __shared__ float red[3][NMAT * 4][64];
 
-  __shared__ float red[3][MT * NMAT * 4][64];
-
-  for (int mbase = 0; mbase < Te; mbase += 16 * MT) {
-    floatx4 acc[MT][NMAT];
-    size_t arow[MT];
-    bool av[MT];
+  for (int mbase = 0; mbase < Te; mbase += 16) {
+    floatx4 acc[NMAT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-      for (int m = 0; m < NMAT; ++m) acc[mt][m] = floatx4{0.f, 0.f, 0.f, 0.f};
-      const int idx = mbase + mt * 16 + n;
-      av[mt] = idx < Te;
-      const int row = av[mt] ? (a.list_row ? a.list_row[base + idx] : base + idx) : 0;
-      arow[mt] = (size_t)row * nblk * 8;
-    }
-    const int mlive = min(MT, (Te - mbase + 15) >> 4);  // wave-uniform
-
+    for (int m = 0; m < NMAT; ++m) acc[m] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const int idx = min(mbase + n, Te - 1);  // lanes past the last token re-read it; outputs unused
+    const int row = a.list_row ? a.list_row[base + idx] : base + idx;
+    const uint4* ap = a.A + (size_t)row * nblk * 8;
     for (int j = wv; j < nsteps; j += 4) {
       const int kb = 4 * j + g;
-      const bool kv = kb < nblk;
-      uint4 qa = make_uint4(0, 0, 0, 0), qb = make_uint4(0, 0, 0, 0);
-      float sa = 0.0f, sb = 0.0f;
-      if (kv) {
-        qa = q0[kb * 16 + n];
-        sa = e8m0_scale(s0[kb * 16 + n]);
-        if (NMAT == 2) {
-          qb = q1[kb * 16 + n];
-          sb = e8m0_scale(s1[kb * 16 + n]);
-        }
+      const int kbc = min(kb, nblk - 1);
+      const uint4 qa = q0[kbc * 16];
+      const uint32_t sa = s0[kbc * 16];
+      uint4 qb = qa;
+      uint32_t sbv = sa;
+      if (NMAT == 2) {
+        qb = q1[kbc * 16];
+        sbv = s1[kbc * 16];
       }
-      U4B8 ah[MT][4], al[MT][4];
+      U4B8 af[8];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        if (mt < mlive) {
-          if (kv && av[mt]) {
-            const uint4* ap = a.A + arow[mt] + (size_t)kb * 8;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              ah[mt][i].u = ap[i];
-              al[mt][i].u = ap[4 + i];
-            }
-          } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              ah[mt][i].u = make_uint4(0, 0, 0, 0);
-              al[mt][i].u = make_uint4(0, 0, 0, 0);
-            }
-          }
-        }
-      }
-      const uint32_t qaw[4] = {qa.x, qa.y, qa.z, qa.w};
-      const uint32_t qbw[4] = {qb.x, qb.y, qb.z, qb.w};
+      for (int i = 0; i < 8; ++i) af[i].u = ap[(size_t)kbc * 8 + i];
+      const float sc0 = kb < nblk ? e8m0_scale(sa) : 0.0f;
+      const float sc1 = kb < nblk ? e8m0_scale(sbv) : 0.0f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const bf16x8 b0 = cvt_fp4x8(qaw[i], sa);
-        bf16x8 b1;
-        if (NMAT == 2) b1 = cvt_fp4x8(qbw[i], sb);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          if (mt < mlive) {
-            acc[mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[mt][i].b, b0, acc[mt][0], 0, 0, 0);
-            acc[mt][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[mt][i].b, b0, acc[mt][0], 0, 0, 0);
-            if (NMAT == 2) {
-              acc[mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[mt][i].b, b1, acc[mt][1], 0, 0, 0);
-              acc[mt][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[mt][i].b, b1, acc[mt][1], 0, 0, 0);
-            }
-          }
+        const bf16x8 b0 = cvt_fp4x8(u4_word(qa, i), sc0);
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i].b, b0, acc[0], 0, 0, 0);
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[4 + i].b, b0, acc[0], 0, 0, 0);
+        if (NMAT == 2) {
+          const bf16x8 b1 = cvt_fp4x8(u4_word(qb, i), sc1);
+          acc[NMAT - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i].b, b1, acc[NMAT - 1], 0, 0, 0);
+          acc[NMAT - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[4 + i].b, b1, acc[NMAT - 1], 0, 0, 0);
         }
       }
     }
-
-    // Sum the four waves' K slices (fixed order: wave 0 + 1 + 2 + 3).
     if (wv > 0) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-        for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) red[wv - 1][(mt * NMAT + m) * 4 + i][lane] = acc[mt][m][i];
+        for (int i = 0; i < 4; ++i) red[wv - 1][m * 4 + i][lane] = acc[m][i];
     }
     __syncthreads();
     if (wv == 0) {
-      const int r = R * 16 + n;  // output feature
+      const int r = R * 16 + n;
+      const ExpertW& w = wd->w;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        if (mt < mlive) {
+      for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-          for (int m = 0; m < NMAT; ++m)
+        for (int i = 0; i < 4; ++i) {
+          const int o = m * 4 + i;
+          acc[m][i] = ((acc[m][i] + red[0][o][lane]) + red[1][o][lane]) + red[2][o][lane];
+        }
+      if (r < a.N) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int o = (mt * NMAT + m) * 4 + i;
-              acc[mt][m][i] = ((acc[mt][m][i] + red[0][o][lane]) + red[1][o][lane]) + red[2][o][lane];
-            }
-          if (r < a.N) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int idx = mbase + mt * 16 + g * 4 + i;  // token within this expert
-              if (idx < Te) {
-                const size_t p = (size_t)(base + idx);
-                if (NMAT == 2) {
-                  const float gate_v = acc[mt][0][i] + (w.b_gate ? w.b_gate[r] : 0.0f);
-                  const float up_v = acc[mt][1][i] + (w.b_up ? w.b_up[r] : 0.0f);
-                  uint16_t hi, lo;
-                  split_bf16(moe_activation(gate_v, up_v, a.act_type), hi, lo);
-                  uint16_t* o = a.act_out + (p * (size_t)(a.N >> 5) + (r >> 5)) * 64 + (r & 31);
-                  o[0] = hi;
-                  o[32] = lo;
-                } else {
-                  a.y_out[p * (size_t)a.N + r] = acc[mt][0][i] + (w.b_down ? w.b_down[r] : 0.0f);
-                }
-              }
+        for (int i = 0; i < 4; ++i) {
+          const int t = mbase + g * 4 + i;
+          if (t < Te) {
+            const size_t p = (size_t)(base + t);
+            if (NMAT == 2) {
+              const float gate_v = acc[0][i] + (w.b_gate ? w.b_gate[r] : 0.0f);
+              const float up_v = acc[NMAT - 1][i] + (w.b_up ? w.b_up[r] : 0.0f);
+              uint16_t hi, lo;
+              split_bf16(moe_activation(gate_v, up_v, a.act_type), hi, lo);
+              uint16_t* o = a.act_out + (p * (size_t)(a.N >> 5) + (r >> 5)) * 64 + (r & 31);
+              o[0] = hi;
+              o[32] = lo;
+            } else {
+              a.y_out[p * (size_t)a.N + r] = acc[0][i] + (w.b_down ? w.b_down[r] : 0.0f);
             }
           }
         }

@@ -3,6 +3,7 @@
 // (histogram -> prefix scan -> ordered scatter) and the weighted combine.
 #pragma once
 #include "common.h"
+#include "expert_stream_kernel.h"
 
 namespace csk {
 
@@ -188,26 +189,52 @@ __global__ __launch_bounds__(256) void dispatch_count_kernel(const int* __restri
 // (moe_weight_fetch_node.h:31-60).
 __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
     const int* __restrict__ ids, const float* __restrict__ pairs, int P, int k, int E,
-    const int* __restrict__ counts, int* __restrict__ offsets, int* __restrict__ active,
-    int* __restrict__ n_active, int* __restrict__ list_tok, float* __restrict__ list_w,
+    const int* __restrict__ counts, const ExpertW* __restrict__ ew, int* __restrict__ offsets,
+    WorkDesc* __restrict__ desc, int* __restrict__ list_tok, float* __restrict__ list_w,
     int* __restrict__ pos_of_slot) {
   const int e = blockIdx.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   __shared__ int sh[8];
-  int c = (threadIdx.x < e) ? counts[threadIdx.x] : 0;  // E <= 256 = blockDim
+  __shared__ int cnt[kMaxExperts], act_e[kMaxExperts], act_off[kMaxExperts];
+  const int mine = (threadIdx.x < E) ? counts[threadIdx.x] : 0;  // E <= 256 = blockDim
+  int c = (threadIdx.x < e) ? mine : 0;
   c = (int)wave_sum((float)c);
   if (lane == 0) sh[wv] = c;
+  if (e == 0) cnt[threadIdx.x] = mine;
   __syncthreads();
   const int off = sh[0] + sh[1] + sh[2] + sh[3];
-  if (e == 0 && threadIdx.x == 0) {
-    int run = 0, na = 0;
-    for (int i = 0; i < E; ++i) {
-      offsets[i] = run;
-      if (counts[i] > 0) active[na++] = i;
-      run += counts[i];
+  if (e == 0) {
+    // workgroup 0 publishes the scan and the work descriptors of the active experts
+    __shared__ int na_sh;
+    if (threadIdx.x == 0) {
+      int run = 0, na = 0;
+      for (int i = 0; i < E; ++i) {
+        offsets[i] = run;
+        if (cnt[i] > 0) {
+          act_e[na] = i;
+          act_off[na] = run;
+          ++na;
+        }
+        run += cnt[i];
+      }
+      offsets[E] = run;
+      na_sh = na;
     }
-    offsets[E] = run;
-    *n_active = na;
+    __syncthreads();
+    if (threadIdx.x < E) {
+      WorkDesc d;
+      if ((int)threadIdx.x < na_sh) {
+        d.e = act_e[threadIdx.x];
+        d.Te = cnt[d.e];
+        d.base = act_off[threadIdx.x];
+        d.pad = 0;
+        d.w = ew[d.e];
+      } else {
+        d.e = 0, d.Te = 0, d.base = 0, d.pad = 0;
+        d.w = ExpertW{};
+      }
+      desc[threadIdx.x] = d;
+    }
   }
   int base = off;
   for (int p0 = 0; p0 < P; p0 += 256) {
