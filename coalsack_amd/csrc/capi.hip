@@ -59,6 +59,10 @@ int dev_alloc(T** p, size_t count) {
 
 inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 
+// Above this many token-expert assignments the token-group list of the
+// weight-streaming kernel is not built.
+constexpr int64_t kStreamMaxP = 2048;
+
 // ---- workspace shared by every layer (single stream, one call at a time) --
 struct Workspace {
   int64_t T = 0, E = 0, k = 0, H = 0, F = 0;
@@ -71,6 +75,8 @@ struct Workspace {
   int* counts = nullptr;    // [E]
   int* offsets = nullptr;   // [E+1]
   WorkDesc* desc = nullptr; // [E] work descriptors of the active experts
+  int* vlist = nullptr;     // [2 * P] token groups of the streaming kernel
+  int* nv = nullptr;        // [1]
   int* list_tok = nullptr;  // [P]
   float* list_w = nullptr;  // [P]
   int* pos = nullptr;       // [P]
@@ -80,7 +86,7 @@ struct Workspace {
   int* n_tiles = nullptr;
 
   void release() {
-    void* ps[] = {xn, xs, xg, logits, pairs, ids, counts, offsets, desc,
+    void* ps[] = {xn, xs, xg, logits, pairs, ids, counts, offsets, desc, vlist, nv,
                   list_tok, list_w, pos, act, y, tiles, n_tiles};
     for (void* p : ps)
       if (p) (void)hipFree(p);
@@ -106,6 +112,8 @@ struct Workspace {
     WS_ALLOC(counts, (size_t)nE);
     WS_ALLOC(offsets, (size_t)nE + 1);
     WS_ALLOC(desc, (size_t)nE);
+    WS_ALLOC(vlist, 2 * P);
+    WS_ALLOC(nv, 1);
     WS_ALLOC(list_tok, P);
     WS_ALLOC(list_w, P);
     WS_ALLOC(pos, P);
@@ -282,26 +290,26 @@ int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, in
   int rc = check_launch("dispatch_count_kernel");
   if (rc != CSK_OK) return rc;
   dispatch_scatter_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(
-      ids, pairs, (int)P, (int)k, (int)E, ws.counts, ew, ws.offsets, ws.desc, ws.list_tok,
-      ws.list_w, ws.pos);
+      ids, pairs, (int)P, (int)k, (int)E, ws.counts, ew, ws.offsets, ws.desc,
+      P <= kStreamMaxP ? ws.vlist : nullptr, ws.nv, ws.list_tok, ws.list_w, ws.pos);
   return check_launch("dispatch_scatter_kernel");
 }
 
 template <int NMAT>
-int launch_stream(ExpertStreamArgs a, int64_t max_active, int64_t T) {
-  if (a.nblk > 96) {  // contraction length above 3072
+int launch_stream(ExpertStreamArgs a, int64_t max_active, int64_t P, Workspace& ws) {
+  (void)max_active;
+  if (a.nblk > 96 || P > kStreamMaxP) {  // contraction length above 3072, or a large batch
     expert_generic_kernel<NMAT><<<dim3((unsigned)a.ntile, (unsigned)max_active), 256, 0, g_stream>>>(a);
     return check_launch("expert_generic_kernel");
   }
-  constexpr int G = 4;
-  // enough workgroups for two per compute unit, each walking through consecutive tiles
-  const int64_t want = 2 * (int64_t)std::max(g_cus, 1);
-  int64_t chunks = std::min<int64_t>(a.ntile, std::max<int64_t>(1, cdiv(want, max_active)));
-  a.tiles_per_wg = (int)cdiv(a.ntile, chunks);
-  chunks = cdiv(a.ntile, a.tiles_per_wg);
-  const dim3 grid((unsigned)chunks, (unsigned)max_active, (unsigned)cdiv(T, G));
-  const size_t lds = (size_t)G * a.nblk * 128 + 2 * 4 * NMAT * 4 * 64 * sizeof(float);
-  expert_stream_kernel<NMAT, G><<<grid, 256, lds, g_stream>>>(a);
+  constexpr int G = kStreamG;
+  a.vlist = ws.vlist;
+  a.nv = ws.nv;
+  // two workgroups per compute unit, but never more than the work units there can be
+  const int64_t npair = NMAT == 2 ? a.ntile : (a.ntile + 1) / 2;
+  const int64_t nwg = std::min<int64_t>(2 * (int64_t)std::max(g_cus, 1), P * npair);
+  const size_t lds = (size_t)G * a.nblk * 128 + 2 * 4 * 8 * 64 * sizeof(float);
+  expert_stream_kernel<NMAT == 2 ? 0 : 1, G><<<dim3((unsigned)nwg), 256, lds, g_stream>>>(a);
   return check_launch("expert_stream_kernel");
 }
 
@@ -325,7 +333,7 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   a.act_out = ws.act;
   a.y_out = nullptr;
   if (timed) mark(CSK_STAGE_GATEUP);
-  int rc = launch_stream<2>(a, max_active, T);
+  int rc = launch_stream<2>(a, max_active, P, ws);
   if (rc != CSK_OK) return rc;
   if (timed) mark(CSK_STAGE_DOWN);
   // down
@@ -336,7 +344,7 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   a.ntile = (int)cdiv(H, 16);
   a.act_out = nullptr;
   a.y_out = ws.y;
-  return launch_stream<1>(a, max_active, T);
+  return launch_stream<1>(a, max_active, P, ws);
 }
 
 int launch_combine(const float* y, const float* pairs, const int* pos, const float* residual,
@@ -695,18 +703,33 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
   if (rc != CSK_OK) return rc;
   const int64_t P = T * L->k;
   const bool norm = (flags & CSK_FWD_RMSNORM) != 0;
-  mark(CSK_STAGE_PREP);
-  rc = launch_prep(hidden, norm ? L->norm_w : nullptr, L->eps, norm ? ws.xn : nullptr, ws.xs, T,
-                   L->H, nullptr, nullptr);
-  if (rc != CSK_OK) return rc;
   const float* xr = norm ? ws.xn : hidden;
-  mark(CSK_STAGE_ROUTER);
-  rc = launch_router(xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, T, L->E, L->H, L->k,
-                     L->sigmoid, ws.logits, ws.pairs, ws.ids);
-  if (rc != CSK_OK) return rc;
-  mark(CSK_STAGE_DISPATCH);
-  rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, L->ew_dev, ws);
-  if (rc != CSK_OK) return rc;
+  if (P <= 1024 && T <= 64) {
+    // small batch: prologue + logits in one launch, top-k + dispatch in another
+    mark(CSK_STAGE_PREP);
+    mark(CSK_STAGE_ROUTER);
+    router_prep_logits_kernel<<<dim3((unsigned)(L->E + 4), (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
+        hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, ws.xs, L->gate_w,
+        L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
+    if ((rc = check_launch("router_prep_logits_kernel")) != CSK_OK) return rc;
+    mark(CSK_STAGE_DISPATCH);
+    route_small_kernel<<<dim3(1), 1024, 0, g_stream>>>(
+        ws.logits, ws.pairs, ws.ids, (int)T, (int)L->E, (int)L->k, L->sigmoid, L->ew_dev, ws.counts,
+        ws.offsets, ws.desc, ws.vlist, ws.nv, ws.list_tok, ws.list_w, ws.pos);
+    if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
+  } else {
+    mark(CSK_STAGE_PREP);
+    rc = launch_prep(hidden, norm ? L->norm_w : nullptr, L->eps, norm ? ws.xn : nullptr, ws.xs, T,
+                     L->H, nullptr, nullptr);
+    if (rc != CSK_OK) return rc;
+    mark(CSK_STAGE_ROUTER);
+    rc = launch_router(xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, T, L->E, L->H, L->k,
+                       L->sigmoid, ws.logits, ws.pairs, ws.ids);
+    if (rc != CSK_OK) return rc;
+    mark(CSK_STAGE_DISPATCH);
+    rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, L->ew_dev, ws);
+    if (rc != CSK_OK) return rc;
+  }
   const uint16_t* xa = ws.xs;
   const int* list_row = ws.list_tok;
   if (L->wbf) {

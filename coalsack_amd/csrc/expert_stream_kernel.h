@@ -33,6 +33,8 @@ struct WorkDesc {
 // unconditional.
 struct ExpertStreamArgs {
   const WorkDesc* desc;
+  const int* vlist;      // [2 * nv]: (expert slot, first token) of each group of kStreamG tokens
+  const int* nv;         // number of such groups
   const int* list_row;   // packed position -> row of A; null: row = packed position
   const uint4* A;        // [rows][nblk][8] x 16 B: 32 bf16 hi then 32 bf16 lo per block
   int nblk;              // K / 32
@@ -84,176 +86,185 @@ __device__ __forceinline__ uint32_t u4_word(const uint4& v, int i) {
 // ---------------------------------------------------------------------------
 // Persistent, software-pipelined kernel (K <= 3072).
 //
-// NMAT = 2: gate and up tiles together, SwiGLU epilogue.  NMAT = 1: down.
-// G = tokens contracted per workgroup (rows 0..G-1 of the 16-row MFMA tile);
-// token group blockIdx.z of expert slot blockIdx.y, tiles
-// [blockIdx.x * tiles_per_wg, ...).
+// MODE 0: a work unit is the pair (gate tile R, up tile R), SwiGLU epilogue.
+// MODE 1: a work unit is the pair of down tiles (2R, 2R+1).
+// G = tokens contracted per pass (rows 0..G-1 of the 16-row MFMA tile).
 //
+// The work -- (token group of an expert) x (tile pair) -- is cut into gridDim.x
+// equal contiguous ranges, so the load is balanced whatever the routing was.
 // Memory-level parallelism bounds this kernel, so it never lets the memory
-// queue drain: the group's activation rows are copied once into LDS
-// (global_load_lds, no registers), and while the matrix cores work on tile t
-// from one register set the 24 weight loads of tile t+1 -- all of a wave's K
+// queue drain: a group's activation rows are copied once into LDS
+// (global_load_lds, no registers), and while the matrix cores work on unit t
+// from one register set the weight loads of unit t+1 -- all of a wave's K
 // steps, issued back to back from clamped addresses so that no wait separates
 // them -- are already in flight into the other set.  The four waves split K;
-// their partial sums meet in double-buffered LDS (one barrier per tile) in the
-// fixed order w0 + w1 + w2 + w3, and wave t mod 4 finishes tile t.
-template <int NMAT, int G>
+// their partial sums meet in double-buffered LDS (one barrier per unit) in the
+// fixed order w0 + w1 + w2 + w3, and wave t mod 4 finishes unit t.
+template <int MODE, int G>
 __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) {
   constexpr int NS = 6;  // K steps per wave: 4 waves x 6 x 128 = 3072 elements
-  constexpr int NV = NMAT * 4;
+  constexpr int NV = 8;  // accumulator floats per lane per unit
   extern __shared__ __align__(16) unsigned char smem[];
   const int nblk = a.nblk;
   const int row_u4 = nblk * 8;                   // uint4 per activation row
   uint4* As = reinterpret_cast<uint4*>(smem);    // [G][row_u4]
   float* red = reinterpret_cast<float*>(smem + (size_t)G * row_u4 * 16);  // [2][4][NV][64]
 
-  const WorkDesc* wd = a.desc + blockIdx.y;
-  const int Te = wd->Te;
-  const int gbase = blockIdx.z * G;
-  if (gbase >= Te) return;
-  const int gcount = min(G, Te - gbase);
-  const int t_begin = blockIdx.x * a.tiles_per_wg;
-  const int t_end = min(a.ntile, t_begin + a.tiles_per_wg);
-  if (t_begin >= t_end) return;
-  const int base = wd->base + gbase;
+  const int npair = MODE == 0 ? a.ntile : (a.ntile + 1) >> 1;
+  const long total = (long)(*a.nv) * npair;
+  const long w_begin = total * blockIdx.x / gridDim.x;
+  const long w_end = total * (blockIdx.x + 1) / gridDim.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
-  const CSK_GLOBAL u32x4* q0 = as_global(reinterpret_cast<const u32x4*>(NMAT == 2 ? wd->w.q_gate : wd->w.q_down)) + n;
-  const CSK_GLOBAL uint8_t* s0 = as_global(NMAT == 2 ? wd->w.s_gate : wd->w.s_down) + n;
-  const CSK_GLOBAL u32x4* q1 = as_global(reinterpret_cast<const u32x4*>(wd->w.q_up)) + n;
-  const CSK_GLOBAL uint8_t* s1 = as_global(wd->w.s_up) + n;
-  const CSK_GLOBAL float* bp0 = as_global(NMAT == 2 ? wd->w.b_gate : wd->w.b_down);
-  const CSK_GLOBAL float* bp1 = as_global(wd->w.b_up);
-
-  // activation rows of this token group -> LDS
-#pragma unroll
-  for (int rr = 0; rr < G; ++rr) {
-    if (rr < gcount) {
-      const int row = a.list_row ? a.list_row[base + rr] : base + rr;
-      const uint4* src = a.A + (size_t)row * row_u4;
-      for (int c0 = wv * 64; c0 < row_u4; c0 += 256) {
-        if (c0 + lane < row_u4)
-          __builtin_amdgcn_global_load_lds(
-              src + c0 + lane,
-              reinterpret_cast<__attribute__((address_space(3))) uint4*>(
-                  reinterpret_cast<uintptr_t>(As + rr * row_u4 + c0)),
-              16, 0, 0);
-      }
-    }
-  }
+  const int arow = min(n, G - 1) * row_u4;  // lanes past G re-read a live row; their outputs are unused
 
   struct WSet {
-    u32x4 q[NS][NMAT];
-    uint32_t sb[NS][NMAT];
+    u32x4 q[NS][2];
+    uint32_t sb[NS][2];
     float b0, b1;
   };
-  auto load_tile = [&](WSet& ws, int tile) {
-    const size_t te = (size_t)tile * nblk * 16;
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      const int kb = min(4 * (wv + 4 * s) + g, nblk - 1);
-      ws.q[s][0] = q0[te + kb * 16];
-      ws.sb[s][0] = s0[te + kb * 16];
-      if (NMAT == 2) {
-        ws.q[s][1] = q1[te + kb * 16];
-        ws.sb[s][1] = s1[te + kb * 16];
-      }
-    }
-    const int r = min(tile * 16 + n, a.N - 1);
-    ws.b0 = bp0[r];  // bias pointers are never null here (an absent bias is a zero vector)
-    if (NMAT == 2) ws.b1 = bp1[r];
-  };
 
-  const int arow = min(n, G - 1) * row_u4;  // lanes past G re-read a live row; their outputs are unused
-  const bool live = g * 4 < gcount;         // this lane's accumulator rows belong to live tokens
+  int par = 0;
+  for (long it = w_begin; it < w_end;) {
+    const int v = (int)(it / npair);
+    const int p_begin = (int)(it - (long)v * npair);
+    const int p_end = (int)min((long)npair, p_begin + (w_end - it));
+    it += p_end - p_begin;
+    const WorkDesc* wd = a.desc + a.vlist[2 * v];
+    const int gbase = a.vlist[2 * v + 1];
+    const int gcount = min(G, wd->Te - gbase);
+    const int base = wd->base + gbase;
+    const CSK_GLOBAL u32x4* q0 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_gate : wd->w.q_down)) + n;
+    const CSK_GLOBAL uint8_t* s0 = as_global(MODE == 0 ? wd->w.s_gate : wd->w.s_down) + n;
+    const CSK_GLOBAL u32x4* q1 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_up : wd->w.q_down)) + n;
+    const CSK_GLOBAL uint8_t* s1 = as_global(MODE == 0 ? wd->w.s_up : wd->w.s_down) + n;
+    const CSK_GLOBAL float* bp0 = as_global(MODE == 0 ? wd->w.b_gate : wd->w.b_down);
+    const CSK_GLOBAL float* bp1 = as_global(MODE == 0 ? wd->w.b_up : wd->w.b_down);
 
-  auto compute_tile = [&](const WSet& ws, int tile, int par) {
-    floatx4 acc[NMAT][2];  // [matrix][hi, lo term]: independent accumulation chains
+    // activation rows of this token group -> LDS (every wave is past its last
+    // read of the previous group: it has crossed that unit's barrier)
 #pragma unroll
-    for (int m = 0; m < NMAT; ++m) acc[m][0] = acc[m][1] = floatx4{0.f, 0.f, 0.f, 0.f};
-    U4B8 ahi[2], alo[2];  // activation fragments run one quarter-step ahead of the matrix cores
-    {
-      const int kb0 = min(4 * wv + g, nblk - 1);
-      ahi[0].u = As[arow + kb0 * 8];
-      alo[0].u = As[arow + kb0 * 8 + 4];
-    }
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      const int kb = 4 * (wv + 4 * s) + g;
-      const bool kvs = kb < nblk;
-      const float sc0 = kvs ? e8m0_scale(ws.sb[s][0]) : 0.0f;
-      const float sc1 = (NMAT == 2 && kvs) ? e8m0_scale(ws.sb[s][1]) : 0.0f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int cur = (s * 4 + i) & 1, nxt = cur ^ 1;
-        if (s * 4 + i + 1 < NS * 4) {
-          const int s2 = (s * 4 + i + 1) >> 2, i2 = (s * 4 + i + 1) & 3;
-          const int kb2 = min(4 * (wv + 4 * s2) + g, nblk - 1);
-          ahi[nxt].u = As[arow + kb2 * 8 + i2];
-          alo[nxt].u = As[arow + kb2 * 8 + 4 + i2];
-        }
-        const bf16x8 b0 = cvt_fp4x8(ws.q[s][0][i], sc0);
-        acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[cur].b, b0, acc[0][0], 0, 0, 0);
-        acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[cur].b, b0, acc[0][1], 0, 0, 0);
-        if (NMAT == 2) {
-          const bf16x8 b1 = cvt_fp4x8(ws.q[s][1][i], sc1);
-          acc[NMAT - 1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[cur].b, b1, acc[NMAT - 1][0], 0, 0, 0);
-          acc[NMAT - 1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[cur].b, b1, acc[NMAT - 1][1], 0, 0, 0);
+    for (int rr = 0; rr < G; ++rr) {
+      if (rr < gcount) {
+        const int row = a.list_row ? a.list_row[base + rr] : base + rr;
+        const uint4* src = a.A + (size_t)row * row_u4;
+        for (int c0 = wv * 64; c0 < row_u4; c0 += 256) {
+          if (c0 + lane < row_u4)
+            __builtin_amdgcn_global_load_lds(
+                src + c0 + lane,
+                reinterpret_cast<__attribute__((address_space(3))) uint4*>(
+                    reinterpret_cast<uintptr_t>(As + rr * row_u4 + c0)),
+                16, 0, 0);
         }
       }
     }
-    float* rbuf = red + (size_t)par * 4 * NV * 64;
-    if (live) {
+
+    // tiles of a unit: (R, R) for gate/up, (2R, 2R+1) for down
+    auto load_unit = [&](WSet& ws, int unit) {
+      const int ta = MODE == 0 ? unit : 2 * unit;
+      const int tb = MODE == 0 ? unit : min(2 * unit + 1, a.ntile - 1);
+      const size_t ea = (size_t)ta * nblk * 16, eb = (size_t)tb * nblk * 16;
 #pragma unroll
-      for (int m = 0; m < NMAT; ++m)
+      for (int s = 0; s < NS; ++s) {
+        const int kb = min(4 * (wv + 4 * s) + g, nblk - 1);
+        ws.q[s][0] = q0[ea + kb * 16];
+        ws.sb[s][0] = s0[ea + kb * 16];
+        ws.q[s][1] = q1[eb + kb * 16];
+        ws.sb[s][1] = s1[eb + kb * 16];
+      }
+      ws.b0 = bp0[min(ta * 16 + n, a.N - 1)];  // bias pointers are never null (absent bias = zero vector)
+      ws.b1 = bp1[min(tb * 16 + n, a.N - 1)];
+    };
+    const bool live = g * 4 < gcount;  // this lane's accumulator rows belong to live tokens
+
+    auto compute_unit = [&](const WSet& ws, int unit) {
+      floatx4 acc[2][2];  // [tile of the pair][hi, lo term]: independent accumulation chains
 #pragma unroll
-        for (int i = 0; i < 4; ++i) rbuf[(wv * NV + m * 4 + i) * 64 + lane] = acc[m][0][i] + acc[m][1][i];
-    }
-    __syncthreads();
-    if (wv == (tile & 3) && live) {
-      const int r = tile * 16 + n;  // output feature
-      float v[NMAT][4];
+      for (int m = 0; m < 2; ++m) acc[m][0] = acc[m][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+      U4B8 ahi[2], alo[2];  // activation fragments run one quarter-step ahead of the matrix cores
+      {
+        const int kb0 = min(4 * wv + g, nblk - 1);
+        ahi[0].u = As[arow + kb0 * 8];
+        alo[0].u = As[arow + kb0 * 8 + 4];
+      }
 #pragma unroll
-      for (int m = 0; m < NMAT; ++m)
+      for (int s = 0; s < NS; ++s) {
+        const int kb = 4 * (wv + 4 * s) + g;
+        const bool kvs = kb < nblk;
+        const float sc0 = kvs ? e8m0_scale(ws.sb[s][0]) : 0.0f;
+        const float sc1 = kvs ? e8m0_scale(ws.sb[s][1]) : 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int o = m * 4 + i;
-          v[m][i] = ((rbuf[(0 * NV + o) * 64 + lane] + rbuf[(1 * NV + o) * 64 + lane]) +
-                     rbuf[(2 * NV + o) * 64 + lane]) + rbuf[(3 * NV + o) * 64 + lane];
+          const int cur = (s * 4 + i) & 1, nxt = cur ^ 1;
+          if (s * 4 + i + 1 < NS * 4) {
+            const int s2 = (s * 4 + i + 1) >> 2, i2 = (s * 4 + i + 1) & 3;
+            const int kb2 = min(4 * (wv + 4 * s2) + g, nblk - 1);
+            ahi[nxt].u = As[arow + kb2 * 8 + i2];
+            alo[nxt].u = As[arow + kb2 * 8 + 4 + i2];
+          }
+          const bf16x8 b0 = cvt_fp4x8(ws.q[s][0][i], sc0);
+          acc[0][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[cur].b, b0, acc[0][0], 0, 0, 0);
+          acc[0][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[cur].b, b0, acc[0][1], 0, 0, 0);
+          const bf16x8 b1 = cvt_fp4x8(ws.q[s][1][i], sc1);
+          acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[cur].b, b1, acc[1][0], 0, 0, 0);
+          acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[cur].b, b1, acc[1][1], 0, 0, 0);
         }
-      if (r < a.N) {
+      }
+      float* rbuf = red + (size_t)par * 4 * NV * 64;
+      par ^= 1;
+      if (live) {
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) rbuf[(wv * NV + m * 4 + i) * 64 + lane] = acc[m][0][i] + acc[m][1][i];
+      }
+      __syncthreads();
+      if (wv == (unit & 3) && live) {
+        float v2[2][4];
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int o = m * 4 + i;
+            v2[m][i] = ((rbuf[(0 * NV + o) * 64 + lane] + rbuf[(1 * NV + o) * 64 + lane]) +
+                        rbuf[(2 * NV + o) * 64 + lane]) + rbuf[(3 * NV + o) * 64 + lane];
+          }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int t = g * 4 + i;  // token slot within the group
           if (t < gcount) {
             const size_t p = (size_t)(base + t);
-            if (NMAT == 2) {
-              uint16_t hi, lo;
-              split_bf16(moe_activation(v[0][i] + ws.b0, v[NMAT - 1][i] + ws.b1, a.act_type), hi, lo);
-              uint16_t* o = a.act_out + (p * (size_t)(a.N >> 5) + (r >> 5)) * 64 + (r & 31);
-              o[0] = hi;
-              o[32] = lo;
+            if (MODE == 0) {
+              const int r = unit * 16 + n;  // output feature
+              if (r < a.N) {
+                uint16_t hi, lo;
+                split_bf16(moe_activation(v2[0][i] + ws.b0, v2[1][i] + ws.b1, a.act_type), hi, lo);
+                uint16_t* o = a.act_out + (p * (size_t)(a.N >> 5) + (r >> 5)) * 64 + (r & 31);
+                o[0] = hi;
+                o[32] = lo;
+              }
             } else {
-              a.y_out[p * (size_t)a.N + r] = v[0][i] + ws.b0;
+              const int ra = 2 * unit * 16 + n, rb = ra + 16;
+              if (ra < a.N) a.y_out[p * (size_t)a.N + ra] = v2[0][i] + ws.b0;
+              if (rb < a.N) a.y_out[p * (size_t)a.N + rb] = v2[1][i] + ws.b1;
             }
           }
         }
       }
-    }
-  };
+    };
 
-  // Prefetches are unconditional (past the last tile they re-read it), so that the
-  // number of loads in flight behind a register set is the same on every path and
-  // the waits in front of the matrix cores stay partial.
-  WSet wa, wb;
-  load_tile(wa, t_begin);
-  __syncthreads();  // (the compiler waits for the LDS copies before the barrier)
-  int par = 0;
-  for (int t = t_begin; t < t_end; t += 2) {
-    load_tile(wb, min(t + 1, t_end - 1));
-    compute_tile(wa, t, par);
-    load_tile(wa, min(t + 2, t_end - 1));
-    if (t + 1 < t_end) compute_tile(wb, t + 1, par ^ 1);
+    // Prefetches are unconditional (past the last unit they re-read it), so that the
+    // number of loads in flight behind a register set is the same on every path and
+    // the waits in front of the matrix cores stay partial.
+    WSet wa, wb;
+    load_unit(wa, p_begin);
+    __syncthreads();  // the LDS copies have landed (the compiler waits for them before the barrier)
+    for (int t = p_begin; t < p_end; t += 2) {
+      load_unit(wb, min(t + 1, p_end - 1));
+      compute_unit(wa, t);
+      load_unit(wa, min(t + 2, p_end - 1));
+      if (t + 1 < p_end) compute_unit(wb, t + 1);
+    }
   }
 }
 

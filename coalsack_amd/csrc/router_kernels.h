@@ -89,6 +89,107 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restr
   }
 }
 
+// --------------------------------------------- small batches: prologue + logits
+// One launch for small T: workgroups x in [0, E) compute the logits of one expert for
+// the four tokens of tile y (the four waves split H, so all loads of a row are in flight at
+// once); workgroups x in [E, E + 4) run the prologue of one token of tile y (RMSNorm, f32 copy,
+// bf16 hi/lo split).  With RMSNorm the expert workgroups recompute each token's
+// normalisation themselves -- 2 H flops per token -- instead of waiting for the
+// prologue.  Restates moe_router_node.h:161-167 and rmsnorm_node.h:62-83.
+__global__ __launch_bounds__(256) void router_prep_logits_kernel(
+    const float* __restrict__ hidden, const float* __restrict__ norm_w, float eps,
+    float* __restrict__ xn, uint16_t* __restrict__ xs, const float* __restrict__ g,
+    const float* __restrict__ b, float* __restrict__ logits, int T, int E, int H) {
+  __shared__ float part[2][4][4];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  if ((int)blockIdx.x >= E) {  // ---- prologue of token t (one of four per token tile)
+    const int t = (blockIdx.x - E) + 4 * blockIdx.y;
+    if (blockIdx.x - E >= 4 || t >= T) return;
+    const float* x = hidden + (size_t)t * H;
+    float den = 1.0f;
+    if (norm_w) {
+      float ss = 0.0f;
+      for (int d = threadIdx.x; d < H; d += 256) ss += x[d] * x[d];
+      ss = wave_sum(ss);
+      if (lane == 0) part[0][wv][0] = ss;
+      __syncthreads();
+      ss = (part[0][0][0] + part[0][1][0]) + (part[0][2][0] + part[0][3][0]);
+      den = sqrtf(ss / (float)H + eps);
+    }
+    for (int d = threadIdx.x; d < H; d += 256) {
+      float v = x[d];
+      if (norm_w) {
+        v = (v / den) * norm_w[d];
+        xn[(size_t)t * H + d] = v;
+      }
+      uint16_t hi, lo;
+      split_bf16(v, hi, lo);
+      uint16_t* o = xs + ((size_t)t * (H / 32) + (d >> 5)) * 64 + (d & 31);
+      o[0] = hi;
+      o[32] = lo;
+    }
+    return;
+  }
+  // ---- logits of expert e for four tokens (token tile blockIdx.y)
+  const int e = blockIdx.x;
+  const int H4 = H >> 2;
+  const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)e * H);
+  const float4* w4 = reinterpret_cast<const float4*>(norm_w);
+  const float bias = b ? b[e] : 0.0f;
+  {
+    const int t0 = blockIdx.y * 4;
+    float den[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    if (norm_w) {
+      float ss[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int c = threadIdx.x; c < H4; c += 256) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int t = min(t0 + i, T - 1);
+          const float4 xv = reinterpret_cast<const float4*>(hidden + (size_t)t * H)[c];
+          ss[i] += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float s = wave_sum(ss[i]);
+        if (lane == 0) part[0][wv][i] = s;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        den[i] = sqrtf(((part[0][0][i] + part[0][1][i]) + (part[0][2][i] + part[0][3][i])) / (float)H + eps);
+    }
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int c = threadIdx.x; c < H4; c += 256) {
+      const float4 gv = g4[c];
+      float4 wv4 = make_float4(1.f, 1.f, 1.f, 1.f);
+      if (norm_w) wv4 = w4[c];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = min(t0 + i, T - 1);
+        float4 xv = reinterpret_cast<const float4*>(hidden + (size_t)t * H)[c];
+        if (norm_w) {
+          xv.x = (xv.x / den[i]) * wv4.x;
+          xv.y = (xv.y / den[i]) * wv4.y;
+          xv.z = (xv.z / den[i]) * wv4.z;
+          xv.w = (xv.w / den[i]) * wv4.w;
+        }
+        acc[i] += xv.x * gv.x + xv.y * gv.y + xv.z * gv.z + xv.w * gv.w;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float s = wave_sum(acc[i]);
+      if (lane == 0) part[1][wv][i] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x < 4 && t0 + (int)threadIdx.x < T) {
+      const int i = threadIdx.x;
+      logits[(size_t)(t0 + i) * E + e] = ((part[1][0][i] + part[1][1][i]) + (part[1][2][i] + part[1][3][i])) + bias;
+    }
+  }
+}
+
 // ------------------------------------------------------------------- top-k
 // One wave per token.  Lane l holds the logits of experts l, l+64, l+128,
 // l+192; each of the k rounds finds the wave-wide maximum (ties -> lowest
@@ -190,8 +291,8 @@ __global__ __launch_bounds__(256) void dispatch_count_kernel(const int* __restri
 __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
     const int* __restrict__ ids, const float* __restrict__ pairs, int P, int k, int E,
     const int* __restrict__ counts, const ExpertW* __restrict__ ew, int* __restrict__ offsets,
-    WorkDesc* __restrict__ desc, int* __restrict__ list_tok, float* __restrict__ list_w,
-    int* __restrict__ pos_of_slot) {
+    WorkDesc* __restrict__ desc, int* __restrict__ vlist, int* __restrict__ nv,
+    int* __restrict__ list_tok, float* __restrict__ list_w, int* __restrict__ pos_of_slot) {
   const int e = blockIdx.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   __shared__ int sh[8];
@@ -219,6 +320,17 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
       }
       offsets[E] = run;
       na_sh = na;
+      // token groups of the weight-streaming kernel: (expert slot, first token)
+      int nvv = 0;
+      if (vlist) {
+        for (int u = 0; u < na; ++u)
+          for (int gb = 0; gb < cnt[act_e[u]]; gb += kStreamG) {
+            vlist[2 * nvv] = u;
+            vlist[2 * nvv + 1] = gb;
+            ++nvv;
+          }
+      }
+      *nv = nvv;
     }
     __syncthreads();
     if (threadIdx.x < E) {
@@ -254,6 +366,151 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
       pos_of_slot[p] = pos;
     }
     base += sh[4] + sh[5] + sh[6] + sh[7];
+  }
+}
+
+// ------------------------------------- small batches: top-k + dispatch, fused
+// One workgroup of 16 waves does, for P = T * k <= 1024 assignments, what
+// router_topk_kernel, dispatch_count_kernel and dispatch_scatter_kernel do in
+// three launches: top-k and weights per token (one wave per token), histogram,
+// exclusive scan, ordered scatter, work descriptors and token groups -- all
+// through LDS.
+__global__ __launch_bounds__(1024) void route_small_kernel(
+    const float* __restrict__ logits, float* __restrict__ pairs, int* __restrict__ ids_out, int T,
+    int E, int k, int sigmoid, const ExpertW* __restrict__ ew, int* __restrict__ counts,
+    int* __restrict__ offsets, WorkDesc* __restrict__ desc, int* __restrict__ vlist,
+    int* __restrict__ nv, int* __restrict__ list_tok, float* __restrict__ list_w,
+    int* __restrict__ pos_of_slot) {
+  __shared__ int ids[1024];
+  __shared__ float wts[1024];
+  __shared__ int cnt[kMaxExperts], off[kMaxExperts], act_e[kMaxExperts];
+  __shared__ int na_sh;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int P = T * k;
+  const float NEG = -__builtin_inff();
+  for (int t = wv; t < T; t += 16) {
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = lane + 64 * j;
+      v[j] = (e < E) ? logits[(size_t)t * E + e] : NEG;
+    }
+    float my_val = 0.0f, vmax = 0.0f;
+    int my_idx = 0;
+    for (int s = 0; s < k; ++s) {
+      float bv = v[0];
+      int bi = lane;
+#pragma unroll
+      for (int j = 1; j < 4; ++j) {
+        if (v[j] > bv) {
+          bv = v[j];
+          bi = lane + 64 * j;
+        }
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) {
+          bv = ov;
+          bi = oi;
+        }
+      }
+      if (s == 0) vmax = bv;
+      if (lane == s) {
+        my_val = bv;
+        my_idx = bi;
+      }
+      if ((bi & 63) == lane) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if ((bi >> 6) == j) v[j] = NEG;
+      }
+    }
+    float w;
+    if (sigmoid) {
+      w = 1.0f / (1.0f + expf(-my_val));
+    } else {
+      w = (lane < k) ? expf(my_val - vmax) : 0.0f;
+      float sum = 0.0f;
+      for (int s = 0; s < k; ++s) sum += __shfl(w, s, 64);  // slot order
+      const float inv = (sum > 0.0f) ? (1.0f / sum) : 0.0f;
+      w *= inv;
+    }
+    if (lane < k) {
+      reinterpret_cast<float2*>(pairs)[(size_t)t * k + lane] = make_float2((float)my_idx, w);
+      ids_out[t * k + lane] = my_idx;
+      ids[t * k + lane] = my_idx;
+      wts[t * k + lane] = w;
+    }
+  }
+  __syncthreads();
+  // histogram: wave wv counts experts wv, wv + 16, ... with ballots over the assignments
+  for (int e = wv; e < E; e += 16) {
+    int c = 0;
+    for (int p0 = 0; p0 < P; p0 += 64) {
+      const int p = p0 + lane;
+      c += __popcll(__ballot(p < P && ids[p] == e));
+    }
+    if (lane == 0) {
+      cnt[e] = c;
+      counts[e] = c;
+    }
+  }
+  __syncthreads();
+  // exclusive scan, active experts, token groups
+  if (threadIdx.x == 0) {
+    int run = 0, na = 0, nvv = 0;
+    for (int i = 0; i < E; ++i) {
+      const int c = cnt[i];
+      off[i] = run;
+      offsets[i] = run;
+      if (c > 0) {
+        for (int gb = 0; gb < c; gb += kStreamG) {
+          vlist[2 * nvv] = na;
+          vlist[2 * nvv + 1] = gb;
+          ++nvv;
+        }
+        act_e[na++] = i;
+      }
+      run += c;
+    }
+    offsets[E] = run;
+    na_sh = na;
+    *nv = nvv;
+  }
+  __syncthreads();
+  // ordered scatter: rank of an assignment = matches before it (ballot prefix)
+  for (int e = wv; e < E; e += 16) {
+    if (cnt[e] == 0) continue;
+    int basep = off[e];
+    for (int p0 = 0; p0 < P; p0 += 64) {
+      const int p = p0 + lane;
+      const bool hit = p < P && ids[p] == e;
+      const unsigned long long m = __ballot(hit);
+      if (hit) {
+        const int pos = basep + __popcll(m & ((1ull << lane) - 1ull));
+        list_tok[pos] = p / k;
+        list_w[pos] = wts[p];
+        pos_of_slot[p] = pos;
+      }
+      basep += __popcll(m);
+    }
+  }
+  if ((int)threadIdx.x < E) {
+    // work descriptor of active slot threadIdx.x
+    WorkDesc d;
+    if ((int)threadIdx.x < na_sh) {
+      d.e = act_e[threadIdx.x];
+      d.Te = cnt[d.e];
+      d.base = off[d.e];
+      d.pad = 0;
+      d.w = ew[d.e];
+    } else {
+      d.e = 0, d.Te = 0, d.base = 0, d.pad = 0;
+      d.w = ExpertW{};
+    }
+    desc[threadIdx.x] = d;
   }
 }
 
