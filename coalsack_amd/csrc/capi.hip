@@ -291,26 +291,42 @@ int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, in
   if (rc != CSK_OK) return rc;
   dispatch_scatter_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(
       ids, pairs, (int)P, (int)k, (int)E, ws.counts, ew, ws.offsets, ws.desc,
-      P <= kStreamMaxP ? ws.vlist : nullptr, ws.nv, ws.list_tok, ws.list_w, ws.pos);
+      P <= kStreamMaxP ? ws.vlist : nullptr, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w,
+      ws.pos);
   return check_launch("dispatch_scatter_kernel");
 }
 
+// Weight-streaming kernel for small batches (every expert sees few tokens, the
+// layer is HBM-bound); grouped GEMM otherwise.
 template <int NMAT>
-int launch_stream(ExpertStreamArgs a, int64_t max_active, int64_t P, Workspace& ws) {
-  (void)max_active;
-  if (a.nblk > 96 || P > kStreamMaxP) {  // contraction length above 3072, or a large batch
-    expert_generic_kernel<NMAT><<<dim3((unsigned)a.ntile, (unsigned)max_active), 256, 0, g_stream>>>(a);
-    return check_launch("expert_generic_kernel");
+int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspace& ws) {
+  if (T <= 64 && a.nblk <= 96) {
+    constexpr int G = kStreamG;
+    a.vlist = ws.vlist;
+    a.nv = ws.nv;
+    // two workgroups per compute unit, but never more than the work units there can be
+    const int64_t npair = NMAT == 2 ? a.ntile : (a.ntile + 1) / 2;
+    const int64_t nwg = std::min<int64_t>(2 * (int64_t)std::max(g_cus, 1), P * npair);
+    const size_t lds = (size_t)G * a.nblk * 128 + 2 * 4 * 8 * 64 * sizeof(float);
+    expert_stream_kernel<NMAT == 2 ? 0 : 1, G><<<dim3((unsigned)nwg), 256, lds, g_stream>>>(a);
+    return check_launch("expert_stream_kernel");
   }
-  constexpr int G = kStreamG;
-  a.vlist = ws.vlist;
-  a.nv = ws.nv;
-  // two workgroups per compute unit, but never more than the work units there can be
-  const int64_t npair = NMAT == 2 ? a.ntile : (a.ntile + 1) / 2;
-  const int64_t nwg = std::min<int64_t>(2 * (int64_t)std::max(g_cus, 1), P * npair);
-  const size_t lds = (size_t)G * a.nblk * 128 + 2 * 4 * 8 * 64 * sizeof(float);
-  expert_stream_kernel<NMAT == 2 ? 0 : 1, G><<<dim3((unsigned)nwg), 256, lds, g_stream>>>(a);
-  return check_launch("expert_stream_kernel");
+  ExpertGemmArgs ga{};
+  ga.desc = a.desc;
+  ga.mtiles = ws.tiles;
+  ga.n_mtiles = ws.n_tiles;
+  ga.list_row = a.list_row;
+  ga.A = a.A;
+  ga.nblk = a.nblk;
+  ga.ntile = a.ntile;
+  ga.N = a.N;
+  ga.act_type = a.act_type;
+  ga.act_out = a.act_out;
+  ga.y_out = a.y_out;
+  const int64_t max_mtiles = P / kGemmBM + std::min<int64_t>(E, P);
+  const dim3 grid((unsigned)cdiv(a.ntile, NMAT == 2 ? 8 : 16), (unsigned)max_mtiles);
+  expert_gemm_kernel<NMAT == 2 ? 0 : 1><<<grid, 256, 2 * 2048 * 16, g_stream>>>(ga);
+  return check_launch("expert_gemm_kernel");
 }
 
 // Experts' MLPs over the dispatched tokens: ws.y[P,H] <- down(act(gate, up)).
@@ -320,7 +336,6 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
                 int act_type, const uint16_t* x_split, const int* list_row, Workspace& ws,
                 bool timed = false) {
   const int64_t P = T * k;
-  const int64_t max_active = std::min<int64_t>(E, P);
   ExpertStreamArgs a{};
   a.desc = ws.desc;
   a.act_type = act_type;
@@ -333,7 +348,7 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   a.act_out = ws.act;
   a.y_out = nullptr;
   if (timed) mark(CSK_STAGE_GATEUP);
-  int rc = launch_stream<2>(a, max_active, P, ws);
+  int rc = launch_experts<2>(a, E, T, P, ws);
   if (rc != CSK_OK) return rc;
   if (timed) mark(CSK_STAGE_DOWN);
   // down
@@ -344,7 +359,7 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   a.ntile = (int)cdiv(H, 16);
   a.act_out = nullptr;
   a.y_out = ws.y;
-  return launch_stream<1>(a, max_active, P, ws);
+  return launch_experts<1>(a, E, T, P, ws);
 }
 
 int launch_combine(const float* y, const float* pairs, const int* pos, const float* residual,
@@ -715,7 +730,7 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
     mark(CSK_STAGE_DISPATCH);
     route_small_kernel<<<dim3(1), 1024, 0, g_stream>>>(
         ws.logits, ws.pairs, ws.ids, (int)T, (int)L->E, (int)L->k, L->sigmoid, L->ew_dev, ws.counts,
-        ws.offsets, ws.desc, ws.vlist, ws.nv, ws.list_tok, ws.list_w, ws.pos);
+        ws.offsets, ws.desc, ws.vlist, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w, ws.pos);
     if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
   } else {
     mark(CSK_STAGE_PREP);

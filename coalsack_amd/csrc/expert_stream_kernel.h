@@ -268,103 +268,4 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
   }
 }
 
-// ---------------------------------------------------------------------------
-// Generic fallback for contraction lengths above 3072: one 16-row tile per
-// workgroup, the four waves striding over K steps, activation fragments read
-// straight from global memory (L2), 16 tokens per pass.
-template <int NMAT>
-__global__ __launch_bounds__(256) void expert_generic_kernel(ExpertStreamArgs a) {
-  const WorkDesc* wd = a.desc + blockIdx.y;
-  const int Te = wd->Te;
-  if (Te == 0) return;
-  const int base = wd->base;
-  const int R = blockIdx.x;
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int n = lane & 15, g = lane >> 4;
-  const int nblk = a.nblk;
-  const size_t tile0 = (size_t)R * nblk * 16 + n;
-  const uint4* q0 = (NMAT == 2 ? wd->w.q_gate : wd->w.q_down) + tile0;
-  const uint8_t* s0 = (NMAT == 2 ? wd->w.s_gate : wd->w.s_down) + tile0;
-  const uint4* q1 = wd->w.q_up + tile0;
-  const uint8_t* s1 = wd->w.s_up + tile0;
-  const int nsteps = (nblk + 3) >> 2;
-  __shared__ float red[3][NMAT * 4][64];
-
-  for (int mbase = 0; mbase < Te; mbase += 16) {
-    floatx4 acc[NMAT];
-#pragma unroll
-    for (int m = 0; m < NMAT; ++m) acc[m] = floatx4{0.f, 0.f, 0.f, 0.f};
-    const int idx = min(mbase + n, Te - 1);  // lanes past the last token re-read it; outputs unused
-    const int row = a.list_row ? a.list_row[base + idx] : base + idx;
-    const uint4* ap = a.A + (size_t)row * nblk * 8;
-    for (int j = wv; j < nsteps; j += 4) {
-      const int kb = 4 * j + g;
-      const int kbc = min(kb, nblk - 1);
-      const uint4 qa = q0[kbc * 16];
-      const uint32_t sa = s0[kbc * 16];
-      uint4 qb = qa;
-      uint32_t sbv = sa;
-      if (NMAT == 2) {
-        qb = q1[kbc * 16];
-        sbv = s1[kbc * 16];
-      }
-      U4B8 af[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) af[i].u = ap[(size_t)kbc * 8 + i];
-      const float sc0 = kb < nblk ? e8m0_scale(sa) : 0.0f;
-      const float sc1 = kb < nblk ? e8m0_scale(sbv) : 0.0f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const bf16x8 b0 = cvt_fp4x8(u4_word(qa, i), sc0);
-        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i].b, b0, acc[0], 0, 0, 0);
-        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[4 + i].b, b0, acc[0], 0, 0, 0);
-        if (NMAT == 2) {
-          const bf16x8 b1 = cvt_fp4x8(u4_word(qb, i), sc1);
-          acc[NMAT - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i].b, b1, acc[NMAT - 1], 0, 0, 0);
-          acc[NMAT - 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[4 + i].b, b1, acc[NMAT - 1], 0, 0, 0);
-        }
-      }
-    }
-    if (wv > 0) {
-#pragma unroll
-      for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) red[wv - 1][m * 4 + i][lane] = acc[m][i];
-    }
-    __syncthreads();
-    if (wv == 0) {
-      const int r = R * 16 + n;
-      const ExpertW& w = wd->w;
-#pragma unroll
-      for (int m = 0; m < NMAT; ++m)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int o = m * 4 + i;
-          acc[m][i] = ((acc[m][i] + red[0][o][lane]) + red[1][o][lane]) + red[2][o][lane];
-        }
-      if (r < a.N) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int t = mbase + g * 4 + i;
-          if (t < Te) {
-            const size_t p = (size_t)(base + t);
-            if (NMAT == 2) {
-              const float gate_v = acc[0][i] + (w.b_gate ? w.b_gate[r] : 0.0f);
-              const float up_v = acc[NMAT - 1][i] + (w.b_up ? w.b_up[r] : 0.0f);
-              uint16_t hi, lo;
-              split_bf16(moe_activation(gate_v, up_v, a.act_type), hi, lo);
-              uint16_t* o = a.act_out + (p * (size_t)(a.N >> 5) + (r >> 5)) * 64 + (r & 31);
-              o[0] = hi;
-              o[32] = lo;
-            } else {
-              a.y_out[p * (size_t)a.N + r] = acc[0][i] + (w.b_down ? w.b_down[r] : 0.0f);
-            }
-          }
-        }
-      }
-    }
-    __syncthreads();
-  }
-}
-
 }  // namespace csk

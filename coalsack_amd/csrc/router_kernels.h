@@ -292,7 +292,8 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
     const int* __restrict__ ids, const float* __restrict__ pairs, int P, int k, int E,
     const int* __restrict__ counts, const ExpertW* __restrict__ ew, int* __restrict__ offsets,
     WorkDesc* __restrict__ desc, int* __restrict__ vlist, int* __restrict__ nv,
-    int* __restrict__ list_tok, float* __restrict__ list_w, int* __restrict__ pos_of_slot) {
+    int* __restrict__ mtiles, int* __restrict__ n_mtiles, int* __restrict__ list_tok,
+    float* __restrict__ list_w, int* __restrict__ pos_of_slot) {
   const int e = blockIdx.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   __shared__ int sh[8];
@@ -331,6 +332,15 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
           }
       }
       *nv = nvv;
+      // M tiles of the grouped GEMM: (expert slot, first token), 64 tokens each
+      int nm = 0;
+      for (int u = 0; u < na; ++u)
+        for (int m0 = 0; m0 < cnt[act_e[u]]; m0 += 64) {
+          mtiles[2 * nm] = u;
+          mtiles[2 * nm + 1] = m0;
+          ++nm;
+        }
+      *n_mtiles = nm;
     }
     __syncthreads();
     if (threadIdx.x < E) {
@@ -379,8 +389,8 @@ __global__ __launch_bounds__(1024) void route_small_kernel(
     const float* __restrict__ logits, float* __restrict__ pairs, int* __restrict__ ids_out, int T,
     int E, int k, int sigmoid, const ExpertW* __restrict__ ew, int* __restrict__ counts,
     int* __restrict__ offsets, WorkDesc* __restrict__ desc, int* __restrict__ vlist,
-    int* __restrict__ nv, int* __restrict__ list_tok, float* __restrict__ list_w,
-    int* __restrict__ pos_of_slot) {
+    int* __restrict__ nv, int* __restrict__ mtiles, int* __restrict__ n_mtiles,
+    int* __restrict__ list_tok, float* __restrict__ list_w, int* __restrict__ pos_of_slot) {
   __shared__ int ids[1024];
   __shared__ float wts[1024];
   __shared__ int cnt[kMaxExperts], off[kMaxExperts], act_e[kMaxExperts];
@@ -460,7 +470,7 @@ __global__ __launch_bounds__(1024) void route_small_kernel(
   __syncthreads();
   // exclusive scan, active experts, token groups
   if (threadIdx.x == 0) {
-    int run = 0, na = 0, nvv = 0;
+    int run = 0, na = 0, nvv = 0, nm = 0;
     for (int i = 0; i < E; ++i) {
       const int c = cnt[i];
       off[i] = run;
@@ -471,6 +481,11 @@ __global__ __launch_bounds__(1024) void route_small_kernel(
           vlist[2 * nvv + 1] = gb;
           ++nvv;
         }
+        for (int m0 = 0; m0 < c; m0 += 64) {
+          mtiles[2 * nm] = na;
+          mtiles[2 * nm + 1] = m0;
+          ++nm;
+        }
         act_e[na++] = i;
       }
       run += c;
@@ -478,6 +493,7 @@ __global__ __launch_bounds__(1024) void route_small_kernel(
     offsets[E] = run;
     na_sh = na;
     *nv = nvv;
+    *n_mtiles = nm;
   }
   __syncthreads();
   // ordered scatter: rank of an assignment = matches before it (ballot prefix)

@@ -73,3 +73,22 @@ def nbits_differ(a, b):
     a = np.ascontiguousarray(a, np.float32).reshape(-1).view(np.uint32)
     b = np.ascontiguousarray(b, np.float32).reshape(-1).view(np.uint32)
     return int(np.count_nonzero(a != b))
+
+
+def oracle_layer_subset(oracle, L, hidden, ntok, norm=False, residual=False, **opts):
+    """Oracle output for the first ntok tokens, replaying on the host only the
+    experts those tokens select (the others stay zero and are never read)."""
+    xin = oracle.rmsnorm(hidden[:ntok], L.norm_w, 1e-5) if norm else hidden[:ntok]
+    pairs = oracle.router(xin, L.gate_w, L.gate_b, L.k, opts.get("sigmoid", False))
+    used = sorted(set(pairs[..., 0].astype(int).ravel().tolist()))
+    per_gu, per_d = L.F * (L.H // 32) * 17, L.H * (L.F // 32) * 17
+    wu = np.zeros(L.E * per_gu, np.uint8)
+    wg = np.zeros(L.E * per_gu, np.uint8)
+    wd = np.zeros(L.E * per_d, np.uint8)
+    for e in used:
+        wu[e * per_gu:(e + 1) * per_gu] = L.blocks(e, 0)
+        wg[e * per_gu:(e + 1) * per_gu] = L.blocks(e, 1)
+        wd[e * per_d:(e + 1) * per_d] = L.blocks(e, 2)
+    return oracle.moe_layer(hidden[:ntok], L.E, L.k, L.H, L.F, L.gate_w, L.gate_b, wu, wg, wd,
+                            L.b_up, L.b_gate, L.b_down, norm_w=L.norm_w if norm else None,
+                            norm_eps=1e-5, residual=residual, **opts)

@@ -6,7 +6,8 @@ import pytest
 
 from coalsack_amd import capi, synth
 from tests.helpers import (all_blocks, assert_layer_close, build_layer,
-                           classify_index_mismatches, oracle_layer, nbits_differ)
+                           classify_index_mismatches, oracle_layer, nbits_differ,
+                           oracle_layer_subset)
 
 pytestmark = pytest.mark.gpu
 
@@ -274,3 +275,59 @@ def test_layer_120b_shape_skewed_16_tokens(lib, oracle):
     weights generated on the device, replayed on the host for the oracle."""
     L = synth.LayerInputs(128, 4, 2880, 2880, seed=42, hot_experts=8)
     _check_layer(lib, oracle, L, 16, device_weights=True)
+
+
+# ----------------------------------------------------- prefill (grouped GEMM)
+
+def _prefill_case(lib, oracle, L, T, ntok_oracle):
+    hidden = synth.hidden_states(T, L.H, seed=T + 3)
+    with build_layer(lib, L, device_weights=True) as layer:
+        got, pairs = layer.forward(hidden, want_pairs=True)
+        counts, toks = layer.last_dispatch(T)
+        again = layer.forward(hidden)
+        # a token's result does not depend on its place in the batch: permuting the
+        # tokens permutes the outputs bit for bit
+        perm = np.random.default_rng(1).permutation(T)
+        got_p = layer.forward(hidden[perm])
+    assert nbits_differ(got, again) == 0
+    assert nbits_differ(got_p, got[perm]) == 0
+    ids = pairs[..., 0].astype(int)
+    assert counts.sum() == T * L.k and np.array_equal(counts, np.bincount(ids.ravel(), minlength=L.E))
+    off = np.concatenate([[0], np.cumsum(counts)])
+    for e in range(L.E):
+        assert np.array_equal(toks[off[e]:off[e + 1]], np.nonzero(np.any(ids == e, axis=1))[0])
+    assert np.allclose(pairs[..., 1].sum(axis=1), 1.0, atol=1e-5)
+    want, wpairs = oracle_layer_subset(oracle, L, hidden, ntok_oracle)
+    real, near = classify_index_mismatches(oracle, hidden[:ntok_oracle], L, pairs[:ntok_oracle], wpairs)
+    assert real == 0, (real, near)
+    same = np.all(pairs[:ntok_oracle, :, 0] == wpairs[..., 0], axis=1)
+    assert_layer_close(got[:ntok_oracle][same], want[same])
+    return counts
+
+
+def test_prefill_20b_2048_tokens(lib, oracle):
+    """BASELINE config 3: 20b shape, 2048 tokens (about 256 tokens per expert)."""
+    L = synth.LayerInputs(32, 4, 2880, 2880, seed=77)
+    counts = _prefill_case(lib, oracle, L, 2048, 12)
+    assert counts.min() > 64  # natural routing: every expert sees several M tiles
+
+
+def test_prefill_120b_skewed_4096_tokens(lib, oracle):
+    """BASELINE config 4 at T=4096: 8 hot experts take about half of the assignments."""
+    L = synth.LayerInputs(128, 4, 2880, 2880, seed=78, hot_experts=8)
+    counts = _prefill_case(lib, oracle, L, 4096, 8)
+    hot = np.sort(counts)[-8:].sum() / counts.sum()
+    assert 0.4 < hot < 0.75, hot  # +2.0 logit offset on logits of std ~1.1
+
+
+def test_prefill_ragged_small_shape(lib, oracle):
+    """Token counts that are not multiples of the 64-token M tile, N not a multiple of
+    the 128-feature N tile, K not a multiple of the 128-element K step."""
+    L = synth.LayerInputs(5, 2, 96, 160, seed=31)
+    hidden = synth.hidden_states(333, L.H, seed=2)
+    with build_layer(lib, L) as layer:
+        got, pairs = layer.forward(hidden, want_pairs=True)
+    want, wpairs = oracle_layer(oracle, L, hidden)
+    same = np.all(pairs[..., 0] == wpairs[..., 0], axis=1)
+    assert same.mean() > 0.99
+    assert_layer_close(got[same], want[same])
