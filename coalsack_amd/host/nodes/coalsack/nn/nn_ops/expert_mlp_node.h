@@ -1,0 +1,202 @@
+// expert_mlp_node backed by the gfx950 library: same class name, constructor,
+// setters, test wrapper, input order, output conventions and error texts as
+// include/coalsack/nn/nn_ops/expert_mlp_node.h of the reference (cited by line
+// below) for MXFP4 weights; the body calls csk_expert_mlp_mxfp4.
+//
+// Weights are uploaded (repacked into the resident device layout) the first
+// time a storage pointer is seen and cached per node: moe_weight_provider
+// hands out the same storage from its own cache on every frame
+// (src/llm/moe_weight_provider.cpp:75-225), so a layer's experts become
+// resident after the first token.  The FP16 branch of the reference node
+// (:269-389) is not part of this path and reports an error.
+#pragma once
+
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "coalsack/nn/nn_op_node.h"
+#include "coalsack/tensor/dynamic_mx_tensor_message.h"
+#include "coalsack_moe.h"
+
+namespace coalsack {
+
+class expert_mlp_node : public graph_node {
+ public:
+  enum class activation_type {  // :27-30
+    MODIFIED_SWIGLU,
+    STANDARD_SWIGLU,
+  };
+
+  explicit expert_mlp_node(int expert_id = 0)  // :32-38
+      : expert_id_(expert_id), output_(std::make_shared<graph_edge>(this)) {
+    set_output(output_);
+  }
+  ~expert_mlp_node() override {
+    for (auto& kv : resident_) csk_mxfp4_free(kv.second.handle);
+  }
+  expert_mlp_node(const expert_mlp_node&) = delete;
+  expert_mlp_node& operator=(const expert_mlp_node&) = delete;
+
+  int get_expert_id() const { return expert_id_; }
+  std::string get_proc_name() const override { return "expert_mlp"; }
+  void set_input_names(const std::vector<std::string>& names) { input_names_ = names; }
+  void set_output_name(const std::string& name) { output_name_ = name; }
+  void set_node_name(const std::string& name) { node_name_ = name; }
+  void set_activation_type(activation_type t) { activation_type_ = t; }
+  activation_type get_activation_type() const { return activation_type_; }
+  void set_weight_before_ffn(bool v) { weight_before_ffn_ = v; }  // :52
+
+  // One token through raw 17-byte-block weights (:63-70).
+  void compute_test_mxfp4(const float* hidden_vec, const uint8_t* w_up_data, const uint8_t* w_gate_data,
+                          const uint8_t* w_down_data, const float* b_up_data, const float* b_gate_data,
+                          const float* b_down_data, float* output_vec, int64_t hidden_dim,
+                          int64_t expert_ffn_dim) {
+    if (expert_ffn_dim % 2 != 0)  // :662-669
+      throw std::runtime_error("compute_token_mxfp4: expert_ffn_dim must be even, got " +
+                               std::to_string(expert_ffn_dim));
+    if (hidden_dim % 2 != 0)
+      throw std::runtime_error("compute_token_mxfp4: hidden_dim must be even, got " +
+                               std::to_string(hidden_dim));
+    const int rc = csk_expert_token_mxfp4(hidden_vec, w_up_data, w_gate_data, w_down_data, b_up_data,
+                                          b_gate_data, b_down_data, output_vec, hidden_dim,
+                                          expert_ffn_dim, act_code());
+    if (rc != CSK_OK) throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
+  }
+
+  void process(std::string /*input_name*/, graph_message_ptr message) override {  // :73-148
+    auto in = std::dynamic_pointer_cast<result_message>(message);
+    const uint64_t frame = in ? in->get_frame_number() : 0;
+    const double stamp = in ? in->get_timestamp() : 0.0;
+    std::shared_ptr<result_message> out;
+    if (in && !in->is_ok()) {
+      out = result_message::error({{output_name_, nullptr}}, "Input error");
+    } else {
+      try {
+        if (!in || input_names_.empty()) throw std::runtime_error("expert_mlp: invalid input");
+        std::vector<graph_message_ptr> fields;
+        for (const auto& name : input_names_) {
+          auto f = in->get_field(name);
+          if (!f) throw std::runtime_error("expert_mlp: missing field " + name);
+          fields.push_back(f);
+        }
+        if (fields.size() < 2 || !std::dynamic_pointer_cast<dynamic_mx_tensor_message>(fields[1]))
+          throw std::runtime_error("expert_mlp: only MXFP4 weights are supported on the GPU path");
+        out = result_message::ok(
+            {{output_name_, std::make_shared<dynamic_tensor_message>(compute_with_mxfp4(fields))}});
+      } catch (const std::exception& e) {
+        out = result_message::error({{output_name_, nullptr}}, e.what());
+      }
+    }
+    out->set_frame_number(frame);
+    out->set_timestamp(stamp);
+    output_->send(out);
+  }
+
+ private:
+  struct resident {
+    csk_mxfp4* handle;
+    int64_t rows, cols;
+  };
+
+  int act_code() const {
+    return activation_type_ == activation_type::MODIFIED_SWIGLU ? CSK_ACT_MODIFIED_SWIGLU
+                                                                : CSK_ACT_STANDARD_SWIGLU;
+  }
+
+  csk_mxfp4* resident_copy(const dynamic_mx_tensor& t) {
+    const uint8_t* key = t.data_ptr();
+    auto it = resident_.find(key);
+    if (it != resident_.end() && it->second.rows == t.dim(0) && it->second.cols == t.dim(1))
+      return it->second.handle;
+    if (it != resident_.end()) {
+      csk_mxfp4_free(it->second.handle);
+      resident_.erase(it);
+    }
+    csk_mxfp4* h = nullptr;
+    if (csk_mxfp4_upload(key, t.dim(0), t.dim(1), &h) != CSK_OK)
+      throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
+    resident_[key] = resident{h, t.dim(0), t.dim(1)};
+    return h;
+  }
+
+  dynamic_tensor compute_with_mxfp4(const std::vector<graph_message_ptr>& msgs) {  // :392-485
+    if (msgs.size() != 5 && msgs.size() != 8)
+      throw std::runtime_error("expert_mlp: expected 5 or 8 inputs for MXFP4, got " +
+                               std::to_string(msgs.size()));
+    const bool has_bias = msgs.size() == 8;
+    auto hidden_msg = std::dynamic_pointer_cast<dynamic_tensor_message>(msgs[0]);
+    auto up_msg = std::dynamic_pointer_cast<dynamic_mx_tensor_message>(msgs[1]);
+    auto gate_msg = std::dynamic_pointer_cast<dynamic_mx_tensor_message>(msgs[2]);
+    auto down_msg = std::dynamic_pointer_cast<dynamic_mx_tensor_message>(msgs[3]);
+    auto router_msg = std::dynamic_pointer_cast<dynamic_tensor_message>(msgs[has_bias ? 7 : 4]);
+    std::shared_ptr<dynamic_tensor_message> b_up, b_gate, b_down;
+    if (has_bias) {
+      b_up = std::dynamic_pointer_cast<dynamic_tensor_message>(msgs[4]);
+      b_gate = std::dynamic_pointer_cast<dynamic_tensor_message>(msgs[5]);
+      b_down = std::dynamic_pointer_cast<dynamic_tensor_message>(msgs[6]);
+    }
+    if (!hidden_msg || !up_msg || !gate_msg || !down_msg || !router_msg)
+      throw std::runtime_error("expert_mlp: invalid input message types for MXFP4");
+    if (has_bias && (!b_up || !b_gate || !b_down))
+      throw std::runtime_error("expert_mlp: invalid bias message types for MXFP4");
+
+    const dynamic_tensor& hidden = hidden_msg->get_tensor();
+    const dynamic_tensor& router = router_msg->get_tensor();
+    const dynamic_mx_tensor& w_up = up_msg->get_mx_tensor();
+    const dynamic_mx_tensor& w_gate = gate_msg->get_mx_tensor();
+    const dynamic_mx_tensor& w_down = down_msg->get_mx_tensor();
+    if (hidden.ndim() != 3) throw std::runtime_error("expert_mlp: hidden_states must be 3D");
+    if (router.ndim() != 4 || router.dim(3) != 2)
+      throw std::runtime_error("expert_mlp: router_output must be 4D [batch, seq_len, top_k, 2]");
+
+    // not selected by any token: a {0}-shaped tensor, before any weight is looked at (:441-443)
+    const int64_t tokens = hidden.dim(0) * hidden.dim(1), top_k = router.dim(2);
+    const float* rp = router.data_ptr<float>();
+    bool any = false;
+    for (int64_t p = 0; p < router.dim(0) * router.dim(1) * top_k && !any; ++p)
+      any = static_cast<int>(rp[2 * p]) == expert_id_;
+    if (!any) return dynamic_tensor(dtype::float32, {0});
+
+    const int64_t hidden_dim = hidden.dim(2);
+    if (w_up.ndim() != 2 || w_gate.ndim() != 2 || w_down.ndim() != 2)
+      throw std::runtime_error("expert_mlp: all weights must be 2D");
+    const int64_t ffn = w_up.dim(0);
+    if (w_up.dim(1) != hidden_dim || w_gate.dim(0) != ffn || w_gate.dim(1) != hidden_dim ||
+        w_down.dim(0) != hidden_dim || w_down.dim(1) != ffn)
+      throw std::runtime_error("expert_mlp: weight dimension mismatch");
+    if (hidden_dim % 32 != 0)
+      throw std::runtime_error("expert_mlp: hidden_dim must be a multiple of 32 for MXFP4, got " +
+                               std::to_string(hidden_dim));
+    if (ffn % 32 != 0)
+      throw std::runtime_error("expert_mlp: expert_ffn_dim must be a multiple of 32 for MXFP4, got " +
+                               std::to_string(ffn));
+
+    dynamic_tensor output(dtype::float32, hidden.shape());
+    int is_empty = 0;
+    const int rc = csk_expert_mlp_mxfp4(
+        expert_id_, hidden.data_ptr<float>(), tokens, hidden_dim, ffn, resident_copy(w_up),
+        resident_copy(w_gate), resident_copy(w_down),
+        has_bias ? b_up->get_tensor().data_ptr<float>() : nullptr,
+        has_bias ? b_gate->get_tensor().data_ptr<float>() : nullptr,
+        has_bias ? b_down->get_tensor().data_ptr<float>() : nullptr, rp, top_k, act_code(),
+        weight_before_ffn_ ? 1 : 0, output.data_ptr<float>(), &is_empty);
+    if (rc != CSK_OK) throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
+    if (is_empty) return dynamic_tensor(dtype::float32, {0});
+    return output;
+  }
+
+  int expert_id_;
+  graph_edge_ptr output_;
+  std::vector<std::string> input_names_;
+  std::string output_name_, node_name_;
+  activation_type activation_type_ = activation_type::MODIFIED_SWIGLU;
+  bool weight_before_ffn_ = false;
+  std::unordered_map<const uint8_t*, resident> resident_;
+};
+
+}  // namespace coalsack
+
+COALSACK_REGISTER_NODE(coalsack::expert_mlp_node, coalsack::graph_node)

@@ -1,0 +1,91 @@
+// moe_router_node backed by the gfx950 library: same class name, setters, test
+// wrappers, input order, output format and error texts as
+// include/coalsack/nn/nn_ops/moe_router_node.h of the reference (cited by line
+// below); the body calls csk_moe_router instead of the scalar CPU loops.
+//
+// Place this directory in front of the reference's include path to swap the
+// node in; it needs only coalsack/nn/nn_op_node.h and the C ABI header.
+#pragma once
+
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "coalsack/nn/nn_op_node.h"
+#include "coalsack_moe.h"
+
+namespace coalsack {
+
+// Inputs: hidden_states [batch, seq_len, hidden_dim] f32, gate_weights
+// [num_experts, hidden_dim] f32, optional gate_bias [num_experts] f32.
+// Output: [batch, seq_len, top_k, 2] f32 = (expert index, routing weight),
+// slots in descending logit order (moe_router_node.h:13-21).
+class moe_router_node : public variadic_op_node {
+ public:
+  moe_router_node() : variadic_op_node("moe_router", 3) {}
+
+  void set_config(int64_t num_experts, int64_t top_k) {  // :27-30
+    num_experts_ = num_experts;
+    top_k_ = top_k;
+  }
+  void set_sigmoid_gating(bool v) { use_sigmoid_gating_ = v; }  // :34
+
+  dynamic_tensor compute_test(const dynamic_tensor& hidden_states, const dynamic_tensor& gate_weights,
+                              const dynamic_tensor& gate_bias) {  // :37-42
+    return compute({hidden_states, gate_weights, gate_bias});
+  }
+  dynamic_tensor compute_test(const dynamic_tensor& hidden_states,
+                              const dynamic_tensor& gate_weights) {  // :44-48
+    return compute({hidden_states, gate_weights});
+  }
+
+ protected:
+  dynamic_tensor compute(const std::vector<dynamic_tensor>& inputs) override {  // :51-124
+    if (inputs.size() != 2 && inputs.size() != 3)
+      throw std::runtime_error(
+          "moe_router: expected 2 or 3 inputs (hidden_states, gate_weights[, gate_bias]), got " +
+          std::to_string(inputs.size()));
+    const dynamic_tensor& hidden = inputs[0];
+    const dynamic_tensor& gate = inputs[1];
+    const bool has_bias = inputs.size() == 3;
+    if (hidden.ndim() != 3)
+      throw std::runtime_error("moe_router: hidden_states must be 3D [batch, seq_len, hidden_dim], got " +
+                               std::to_string(hidden.ndim()) + "D");
+    if (gate.ndim() != 2)
+      throw std::runtime_error("moe_router: gate_weights must be 2D [num_experts, hidden_dim], got " +
+                               std::to_string(gate.ndim()) + "D");
+    if (has_bias && inputs[2].ndim() != 1)
+      throw std::runtime_error("moe_router: gate_bias must be 1D [num_experts], got " +
+                               std::to_string(inputs[2].ndim()) + "D");
+    const int64_t batch = hidden.dim(0), seq_len = hidden.dim(1), hidden_dim = hidden.dim(2);
+    if (gate.dim(0) != num_experts_ || gate.dim(1) != hidden_dim)
+      throw std::runtime_error("moe_router: gate_weights shape mismatch, expected [" +
+                               std::to_string(num_experts_) + ", " + std::to_string(hidden_dim) +
+                               "], got [" + std::to_string(gate.dim(0)) + ", " +
+                               std::to_string(gate.dim(1)) + "]");
+    if (has_bias && inputs[2].dim(0) != num_experts_)
+      throw std::runtime_error("moe_router: gate_bias must have num_experts=" +
+                               std::to_string(num_experts_) + " elements, got " +
+                               std::to_string(inputs[2].dim(0)));
+    // the GPU path computes in f32; the reference's float64 branch (:116-119) is not offered
+    if (hidden.get_dtype() != dtype::float32 || gate.get_dtype() != dtype::float32)
+      throw std::runtime_error("moe_router: only float32 supported on the GPU path");
+
+    dynamic_tensor output(dtype::float32, {batch, seq_len, top_k_, 2});
+    const int rc = csk_moe_router(hidden.data_ptr<float>(), batch * seq_len, hidden_dim,
+                                  gate.data_ptr<float>(), num_experts_,
+                                  has_bias ? inputs[2].data_ptr<float>() : nullptr, top_k_,
+                                  use_sigmoid_gating_ ? 1 : 0, output.data_ptr<float>());
+    if (rc != CSK_OK) throw std::runtime_error(std::string("moe_router: ") + csk_last_error());
+    return output;
+  }
+
+ private:
+  int64_t num_experts_ = 0;
+  int64_t top_k_ = 0;
+  bool use_sigmoid_gating_ = false;
+};
+
+}  // namespace coalsack
+
+COALSACK_REGISTER_NODE(coalsack::moe_router_node, coalsack::graph_node)

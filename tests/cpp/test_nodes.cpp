@@ -1,0 +1,341 @@
+// Tests of the drop-in node classes (coalsack_amd/host/nodes) in the style of
+// the reference's test/test_moe_router.cpp, test/test_expert_mlp.cpp and
+// test/test_frame_sync.cpp, without googletest.
+//   test_nodes --cpu   argument / error-path behaviour (no GPU call is reached)
+//   test_nodes --gpu   numerics on the GPU against the CPU checker (oracle/)
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "coalsack/nn/nn_ops/expert_merge_node.h"
+#include "coalsack/nn/nn_ops/expert_mlp_node.h"
+#include "coalsack/nn/nn_ops/moe_router_node.h"
+
+using namespace coalsack;
+
+extern "C" {  // the CPU checker, oracle/moe_oracle.c
+int orc_router(const float*, int64_t, int64_t, const float*, int64_t, const float*, int64_t, int, float*);
+int orc_expert_token_mxfp4(const float*, const uint8_t*, const uint8_t*, const uint8_t*, const float*,
+                           const float*, const float*, float*, int64_t, int64_t, int);
+int orc_expert_mlp_mxfp4(int, const float*, int64_t, int64_t, int64_t, const uint8_t*, const uint8_t*,
+                         const uint8_t*, const float*, const float*, const float*, const float*, int64_t,
+                         int, int, float*, int*);
+int orc_expert_merge(const float*, int64_t, int64_t, int64_t, int64_t, const float* const*, int, float*);
+}
+
+static int g_failed = 0, g_checks = 0;
+#define CHECK(cond)                                                              \
+  do {                                                                           \
+    ++g_checks;                                                                  \
+    if (!(cond)) {                                                               \
+      ++g_failed;                                                                \
+      std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);            \
+    }                                                                            \
+  } while (0)
+
+static bool throws_with(const std::function<void()>& fn, const std::string& text) {
+  try {
+    fn();
+  } catch (const std::exception& e) {
+    if (std::string(e.what()).find(text) != std::string::npos) return true;
+    std::printf("  unexpected message: %s\n", e.what());
+    return false;
+  }
+  return false;
+}
+
+static dynamic_tensor random_tensor(const std::vector<int64_t>& shape, std::mt19937& gen, float lo, float hi) {
+  dynamic_tensor t(dtype::float32, shape);
+  std::uniform_real_distribution<float> d(lo, hi);
+  for (int64_t i = 0; i < t.numel(); ++i) t.data_ptr<float>()[i] = d(gen);
+  return t;
+}
+
+static dynamic_mx_tensor random_mx(int64_t rows, int64_t cols, std::mt19937& gen) {
+  dynamic_mx_tensor t({rows, cols});
+  std::uniform_int_distribution<int> byte(0, 255), scale(117, 121);
+  uint8_t* p = t.data_ptr();
+  for (size_t b = 0; b < t.num_blocks(); ++b) {
+    p[17 * b] = (uint8_t)scale(gen);
+    for (int j = 1; j < 17; ++j) p[17 * b + j] = (uint8_t)byte(gen);
+  }
+  return t;
+}
+
+// captures what a node sends, like message_capture_node of test/test_frame_sync.cpp
+struct capture_node : graph_node {
+  std::vector<std::shared_ptr<result_message>> got;
+  std::string get_proc_name() const override { return "capture"; }
+  void process(std::string, graph_message_ptr m) override {
+    got.push_back(std::dynamic_pointer_cast<result_message>(m));
+  }
+};
+
+// ------------------------------------------------------------------ CPU mode
+
+static void cpu_router_argument_errors() {
+  std::printf("router: argument errors\n");
+  moe_router_node node;
+  node.set_config(8, 2);
+  dynamic_tensor h3(dtype::float32, {1, 2, 4}), h2(dtype::float32, {2, 4});
+  dynamic_tensor g(dtype::float32, {8, 4}), g_bad(dtype::float32, {7, 4}), g1(dtype::float32, {32});
+  dynamic_tensor b(dtype::float32, {8}), b_bad(dtype::float32, {5}), b2(dtype::float32, {8, 1});
+  CHECK(throws_with([&] { node.compute_test(h2, g); }, "moe_router: hidden_states must be 3D"));
+  CHECK(throws_with([&] { node.compute_test(h3, g1); }, "moe_router: gate_weights must be 2D"));
+  CHECK(throws_with([&] { node.compute_test(h3, g_bad); }, "moe_router: gate_weights shape mismatch, expected [8, 4], got [7, 4]"));
+  CHECK(throws_with([&] { node.compute_test(h3, g, b_bad); }, "moe_router: gate_bias must have num_experts=8 elements, got 5"));
+  CHECK(throws_with([&] { node.compute_test(h3, g, b2); }, "moe_router: gate_bias must be 1D"));
+  // through process(): the exception becomes an error result with a null field (nn_op_node.h:306-314)
+  capture_node cap;
+  cap.set_input(node.get_output());
+  node.set_input_names({"h", "g"});
+  node.set_output_name("router_out");
+  auto msg = result_message::ok({{"h", std::make_shared<dynamic_tensor_message>(h2)},
+                                 {"g", std::make_shared<dynamic_tensor_message>(g)}});
+  msg->set_frame_number(7);
+  node.process("default", msg);
+  CHECK(cap.got.size() == 1 && cap.got[0]->is_error() && cap.got[0]->get_frame_number() == 7);
+  CHECK(cap.got[0]->get_fields().count("router_out") == 1 && cap.got[0]->get_field("router_out") == nullptr);
+  CHECK(cap.got[0]->get_error_message().find("must be 3D") != std::string::npos);
+}
+
+static void cpu_expert_node_paths() {
+  std::printf("expert_mlp: error propagation, missing field, unselected expert\n");
+  std::mt19937 gen(42);
+  expert_mlp_node node(5);
+  capture_node cap;
+  cap.set_input(node.get_output());
+  node.set_input_names({"hidden", "w_up", "w_gate", "w_down", "router"});
+  node.set_output_name("e5");
+  CHECK(node.get_expert_id() == 5 && node.get_proc_name() == "expert_mlp");
+  // upstream error is forwarded, compute is skipped (expert_mlp_node.h:82-91)
+  node.process("default", result_message::error({{"hidden", nullptr}}, "boom"));
+  CHECK(cap.got.size() == 1 && cap.got[0]->is_error() && cap.got[0]->get_error_message() == "Input error");
+  // missing field (:104-106)
+  auto hidden = std::make_shared<dynamic_tensor_message>(random_tensor({1, 3, 64}, gen, -1, 1));
+  node.process("default", result_message::ok({{"hidden", hidden}}));
+  CHECK(cap.got.size() == 2 && cap.got[1]->is_error() &&
+        cap.got[1]->get_error_message() == "expert_mlp: missing field w_up");
+  // no token selects expert 5: ok message with a {0}-shaped f32 tensor (:441-443), no GPU work
+  auto w = std::make_shared<dynamic_mx_tensor_message>(random_mx(64, 64, gen));
+  dynamic_tensor router(dtype::float32, {1, 3, 2, 2});
+  for (int p = 0; p < 6; ++p) {
+    router.data_ptr<float>()[2 * p] = (float)(p % 4);
+    router.data_ptr<float>()[2 * p + 1] = 0.5f;
+  }
+  auto msg = result_message::ok({{"hidden", hidden}, {"w_up", w}, {"w_gate", w}, {"w_down", w},
+                                 {"router", std::make_shared<dynamic_tensor_message>(router)}});
+  msg->set_frame_number(3);
+  msg->set_timestamp(1.5);
+  node.process("default", msg);
+  CHECK(cap.got.size() == 3 && cap.got[2]->is_ok() && cap.got[2]->get_frame_number() == 3 &&
+        cap.got[2]->get_timestamp() == 1.5);
+  auto out = std::dynamic_pointer_cast<dynamic_tensor_message>(cap.got[2]->get_field("e5"));
+  CHECK(out && out->get_tensor().ndim() == 1 && out->get_tensor().dim(0) == 0);
+  // bad router shape (:436-438) and wrong input count (:394-397)
+  dynamic_tensor router3(dtype::float32, {1, 3, 4});
+  node.process("default", result_message::ok({{"hidden", hidden}, {"w_up", w}, {"w_gate", w}, {"w_down", w},
+                                              {"router", std::make_shared<dynamic_tensor_message>(router3)}}));
+  CHECK(cap.got[3]->is_error() &&
+        cap.got[3]->get_error_message() == "expert_mlp: router_output must be 4D [batch, seq_len, top_k, 2]");
+  node.set_input_names({"hidden", "w_up", "w_gate", "w_down"});
+  node.process("default", msg);
+  CHECK(cap.got[4]->is_error() && cap.got[4]->get_error_message() == "expert_mlp: expected 5 or 8 inputs for MXFP4, got 4");
+}
+
+static void cpu_merge_argument_errors() {
+  std::printf("expert_merge: argument errors\n");
+  expert_merge_node node;
+  node.set_config(4, 2);
+  dynamic_tensor router(dtype::float32, {1, 2, 2, 2}), empty(dtype::float32, {0});
+  CHECK(throws_with([&] { node.compute_test({router, empty}); }, "expert_merge: expected 5 inputs, got 2"));
+  dynamic_tensor router_bad(dtype::float32, {1, 2, 3, 2});
+  CHECK(throws_with([&] { node.compute_test({router_bad, empty, empty, empty, empty}); },
+                    "expert_merge: router output must have shape [batch, seq_len, 2, 2]"));
+  CHECK(throws_with([&] { node.compute_test({router, empty, empty, empty, empty}); },
+                    "expert_merge: no non-empty expert outputs found"));
+  dynamic_tensor a(dtype::float32, {1, 2, 8}), b(dtype::float32, {1, 3, 8});
+  CHECK(throws_with([&] { node.compute_test({router, a, b, empty, empty}); },
+                    "expert_merge: all non-empty expert outputs must have same shape"));
+}
+
+// ------------------------------------------------------------------ GPU mode
+
+static void gpu_router_tests() {
+  std::printf("router: Basic / TopKSelection / GptOssScale / WeightNormalization\n");
+  std::mt19937 gen(42);
+  {  // test/test_moe_router.cpp:24-79
+    moe_router_node node;
+    node.set_config(8, 2);
+    auto h = random_tensor({1, 2, 4}, gen, -1, 1), g = random_tensor({8, 4}, gen, -1, 1);
+    dynamic_tensor b(dtype::float32, {8});
+    std::memset(b.data_ptr<float>(), 0, b.bytes());
+    auto out = node.compute_test(h, g, b);
+    CHECK((out.shape() == std::vector<int64_t>{1, 2, 2, 2}));
+    for (int s = 0; s < 2; ++s) {
+      float sum = 0;
+      for (int k = 0; k < 2; ++k) {
+        const float idx = out.data_ptr<float>()[(s * 2 + k) * 2], w = out.data_ptr<float>()[(s * 2 + k) * 2 + 1];
+        CHECK(idx >= 0 && idx < 8 && w > 0);
+        sum += w;
+      }
+      CHECK(std::fabs(sum - 1.0f) < 1e-5f);
+    }
+  }
+  {  // :82-138: hidden = 1, gate row e = e / H  =>  experts 5, 4, 3
+    moe_router_node node;
+    node.set_config(6, 3);
+    dynamic_tensor h(dtype::float32, {1, 1, 4}), g(dtype::float32, {6, 4});
+    for (int i = 0; i < 4; ++i) h.data_ptr<float>()[i] = 1.0f;
+    for (int e = 0; e < 6; ++e)
+      for (int d = 0; d < 4; ++d) g.data_ptr<float>()[e * 4 + d] = (float)e / 4;
+    auto out = node.compute_test(h, g);
+    CHECK((int)out.data_ptr<float>()[0] == 5 && (int)out.data_ptr<float>()[2] == 4 && (int)out.data_ptr<float>()[4] == 3);
+  }
+  {  // :141-203 gpt-oss scale, and agreement with the CPU checker
+    moe_router_node node;
+    node.set_config(32, 4);
+    auto h = random_tensor({2, 8, 128}, gen, -1, 1), g = random_tensor({32, 128}, gen, -0.2f, 0.2f);
+    auto b = random_tensor({32}, gen, -0.01f, 0.01f);
+    auto out = node.compute_test(h, g, b);
+    std::vector<float> want(16 * 4 * 2);
+    orc_router(h.data_ptr<float>(), 16, 128, g.data_ptr<float>(), 32, b.data_ptr<float>(), 4, 0, want.data());
+    for (int t = 0; t < 16; ++t) {
+      float sum = 0;
+      for (int k = 0; k < 4; ++k) {
+        const float* o = out.data_ptr<float>() + (t * 4 + k) * 2;
+        CHECK(o[0] == want[(t * 4 + k) * 2] && std::fabs(o[1] - want[(t * 4 + k) * 2 + 1]) < 1e-5f && o[1] <= 1.0f);
+        sum += o[1];
+      }
+      CHECK(std::fabs(sum - 1.0f) < 1e-4f);
+    }
+  }
+}
+
+static void gpu_expert_known_answer() {
+  std::printf("expert_mlp: ModifiedSwigluActivation (gate = 1.0, up = 1.5, identity down)\n");
+  // test/test_expert_mlp.cpp:118-200 recast for MXFP4 storage
+  const int64_t H = 32, F = 32;
+  std::vector<uint8_t> wz(F * 17, 0), wd(H * 17, 0);
+  for (int r = 0; r < 32; ++r) {
+    wz[r * 17] = 128;
+    wd[r * 17] = 128;
+    if (r < 16) wd[r * 17 + 1 + r] |= 1;  // code 1 = +1.0 at element r
+    else wd[r * 17 + 1 + r - 16] |= 1 << 4;
+  }
+  std::vector<float> x(H, 1.0f), bu(F, 1.5f), bg(F, 1.0f), bd(H, 0.0f), out(H);
+  expert_mlp_node node(0);
+  node.compute_test_mxfp4(x.data(), wz.data(), wz.data(), wd.data(), bu.data(), bg.data(), bd.data(), out.data(), H, F);
+  const float want = 1.0f / (1.0f + std::exp(-1.702f)) * 2.5f;
+  for (int i = 0; i < H; ++i) CHECK(std::fabs(out[i] - want) < 1e-3f);
+  node.set_activation_type(expert_mlp_node::activation_type::STANDARD_SWIGLU);
+  node.compute_test_mxfp4(x.data(), wz.data(), wz.data(), wd.data(), bu.data(), bg.data(), bd.data(), out.data(), H, F);
+  const float want2 = 1.0f / (1.0f + std::exp(-1.0f)) * 1.5f;
+  for (int i = 0; i < H; ++i) CHECK(std::fabs(out[i] - want2) < 1e-3f);
+}
+
+// router -> E expert nodes -> merge, wired with edges and result messages the way
+// llm_engine builds the block (src/llm/llm_engine.cpp:721-753), against the CPU checker.
+static void gpu_node_chain() {
+  std::printf("router -> experts -> merge through result messages\n");
+  std::mt19937 gen(7);
+  const int64_t E = 6, K = 2, H = 64, F = 96, B = 1, S = 9, T = B * S;
+  auto hidden = random_tensor({B, S, H}, gen, -1, 1);
+  auto gate = random_tensor({E, H}, gen, -0.3f, 0.3f);
+  auto gate_b = random_tensor({E}, gen, -0.01f, 0.01f);
+  std::vector<dynamic_mx_tensor> wu, wg, wd;
+  std::vector<dynamic_tensor> bu, bg, bd;
+  for (int e = 0; e < E; ++e) {
+    wu.push_back(random_mx(F, H, gen));
+    wg.push_back(random_mx(F, H, gen));
+    wd.push_back(random_mx(H, F, gen));
+    bu.push_back(random_tensor({F}, gen, -0.01f, 0.01f));
+    bg.push_back(random_tensor({F}, gen, -0.01f, 0.01f));
+    bd.push_back(random_tensor({H}, gen, -0.01f, 0.01f));
+  }
+  moe_router_node router;
+  router.set_config(E, K);
+  router.set_input_names({"hidden", "gate_w", "gate_b"});
+  router.set_output_name("router_out");
+  capture_node rcap;
+  rcap.set_input(router.get_output());
+  auto mk = [](const dynamic_tensor& t) { return std::make_shared<dynamic_tensor_message>(t); };
+  router.process("default", result_message::ok({{"hidden", mk(hidden)}, {"gate_w", mk(gate)}, {"gate_b", mk(gate_b)}}));
+  CHECK(rcap.got.size() == 1 && rcap.got[0]->is_ok());
+  auto router_out = std::dynamic_pointer_cast<dynamic_tensor_message>(rcap.got[0]->get_field("router_out"));
+  CHECK(router_out && (router_out->get_tensor().shape() == std::vector<int64_t>{B, S, K, 2}));
+  const float* pairs = router_out->get_tensor().data_ptr<float>();
+
+  std::vector<dynamic_tensor> merge_inputs{router_out->get_tensor()};
+  std::vector<std::vector<float>> want_outs(E);
+  std::vector<const float*> want_ptrs(E, nullptr);
+  int n_empty = 0;
+  for (int e = 0; e < E; ++e) {
+    expert_mlp_node node(e);
+    node.set_input_names({"hidden", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "router"});
+    node.set_output_name("out");
+    capture_node cap;
+    cap.set_input(node.get_output());
+    auto msg = result_message::ok({{"hidden", mk(hidden)},
+                                   {"w_up", std::make_shared<dynamic_mx_tensor_message>(wu[e])},
+                                   {"w_gate", std::make_shared<dynamic_mx_tensor_message>(wg[e])},
+                                   {"w_down", std::make_shared<dynamic_mx_tensor_message>(wd[e])},
+                                   {"b_up", mk(bu[e])}, {"b_gate", mk(bg[e])}, {"b_down", mk(bd[e])},
+                                   {"router", router_out}});
+    node.process("default", msg);
+    node.process("default", msg);  // second frame: weights are already resident
+    CHECK(cap.got.size() == 2 && cap.got[0]->is_ok() && cap.got[1]->is_ok());
+    auto out = std::dynamic_pointer_cast<dynamic_tensor_message>(cap.got[1]->get_field("out"))->get_tensor();
+    want_outs[e].resize(T * H);
+    int empty = 0;
+    orc_expert_mlp_mxfp4(e, hidden.data_ptr<float>(), T, H, F, wu[e].data_ptr(), wg[e].data_ptr(), wd[e].data_ptr(),
+                         bu[e].data_ptr<float>(), bg[e].data_ptr<float>(), bd[e].data_ptr<float>(), pairs, K, 0, 0,
+                         want_outs[e].data(), &empty);
+    if (empty) {
+      ++n_empty;
+      CHECK(out.ndim() == 1 && out.dim(0) == 0);
+    } else {
+      CHECK((out.shape() == std::vector<int64_t>{B, S, H}));
+      want_ptrs[e] = want_outs[e].data();
+      float worst = 0;
+      for (int64_t i = 0; i < T * H; ++i)
+        worst = std::fmax(worst, std::fabs(out.data_ptr<float>()[i] - want_outs[e][i]) / std::fmax(1.0f, std::fabs(want_outs[e][i])));
+      CHECK(worst <= 1e-3f);
+    }
+    merge_inputs.push_back(out);
+  }
+  std::printf("  %d of %d experts unselected\n", n_empty, (int)E);
+  expert_merge_node merge;
+  merge.set_config(E, K);
+  auto merged = merge.compute_test(merge_inputs);
+  std::vector<float> want(T * H);
+  CHECK(orc_expert_merge(pairs, T, K, E, H, want_ptrs.data(), 0, want.data()) == 0);
+  float worst = 0;
+  for (int64_t i = 0; i < T * H; ++i)
+    worst = std::fmax(worst, std::fabs(merged.data_ptr<float>()[i] - want[i]) / std::fmax(1.0f, std::fabs(want[i])));
+  std::printf("  merged layer output: max rel err %.3g\n", worst);
+  CHECK(worst <= 1e-3f);
+}
+
+int main(int argc, char** argv) {
+  const bool gpu = argc > 1 && std::string(argv[1]) == "--gpu";
+  if (gpu) {
+    if (csk_init(0) != CSK_OK) {
+      std::printf("csk_init failed: %s\n", csk_last_error());
+      return 2;
+    }
+    gpu_router_tests();
+    gpu_expert_known_answer();
+    gpu_node_chain();
+  } else {
+    cpu_router_argument_errors();
+    cpu_expert_node_paths();
+    cpu_merge_argument_errors();
+  }
+  std::printf("%d checks, %d failed\n", g_checks, g_failed);
+  return g_failed ? 1 : 0;
+}
