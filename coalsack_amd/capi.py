@@ -28,6 +28,7 @@ SIGNATURES = {
     "csk_dev_free": (None, [_P]),
     "csk_copy_h2d": (C.c_int, [_P, _P, C.c_size_t]),
     "csk_copy_d2h": (C.c_int, [_P, _P, C.c_size_t]),
+    "csk_copy_d2d": (C.c_int, [_P, _P, C.c_size_t]),
     "csk_synchronize": (C.c_int, []),
     "csk_event_create": (_P, []),
     "csk_event_destroy": (None, [_P]),
@@ -140,6 +141,9 @@ class Library:
         out = np.empty(shape, dtype=dtype)
         self.check(self.dll.csk_copy_d2h(_ptr(out), p, out.nbytes))
         return out
+
+    def copy_d2d(self, dst, src, nbytes):
+        self.check(self.dll.csk_copy_d2d(dst, src, nbytes))
 
     def synchronize(self):
         self.check(self.dll.csk_synchronize())

@@ -461,6 +461,21 @@ extern "C" int csk_copy_d2h(void* dst, const void* src, size_t bytes) {
   HIP_TRY(hipStreamSynchronize(g_stream));
   return CSK_OK;
 }
+namespace {
+__global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, long n) {
+  const long stride = (long)gridDim.x * 256;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+}
+}  // namespace
+extern "C" int csk_copy_d2d(void* dst, const void* src, size_t bytes) {
+  REQUIRE_INIT();
+  if (!dst || !src || bytes % 16) return fail(CSK_ERR_ARG, "csk_copy_d2d: null pointer or size not a multiple of 16");
+  if (bytes == 0) return CSK_OK;
+  const long n = (long)(bytes / 16);
+  const long blocks = std::min<long>(cdiv(n, 256), 8L * std::max(g_cus, 1));
+  copy_kernel<<<dim3((unsigned)blocks), 256, 0, g_stream>>>((const uint4*)src, (uint4*)dst, n);
+  return check_launch("copy_kernel");
+}
 extern "C" int csk_synchronize(void) {
   REQUIRE_INIT();
   HIP_TRY(hipStreamSynchronize(g_stream));

@@ -60,6 +60,10 @@ void* csk_dev_alloc(size_t bytes);
 void csk_dev_free(void* p);
 int csk_copy_h2d(void* dst_device, const void* src_host, size_t bytes);
 int csk_copy_d2h(void* dst_host, const void* src_device, size_t bytes);
+/* Device-to-device copy by a plain grid-stride kernel (16-byte accesses), asynchronous on the
+ * library's stream; bytes must be a multiple of 16.  Also the known-size reference that profiler
+ * byte counters are calibrated against. */
+int csk_copy_d2d(void* dst_device, const void* src_device, size_t bytes);
 int csk_synchronize(void);
 typedef struct csk_event csk_event;
 csk_event* csk_event_create(void);
