@@ -62,6 +62,7 @@ inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 // Above this many token-expert assignments the token-group list of the
 // weight-streaming kernel is not built.
 constexpr int64_t kStreamMaxP = 2048;
+constexpr int kStreamWgPerCu = 3;  // resident workgroups of the streaming kernel per compute unit
 
 // ---- workspace shared by every layer (single stream, one call at a time) --
 struct Workspace {
@@ -304,10 +305,10 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
     constexpr int G = kStreamG;
     a.vlist = ws.vlist;
     a.nv = ws.nv;
-    // two workgroups per compute unit, but never more than the work units there can be
+    // kStreamWgPerCu workgroups per compute unit, but never more than the work units there can be
     const int64_t npair = NMAT == 2 ? a.ntile : (a.ntile + 1) / 2;
-    const int64_t nwg = std::min<int64_t>(2 * (int64_t)std::max(g_cus, 1), P * npair);
-    const size_t lds = (size_t)G * a.nblk * 128 + 2 * 4 * 8 * 64 * sizeof(float);
+    const int64_t nwg = std::min<int64_t>(kStreamWgPerCu * (int64_t)std::max(g_cus, 1), P * npair);
+    const size_t lds = (size_t)G * a.nblk * 128 + 2 * 4 * 8 * 16 * sizeof(float);
     expert_stream_kernel<NMAT == 2 ? 0 : 1, G><<<dim3((unsigned)nwg), 256, lds, g_stream>>>(a);
     return check_launch("expert_stream_kernel");
   }

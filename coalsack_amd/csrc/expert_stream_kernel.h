@@ -1,14 +1,12 @@
 // Expert MLP for the weight-streaming (decode) regime.
 //
-// A workgroup owns TPW consecutive 16-row tiles of one active expert's matrix
-// (gate and up together, or down) and streams them from HBM exactly once:
-// 64 lanes x 16 bytes = 1 KiB of contiguous nibbles per matrix per tile per
-// step.  The four waves take interleaved K steps (128 elements each); a wave
-// loads its slice of the activations once per step and reuses it for all TPW
-// tiles.  MXFP4 is expanded in registers by v_cvt_scalef32_pk_bf16_fp4 (exact:
-// an E2M1 value times a power of two always fits bf16) and contracted on the
-// matrix cores against up to 16*MT tokens of that expert.  Activations arrive
-// as two bf16 terms (hi + lo, 16 mantissa bits), so each product is that of the
+// Every active expert's matrices are streamed from HBM once per group of up to
+// four of its tokens: 64 lanes x 16 bytes = 1 KiB of contiguous nibbles per
+// 16-row tile per K step, the four waves of a workgroup taking interleaved K
+// steps (128 elements each).  MXFP4 is expanded in registers by
+// v_cvt_scalef32_pk_bf16_fp4 (exact: an E2M1 value times a power of two always
+// fits bf16) and contracted on the matrix cores.  Activations arrive as two
+// bf16 terms (hi + lo, 16 mantissa bits), so each product is that of the
 // reference's fp32 activation and exactly dequantised weight to within 2^-17;
 // accumulation is fp32.  The K slices of the four waves meet in LDS in a fixed
 // order.
@@ -41,7 +39,6 @@ struct ExpertStreamArgs {
   int ntile;             // ceil(N / 16)
   int N;                 // output features (F for gate/up, H for down)
   int act_type;
-  int tiles_per_wg;      // consecutive row tiles one workgroup walks through
   uint16_t* act_out;     // gate/up: [P][N/32][64] bf16 hi|lo
   float* y_out;          // down: [P][N] f32
 };
@@ -94,10 +91,10 @@ __device__ __forceinline__ uint32_t u4_word(const uint4& v, int i) {
 // equal contiguous ranges, so the load is balanced whatever the routing was.
 // Memory-level parallelism bounds this kernel, so it never lets the memory
 // queue drain: a group's activation rows are copied once into LDS
-// (global_load_lds, no registers), and while the matrix cores work on unit t
-// from one register set the weight loads of unit t+1 -- all of a wave's K
-// steps, issued back to back from clamped addresses so that no wait separates
-// them -- are already in flight into the other set.  The four waves split K;
+// (global_load_lds, no registers), and the weight registers are refilled step
+// by step as the matrix cores consume them: the loads of unit t+1 -- issued
+// unconditionally from clamped addresses so that no full wait separates them
+// -- are in flight while unit t is contracted.  The four waves split K;
 // their partial sums meet in double-buffered LDS (one barrier per unit) in the
 // fixed order w0 + w1 + w2 + w3, and wave t mod 4 finishes unit t.
 template <int MODE, int G>
@@ -108,7 +105,7 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
   const int nblk = a.nblk;
   const int row_u4 = nblk * 8;                   // uint4 per activation row
   uint4* As = reinterpret_cast<uint4*>(smem);    // [G][row_u4]
-  float* red = reinterpret_cast<float*>(smem + (size_t)G * row_u4 * 16);  // [2][4][NV][64]
+  float* red = reinterpret_cast<float*>(smem + (size_t)G * row_u4 * 16);  // [2][4][NV][16]: live lanes only
 
   const int npair = MODE == 0 ? a.ntile : (a.ntile + 1) >> 1;
   const long total = (long)(*a.nv) * npair;
@@ -160,24 +157,28 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
     }
 
     // tiles of a unit: (R, R) for gate/up, (2R, 2R+1) for down
-    auto load_unit = [&](WSet& ws, int unit) {
+    auto load_step = [&](WSet& ws, int unit, int s) {
       const int ta = MODE == 0 ? unit : 2 * unit;
       const int tb = MODE == 0 ? unit : min(2 * unit + 1, a.ntile - 1);
       const size_t ea = (size_t)ta * nblk * 16, eb = (size_t)tb * nblk * 16;
-#pragma unroll
-      for (int s = 0; s < NS; ++s) {
-        const int kb = min(4 * (wv + 4 * s) + g, nblk - 1);
-        ws.q[s][0] = q0[ea + kb * 16];
-        ws.sb[s][0] = s0[ea + kb * 16];
-        ws.q[s][1] = q1[eb + kb * 16];
-        ws.sb[s][1] = s1[eb + kb * 16];
-      }
-      ws.b0 = bp0[min(ta * 16 + n, a.N - 1)];  // bias pointers are never null (absent bias = zero vector)
-      ws.b1 = bp1[min(tb * 16 + n, a.N - 1)];
+      const int kb = min(4 * (wv + 4 * s) + g, nblk - 1);
+      ws.q[s][0] = q0[ea + kb * 16];
+      ws.sb[s][0] = s0[ea + kb * 16];
+      ws.q[s][1] = q1[eb + kb * 16];
+      ws.sb[s][1] = s1[eb + kb * 16];
     };
-    const bool live = g * 4 < gcount;  // this lane's accumulator rows belong to live tokens
+    auto load_bias = [&](float& b0, float& b1, int unit) {
+      const int ta = MODE == 0 ? unit : 2 * unit;
+      const int tb = MODE == 0 ? unit : min(2 * unit + 1, a.ntile - 1);
+      b0 = bp0[min(ta * 16 + n, a.N - 1)];  // bias pointers are never null (absent bias = zero vector)
+      b1 = bp1[min(tb * 16 + n, a.N - 1)];
+    };
+    static_assert(G <= 4, "live accumulator rows are those of lanes g == 0");
+    const bool live = g == 0;  // tokens 0..G-1 are accumulator rows 0..3 of lanes 0..15
 
-    auto compute_unit = [&](const WSet& ws, int unit) {
+    // Contracts unit `unit` out of ws and, step by step, refills ws with unit `next`.
+    auto compute_unit = [&](WSet& ws, int unit, int next) {
+      const float bias0 = ws.b0, bias1 = ws.b1;
       floatx4 acc[2][2];  // [tile of the pair][hi, lo term]: independent accumulation chains
 #pragma unroll
       for (int m = 0; m < 2; ++m) acc[m][0] = acc[m][1] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -209,14 +210,16 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
           acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[cur].b, b1, acc[1][0], 0, 0, 0);
           acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[cur].b, b1, acc[1][1], 0, 0, 0);
         }
+        load_step(ws, next, s);  // this step's registers are free: start the next unit's loads
       }
-      float* rbuf = red + (size_t)par * 4 * NV * 64;
+      load_bias(ws.b0, ws.b1, next);
+      float* rbuf = red + (size_t)par * 4 * NV * 16;
       par ^= 1;
       if (live) {
 #pragma unroll
         for (int m = 0; m < 2; ++m)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) rbuf[(wv * NV + m * 4 + i) * 64 + lane] = acc[m][0][i] + acc[m][1][i];
+          for (int i = 0; i < 4; ++i) rbuf[(wv * NV + m * 4 + i) * 16 + n] = acc[m][0][i] + acc[m][1][i];
       }
       __syncthreads();
       if (wv == (unit & 3) && live) {
@@ -226,8 +229,8 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int o = m * 4 + i;
-            v2[m][i] = ((rbuf[(0 * NV + o) * 64 + lane] + rbuf[(1 * NV + o) * 64 + lane]) +
-                        rbuf[(2 * NV + o) * 64 + lane]) + rbuf[(3 * NV + o) * 64 + lane];
+            v2[m][i] = ((rbuf[(0 * NV + o) * 16 + n] + rbuf[(1 * NV + o) * 16 + n]) +
+                        rbuf[(2 * NV + o) * 16 + n]) + rbuf[(3 * NV + o) * 16 + n];
           }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -238,33 +241,32 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
               const int r = unit * 16 + n;  // output feature
               if (r < a.N) {
                 uint16_t hi, lo;
-                split_bf16(moe_activation(v2[0][i] + ws.b0, v2[1][i] + ws.b1, a.act_type), hi, lo);
+                split_bf16(moe_activation(v2[0][i] + bias0, v2[1][i] + bias1, a.act_type), hi, lo);
                 uint16_t* o = a.act_out + (p * (size_t)(a.N >> 5) + (r >> 5)) * 64 + (r & 31);
                 o[0] = hi;
                 o[32] = lo;
               }
             } else {
               const int ra = 2 * unit * 16 + n, rb = ra + 16;
-              if (ra < a.N) a.y_out[p * (size_t)a.N + ra] = v2[0][i] + ws.b0;
-              if (rb < a.N) a.y_out[p * (size_t)a.N + rb] = v2[1][i] + ws.b1;
+              if (ra < a.N) a.y_out[p * (size_t)a.N + ra] = v2[0][i] + bias0;
+              if (rb < a.N) a.y_out[p * (size_t)a.N + rb] = v2[1][i] + bias1;
             }
           }
         }
       }
     };
 
-    // Prefetches are unconditional (past the last unit they re-read it), so that the
-    // number of loads in flight behind a register set is the same on every path and
-    // the waits in front of the matrix cores stay partial.
-    WSet wa, wb;
-    load_unit(wa, p_begin);
+    // One register set, refilled step by step as it is consumed: the loads of unit
+    // t+1 are issued during unit t and stay one unit ahead of their use.  Refills
+    // are unconditional (past the last unit they re-read it), so that the number of
+    // loads in flight is the same on every path and the waits in front of the
+    // matrix cores stay partial.
+    WSet ws;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) load_step(ws, p_begin, s);
+    load_bias(ws.b0, ws.b1, p_begin);
     __syncthreads();  // the LDS copies have landed (the compiler waits for them before the barrier)
-    for (int t = p_begin; t < p_end; t += 2) {
-      load_unit(wb, min(t + 1, p_end - 1));
-      compute_unit(wa, t);
-      load_unit(wa, min(t + 2, p_end - 1));
-      if (t + 1 < p_end) compute_unit(wb, t + 1);
-    }
+    for (int t = p_begin; t < p_end; ++t) compute_unit(ws, t, min(t + 1, p_end - 1));
   }
 }
 
