@@ -62,7 +62,7 @@ inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 // Above this many token-expert assignments the token-group list of the
 // weight-streaming kernel is not built.
 constexpr int64_t kStreamMaxP = 2048;
-constexpr int kStreamWgPerCu = 3;  // resident workgroups of the streaming kernel per compute unit
+constexpr int kStreamWgPerCu = 2;  // resident workgroups of the streaming kernel per compute unit
 
 // ---- workspace shared by every layer (single stream, one call at a time) --
 struct Workspace {
@@ -152,6 +152,7 @@ struct csk_mxfp4 {
   int64_t ntile = 0, nblk = 0;
   bool owned = true;
   long entries() const { return (long)(ntile * nblk * 16); }
+  long scale_bytes() const { return (long)ntile * 256 * scale_slots((int)nblk); }
 };
 
 struct csk_layer {
@@ -175,12 +176,15 @@ struct csk_layer {
   long ent_gu() const { return (long)(ntF * nblkH * 16); }  // gate or up: [F,H]
   long ent_d() const { return (long)(ntH * nblkF * 16); }   // down: [H,F]
   long ent_expert() const { return 2 * ent_gu() + ent_d(); }
+  long sc_gu() const { return (long)ntF * 256 * scale_slots((int)nblkH); }  // scale bytes of gate or up
+  long sc_d() const { return (long)ntH * 256 * scale_slots((int)nblkF); }
+  long sc_expert() const { return 2 * sc_gu() + sc_d(); }
   csk_mxfp4 view(int64_t e, int which) const {
     csk_mxfp4 m;
     const long base = (long)e * ent_expert();
     const long off = which == CSK_W_GATE ? 0 : (which == CSK_W_UP ? ent_gu() : 2 * ent_gu());
     m.q = q_all + base + off;
-    m.s = s_all + base + off;
+    m.s = s_all + (long)e * sc_expert() + (which == CSK_W_GATE ? 0 : (which == CSK_W_UP ? sc_gu() : 2 * sc_gu()));
     m.rows = which == CSK_W_DOWN ? H : F;
     m.K = which == CSK_W_DOWN ? F : H;
     m.ntile = which == CSK_W_DOWN ? ntH : ntF;
@@ -522,7 +526,8 @@ extern "C" int csk_mxfp4_upload(const uint8_t* blocks, int64_t rows, int64_t K, 
   m->nblk = K / 32;
   m->ntile = cdiv(rows, 16);
   int rc = dev_alloc(&m->q, (size_t)m->entries());
-  if (rc == CSK_OK) rc = dev_alloc(&m->s, (size_t)m->entries());
+  if (rc == CSK_OK) rc = dev_alloc(&m->s, (size_t)m->scale_bytes());
+  if (rc == CSK_OK && hipMemset(m->s, 127, (size_t)m->scale_bytes()) != hipSuccess) rc = fail(CSK_ERR_HIP, "hipMemset failed");
   if (rc == CSK_OK) rc = pack_into(blocks, *m);
   if (rc != CSK_OK) {
     csk_mxfp4_free(m);
@@ -566,7 +571,8 @@ extern "C" int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_
   rc = dev_alloc(&L->gate_w, (size_t)E * H);
   if (rc == CSK_OK) rc = dev_alloc(&L->gate_b, (size_t)E);
   if (rc == CSK_OK) rc = dev_alloc(&L->q_all, (size_t)E * L->ent_expert());
-  if (rc == CSK_OK) rc = dev_alloc(&L->s_all, (size_t)E * L->ent_expert());
+  if (rc == CSK_OK) rc = dev_alloc(&L->s_all, (size_t)E * L->sc_expert());
+  if (rc == CSK_OK && hipMemset(L->s_all, 127, (size_t)E * L->sc_expert()) != hipSuccess) rc = fail(CSK_ERR_HIP, "hipMemset failed");
   if (rc == CSK_OK) rc = dev_alloc(&L->bias_all, (size_t)E * (2 * F + H));
   if (rc == CSK_OK) rc = dev_alloc(&L->ew_dev, (size_t)E);
   if (rc == CSK_OK) rc = dev_alloc(&L->norm_w, (size_t)H);

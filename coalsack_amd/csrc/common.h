@@ -9,6 +9,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // 16 bytes, address-space friendly
 
 constexpr int kWave = 64;
@@ -22,7 +23,10 @@ constexpr int kStreamG = 4;      // tokens per pass of the weight-streaming expe
 //   q: [rows/16][K/32][16] x 16 bytes -- byte b of an entry holds elements
 //      2b (low nibble) and 2b+1 (high nibble) of one 32-element block, which
 //      is the order v_cvt_scalef32_pk_*_fp4 consumes;
-//   s: [rows/16][K/32][16] scale bytes (E8M0).
+//   s: scale bytes (E8M0), per tile [4 waves][64 lanes][slots]: the scale of block kb
+//      of row n sits with wave (kb/4)%4, lane (kb%4)*16+n, slot kb/16, so that the
+//      wave that owns K steps w, w+4, ... fetches all its scales of a tile with one
+//      8-byte load per lane (slots = K steps per wave, rounded up to 8).
 // A wave reading entries [kb..kb+3][0..15] of one tile fetches 1 KiB of
 // contiguous nibbles; lane (g = lane/16, n = lane%16) owns block kb+g of row n.
 struct ExpertW {
@@ -44,6 +48,16 @@ struct ExpertW {
 template <class T>
 __device__ __forceinline__ const CSK_GLOBAL T* as_global(const T* p) {
   return (const CSK_GLOBAL T*)p;
+}
+
+// Scale-plane geometry (see ExpertW).
+__host__ __device__ inline int scale_slots(int nblk) {
+  const int per_wave = (((nblk + 3) >> 2) + 3) >> 2;
+  return (per_wave + 7) & ~7;
+}
+__host__ __device__ inline size_t scale_index(long tile, int kb, int n, int slots) {
+  const int j = kb >> 2;
+  return ((size_t)tile * 256 + (size_t)(j & 3) * 64 + (kb & 3) * 16 + n) * slots + (j >> 2);
 }
 
 // E8M0 byte -> scale of true E2M1 values, 2^(b-127); exact for b in 1..254.

@@ -57,6 +57,7 @@ __global__ __launch_bounds__(256) void expert_gemm_kernel(ExpertGemmArgs a) {
   const int n = lane & 15, g = lane >> 4;
   const int nblk = a.nblk;
   const int nsteps = (nblk + 3) >> 2;
+  const int slots = scale_slots(nblk);
 
   // this wave's four weight row tiles
   int tiles[4];
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(256) void expert_gemm_kernel(ExpertGemmArgs a) {
     const uint4* qb = MODE == 0 ? (e < 2 ? wd->w.q_gate : wd->w.q_up) : wd->w.q_down;
     const uint8_t* sb = MODE == 0 ? (e < 2 ? wd->w.s_gate : wd->w.s_up) : wd->w.s_down;
     qp[e] = as_global(reinterpret_cast<const u32x4*>(qb)) + (size_t)tc * nblk * 16 + n;
-    sp[e] = as_global(sb) + (size_t)tc * nblk * 16 + n;
+    sp[e] = as_global(sb) + scale_index(tc, 0, n, slots);
   }
   if (tiles[0] >= a.ntile) {
     // the whole wave is past N; it still takes part in the copies and barriers below
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(256) void expert_gemm_kernel(ExpertGemmArgs a) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       b.q[e] = qp[e][kb * 16];
-      b.s[e] = sp[e][kb * 16];
+      b.s[e] = sp[e][scale_index(0, kb, 0, slots)];
     }
   };
 

@@ -87,8 +87,9 @@ __device__ __forceinline__ uint32_t u4_word(const uint4& v, int i) {
 // MODE 1: a work unit is the pair of down tiles (2R, 2R+1).
 // G = tokens contracted per pass (rows 0..G-1 of the 16-row MFMA tile).
 //
-// The work -- (token group of an expert) x (tile pair) -- is cut into gridDim.x
-// equal contiguous ranges, so the load is balanced whatever the routing was.
+// The work is (token group of an expert) x (tile pair): every group costs the
+// same, so teams of gridDim.x / groups workgroups take one group each and
+// interleave its units, and the load is balanced whatever the routing was.
 // Memory-level parallelism bounds this kernel, so it never lets the memory
 // queue drain: a group's activation rows are copied once into LDS
 // (global_load_lds, no registers), and the weight registers are refilled step
@@ -108,33 +109,35 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
   float* red = reinterpret_cast<float*>(smem + (size_t)G * row_u4 * 16);  // [2][4][NV][16]: live lanes only
 
   const int npair = MODE == 0 ? a.ntile : (a.ntile + 1) >> 1;
-  const long total = (long)(*a.nv) * npair;
-  const long w_begin = total * blockIdx.x / gridDim.x;
-  const long w_end = total * (blockIdx.x + 1) / gridDim.x;
+  // Teams of W workgroups share one token group and interleave its units
+  // (workgroup j takes units j, j + W, ...), so that at any moment a team reads one
+  // contiguous window of the expert's planes.
+  const int nvv = *a.nv;
+  const int W = max(1, (int)gridDim.x / max(nvv, 1));
+  const int teams = gridDim.x / W;
+  const int team = blockIdx.x / W, tj = blockIdx.x % W;
+  if (team >= teams || tj >= npair) return;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
   const int arow = min(n, G - 1) * row_u4;  // lanes past G re-read a live row; their outputs are unused
 
   struct WSet {
     u32x4 q[NS][2];
-    uint32_t sb[NS][2];
+    u32x2 sc[2];  // this wave's scale bytes of the two tiles, one byte per K step
     float b0, b1;
   };
 
   int par = 0;
-  for (long it = w_begin; it < w_end;) {
-    const int v = (int)(it / npair);
-    const int p_begin = (int)(it - (long)v * npair);
-    const int p_end = (int)min((long)npair, p_begin + (w_end - it));
-    it += p_end - p_begin;
+  for (int v = team; v < nvv; v += teams) {
+    const int p_begin = tj, p_end = npair;
     const WorkDesc* wd = a.desc + a.vlist[2 * v];
     const int gbase = a.vlist[2 * v + 1];
     const int gcount = min(G, wd->Te - gbase);
     const int base = wd->base + gbase;
     const CSK_GLOBAL u32x4* q0 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_gate : wd->w.q_down)) + n;
-    const CSK_GLOBAL uint8_t* s0 = as_global(MODE == 0 ? wd->w.s_gate : wd->w.s_down) + n;
+    const CSK_GLOBAL u32x2* s0 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? wd->w.s_gate : wd->w.s_down)) + wv * 64 + lane;
     const CSK_GLOBAL u32x4* q1 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_up : wd->w.q_down)) + n;
-    const CSK_GLOBAL uint8_t* s1 = as_global(MODE == 0 ? wd->w.s_up : wd->w.s_down) + n;
+    const CSK_GLOBAL u32x2* s1 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? wd->w.s_up : wd->w.s_down)) + wv * 64 + lane;
     const CSK_GLOBAL float* bp0 = as_global(MODE == 0 ? wd->w.b_gate : wd->w.b_down);
     const CSK_GLOBAL float* bp1 = as_global(MODE == 0 ? wd->w.b_up : wd->w.b_down);
 
@@ -163,13 +166,14 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
       const size_t ea = (size_t)ta * nblk * 16, eb = (size_t)tb * nblk * 16;
       const int kb = min(4 * (wv + 4 * s) + g, nblk - 1);
       ws.q[s][0] = q0[ea + kb * 16];
-      ws.sb[s][0] = s0[ea + kb * 16];
       ws.q[s][1] = q1[eb + kb * 16];
-      ws.sb[s][1] = s1[eb + kb * 16];
     };
-    auto load_bias = [&](float& b0, float& b1, int unit) {
+    // per-unit scalars: the wave's scale bytes (scale plane: [tile][wave][lane][8]) and biases
+    auto load_unit_scalars = [&](u32x2& sc0, u32x2& sc1, float& b0, float& b1, int unit) {
       const int ta = MODE == 0 ? unit : 2 * unit;
       const int tb = MODE == 0 ? unit : min(2 * unit + 1, a.ntile - 1);
+      sc0 = s0[(size_t)ta * 256];
+      sc1 = s1[(size_t)tb * 256];
       b0 = bp0[min(ta * 16 + n, a.N - 1)];  // bias pointers are never null (absent bias = zero vector)
       b1 = bp1[min(tb * 16 + n, a.N - 1)];
     };
@@ -179,6 +183,7 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
     // Contracts unit `unit` out of ws and, step by step, refills ws with unit `next`.
     auto compute_unit = [&](WSet& ws, int unit, int next) {
       const float bias0 = ws.b0, bias1 = ws.b1;
+      const u32x2 scb0 = ws.sc[0], scb1 = ws.sc[1];
       floatx4 acc[2][2];  // [tile of the pair][hi, lo term]: independent accumulation chains
 #pragma unroll
       for (int m = 0; m < 2; ++m) acc[m][0] = acc[m][1] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -192,8 +197,10 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
       for (int s = 0; s < NS; ++s) {
         const int kb = 4 * (wv + 4 * s) + g;
         const bool kvs = kb < nblk;
-        const float sc0 = kvs ? e8m0_scale(ws.sb[s][0]) : 0.0f;
-        const float sc1 = kvs ? e8m0_scale(ws.sb[s][1]) : 0.0f;
+        const uint32_t byte0 = ((s < 4 ? scb0.x : scb0.y) >> (8 * (s & 3))) & 0xFFu;
+        const uint32_t byte1 = ((s < 4 ? scb1.x : scb1.y) >> (8 * (s & 3))) & 0xFFu;
+        const float sc0 = kvs ? e8m0_scale(byte0) : 0.0f;
+        const float sc1 = kvs ? e8m0_scale(byte1) : 0.0f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int cur = (s * 4 + i) & 1, nxt = cur ^ 1;
@@ -212,7 +219,7 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
         }
         load_step(ws, next, s);  // this step's registers are free: start the next unit's loads
       }
-      load_bias(ws.b0, ws.b1, next);
+      load_unit_scalars(ws.sc[0], ws.sc[1], ws.b0, ws.b1, next);
       float* rbuf = red + (size_t)par * 4 * NV * 16;
       par ^= 1;
       if (live) {
@@ -261,12 +268,13 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
     // are unconditional (past the last unit they re-read it), so that the number of
     // loads in flight is the same on every path and the waits in front of the
     // matrix cores stay partial.
+    const int t_last = p_begin + ((p_end - 1 - p_begin) / W) * W;  // last unit of this workgroup
     WSet ws;
 #pragma unroll
     for (int s = 0; s < NS; ++s) load_step(ws, p_begin, s);
-    load_bias(ws.b0, ws.b1, p_begin);
+    load_unit_scalars(ws.sc[0], ws.sc[1], ws.b0, ws.b1, p_begin);
     __syncthreads();  // the LDS copies have landed (the compiler waits for them before the barrier)
-    for (int t = p_begin; t < p_end; ++t) compute_unit(ws, t, min(t + 1, p_end - 1));
+    for (int t = p_begin; t < p_end; t += W) compute_unit(ws, t, min(t + W, t_last));
   }
 }
 

@@ -55,15 +55,17 @@ __global__ void pack_mxfp4_kernel(const uint8_t* __restrict__ src, uint4* __rest
   const int n = (int)(i & 15);
   const long tk = i >> 4;
   const int kb = (int)(tk % nblk);
-  const long row = (tk / nblk) * 16 + n;
+  const long tile = tk / nblk;
+  const long row = tile * 16 + n;
+  const size_t si = scale_index(tile, kb, n, scale_slots(nblk));
   if (row >= rows) {
     q[i] = make_uint4(0, 0, 0, 0);
-    s[i] = 127;
+    s[si] = 127;
     return;
   }
   const uint8_t* blk = src + (row * nblk + kb) * 17;
   q[i] = ref_block_to_entry(blk);
-  s[i] = blk[0];
+  s[si] = blk[0];
 }
 
 __global__ void export_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t* __restrict__ s,
@@ -73,9 +75,11 @@ __global__ void export_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t* 
   const int n = (int)(i & 15);
   const long tk = i >> 4;
   const int kb = (int)(tk % nblk);
-  const long row = (tk / nblk) * 16 + n;
+  const long tile = tk / nblk;
+  const long row = tile * 16 + n;
+  const size_t si = scale_index(tile, kb, n, scale_slots(nblk));
   if (row >= rows) return;
-  entry_to_ref_block(q[i], s[i], dst + (row * nblk + kb) * 17);
+  entry_to_ref_block(q[i], s[si], dst + (row * nblk + kb) * 17);
 }
 
 // Dequantise through the same conversion instruction the expert kernels use
@@ -90,10 +94,12 @@ __global__ void dequant_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t*
   const int n = (int)(i & 15);
   const long tk = i >> 4;
   const int kb = (int)(tk % nblk);
-  const long row = (tk / nblk) * 16 + n;
+  const long tile = tk / nblk;
+  const long row = tile * 16 + n;
+  const size_t si = scale_index(tile, kb, n, scale_slots(nblk));
   if (row >= rows) return;
   const uint4 e = q[i];
-  const float sc = e8m0_scale(s[i]);
+  const float sc = e8m0_scale(s[si]);
   const uint32_t w[4] = {e.x, e.y, e.z, e.w};
   float* o = dst + (row * nblk + kb) * 32;
 #pragma unroll
@@ -126,10 +132,12 @@ __global__ void synth_mxfp4_kernel(uint4* __restrict__ q, uint8_t* __restrict__ 
   const int n = (int)(i & 15);
   const long tk = i >> 4;
   const int kb = (int)(tk % nblk);
-  const long row = (tk / nblk) * 16 + n;
+  const long tile = tk / nblk;
+  const long row = tile * 16 + n;
+  const size_t si = scale_index(tile, kb, n, scale_slots(nblk));
   if (row >= rows) {
     q[i] = make_uint4(0, 0, 0, 0);
-    s[i] = 127;
+    s[si] = 127;
     return;
   }
   const uint64_t b = (uint64_t)(row * nblk + kb);
@@ -142,7 +150,7 @@ __global__ void synth_mxfp4_kernel(uint4* __restrict__ q, uint8_t* __restrict__ 
     blk[9 + j] = (uint8_t)(h2 >> (8 * j));
   }
   q[i] = ref_block_to_entry(blk);
-  s[i] = blk[0];
+  s[si] = blk[0];
 }
 
 }  // namespace csk
