@@ -309,9 +309,11 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
     constexpr int G = kStreamG;
     a.vlist = ws.vlist;
     a.nv = ws.nv;
-    // kStreamWgPerCu workgroups per compute unit, but never more than the work units there can be
+    // kStreamWgPerCu workgroups per compute unit in steady state; a batch so small that
+    // every work unit can have a workgroup of its own (three fit a compute unit) gets that
     const int64_t npair = NMAT == 2 ? a.ntile : (a.ntile + 1) / 2;
-    const int64_t nwg = std::min<int64_t>(kStreamWgPerCu * (int64_t)std::max(g_cus, 1), P * npair);
+    const int64_t cus = std::max(g_cus, 1);
+    const int64_t nwg = P * npair <= 3 * cus ? P * npair : kStreamWgPerCu * cus;
     const size_t lds = (size_t)G * a.nblk * 128 + 2 * 4 * 8 * 16 * sizeof(float);
     expert_stream_kernel<NMAT == 2 ? 0 : 1, G><<<dim3((unsigned)nwg), 256, lds, g_stream>>>(a);
     return check_launch("expert_stream_kernel");

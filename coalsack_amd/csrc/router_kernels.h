@@ -468,32 +468,60 @@ __global__ __launch_bounds__(1024) void route_small_kernel(
     }
   }
   __syncthreads();
-  // exclusive scan, active experts, token groups
-  if (threadIdx.x == 0) {
-    int run = 0, na = 0, nvv = 0, nm = 0;
-    for (int i = 0; i < E; ++i) {
-      const int c = cnt[i];
-      off[i] = run;
-      offsets[i] = run;
-      if (c > 0) {
-        for (int gb = 0; gb < c; gb += kStreamG) {
-          vlist[2 * nvv] = na;
-          vlist[2 * nvv + 1] = gb;
-          ++nvv;
-        }
-        for (int m0 = 0; m0 < c; m0 += 64) {
-          mtiles[2 * nm] = na;
-          mtiles[2 * nm + 1] = m0;
-          ++nm;
-        }
-        act_e[na++] = i;
-      }
-      run += c;
+  // exclusive scan, active experts, token groups, M tiles: wave 0, four consecutive
+  // experts per lane, wave-wide prefix sums
+  if (wv == 0) {
+    int c[4], tot = 0, nact = 0, ngrp = 0, nmt = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = lane * 4 + j;
+      c[j] = e < E ? cnt[e] : 0;
+      tot += c[j];
+      nact += c[j] > 0;
+      ngrp += (c[j] + kStreamG - 1) / kStreamG;
+      nmt += (c[j] + 63) / 64;
     }
-    offsets[E] = run;
-    na_sh = na;
-    *nv = nvv;
-    *n_mtiles = nm;
+    int s_tot = tot, s_act = nact, s_grp = ngrp, s_mt = nmt;  // inclusive scans over lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t0 = __shfl_up(s_tot, o, 64), t1 = __shfl_up(s_act, o, 64);
+      const int t2 = __shfl_up(s_grp, o, 64), t3 = __shfl_up(s_mt, o, 64);
+      if (lane >= o) {
+        s_tot += t0;
+        s_act += t1;
+        s_grp += t2;
+        s_mt += t3;
+      }
+    }
+    int run = s_tot - tot, slot = s_act - nact, gi = s_grp - ngrp, mi = s_mt - nmt;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = lane * 4 + j;
+      if (e < E) {
+        off[e] = run;
+        offsets[e] = run;
+        if (c[j] > 0) {
+          for (int gb = 0; gb < c[j]; gb += kStreamG) {
+            vlist[2 * gi] = slot;
+            vlist[2 * gi + 1] = gb;
+            ++gi;
+          }
+          for (int m0 = 0; m0 < c[j]; m0 += 64) {
+            mtiles[2 * mi] = slot;
+            mtiles[2 * mi + 1] = m0;
+            ++mi;
+          }
+          act_e[slot++] = e;
+        }
+        run += c[j];
+      }
+    }
+    if (lane == 63) {
+      offsets[E] = s_tot;
+      na_sh = s_act;
+      *nv = s_grp;
+      *n_mtiles = s_mt;
+    }
   }
   __syncthreads();
   // ordered scatter: rank of an assignment = matches before it (ballot prefix)
