@@ -330,8 +330,9 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
   ga.act_type = a.act_type;
   ga.act_out = a.act_out;
   ga.y_out = a.y_out;
+  ga.n_ntiles = (int)cdiv(a.ntile, NMAT == 2 ? 8 : 16);
   const int64_t max_mtiles = P / kGemmBM + std::min<int64_t>(E, P);
-  const dim3 grid((unsigned)cdiv(a.ntile, NMAT == 2 ? 8 : 16), (unsigned)max_mtiles);
+  const dim3 grid((unsigned)(cdiv(max_mtiles * ga.n_ntiles, kDies) * kDies));
   expert_gemm_kernel<NMAT == 2 ? 0 : 1><<<grid, 256, 2 * 2048 * 16, g_stream>>>(ga);
   return check_launch("expert_gemm_kernel");
 }

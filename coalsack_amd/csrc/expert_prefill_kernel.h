@@ -26,6 +26,7 @@
 namespace csk {
 
 constexpr int kGemmBM = 64;  // tokens per M tile
+constexpr int kDies = 8;     // accelerator dies (XCDs) of the part, each with a private L2
 
 struct ExpertGemmArgs {
   const WorkDesc* desc;
@@ -35,6 +36,7 @@ struct ExpertGemmArgs {
   const uint4* A;        // [rows][nblk][8] x 16 B: 32 bf16 hi then 32 bf16 lo per block
   int nblk;              // K / 32
   int ntile;             // ceil(N / 16) weight row tiles
+  int n_ntiles;          // N tiles per M tile: ceil(ntile / 8) (MODE 0) or ceil(ntile / 16)
   int N;
   int act_type;
   uint16_t* act_out;     // MODE 0
@@ -47,9 +49,19 @@ template <int MODE>
 __global__ __launch_bounds__(256) void expert_gemm_kernel(ExpertGemmArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   uint4* As = reinterpret_cast<uint4*>(smem);  // [2 stages][64 tokens][32 chunks]
-  if ((int)blockIdx.y >= *a.n_mtiles) return;
-  const WorkDesc* wd = a.desc + a.mtiles[2 * blockIdx.y];
-  const int m0 = a.mtiles[2 * blockIdx.y + 1];
+  // Work unit = (M tile, N tile), numbered M-tile major.  Workgroups are handed to
+  // the eight accelerator dies round-robin by linear id, and each die has its own L2:
+  // die x takes the x-th contiguous eighth of the unit sequence, so that the
+  // workgroups resident on one die at one time share a few activation panels and a few
+  // experts' weights, which then come from that L2 instead of from memory.
+  const int n_units = *a.n_mtiles * a.n_ntiles;
+  const int per_die = (n_units + kDies - 1) / kDies;
+  const int slot = blockIdx.x / kDies;
+  const int unit = (blockIdx.x % kDies) * per_die + slot;
+  if (slot >= per_die || unit >= n_units) return;
+  const int mt = unit / a.n_ntiles, nt = unit - mt * a.n_ntiles;
+  const WorkDesc* wd = a.desc + a.mtiles[2 * mt];
+  const int m0 = a.mtiles[2 * mt + 1];
   const int Te = wd->Te;
   const int base = wd->base + m0;
   const int mcount = min(kGemmBM, Te - m0);
@@ -66,8 +78,8 @@ __global__ __launch_bounds__(256) void expert_gemm_kernel(ExpertGemmArgs a) {
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     int t;
-    if (MODE == 0) t = blockIdx.x * 8 + wv * 2 + (e & 1);
-    else t = blockIdx.x * 16 + wv * 4 + e;
+    if (MODE == 0) t = nt * 8 + wv * 2 + (e & 1);
+    else t = nt * 16 + wv * 4 + e;
     tiles[e] = t;
     const int tc = min(t, a.ntile - 1);
     const uint4* qb = MODE == 0 ? (e < 2 ? wd->w.q_gate : wd->w.q_up) : wd->w.q_down;
