@@ -142,12 +142,23 @@ def bench_stack(lib, synth, shape, T, steps, warmup, n_layers, seed=1234):
         stack_forward(lib, layers, d_h, T)
     ms = time_forward(lib, fn, steps, warmup)
     out = lib.to_host(d_h, hidden.shape)
+    # untimed pass, layer by layer, to count the distinct experts each layer streams
+    from coalsack_amd.capi import FWD_RMSNORM, FWD_RESIDUAL
+    lib.copy_d2d(d_h, d_h0, hidden.nbytes)
+    total_bytes, distinct = 0, []
+    for layer in layers:
+        layer.forward_device(d_h, T, d_h, FWD_RMSNORM | FWD_RESIDUAL)
+        counts, _ = layer.last_dispatch(T)
+        U = int(np.count_nonzero(counts))
+        distinct.append(U)
+        total_bytes += layer_bytes(shape["E"], shape["k"], shape["H"], shape["F"], T, U) + shape["H"] * 4
     lib.dev_free(d_h)
     lib.dev_free(d_h0)
     for layer in layers:
         layer.close()
     return dict(T=T, layers=n_layers, ms_per_step=ms, tokens_per_s=T / (ms * 1e-3),
-                finite=bool(np.all(np.isfinite(out))))
+                finite=bool(np.all(np.isfinite(out))), stack_bytes=total_bytes,
+                distinct_experts_per_layer=distinct)
 
 
 def cpu_baseline(L, hidden, gpu_out, budget_s=12.0):
@@ -217,8 +228,14 @@ def main():
                     higher_is_better=True, scaling="weak", vs_baseline=None, dtype="mxfp4 x bf16(2-term) -> f32",
                     data="synthetic",
                     config=dict(workload=f"c5_stack: 36 x 120b-shaped MoE layer (RMSNorm + residual), T={T}",
-                                tokens=T, device=dev_name),
-                    roofline=None, cpu_baseline=None, finite=res["finite"])
+                                tokens=T, device=dev_name,
+                                distinct_experts_per_layer=res["distinct_experts_per_layer"]),
+                    roofline=dict(bound="hbm", kernel="whole stack (all kernels of 36 layers)",
+                                  achieved=res["stack_bytes"] / (res["ms_per_step"] * 1e-3) / 1e9,
+                                  peak=HBM_PEAK_GBS, unit="GB/s", traffic=None,
+                                  frac=res["stack_bytes"] / (res["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                  algorithmic_bytes=res["stack_bytes"]),
+                    cpu_baseline=None, finite=res["finite"])
         print(json.dumps(line))
         return
 
