@@ -268,6 +268,21 @@ int launch_prep(const float* src, const float* norm_w, float eps, float* xn, uin
   return check_launch("prep_kernel");
 }
 
+// x [*, H] fp32 -> three-term FP6 rows (the grouped GEMM's activation operand).
+int launch_mx3(const float* x, uint16_t* x3, int64_t rows, int64_t H, const int* gather_tok,
+               const float* gather_w) {
+  if (rows == 0) return CSK_OK;
+  const int64_t nb = rows * (H / 32);
+  mx3_rows_kernel<<<dim3((unsigned)cdiv(nb, 256)), 256, 0, g_stream>>>(
+      x, reinterpret_cast<u32x4*>(x3), rows, (int)(H / 32), gather_tok, gather_w);
+  return check_launch("mx3_rows_kernel");
+}
+
+// Small batches stream the weights once (HBM-bound, bf16 two-term activations); larger
+// ones run the grouped GEMM on the block-scaled matrix instruction (three-term FP6
+// activations).  One decision per forward: it fixes the activation format of both GEMMs.
+bool stream_path(int64_t T, int64_t H, int64_t F) { return T <= 64 && H / 32 <= 96 && F / 32 <= 96; }
+
 int launch_router(const float* x, const float* gate_w, const float* gate_b, int64_t T, int64_t E,
                   int64_t H, int64_t k, int sigmoid, float* logits, float* pairs, int* ids) {
   if (T == 0) return CSK_OK;
@@ -304,8 +319,8 @@ int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, in
 // Weight-streaming kernel for small batches (every expert sees few tokens, the
 // layer is HBM-bound); grouped GEMM otherwise.
 template <int NMAT>
-int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspace& ws) {
-  if (T <= 64 && a.nblk <= 96) {
+int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspace& ws, bool stream) {
+  if (stream) {
     constexpr int G = kStreamG;
     a.vlist = ws.vlist;
     a.nv = ws.nv;
@@ -318,7 +333,7 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
     expert_stream_kernel<NMAT == 2 ? 0 : 1, G><<<dim3((unsigned)nwg), 256, lds, g_stream>>>(a);
     return check_launch("expert_stream_kernel");
   }
-  ExpertGemmArgs ga{};
+  ExpertGemmMxArgs ga{};
   ga.desc = a.desc;
   ga.mtiles = ws.tiles;
   ga.n_mtiles = ws.n_tiles;
@@ -328,13 +343,13 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
   ga.ntile = a.ntile;
   ga.N = a.N;
   ga.act_type = a.act_type;
-  ga.act_out = a.act_out;
+  ga.act_out = reinterpret_cast<u32x4*>(a.act_out);
   ga.y_out = a.y_out;
-  ga.n_ntiles = (int)cdiv(a.ntile, NMAT == 2 ? 8 : 16);
+  ga.n_ntiles = (int)cdiv(a.ntile, (NMAT == 2 ? 2 : 4) * kMxWaves);
   const int64_t max_mtiles = P / kGemmBM + std::min<int64_t>(E, P);
   const dim3 grid((unsigned)(cdiv(max_mtiles * ga.n_ntiles, kDies) * kDies));
-  expert_gemm_kernel<NMAT == 2 ? 0 : 1><<<grid, 256, 2 * 2048 * 16, g_stream>>>(ga);
-  return check_launch("expert_gemm_kernel");
+  expert_gemm_mx_kernel<NMAT == 2 ? 0 : 1><<<grid, 64 * kMxWaves, 3 * kMxStageChunks * 16, g_stream>>>(ga);
+  return check_launch("expert_gemm_mx_kernel");
 }
 
 // Experts' MLPs over the dispatched tokens: ws.y[P,H] <- down(act(gate, up)).
@@ -344,6 +359,7 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
                 int act_type, const uint16_t* x_split, const int* list_row, Workspace& ws,
                 bool timed = false) {
   const int64_t P = T * k;
+  const bool stream = stream_path(T, H, F);
   ExpertStreamArgs a{};
   a.desc = ws.desc;
   a.act_type = act_type;
@@ -356,7 +372,7 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   a.act_out = ws.act;
   a.y_out = nullptr;
   if (timed) mark(CSK_STAGE_GATEUP);
-  int rc = launch_experts<2>(a, E, T, P, ws);
+  int rc = launch_experts<2>(a, E, T, P, ws, stream);
   if (rc != CSK_OK) return rc;
   if (timed) mark(CSK_STAGE_DOWN);
   // down
@@ -367,7 +383,7 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   a.ntile = (int)cdiv(H, 16);
   a.act_out = nullptr;
   a.y_out = ws.y;
-  return launch_experts<1>(a, E, T, P, ws);
+  return launch_experts<1>(a, E, T, P, ws, stream);
 }
 
 int launch_combine(const float* y, const float* pairs, const int* pos, const float* residual,
@@ -757,11 +773,22 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
         ws.logits, ws.pairs, ws.ids, (int)T, (int)L->E, (int)L->k, L->sigmoid, L->ew_dev, ws.counts,
         ws.offsets, ws.desc, ws.vlist, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w, ws.pos);
     if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
+    if (!stream_path(T, L->H, L->F) && !L->wbf) {
+      // few tokens but rows too long for the streaming kernel: the GEMM wants the FP6 form
+      if ((rc = launch_mx3(xr, ws.xs, T, L->H, nullptr, nullptr)) != CSK_OK) return rc;
+    }
   } else {
     mark(CSK_STAGE_PREP);
-    rc = launch_prep(hidden, norm ? L->norm_w : nullptr, L->eps, norm ? ws.xn : nullptr, ws.xs, T,
-                     L->H, nullptr, nullptr);
-    if (rc != CSK_OK) return rc;
+    const bool stream = stream_path(T, L->H, L->F);
+    if (norm || stream) {
+      rc = launch_prep(hidden, norm ? L->norm_w : nullptr, L->eps, norm ? ws.xn : nullptr,
+                       stream ? ws.xs : nullptr, T, L->H, nullptr, nullptr);
+      if (rc != CSK_OK) return rc;
+    }
+    if (!stream && !L->wbf) {
+      rc = launch_mx3(xr, ws.xs, T, L->H, nullptr, nullptr);
+      if (rc != CSK_OK) return rc;
+    }
     mark(CSK_STAGE_ROUTER);
     rc = launch_router(xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, T, L->E, L->H, L->k,
                        L->sigmoid, ws.logits, ws.pairs, ws.ids);
@@ -773,7 +800,9 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
   const uint16_t* xa = ws.xs;
   const int* list_row = ws.list_tok;
   if (L->wbf) {
-    rc = launch_prep(xr, nullptr, 0.f, nullptr, ws.xg, P, L->H, ws.list_tok, ws.list_w);
+    rc = stream_path(T, L->H, L->F)
+             ? launch_prep(xr, nullptr, 0.f, nullptr, ws.xg, P, L->H, ws.list_tok, ws.list_w)
+             : launch_mx3(xr, ws.xg, P, L->H, ws.list_tok, ws.list_w);
     if (rc != CSK_OK) return rc;
     xa = ws.xg;
     list_row = nullptr;
@@ -946,12 +975,16 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
     // The expert's token count is only known on the device, and at most T
     // tokens can select it: gather T rows.  Positions past the count read the
     // zeroed tail of the lists (token 0, weight 0) and are never consumed.
-    rc = launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xg, T, H, ws.list_tok, ws.list_w);
+    rc = stream_path(T, H, F)
+             ? launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xg, T, H, ws.list_tok, ws.list_w)
+             : launch_mx3(dx.as<float>(), ws.xg, T, H, ws.list_tok, ws.list_w);
     if (rc != CSK_OK) return rc;
     xa = ws.xg;
     list_row = nullptr;
   } else {
-    rc = launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xs, T, H, nullptr, nullptr);
+    rc = stream_path(T, H, F)
+             ? launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xs, T, H, nullptr, nullptr)
+             : launch_mx3(dx.as<float>(), ws.xs, T, H, nullptr, nullptr);
     if (rc != CSK_OK) return rc;
     xa = ws.xs;
     list_row = ws.list_tok;

@@ -1,54 +1,70 @@
-// Expert MLP for the compute-bound (prefill) regime: grouped GEMM over the
-// dispatched tokens on the matrix cores.
+// Expert MLP for the compute-bound (prefill) regime on the block-scaled matrix
+// instruction: v_mfma_scale_f32_32x32x64_f8f6f4 with A = activations as three
+// FP6 (E2M3) terms (mx3.h) and B = the MXFP4 weights exactly as they are stored.
 //
-// A workgroup owns one M tile (64 tokens of one expert) x one N tile (128
-// output features: gate and up rows together, or 256 down rows) and walks K in
-// steps of 128 elements.  Per step
-//   * the activation tile (64 tokens x 128 elements, two bf16 terms = 32 KiB)
-//     is copied into LDS by global_load_lds, gathered by token, with a 16-byte
-//     XOR swizzle chosen at the *source* side (each lane picks which chunk it
-//     fetches) so that the 16 lanes of a fragment read hit 16 different bank
-//     groups;
-//   * each wave loads its four weight entries (16 rows x 4 blocks x 16 B, the
-//     resident packed layout is already fragment order) straight into
-//     registers, one step ahead, and expands them with
-//     v_cvt_scalef32_pk_bf16_fp4;
-//   * 128 MFMAs (16x16x32 bf16) per wave contract hi and lo terms into fp32.
-// Two LDS stages, one barrier per step.  The epilogue fuses bias + SwiGLU (and
-// the bf16 split the next GEMM reads) or bias + store.
+// Measured on this part with random operands: 5.6-6.2 PFLOP/s for FP6 x FP4 in
+// the 32x32x64 form, against 1.9 PFLOP/s for bf16 32x32x16 (1.3 for 16x16x32);
+// three FP6 terms instead of two bf16 terms therefore cost about half the matrix
+// time, need no weight expansion (no conversion instruction at all), and the
+// activation tile is 24 KiB per stage instead of 32.
+//
+// Operand ownership of the instruction (found by one-hot probing): lane l holds
+// row l%32 of A (a token) or column l%32 of B (a weight row) and the 32 K values
+// of block l/32 of the 64; position p of A pairs with position p of B; each lane
+// passes the E8M0 scale of its own block.  A weight "column" l%32 is row l%16 of
+// tile (l%32)/16 of a pair of packed 16-row tiles, and its 16-byte packed entry
+// (32 nibbles in element order) is the operand.
+//
+// A workgroup of eight waves owns 64 tokens of one expert x 256 features (gate and
+// up rows together) or 512 down rows, and walks K in steps of 128 (4 blocks); the
+// kernel is bound by what the compute units can pull from L2, and the activation
+// tile is fetched once per workgroup, so the wide tile is what sets its speed.  The
+// activation tile (64 tokens x 4 blocks x 3 terms x 32 B) goes to LDS by
+// global_load_lds with a 16-byte XOR swizzle applied on the source side; weights
+// go straight to registers; both are requested two steps ahead (three LDS stages, one
+// barrier per step).
+// The gate/up epilogue applies bias + SwiGLU, stages the 64 x 128 tile in LDS as
+// fp32 and re-quantises it to the three-term format the down GEMM reads.
 //
 // Restates include/coalsack/nn/nn_ops/expert_mlp_node.h:651-732 with the token
 // loop of :503-529 as the M dimension.
 #pragma once
 #include "common.h"
 #include "expert_stream_kernel.h"
+#include "mx3.h"
 
 namespace csk {
 
-constexpr int kGemmBM = 64;  // tokens per M tile
-constexpr int kDies = 8;     // accelerator dies (XCDs) of the part, each with a private L2
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32_unaligned __attribute__((aligned(1)));
 
-struct ExpertGemmArgs {
+struct ExpertGemmMxArgs {
   const WorkDesc* desc;
   const int* mtiles;     // [2 * n]: (expert slot, first token) of each M tile
   const int* n_mtiles;
   const int* list_row;   // packed position -> row of A; null: row = packed position
-  const uint4* A;        // [rows][nblk][8] x 16 B: 32 bf16 hi then 32 bf16 lo per block
+  const uint4* A;        // [rows][nblk][6] x 16 B (mx3.h)
   int nblk;              // K / 32
   int ntile;             // ceil(N / 16) weight row tiles
-  int n_ntiles;          // N tiles per M tile: ceil(ntile / 8) (MODE 0) or ceil(ntile / 16)
+  int n_ntiles;          // N tiles per M tile: ceil(ntile / 16) (MODE 0) or ceil(ntile / 32)
   int N;
   int act_type;
-  uint16_t* act_out;     // MODE 0
-  float* y_out;          // MODE 1
+  u32x4* act_out;        // MODE 0: [P][N / 32][6] x 16 B
+  float* y_out;          // MODE 1: [P][N]
 };
 
-// MODE 0: N tile = 128 features; wave w owns gate tiles {8x+2w, 8x+2w+1} and the
-//         same up tiles.  MODE 1: N tile = 256 rows; wave w owns down tiles 16x+4w..+3.
+constexpr int kGemmBM = 64;  // tokens per M tile
+constexpr int kDies = 8;     // accelerator dies (XCDs) of the part, each with a private L2
+
+constexpr int kMxStageChunks = kGemmBM * 4 * kMx3ChunksPerBlock;  // 1536 x 16 B = 24 KiB
+constexpr int kMxRowChunks = 4 * kMx3ChunksPerBlock;              // 24 chunks per token per step
+constexpr int kMxWaves = 4;                                       // waves per workgroup
+constexpr int kMxCopies = kMxStageChunks / 64 / kMxWaves;         // copy instructions per wave per step
+
 template <int MODE>
-__global__ __launch_bounds__(256) void expert_gemm_kernel(ExpertGemmArgs a) {
+__global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_kernel(ExpertGemmMxArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
-  uint4* As = reinterpret_cast<uint4*>(smem);  // [2 stages][64 tokens][32 chunks]
+  uint4* As = reinterpret_cast<uint4*>(smem);  // [3 stages][64 tokens][24 chunks]
   // Work unit = (M tile, N tile), numbered M-tile major.  Workgroups are handed to
   // the eight accelerator dies round-robin by linear id, and each die has its own L2:
   // die x takes the x-th contiguous eighth of the unit sequence, so that the
@@ -66,140 +82,213 @@ __global__ __launch_bounds__(256) void expert_gemm_kernel(ExpertGemmArgs a) {
   const int base = wd->base + m0;
   const int mcount = min(kGemmBM, Te - m0);
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int n = lane & 15, g = lane >> 4;
+  const int n32 = lane & 31, kg = lane >> 5;
+  const int n16 = n32 & 15, th = n32 >> 4;  // row within a packed tile, tile of the pair
   const int nblk = a.nblk;
   const int nsteps = (nblk + 3) >> 2;
   const int slots = scale_slots(nblk);
 
-  // this wave's four weight row tiles
-  int tiles[4];
-  const CSK_GLOBAL u32x4* qp[4];
-  const CSK_GLOBAL uint8_t* sp[4];
+  // this wave's two 32-row groups (each a pair of packed tiles)
+  int tiles[2];  // this lane's packed tile in each group
+  const CSK_GLOBAL u32x4* qp[2];
+  const CSK_GLOBAL uint8_t* sp[2];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
+  for (int s = 0; s < 2; ++s) {
     int t;
-    if (MODE == 0) t = nt * 8 + wv * 2 + (e & 1);
-    else t = nt * 16 + wv * 4 + e;
-    tiles[e] = t;
+    if (MODE == 0) t = nt * (2 * kMxWaves) + wv * 2 + th;
+    else t = nt * (4 * kMxWaves) + wv * 4 + 2 * s + th;
+    tiles[s] = t;
     const int tc = min(t, a.ntile - 1);
-    const uint4* qb = MODE == 0 ? (e < 2 ? wd->w.q_gate : wd->w.q_up) : wd->w.q_down;
-    const uint8_t* sb = MODE == 0 ? (e < 2 ? wd->w.s_gate : wd->w.s_up) : wd->w.s_down;
-    qp[e] = as_global(reinterpret_cast<const u32x4*>(qb)) + (size_t)tc * nblk * 16 + n;
-    sp[e] = as_global(sb) + scale_index(tc, 0, n, slots);
-  }
-  if (tiles[0] >= a.ntile) {
-    // the whole wave is past N; it still takes part in the copies and barriers below
+    const uint4* qb = MODE == 0 ? (s == 0 ? wd->w.q_gate : wd->w.q_up) : wd->w.q_down;
+    const uint8_t* sb = MODE == 0 ? (s == 0 ? wd->w.s_gate : wd->w.s_up) : wd->w.s_down;
+    qp[s] = as_global(reinterpret_cast<const u32x4*>(qb)) + (size_t)tc * nblk * 16 + n16;
+    sp[s] = as_global(sb) + scale_index(tc, 0, n16, slots);
   }
 
-  // rows this lane copies: instruction c (0..7) of wave wv moves tokens 2*(8*wv+c), +1
-  const uint4* arow[8];
+  // Copy instruction c of wave wv fills chunks [(kMxCopies wv + c) * 64, +64) of the
+  // stage, in token-major order; the lane's chunk is physical position pc of token tl
+  // and holds logical chunk lc (XOR swizzle on the low three bits).
+  const uint4* arow[kMxCopies];  // source of this lane's chunk at step 0, minus the block term
+  int ablk[kMxCopies];           // block of the step the chunk belongs to
 #pragma unroll
-  for (int c = 0; c < 8; ++c) {
-    const int tl = min(2 * (8 * wv + c) + (lane >> 5), mcount - 1);  // tokens past the tile re-read its last one
-    const int row = a.list_row ? a.list_row[base + tl] : base + tl;
-    arow[c] = a.A + (size_t)row * nblk * 8;
+  for (int c = 0; c < kMxCopies; ++c) {
+    const int lin = (kMxCopies * wv + c) * 64 + lane;
+    const int tl = lin / kMxRowChunks, pc = lin - tl * kMxRowChunks;
+    const int lc = (pc & ~7) | ((pc & 7) ^ ((tl >> 1) & 7));
+    const int bs = lc / kMx3ChunksPerBlock;
+    const int tlc = min(tl, mcount - 1);  // tokens past the tile re-read its last one
+    const int row = a.list_row ? a.list_row[base + tlc] : base + tlc;
+    arow[c] = a.A + (size_t)row * nblk * kMx3ChunksPerBlock + (lc - bs * kMx3ChunksPerBlock);
+    ablk[c] = bs;
   }
   auto copy_a = [&](int stage, int j) {
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      const int q = 8 * wv + c;                    // copy instruction index within the stage
-      const int tl = 2 * q + (lane >> 5);          // token slot this lane serves
-      const int ci = (lane & 31) ^ (tl & 15);      // logical chunk stored at this lane's position
-      const int kb = min(4 * j + (ci >> 3), nblk - 1);
+    for (int c = 0; c < kMxCopies; ++c) {
+      const int kb = min(4 * j + ablk[c], nblk - 1);  // a block past K re-reads the last one (its weights are zeroed)
       __builtin_amdgcn_global_load_lds(
-          arow[c] + (size_t)kb * 8 + (ci & 7),
+          arow[c] + (size_t)kb * kMx3ChunksPerBlock,
           reinterpret_cast<__attribute__((address_space(3))) uint4*>(
-              reinterpret_cast<uintptr_t>(As + stage * 2048 + q * 64)),
+              reinterpret_cast<uintptr_t>(As + stage * kMxStageChunks + (kMxCopies * wv + c) * 64)),
           16, 0, 0);
     }
   };
   struct BSet {
-    u32x4 q[4];
-    uint32_t s[4];
+    u32x4 q[2][2];     // [64-wide K chunk of the step][row group]
+    uint32_t s[2][2];  // byte 0 = the block's scale byte (the matrix instruction reads only that byte)
   };
   auto load_b = [&](BSet& b, int j) {
-    const int kb = min(4 * j + g, nblk - 1);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      b.q[e] = qp[e][kb * 16];
-      b.s[e] = sp[e][scale_index(0, kb, 0, slots)];
+    for (int kc = 0; kc < 2; ++kc) {
+      const int kb = min(4 * j + 2 * kc + kg, nblk - 1);
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        b.q[kc][s] = qp[s][kb * 16];
+        // a dword load at the byte's own (unaligned) address: no widening instruction, so
+        // nothing waits for the value before the matrix instruction that uses it
+        b.s[kc][s] = *reinterpret_cast<const CSK_GLOBAL u32_unaligned*>(sp[s] + scale_index(0, kb, 0, slots));
+      }
     }
   };
 
-  floatx4 acc[4][4];  // [m sub-tile][weight tile]
+  floatx16 acc[2][2];  // [32-token sub-tile][row group]
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+  for (int ms = 0; ms < 2; ++ms)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) acc[mt][e] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[ms][s][r] = 0.0f;
 
+  const int sw = (n32 >> 1) & 7;
+  // Fragment i = (kc, term, 32-token sub-tile) of a step feeds two matrix instructions
+  // (the two row groups).  Fragments are requested from LDS two ahead of their use, so
+  // the LDS latency is covered by the four matrix instructions in between.
   auto compute = [&](const BSet& b, int stage, int j) {
-    const bool kv = 4 * j + g < nblk;
-    float sc[4];
+    const u32x4* at = reinterpret_cast<const u32x4*>(As) + stage * kMxStageChunks;
+    i32x8 bw[2][2];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) sc[e] = kv ? e8m0_scale(b.s[e]) : 0.0f;
-    const uint4* at = As + stage * 2048;
+    for (int kc = 0; kc < 2; ++kc) {
+      const bool kv = 4 * j + 2 * kc + kg < nblk;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      U4B8 ah[4], al[4];
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
-        const int tok = mt * 16 + n;
-        ah[mt].u = at[tok * 32 + ((g * 8 + i) ^ n)];
-        al[mt].u = at[tok * 32 + ((g * 8 + 4 + i) ^ n)];
+      for (int s = 0; s < 2; ++s) {
+        const u32x4 q = kv ? b.q[kc][s] : u32x4{0u, 0u, 0u, 0u};
+        bw[kc][s] = (i32x8)__builtin_shufflevector(q, q, 0, 1, 2, 3, -1, -1, -1, -1);  // FP4 reads four registers
       }
+    }
+    u32x4 flo[3], fhi[3];
+    auto read_frag = [&](int i) {
+      const int kc = i / 6, t = (i % 6) >> 1, ms = i & 1;
+      const int c0 = ((2 * kc + kg) * kMx3Terms + t) * 2;
+      const int tok = ms * 32 + n32;
+      flo[i % 3] = at[tok * kMxRowChunks + ((c0 & ~7) | ((c0 & 7) ^ sw))];
+      fhi[i % 3] = at[tok * kMxRowChunks + (((c0 + 1) & ~7) | (((c0 + 1) & 7) ^ sw))];
+    };
+    read_frag(0);
+    read_frag(1);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bf16x8 bw = cvt_fp4x8(b.q[e][i], sc[e]);
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-          acc[mt][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah[mt].b, bw, acc[mt][e], 0, 0, 0);
-          acc[mt][e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[mt].b, bw, acc[mt][e], 0, 0, 0);
-        }
-      }
+    for (int i = 0; i < 12; ++i) {
+      const int kc = i / 6, ms = i & 1;
+      if (i + 2 < 12) read_frag(i + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      // FP6 reads the first six registers; fhi[2] (register 6) is the term's scale byte
+      const i32x8 aw = (i32x8)__builtin_shufflevector(flo[i % 3], fhi[i % 3], 0, 1, 2, 3, 4, 5, 6, 7);
+      acc[ms][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aw, bw[kc][0], acc[ms][0], 2, 4, 0,
+                                                                   (int)fhi[i % 3][2], 0, (int)b.s[kc][0]);
+      acc[ms][1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aw, bw[kc][1], acc[ms][1], 2, 4, 0,
+                                                                   (int)fhi[i % 3][2], 0, (int)b.s[kc][1]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  BSet ba, bb;
+  // Three LDS stages, loads two steps ahead.  A __syncthreads() would drain every
+  // outstanding load (its fence waits for vmcnt(0)), so the step boundary is an explicit
+  // count + bare barrier: a wave's loads of step j are older than the kStepLoads loads of
+  // step j+1, memory counters retire in order, so vmcnt(kStepLoads) means "my part of
+  // step j has landed", and the barrier extends that to the other waves' parts and
+  // tells that every wave is done reading the stage about to be overwritten.
+  constexpr int kStepLoads = kMxCopies + 2 * 2 * 2;  // copy_a + load_b instructions per step
+  constexpr int kWaitStep = (kStepLoads & 15) | (7 << 4) | (15 << 8) | ((kStepLoads >> 4) << 14);
+  // The first two steps are requested and awaited in full before the loop, so that the
+  // loop is entered with nothing in flight and its body is the steady state from the
+  // first iteration on (loads still pending at the loop entry would make the compiler's
+  // own wait insertion fall back to vmcnt(0) inside the loop).
+  BSet bs[3];
   copy_a(0, 0);
-  load_b(ba, 0);
-  for (int j = 0; j < nsteps; j += 2) {
-    __syncthreads();  // stage 0 has landed; every wave is done with stage 1
-    copy_a(1, min(j + 1, nsteps - 1));
-    load_b(bb, min(j + 1, nsteps - 1));
-    compute(ba, 0, j);
-    __syncthreads();  // stage 1 has landed; every wave is done with stage 0
-    copy_a(0, min(j + 2, nsteps - 1));
-    load_b(ba, min(j + 2, nsteps - 1));
-    if (j + 1 < nsteps) compute(bb, 1, j + 1);
+  load_b(bs[0], 0);
+  copy_a(1, min(1, nsteps - 1));
+  load_b(bs[1], min(1, nsteps - 1));
+  __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0)
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int kc = 0; kc < 2; ++kc)
+#pragma unroll
+      for (int g = 0; g < 2; ++g)  // "use" the loaded registers so the compiler, too, knows they have arrived
+        asm volatile("" : "+v"(bs[i].q[kc][g]), "+v"(bs[i].s[kc][g]));
+  __builtin_amdgcn_sched_barrier(0);
+  auto step = [&](int u, int jj) {
+    __builtin_amdgcn_s_waitcnt(kWaitStep);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    copy_a((u + 2) % 3, min(jj + 2, nsteps - 1));
+    load_b(bs[(u + 2) % 3], min(jj + 2, nsteps - 1));
+    __builtin_amdgcn_sched_barrier(0);
+    compute(bs[u], u, jj);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // no control-flow joins between the steps of the steady state
+  for (int j = 0;; j += 3) {
+    step(0, j);
+    if (j + 1 >= nsteps) break;
+    step(1, j + 1);
+    if (j + 2 >= nsteps) break;
+    step(2, j + 2);
+    if (j + 3 >= nsteps) break;
   }
 
-  // epilogue: lane (n, g) holds tokens mt*16 + 4g + i of weight row n of each tile
+  // epilogue: lane holds weight row n32 of each group; accumulator register r is token
+  // (r % 4) + 8 * (r / 4) + 4 * kg of the 32-token sub-tile
+  if (MODE == 0) {
+    // bias + activation into LDS as fp32 [token][block = wave][32 + 1], then one thread per
+    // (token, block) re-quantises 32 features to the three-term format
+    __syncthreads();  // the copies issued for the step after the last have landed; all waves are past their reads
+    float* stage = reinterpret_cast<float*>(smem);
+    const int row = tiles[0] * 16 + n16;  // feature
+    const bool rv = tiles[0] < a.ntile && row < a.N;
+    const float bg = rv ? wd->w.b_gate[row] : 0.0f;
+    const float bu = rv ? wd->w.b_up[row] : 0.0f;
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
+    for (int ms = 0; ms < 2; ++ms) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int tl = mt * 16 + g * 4 + i;
-      if (tl >= mcount) continue;
-      const size_t p = (size_t)(base + tl);
-      if (MODE == 0) {
+      for (int r = 0; r < 16; ++r) {
+        const int tl = ms * 32 + (r & 3) + 8 * (r >> 2) + 4 * kg;
+        stage[(tl * kMxWaves + wv) * 33 + n32] = moe_activation(acc[ms][0][r] + bg, acc[ms][1][r] + bu, a.act_type);
+      }
+    }
+    __syncthreads();
+    const int tl = threadIdx.x / kMxWaves, blk = threadIdx.x % kMxWaves;
+    const int kb = nt * kMxWaves + blk;
+    if (tl < mcount && kb * 32 < a.N) {
+      float v[32];
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const int r = tiles[e] * 16 + n;
-          if (tiles[e] < a.ntile && r < a.N) {
-            const float gate_v = acc[mt][e][i] + wd->w.b_gate[r];
-            const float up_v = acc[mt][e + 2][i] + wd->w.b_up[r];
-            uint16_t hi, lo;
-            split_bf16(moe_activation(gate_v, up_v, a.act_type), hi, lo);
-            uint16_t* o = a.act_out + (p * (size_t)(a.N >> 5) + (r >> 5)) * 64 + (r & 31);
-            o[0] = hi;
-            o[32] = lo;
-          }
-        }
-      } else {
+      for (int i = 0; i < 32; ++i) v[i] = stage[(tl * kMxWaves + blk) * 33 + i];
+      u32x4 out[kMx3ChunksPerBlock];
+      mx3_quantize_block(v, out);
+      u32x4* o = a.act_out + ((size_t)(base + tl) * (a.N >> 5) + kb) * kMx3ChunksPerBlock;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = tiles[e] * 16 + n;
-          if (tiles[e] < a.ntile && r < a.N) a.y_out[p * (size_t)a.N + r] = acc[mt][e][i] + wd->w.b_down[r];
+      for (int c = 0; c < kMx3ChunksPerBlock; ++c) o[c] = out[c];
+    }
+  } else {
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int tl = ms * 32 + (r & 3) + 8 * (r >> 2) + 4 * kg;
+        if (tl >= mcount) continue;
+        const size_t p = (size_t)(base + tl);
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          const int row = tiles[s] * 16 + n16;
+          if (tiles[s] < a.ntile && row < a.N) a.y_out[p * (size_t)a.N + row] = acc[ms][s][r] + wd->w.b_down[row];
         }
       }
     }

@@ -3,6 +3,7 @@
 // (histogram -> prefix scan -> ordered scatter) and the weighted combine.
 #pragma once
 #include "common.h"
+#include "mx3.h"
 #include "expert_stream_kernel.h"
 
 namespace csk {
