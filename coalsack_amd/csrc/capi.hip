@@ -294,7 +294,7 @@ int launch_router(const float* x, const float* gate_w, const float* gate_b, int6
     router_logits_kernel<4><<<dim3(gx, (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
         x, gate_w, gate_b, logits, (int)T, (int)E, (int)H);
   } else {
-    router_logits_kernel<8><<<dim3(gx, (unsigned)cdiv(T, 8)), 256, 0, g_stream>>>(
+    router_logits_mfma_kernel<<<dim3((unsigned)cdiv(T, 32), (unsigned)cdiv(E, 32)), 256, 0, g_stream>>>(
         x, gate_w, gate_b, logits, (int)T, (int)E, (int)H);
   }
   int rc = check_launch("router_logits_kernel");

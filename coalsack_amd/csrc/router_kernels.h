@@ -90,6 +90,72 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restr
   }
 }
 
+// ------------------------------------------------- router logits, many tokens
+// The same logits as an fp32 GEMM on the matrix cores (v_mfma_f32_32x32x2_f32: fp32
+// operands, fp32 accumulation, so nothing is rounded to a narrower type).  A workgroup
+// owns 32 tokens x 32 experts; its four waves take interleaved 16-wide slices of H and
+// their partial tiles are added in LDS in a fixed order.  Operand ownership: lane l
+// holds row l%32 (token, or expert) and k index l/32 of the two; each lane loads eight
+// consecutive values of its row per iteration and feeds them to eight instructions --
+// any assignment of k to (instruction, lane half) is valid as long as both operands
+// use the same one.
+__global__ __launch_bounds__(256) void router_logits_mfma_kernel(const float* __restrict__ x,
+                                                                 const float* __restrict__ g,
+                                                                 const float* __restrict__ b,
+                                                                 float* __restrict__ logits, int T,
+                                                                 int E, int H) {
+  __shared__ float part[4][32][33];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int r32 = lane & 31, half = lane >> 5;
+  const int t0 = blockIdx.x * 32, e0 = blockIdx.y * 32;
+  const float* xr = x + (size_t)min(t0 + r32, T - 1) * H + 8 * half;
+  const float* gr = g + (size_t)min(e0 + r32, E - 1) * H + 8 * half;
+  floatx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  // loads run two iterations ahead of the arithmetic (three rolling register sets)
+  const int nit = (H - 16 * wv + 63) / 64;
+  float4 xa[3], xb[3], ga[3], gb[3];
+  auto load = [&](int u, int i) {
+    const int k0 = 16 * wv + 64 * min(i, nit - 1);
+    xa[u] = *reinterpret_cast<const float4*>(xr + k0);
+    xb[u] = *reinterpret_cast<const float4*>(xr + k0 + 4);
+    ga[u] = *reinterpret_cast<const float4*>(gr + k0);
+    gb[u] = *reinterpret_cast<const float4*>(gr + k0 + 4);
+  };
+  if (nit > 0) {
+    load(0, 0);
+    load(1, 1);
+  }
+  for (int i = 0; i < nit; i += 3) {
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      if (i + u < nit) {
+        load((u + 2) % 3, i + u + 2);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].x, ga[u].x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].y, ga[u].y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].z, ga[u].z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].w, ga[u].w, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[u].x, gb[u].x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[u].y, gb[u].y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[u].z, gb[u].z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[u].w, gb[u].w, acc, 0, 0, 0);
+      }
+    }
+  }
+  // accumulator register r of lane (expert column r32, half) is token (r%4) + 8 (r/4) + 4 half
+#pragma unroll
+  for (int r = 0; r < 16; ++r) part[wv][(r & 3) + 8 * (r >> 2) + 4 * half][r32] = acc[r];
+  __syncthreads();
+  for (int i = threadIdx.x; i < 32 * 32; i += 256) {
+    const int tl = i >> 5, el = i & 31;
+    if (t0 + tl < T && e0 + el < E) {
+      const float s = (part[0][tl][el] + part[1][tl][el]) + (part[2][tl][el] + part[3][tl][el]);
+      logits[(size_t)(t0 + tl) * E + e0 + el] = s + (b ? b[e0 + el] : 0.0f);
+    }
+  }
+}
+
 // --------------------------------------------- small batches: prologue + logits
 // One launch for small T: workgroups x in [0, E) compute the logits of one expert for
 // the four tokens of tile y (the four waves split H, so all loads of a row are in flight at
