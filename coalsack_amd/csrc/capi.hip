@@ -306,9 +306,6 @@ int launch_router(const float* x, const float* gate_w, const float* gate_b, int6
 
 int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, int64_t E,
                     const ExpertW* ew, Workspace& ws) {
-  dispatch_count_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(ids, (int)P, ws.counts);
-  int rc = check_launch("dispatch_count_kernel");
-  if (rc != CSK_OK) return rc;
   dispatch_scatter_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(
       ids, pairs, (int)P, (int)k, (int)E, ws.counts, ew, ws.offsets, ws.desc,
       P <= kStreamMaxP ? ws.vlist : nullptr, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w,
@@ -389,7 +386,7 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
 int launch_combine(const float* y, const float* pairs, const int* pos, const float* residual,
                    float* out, int64_t T, int64_t k, int64_t H, int pre_weighted) {
   if (T == 0) return CSK_OK;
-  combine_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)T), 256, 0, g_stream>>>(
+  combine_kernel<<<dim3((unsigned)cdiv(H, 1024), (unsigned)T), 256, 0, g_stream>>>(
       y, pairs, pos, residual, out, (int)T, (int)k, (int)H, pre_weighted);
   return check_launch("combine_kernel");
 }

@@ -335,79 +335,109 @@ __global__ void pairs_to_ids_kernel(const float* __restrict__ pairs, int* __rest
 }
 
 // ----------------------------------------------------------------- dispatch
-// Step 1, histogram: workgroup e counts the assignments that name expert e.
-__global__ __launch_bounds__(256) void dispatch_count_kernel(const int* __restrict__ ids, int P,
-                                                             int* __restrict__ counts) {
-  const int e = blockIdx.x;
-  int c = 0;
-  for (int p = threadIdx.x; p < P; p += 256) c += (ids[p] == e);
-  c = (int)wave_sum((float)c);  // exact below 2^24
-  __shared__ int part[4];
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
-  __syncthreads();
-  if (threadIdx.x == 0) counts[e] = part[0] + part[1] + part[2] + part[3];
-}
-
-// Steps 2+3, exclusive scan and ordered scatter: workgroup e derives its
-// offset from the histogram, then walks the assignments in order and writes
-// the ones naming e at offset + rank, so each expert's list is ascending in
-// token index -- the order the reference's per-expert token loop visits them
-// (expert_mlp_node.h:503-529).  Workgroup 0 also publishes offsets[0..E] and
-// the compact list of experts with at least one token
-// (moe_weight_fetch_node.h:31-60).
+// Workgroup e builds the whole per-expert histogram in LDS (every workgroup does: the
+// ids are L2-resident and LDS atomics are cheap, which saves a launch and any global
+// atomics), derives its offset, then writes the assignments naming e at offset + rank in
+// ascending order, so each expert's list is ascending in token index -- the order the
+// reference's per-expert token loop visits them (expert_mlp_node.h:503-529).  Workgroup 0
+// also publishes counts, offsets[0..E] and the compact list of experts with at least one
+// token (moe_weight_fetch_node.h:31-60).
 __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
     const int* __restrict__ ids, const float* __restrict__ pairs, int P, int k, int E,
-    const int* __restrict__ counts, const ExpertW* __restrict__ ew, int* __restrict__ offsets,
+    int* __restrict__ counts, const ExpertW* __restrict__ ew, int* __restrict__ offsets,
     WorkDesc* __restrict__ desc, int* __restrict__ vlist, int* __restrict__ nv,
     int* __restrict__ mtiles, int* __restrict__ n_mtiles, int* __restrict__ list_tok,
     float* __restrict__ list_w, int* __restrict__ pos_of_slot) {
   const int e = blockIdx.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   __shared__ int sh[8];
-  __shared__ int cnt[kMaxExperts], act_e[kMaxExperts], act_off[kMaxExperts];
-  const int mine = (threadIdx.x < E) ? counts[threadIdx.x] : 0;  // E <= 256 = blockDim
-  int c = (threadIdx.x < e) ? mine : 0;
+  __shared__ int cnt[kMaxExperts], off_sh[kMaxExperts], act_e[kMaxExperts];
+  __shared__ int na_sh;
+  cnt[threadIdx.x] = 0;  // kMaxExperts == blockDim
+  __syncthreads();
+  // each wave scans its own quarter of the assignments: the histogram, and how many name e
+  const int per_wave = ((P + 255) / 256) * 64;
+  const int p_lo = wv * per_wave, p_hi = min(P, p_lo + per_wave);
+  int hits = 0;
+  for (int p0 = p_lo; p0 < p_hi; p0 += 64 * 8) {  // eight loads in flight per lane
+    int id[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int p = p0 + 64 * j + lane;
+      id[j] = p < p_hi ? ids[p] : -1;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (id[j] >= 0) atomicAdd(&cnt[id[j]], 1);
+      hits += __popcll(__ballot(id[j] == e));
+    }
+  }
+  if (lane == 0) sh[4 + wv] = hits;
+  __syncthreads();
+  const int mine = cnt[threadIdx.x];
+  int c = ((int)threadIdx.x < e) ? mine : 0;
   c = (int)wave_sum((float)c);
   if (lane == 0) sh[wv] = c;
-  if (e == 0) cnt[threadIdx.x] = mine;
+  if (e == 0 && (int)threadIdx.x < E) counts[threadIdx.x] = mine;
   __syncthreads();
-  const int off = sh[0] + sh[1] + sh[2] + sh[3];
   if (e == 0) {
-    // workgroup 0 publishes the scan and the work descriptors of the active experts
-    __shared__ int na_sh;
-    if (threadIdx.x == 0) {
-      int run = 0, na = 0;
-      for (int i = 0; i < E; ++i) {
-        offsets[i] = run;
-        if (cnt[i] > 0) {
-          act_e[na] = i;
-          act_off[na] = run;
-          ++na;
-        }
-        run += cnt[i];
+    // workgroup 0 publishes the scan, the active experts, the streaming kernel's token
+    // groups and the GEMM's M tiles: wave 0, four consecutive experts per lane,
+    // wave-wide prefix sums
+    if (wv == 0) {
+      int cc[4], tot = 0, nact = 0, ngrp = 0, nmt = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int ee = lane * 4 + j;
+        cc[j] = ee < E ? cnt[ee] : 0;
+        tot += cc[j];
+        nact += cc[j] > 0;
+        ngrp += (cc[j] + kStreamG - 1) / kStreamG;
+        nmt += (cc[j] + 63) / 64;
       }
-      offsets[E] = run;
-      na_sh = na;
-      // token groups of the weight-streaming kernel: (expert slot, first token)
-      int nvv = 0;
-      if (vlist) {
-        for (int u = 0; u < na; ++u)
-          for (int gb = 0; gb < cnt[act_e[u]]; gb += kStreamG) {
-            vlist[2 * nvv] = u;
-            vlist[2 * nvv + 1] = gb;
-            ++nvv;
+      int s_tot = tot, s_act = nact, s_grp = ngrp, s_mt = nmt;  // inclusive scans over lanes
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int t0 = __shfl_up(s_tot, o, 64), t1 = __shfl_up(s_act, o, 64);
+        const int t2 = __shfl_up(s_grp, o, 64), t3 = __shfl_up(s_mt, o, 64);
+        if (lane >= o) {
+          s_tot += t0;
+          s_act += t1;
+          s_grp += t2;
+          s_mt += t3;
+        }
+      }
+      int run = s_tot - tot, slot = s_act - nact, gi = s_grp - ngrp, mi = s_mt - nmt;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int ee = lane * 4 + j;
+        if (ee < E) {
+          off_sh[ee] = run;
+          offsets[ee] = run;
+          if (cc[j] > 0) {
+            if (vlist) {
+              for (int gb = 0; gb < cc[j]; gb += kStreamG) {
+                vlist[2 * gi] = slot;
+                vlist[2 * gi + 1] = gb;
+                ++gi;
+              }
+            }
+            for (int m0 = 0; m0 < cc[j]; m0 += 64) {
+              mtiles[2 * mi] = slot;
+              mtiles[2 * mi + 1] = m0;
+              ++mi;
+            }
+            act_e[slot++] = ee;
           }
-      }
-      *nv = nvv;
-      // M tiles of the grouped GEMM: (expert slot, first token), 64 tokens each
-      int nm = 0;
-      for (int u = 0; u < na; ++u)
-        for (int m0 = 0; m0 < cnt[act_e[u]]; m0 += 64) {
-          mtiles[2 * nm] = u;
-          mtiles[2 * nm + 1] = m0;
-          ++nm;
+          run += cc[j];
         }
-      *n_mtiles = nm;
+      }
+      if (lane == 63) {
+        offsets[E] = s_tot;
+        na_sh = s_act;
+        *nv = vlist ? s_grp : 0;
+        *n_mtiles = s_mt;
+      }
     }
     __syncthreads();
     if (threadIdx.x < E) {
@@ -415,7 +445,7 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
       if ((int)threadIdx.x < na_sh) {
         d.e = act_e[threadIdx.x];
         d.Te = cnt[d.e];
-        d.base = act_off[threadIdx.x];
+        d.base = off_sh[d.e];
         d.pad = 0;
         d.w = ew[d.e];
       } else {
@@ -425,30 +455,35 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
       desc[threadIdx.x] = d;
     }
   }
-  int base = off;
-  for (int p0 = 0; p0 < P; p0 += 256) {
-    const int p = p0 + threadIdx.x;
-    const bool hit = (p < P) && (ids[p] == e);
-    const unsigned long long m = __ballot(hit);
-    const int below = __popcll(m & ((1ull << lane) - 1ull));
-    __syncthreads();
-    if (lane == 0) sh[4 + wv] = __popcll(m);
-    __syncthreads();
-    int woff = 0;
-    for (int i = 0; i < wv; ++i) woff += sh[4 + i];
-    if (hit) {
-      const int pos = base + woff + below;
-      list_tok[pos] = p / k;
-      list_w[pos] = pairs[2 * (size_t)p + 1];
-      pos_of_slot[p] = pos;
+  // ... then writes them, in order, behind those of the waves before it
+  int base = sh[0] + sh[1] + sh[2] + sh[3];
+  for (int i = 0; i < wv; ++i) base += sh[4 + i];
+  for (int p0 = p_lo; p0 < p_hi; p0 += 64 * 8) {
+    int id[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int p = p0 + 64 * j + lane;
+      id[j] = p < p_hi ? ids[p] : -1;
     }
-    base += sh[4] + sh[5] + sh[6] + sh[7];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int p = p0 + 64 * j + lane;
+      const bool hit = id[j] == e;
+      const unsigned long long m = __ballot(hit);
+      if (hit) {
+        const int pos = base + __popcll(m & ((1ull << lane) - 1ull));
+        list_tok[pos] = p / k;
+        list_w[pos] = pairs[2 * (size_t)p + 1];
+        pos_of_slot[p] = pos;
+      }
+      base += __popcll(m);
+    }
   }
 }
 
 // ------------------------------------- small batches: top-k + dispatch, fused
 // One workgroup of 16 waves does, for P = T * k <= 1024 assignments, what
-// router_topk_kernel, dispatch_count_kernel and dispatch_scatter_kernel do in
+// router_topk_kernel and dispatch_scatter_kernel do in
 // three launches: top-k and weights per token (one wave per token), histogram,
 // exclusive scan, ordered scatter, work descriptors and token groups -- all
 // through LDS.
@@ -639,23 +674,26 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
                                                       int pre_weighted) {
 #pragma clang fp contract(off)  // w * y and the add round separately, as in the reference
   const int t = blockIdx.y;
-  const int d = blockIdx.x * 256 + threadIdx.x;
+  const int d = (blockIdx.x * 256 + threadIdx.x) * 4;  // four adjacent columns per thread (H % 32 == 0)
   if (d >= H) return;
-  float acc = 0.0f;
+  float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
   for (int s = 0; s < k; ++s) {
     const int pos = pos_of_slot[(size_t)t * k + s];
     if (pos < 0) continue;  // empty expert tensor: skipped (expert_merge_node.h:111-113)
-    const float v = y[(size_t)pos * H + d];
+    const float4 v = *reinterpret_cast<const float4*>(y + (size_t)pos * H + d);
     if (pre_weighted) {
-      acc = acc + v;
+      acc.x = acc.x + v.x, acc.y = acc.y + v.y, acc.z = acc.z + v.z, acc.w = acc.w + v.w;
     } else {
       const float w = pairs[2 * ((size_t)t * k + s) + 1];
-      const float wv = w * v;
-      acc = acc + wv;
+      const float4 wv = make_float4(w * v.x, w * v.y, w * v.z, w * v.w);
+      acc.x = acc.x + wv.x, acc.y = acc.y + wv.y, acc.z = acc.z + wv.z, acc.w = acc.w + wv.w;
     }
   }
-  if (residual) acc = residual[(size_t)t * H + d] + acc;
-  out[(size_t)t * H + d] = acc;
+  if (residual) {
+    const float4 r = *reinterpret_cast<const float4*>(residual + (size_t)t * H + d);
+    acc.x = r.x + acc.x, acc.y = r.y + acc.y, acc.z = r.z + acc.z, acc.w = r.w + acc.w;
+  }
+  *reinterpret_cast<float4*>(out + (size_t)t * H + d) = acc;
 }
 
 // Dense per-expert output of the node-level call (expert_mlp_node.h:503-529):
