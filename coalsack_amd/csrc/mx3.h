@@ -25,7 +25,14 @@ namespace csk {
 constexpr int kMx3Terms = 3;
 constexpr int kMx3ChunksPerBlock = 2 * kMx3Terms;  // 16-byte chunks per 32-value block
 
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x32 __attribute__((ext_vector_type(32)));
+typedef uint32_t u32x6 __attribute__((ext_vector_type(6)));
+
 // Quantises one block held in registers; out[2t], out[2t+1] are the chunks of term t.
+// v_cvt_scalef32_2xpk16_fp6_f32 divides by the scale, rounds to nearest even, saturates
+// at +-7.5 and packs value i of its first operand at position 2i, of its second at
+// 2i+1; v_cvt_scalef32_pk32_f32_fp6 is its inverse in position order (both probed).
 __device__ __forceinline__ void mx3_quantize_block(float (&r)[32], u32x4 (&out)[kMx3ChunksPerBlock]) {
 #pragma unroll
   for (int t = 0; t < kMx3Terms; ++t) {
@@ -35,29 +42,21 @@ __device__ __forceinline__ void mx3_quantize_block(float (&r)[32], u32x4 (&out)[
     const uint32_t eb = (__float_as_uint(m) >> 23) & 0xffu;
     // block maximum / scale in [4, 8); blocks below 2^-124 are stored as zeros
     const uint32_t s = eb < 3u ? 127u : min(eb - 2u, 252u);
-    const float inv = __uint_as_float((254u - s) << 23);  // 2^(127-s)
-    const float sc = __uint_as_float(s << 23);            // 2^(s-127)
-    uint32_t w[6] = {0u, 0u, 0u, 0u, 0u, 0u};
+    const float sc = __uint_as_float(s << 23);  // 2^(s-127)
+    f32x16 ev, od;
 #pragma unroll
-    for (int j = 0; j < 32; ++j) {
-      const float v = r[j] * inv;
-      const float a = fabsf(v);
-      // codes are monotone in |value|: 0..7 -> k/8, 8..15 -> 1+k/8, 16..23 -> 2+k/4, 24..31 -> 4+k/2
-      const float q8 = rintf(a * 8.0f);  // a < 1: multiple of 1/8 (8 -> code 8 = 1.0)
-      const uint32_t bits = __float_as_uint(a);
-      uint32_t u = (bits + 0x7FFFFu + ((bits >> 20) & 1u)) >> 20;  // a >= 1: keep 3 mantissa bits, RNE
-      u = min(u, 1008u + 31u);
-      const bool small = a < 1.0f;
-      const uint32_t code = small ? (uint32_t)q8 : u - 1008u;
-      const float val = small ? q8 * 0.125f : __uint_as_float(u << 20);
-      r[j] = r[j] - copysignf(val, v) * sc;  // exact: val * sc is a power-of-two scaling
-      const uint32_t c6 = code | ((__float_as_uint(v) >> 31) << 5);
-      const int bit = 6 * j;
-      w[bit >> 5] |= c6 << (bit & 31);
-      if ((bit & 31) > 26) w[(bit >> 5) + 1] |= c6 >> (32 - (bit & 31));
+    for (int j = 0; j < 16; ++j) {
+      ev[j] = r[2 * j];
+      od[j] = r[2 * j + 1];
     }
-    out[2 * t] = u32x4{w[0], w[1], w[2], w[3]};
-    out[2 * t + 1] = u32x4{w[4], w[5], s, 0u};
+    const u32x6 q = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(ev, od, sc);
+    if (t + 1 < kMx3Terms) {
+      const f32x32 d = __builtin_amdgcn_cvt_scalef32_pk32_f32_fp6(q, sc);
+#pragma unroll
+      for (int j = 0; j < 32; ++j) r[j] = r[j] - d[j];  // exact: d is r rounded to 4 bits
+    }
+    out[2 * t] = u32x4{q[0], q[1], q[2], q[3]};
+    out[2 * t + 1] = u32x4{q[4], q[5], s, 0u};
   }
 }
 
