@@ -252,7 +252,7 @@ def main():
     if prefill:
         st = res["stage_ms"]
         fl = T * shape["k"] * 4 * shape["H"] * shape["F"]  # gate + up flops
-        roof = dict(bound="mfma", kernel="gate/up grouped GEMM", achieved=fl / (st["gateup"] * 1e-3) / 1e12,
+        roof = dict(bound="mfma", kernel="expert_gemm_mx_kernel<0> (gate/up + SwiGLU)", achieved=fl / (st["gateup"] * 1e-3) / 1e12,
                     peak=MFMA_FP4_PEAK_TFLOPS, unit="TFLOP/s", traffic=None)
     else:
         roof = dict(bound="hbm", kernel="expert_stream_kernel<2,*> (gate/up + SwiGLU)",
@@ -285,7 +285,9 @@ def main():
     line = dict(
         metric="MoE layer tokens/s", value=res["tokens_per_s"], unit="tokens/s", n_gpus=1, steps=a.steps,
         warmup=a.warmup, ms_per_step=res["ms_per_step"], higher_is_better=True, scaling="weak",
-        vs_baseline=None, dtype="mxfp4 x bf16(2-term) -> f32", data="synthetic",
+        vs_baseline=None,
+        dtype=("mxfp4 x fp6(3-term, block-scaled) -> f32" if prefill else "mxfp4 x bf16(2-term) -> f32"),
+        data="synthetic",
         config=dict(workload=f"{a.workload}: E={shape['E']} top-{shape['k']} H={shape['H']} F={shape['F']} "
                              f"MXFP4, T={T}" + (", 8 hot experts" if shape["hot"] else ""),
                     tokens=T, distinct_experts=res["distinct_experts"], device=dev_name, compute_units=cus),
