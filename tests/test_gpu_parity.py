@@ -73,7 +73,8 @@ def test_router_known_answer(lib):
 
 @pytest.mark.parametrize("T,H,E,k,bias,sigmoid", [
     (2, 4, 8, 2, True, False), (8, 128, 32, 4, True, False), (33, 2880, 128, 4, True, False),
-    (5, 96, 7, 3, False, False), (64, 2880, 32, 4, True, True), (700, 256, 200, 8, True, False)])
+    (5, 96, 7, 3, False, False), (64, 2880, 32, 4, True, True), (700, 256, 200, 8, True, False),
+    (100, 96, 40, 3, True, False), (65, 32, 5, 1, False, True), (257, 2880, 128, 4, True, False)])
 def test_router_matches_oracle(lib, oracle, T, H, E, k, bias, sigmoid):
     rng = np.random.default_rng(T * 1000 + E)
     h = rng.normal(0, 1, (T, H)).astype(np.float32)
@@ -134,9 +135,10 @@ def test_expert_token_matches_oracle(lib, oracle, H, F, bias, act):
     assert np.max(np.abs(got - want)) <= 1e-4 * max(1.0, np.abs(want).max())
 
 
-@pytest.mark.parametrize("wbf", [False, True])
-def test_expert_node_rows_and_empty(lib, oracle, wbf):
-    H, F, T, k = 64, 96, 37, 2
+@pytest.mark.parametrize("wbf,T", [(False, 37), (True, 37), (False, 150), (True, 150)])
+def test_expert_node_rows_and_empty(lib, oracle, wbf, T):
+    """T = 37 runs the streaming kernels, T = 150 the grouped GEMM."""
+    H, F, k = 64, 96, 2
     rng = np.random.default_rng(1)
     w = [synth.mxfp4_blocks(3, 0, 4, i, F if i < 2 else H, H if i < 2 else F) for i in range(3)]
     hs = [lib.mxfp4_upload(w[0], F, H), lib.mxfp4_upload(w[1], F, H), lib.mxfp4_upload(w[2], H, F)]
@@ -262,6 +264,28 @@ def test_layer_variants(lib, oracle, opts):
     residual = opts.pop("residual", False)
     L = synth.LayerInputs(8, 2, 128, 160, seed=9, with_norm=True)
     _check_layer(lib, oracle, L, 21, bias=bias, norm=norm, residual=residual, **opts)
+
+
+@pytest.mark.parametrize("opts", [dict(act=1), dict(sigmoid=True), dict(weight_before_ffn=True),
+                                  dict(bias=False), dict(norm=True, residual=True),
+                                  dict(weight_before_ffn=True, norm=True, residual=True)])
+def test_layer_variants_grouped_gemm(lib, oracle, opts):
+    """The same variants at a batch that takes the grouped-GEMM path (T > 64), on a shape
+    whose expert count, feature count and K are not multiples of the tile sizes."""
+    opts = dict(opts)
+    bias = opts.pop("bias", True)
+    norm = opts.pop("norm", False)
+    residual = opts.pop("residual", False)
+    L = synth.LayerInputs(7, 3, 160, 224, seed=19, with_norm=True)
+    _check_layer(lib, oracle, L, 131, bias=bias, norm=norm, residual=residual, **opts)
+
+
+def test_layer_few_tokens_long_rows(lib, oracle):
+    """Rows longer than the streaming kernel's LDS budget: few tokens still take the GEMM."""
+    L = synth.LayerInputs(4, 2, 3200, 64, seed=23, with_norm=True)
+    _check_layer(lib, oracle, L, 6, norm=True, residual=True)
+    L = synth.LayerInputs(4, 2, 64, 3200, seed=24)
+    _check_layer(lib, oracle, L, 5)
 
 
 def test_layer_many_tokens_per_expert(lib, oracle):
