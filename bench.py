@@ -37,6 +37,8 @@ SHAPES = {
     "c3_20b_prefill": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=2048, sweep=[]),
     "c4_120b": dict(E=128, k=4, H=2880, F=2880, hot=8, default_T=16, sweep=[1, 16]),
     "c5_stack": dict(E=128, k=4, H=2880, F=2880, hot=8, default_T=8, sweep=[1, 8, 64], layers=36),
+    # next-row workload: one 20b-shaped block read from a GGUF file into a resident layer
+    "gguf_ingest": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=4, sweep=[]),
 }
 
 
@@ -70,6 +72,33 @@ def make_layer(lib, synth, shape, seed, layer_index=0, norm=False):
     if norm:
         layer.set_norm(L.norm_w, 1e-5)
     return L, layer
+
+
+def bench_gguf_ingest(lib, synth, shape, reps=3):
+    """Writes a synthetic one-block GGUF file (MXFP4 experts, biases, router, norm) and
+    times csk_layer_from_gguf: file -> host -> HBM -> repacked resident planes."""
+    import tempfile
+    from coalsack_amd import gguf_writer as gw
+    L = synth.LayerInputs(shape["E"], shape["k"], shape["H"], shape["F"], seed=7, with_norm=True)
+    meta = [("general.architecture", gw.STR, "gpt-oss"), ("gpt-oss.expert_count", gw.U32, L.E),
+            ("gpt-oss.expert_used_count", gw.U32, L.k)]
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "block.gguf")
+        gw.write_gguf(path, meta, gw.moe_block_tensors(L, 0))
+        nbytes = os.path.getsize(path)
+        times = []
+        with lib.gguf(path) as g:
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                layer = g.layer(0)
+                lib.synchronize()
+                times.append(time.perf_counter() - t0)
+                hidden = synth.hidden_states(4, L.H, seed=1)
+                out = layer.forward(hidden)
+                ok = bool(np.array_equal(layer.export(L.E - 1, 2), L.blocks(L.E - 1, 2)))
+                layer.close()
+    return dict(file_bytes=nbytes, seconds=min(times), all_seconds=times, roundtrip_ok=ok,
+                finite=bool(np.all(np.isfinite(out))))
 
 
 def time_forward(lib, fn, steps, warmup):
@@ -220,6 +249,18 @@ def main():
     dev_name, cus, mem = lib.device_info()
     shape = SHAPES[a.workload]
     T = a.tokens or shape["default_T"]
+
+    if a.workload == "gguf_ingest":
+        res = bench_gguf_ingest(lib, synth, shape)
+        line = dict(metric="GGUF MoE block ingest GB/s", value=res["file_bytes"] / res["seconds"] / 1e9,
+                    unit="GB/s", n_gpus=1, steps=len(res["all_seconds"]), warmup=0,
+                    ms_per_step=res["seconds"] * 1e3, higher_is_better=True, scaling="weak",
+                    vs_baseline=None, dtype="u8", data="synthetic",
+                    config=dict(workload="gguf_ingest: one 20b-shaped block (32 experts, MXFP4 + biases + router + norm) "
+                                         "file -> resident layer", file_bytes=res["file_bytes"], device=dev_name),
+                    roofline=None, cpu_baseline=None, roundtrip_ok=res["roundtrip_ok"], finite=res["finite"])
+        print(json.dumps(line))
+        return
 
     if a.workload == "c5_stack":
         res = bench_stack(lib, synth, shape, T, a.steps, a.warmup, shape["layers"])

@@ -49,6 +49,16 @@ SIGNATURES = {
     "csk_layer_fill_synthetic": (C.c_int, [_P, C.c_uint64, _I64, C.c_int, C.c_int]),
     "csk_layer_dequant": (C.c_int, [_P, _I64, C.c_int, _P]),
     "csk_layer_export": (C.c_int, [_P, _I64, C.c_int, _P]),
+    "csk_gguf_open": (C.c_int, [C.c_char_p, C.POINTER(_P)]),
+    "csk_gguf_close": (None, [_P]),
+    "csk_gguf_tensor_count": (C.c_int, [_P, C.POINTER(_I64)]),
+    "csk_gguf_tensor_name": (C.c_int, [_P, _I64, C.c_char_p, C.c_size_t]),
+    "csk_gguf_tensor_info": (C.c_int, [_P, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(C.c_int32),
+                                        C.POINTER(C.c_uint64), C.POINTER(C.c_uint64),
+                                        C.POINTER(C.c_uint64)]),
+    "csk_gguf_get_u32": (C.c_int, [_P, C.c_char_p, C.POINTER(C.c_uint32)]),
+    "csk_gguf_get_str": (C.c_int, [_P, C.c_char_p, C.c_char_p, C.c_size_t]),
+    "csk_layer_from_gguf": (C.c_int, [_P, _I64, C.POINTER(_P)]),
     "csk_moe_forward": (C.c_int, [_P, _P, _I64, _P, C.c_int]),
     "csk_moe_forward_host": (C.c_int, [_P, _P, _I64, _P, _P, C.c_int]),
     "csk_moe_stack_forward": (C.c_int, [C.POINTER(_P), _I64, _P, _I64]),
@@ -254,6 +264,66 @@ class Library:
     def layer(self, E, k, H, F):
         return Layer(self, E, k, H, F)
 
+    def gguf(self, path):
+        return Gguf(self, path)
+
+
+class Gguf:
+    """An open GGUF file (csk_gguf_*): metadata and tensor table, no GPU needed."""
+
+    def __init__(self, lib, path):
+        self.lib = lib
+        self.h = _P()
+        lib.check(lib.dll.csk_gguf_open(os.fsencode(path), C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            self.lib.dll.csk_gguf_close(self.h)
+            self.h = _P()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    def tensor_names(self):
+        n = _I64()
+        self.lib.check(self.lib.dll.csk_gguf_tensor_count(self.h, C.byref(n)))
+        buf = C.create_string_buffer(512)
+        out = []
+        for i in range(n.value):
+            self.lib.check(self.lib.dll.csk_gguf_tensor_name(self.h, i, buf, 512))
+            out.append(buf.value.decode())
+        return out
+
+    def tensor_info(self, name):
+        t, nd, off, nb = C.c_uint32(), C.c_int32(), C.c_uint64(), C.c_uint64()
+        dims = (C.c_uint64 * 4)()
+        self.lib.check(self.lib.dll.csk_gguf_tensor_info(self.h, name.encode(), C.byref(t), C.byref(nd),
+                                                         dims, C.byref(off), C.byref(nb)))
+        return dict(type=t.value, dims=list(dims)[:nd.value], offset=off.value, nbytes=nb.value)
+
+    def get_u32(self, key):
+        v = C.c_uint32()
+        self.lib.check(self.lib.dll.csk_gguf_get_u32(self.h, key.encode(), C.byref(v)))
+        return v.value
+
+    def get_str(self, key):
+        buf = C.create_string_buffer(1024)
+        self.lib.check(self.lib.dll.csk_gguf_get_str(self.h, key.encode(), buf, 1024))
+        return buf.value.decode()
+
+    def layer(self, block):
+        """Resident MoE layer of transformer block `block` (csk_layer_from_gguf)."""
+        h = _P()
+        self.lib.check(self.lib.dll.csk_layer_from_gguf(self.h, block, C.byref(h)))
+        arch = self.get_str("general.architecture")
+        gi = self.tensor_info(f"blk.{block}.ffn_gate_inp.weight")
+        up = self.tensor_info(f"blk.{block}.ffn_up_exps.weight")
+        return Layer.adopt(self.lib, h, gi["dims"][1], self.get_u32(arch + ".expert_used_count"),
+                           gi["dims"][0], up["dims"][1])
+
 
 class Layer:
     """One resident MoE layer (csk_layer_*)."""
@@ -262,6 +332,13 @@ class Layer:
         self.lib, self.E, self.k, self.H, self.F = lib, E, k, H, F
         self.h = _P()
         lib.check(lib.dll.csk_layer_create(E, k, H, F, C.byref(self.h)))
+
+    @classmethod
+    def adopt(cls, lib, handle, E, k, H, F):
+        """Wraps a layer handle the library created itself."""
+        self = cls.__new__(cls)
+        self.lib, self.E, self.k, self.H, self.F, self.h = lib, E, k, H, F, handle
+        return self
 
     def close(self):
         if self.h:

@@ -424,6 +424,8 @@ extern "C" int csk_init(int device) {
 }
 
 extern "C" const char* csk_last_error(void) { return g_err.c_str(); }
+// for the library's other translation units (not part of the public header)
+extern "C" void csk_set_error_(const char* msg) { g_err = msg ? msg : ""; }
 
 extern "C" int csk_device_info(char* name, size_t cap, int* compute_units, size_t* hbm_bytes) {
   REQUIRE_INIT();

@@ -133,6 +133,33 @@ int csk_layer_fill_synthetic(csk_layer* L, uint64_t seed, int64_t layer_index, i
 int csk_layer_dequant(const csk_layer* L, int64_t e, int which, float* host_out);
 int csk_layer_export(const csk_layer* L, int64_t e, int which, uint8_t* blocks17_host);
 
+/* ---------------------------------------------------------------- GGUF ingest
+ * Reads a GGUF file's key/value section and tensor table (no tensor data) --
+ * gguf_loader::load, src/gguf/gguf_loader.cpp:383-518.  Needs no GPU and no
+ * csk_init.  One file; split (sharded) checkpoints are opened shard by shard. */
+typedef struct csk_gguf csk_gguf;
+int csk_gguf_open(const char* path, csk_gguf** out);
+void csk_gguf_close(csk_gguf* g);
+int csk_gguf_tensor_count(const csk_gguf* g, int64_t* n);
+int csk_gguf_tensor_name(const csk_gguf* g, int64_t index, char* buf, size_t cap);
+/* gguf_loader::get_tensor_info: dims in file order (fastest-varying first, padded
+ * with 1), absolute file offset of the data, size in bytes (0: unknown type). */
+int csk_gguf_tensor_info(const csk_gguf* g, const char* name, uint32_t* ggml_type, int32_t* n_dims,
+                         uint64_t* dims4, uint64_t* file_offset, uint64_t* nbytes);
+/* gguf_loader::get_uint32 / get_string (any integer width is accepted) */
+int csk_gguf_get_u32(const csk_gguf* g, const char* key, uint32_t* value);
+int csk_gguf_get_str(const csk_gguf* g, const char* key, char* buf, size_t cap);
+/* Resident MoE layer of transformer block `block`, built from
+ *   blk.N.ffn_gate_inp.{weight,bias}, blk.N.ffn_{up,gate,down}_exps.{weight,bias},
+ *   blk.N.post_attention_norm.weight (llama4: ffn_norm.weight)
+ * with <arch>.expert_count / expert_used_count and the architecture switches of
+ * llm_engine::load_config_from_gguf (src/llm/llm_engine.cpp:135-225).  Expert e
+ * of a stacked tensor is the slice at offset + e * rows * (K/32) * 17 --
+ * moe_weight_provider::get, src/llm/moe_weight_provider.cpp:160-188; it takes
+ * the place of that provider and its LRU cache: all experts stay in HBM.
+ * MXFP4 expert tensors only. */
+int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out);
+
 /* Router -> dispatch -> expert MLPs -> merge for T tokens, everything on the
  * GPU: hidden and out are device pointers [T,H] f32 (out may not alias
  * hidden).  Stands in for the node chain llm_engine wires per layer

@@ -1,0 +1,122 @@
+"""GGUF ingest: header / metadata / tensor-table parsing (CPU) and resident layers
+built from a file (GPU).  Files are written by coalsack_amd/gguf_writer.py."""
+import numpy as np
+import pytest
+
+from coalsack_amd import capi, synth
+from coalsack_amd import gguf_writer as gw
+from tests.helpers import build_layer, nbits_differ, oracle_layer, assert_layer_close
+
+
+def _meta(arch="gpt-oss", E=6, k=2, alignment=None):
+    m = [("general.architecture", gw.STR, arch),
+         ("general.name", gw.STR, "synthetic"),
+         (arch + ".expert_count", gw.U32, E),
+         (arch + ".expert_used_count", gw.U32, k),
+         (arch + ".block_count", gw.U64, 2),
+         ("some.i8", gw.I8, -3), ("some.f64", gw.F64, 2.5), ("some.bool", gw.BOOL, 1),
+         ("tokenizer.ggml.tokens", gw.ARR, (gw.STR, ["a", "bc", "", "def"])),
+         ("tokenizer.ggml.scores", gw.ARR, (gw.F32, [0.5, -1.0, 2.0])),
+         ("tokenizer.ggml.token_type", gw.ARR, (gw.I32, [1, 2, 3, 4, 5])),
+         ("odd.u16s", gw.ARR, (gw.U16, [7, 8, 9]))]
+    if alignment:
+        m.append(("general.alignment", gw.U32, alignment))
+    return m
+
+
+@pytest.mark.parametrize("alignment", [None, 64])
+def test_parse_header_metadata_and_tensor_table(tmp_path, alignment):
+    lib = capi.Library()  # no csk_init: parsing needs no GPU
+    L = synth.LayerInputs(6, 2, 64, 96, seed=5, with_norm=True)
+    tensors = [("token_embd.weight", gw.GGML_F16, [64, 10], np.zeros(640, np.float16).tobytes())]
+    tensors += gw.moe_block_tensors(L, 0) + gw.moe_block_tensors(L, 1, bias=False)
+    path = str(tmp_path / "m.gguf")
+    data_start = gw.write_gguf(path, _meta(alignment=alignment), tensors, alignment or 32)
+    with lib.gguf(path) as g:
+        assert g.get_str("general.architecture") == "gpt-oss"
+        assert g.get_u32("gpt-oss.expert_count") == 6 and g.get_u32("gpt-oss.block_count") == 2
+        assert g.tensor_names() == [t[0] for t in tensors]
+        pos = 0
+        raw = open(path, "rb").read()
+        for name, gtype, dims, data in tensors:
+            info = g.tensor_info(name)
+            assert info["type"] == gtype and info["dims"] == dims
+            assert info["offset"] == data_start + pos and info["nbytes"] == len(data)
+            assert raw[info["offset"]:info["offset"] + len(data)] == bytes(data)
+            pos += (len(data) + (alignment or 32) - 1) // (alignment or 32) * (alignment or 32)
+        up = g.tensor_info("blk.0.ffn_up_exps.weight")
+        assert up["nbytes"] == 6 * 96 * (64 // 32) * 17  # experts x rows x blocks x 17 B
+        with pytest.raises(capi.CskError, match="Tensor not found"):
+            g.tensor_info("blk.9.ffn_up_exps.weight")
+        with pytest.raises(capi.CskError, match="Missing required parameter"):
+            g.get_u32("gpt-oss.nope")
+
+
+def test_rejects_bad_files(tmp_path):
+    lib = capi.Library()
+    p = tmp_path / "bad.gguf"
+    p.write_bytes(b"GGML" + b"\0" * 64)
+    with pytest.raises(capi.CskError, match="bad magic"):
+        lib.gguf(str(p))
+    L = synth.LayerInputs(2, 1, 32, 32, seed=1)
+    path = str(tmp_path / "t.gguf")
+    gw.write_gguf(path, _meta(E=2, k=1), gw.moe_block_tensors(L, 0, norm=False))
+    whole = open(path, "rb").read()
+    (tmp_path / "cut.gguf").write_bytes(whole[:len(whole) - 40])
+    with pytest.raises(capi.CskError, match="past the end"):
+        lib.gguf(str(tmp_path / "cut.gguf"))
+    (tmp_path / "cut2.gguf").write_bytes(whole[:50])
+    with pytest.raises(capi.CskError, match="truncated"):
+        lib.gguf(str(tmp_path / "cut2.gguf"))
+    with pytest.raises(capi.CskError, match="cannot open"):
+        lib.gguf(str(tmp_path / "missing.gguf"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T", [5, 90])
+def test_layer_from_gguf_equals_layer_built_by_hand(lib, oracle, tmp_path, T):
+    """Same bytes through the file and through csk_layer_set_*: identical resident
+    weights and bit-identical outputs; and the file-built layer matches the CPU path."""
+    E, k, H, F = 6, 2, 96, 160
+    L0 = synth.LayerInputs(E, k, H, F, seed=11, with_norm=True)
+    L1 = synth.LayerInputs(E, k, H, F, seed=12, layer=1, with_norm=True)
+    path = str(tmp_path / "two_blocks.gguf")
+    gw.write_gguf(path, _meta(E=E, k=k), gw.moe_block_tensors(L0, 0) + gw.moe_block_tensors(L1, 1, bias=False))
+    hidden = synth.hidden_states(T, H, seed=3)
+    flags = capi.FWD_RMSNORM | capi.FWD_RESIDUAL
+    with lib.gguf(path) as g:
+        for blk, L, bias in ((0, L0, True), (1, L1, False)):
+            with g.layer(blk) as layer, build_layer(lib, L, bias=bias, norm=True) as hand:
+                assert (layer.E, layer.k, layer.H, layer.F) == (E, k, H, F)
+                for e in (0, E - 1):
+                    for which in range(3):
+                        assert np.array_equal(layer.export(e, which), L.blocks(e, which))
+                got = layer.forward(hidden, flags)
+                assert nbits_differ(got, hand.forward(hidden, flags)) == 0
+                want, _ = oracle_layer(oracle, L, hidden, bias=bias, norm=True, residual=True)
+                assert_layer_close(got, want)
+
+
+@pytest.mark.gpu
+def test_layer_from_gguf_llama4_switches_and_errors(lib, oracle, tmp_path):
+    E, k, H, F = 4, 1, 64, 64
+    L = synth.LayerInputs(E, k, H, F, seed=21, with_norm=True)
+    path = str(tmp_path / "l4.gguf")
+    gw.write_gguf(path, _meta("llama4", E, k),
+                  gw.moe_block_tensors(L, 0, bias=False, router_bias=False, norm_name="ffn_norm.weight"))
+    hidden = synth.hidden_states(7, H, seed=4)
+    with lib.gguf(path) as g, g.layer(0) as layer:
+        got = layer.forward(hidden, capi.FWD_RMSNORM)
+    L.gate_b = np.zeros(E, np.float32)
+    want, _ = oracle_layer(oracle, L, hidden, bias=False, norm=True, sigmoid=True, weight_before_ffn=True)
+    assert_layer_close(got, want)
+    # an F16 expert tensor is refused, not misread
+    bad = [(n, (gw.GGML_F16 if n.endswith("ffn_up_exps.weight") else t), d, b)
+           for n, t, d, b in gw.moe_block_tensors(L, 0, bias=False, router_bias=False)]
+    bad[1] = (bad[1][0], gw.GGML_F16, bad[1][2], np.zeros(E * F * H, np.float16).tobytes())
+    gw.write_gguf(str(tmp_path / "f16.gguf"), _meta(E=E, k=k), bad)
+    with lib.gguf(str(tmp_path / "f16.gguf")) as g:
+        with pytest.raises(capi.CskError, match="only MXFP4"):
+            g.layer(0)
+        with pytest.raises(capi.CskError, match="Tensor not found"):
+            g.layer(3)
