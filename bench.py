@@ -128,23 +128,49 @@ def stage_profile(lib, fn, steps):
     return {kk: v / steps for kk, v in acc.items()}
 
 
+def close_calls(L, hidden, k):
+    """Tokens whose k+1 largest router logits contain two closer than the library's
+    close-call threshold (8 * 2^-24 * sqrt(H), relative to max(1, |logit|)): those are
+    recomputed in the reference's summation order, which costs tens of microseconds."""
+    lg = hidden.astype(np.float64) @ L.gate_w.astype(np.float64).T + L.gate_b
+    srt = -np.sort(-lg, axis=1)[:, :k + 1]
+    gaps = (srt[:, :-1] - srt[:, 1:]) / np.maximum(1.0, np.abs(srt[:, :-1]))
+    return int(np.count_nonzero(gaps.min(axis=1) <= 8 * 5.96e-8 * np.sqrt(hidden.shape[1])))
+
+
 def bench_layer(lib, synth, shape, T, steps, warmup, seed=1234):
+    """Times the forward over `nb` different token batches in rotation (decode sizes: the
+    set of selected experts, and with it the bytes streamed, varies from batch to batch)."""
     L, layer = make_layer(lib, synth, shape, seed)
-    hidden = synth.hidden_states(T, L.H, seed=T)
-    d_in = lib.to_device(hidden)
-    d_out = lib.dev_alloc(hidden.nbytes)
-    fn = lambda: layer.forward_device(d_in, T, d_out)  # noqa: E731
-    ms = time_forward(lib, fn, steps, warmup)
-    stages = stage_profile(lib, fn, max(5, min(steps, 50)))
-    counts, _ = layer.last_dispatch(T)
-    U = int(np.count_nonzero(counts))
+    nb = 8 if T < 512 else 1
+    hiddens = [synth.hidden_states(T, L.H, seed=T + 1000 * i) for i in range(nb)]
+    d_ins = [lib.to_device(h) for h in hiddens]
+    d_out = lib.dev_alloc(hiddens[0].nbytes)
+    turn = [0]
+
+    def fn():
+        layer.forward_device(d_ins[turn[0] % nb], T, d_out)
+        turn[0] += 1
+    steps = (steps + nb - 1) // nb * nb
+    ms = time_forward(lib, fn, steps, (warmup + nb - 1) // nb * nb)
+    stages = stage_profile(lib, fn, (max(5, min(steps, 50)) + nb - 1) // nb * nb)
+    Us, tmax = [], 0
+    for i in range(nb - 1, -1, -1):  # batch 0 last: its output is the one checked
+        layer.forward_device(d_ins[i], T, d_out)
+        counts, _ = layer.last_dispatch(T)
+        Us.append(int(np.count_nonzero(counts)))
+        tmax = max(tmax, int(counts.max()))
+    U = float(np.mean(Us))
+    hidden = hiddens[0]
     out = lib.to_host(d_out, (T, L.H))
-    lib.dev_free(d_in)
+    for d in d_ins:
+        lib.dev_free(d)
     lib.dev_free(d_out)
     layer.close()
     res = dict(T=T, ms_per_step=ms, tokens_per_s=T / (ms * 1e-3), distinct_experts=U,
                stage_ms=stages, finite=bool(np.all(np.isfinite(out))),
-               max_tokens_per_expert=int(counts.max()))
+               max_tokens_per_expert=tmax, batches=nb, steps=steps,
+               close_call_tokens=sum(close_calls(L, h, L.k) for h in hiddens))
     res["layer_bytes"] = layer_bytes(L.E, L.k, L.H, L.F, T, U)
     res["layer_hbm_frac"] = res["layer_bytes"] / (ms * 1e-3) / (HBM_PEAK_GBS * 1e9)
     res["layer_flops"] = layer_flops(L.E, L.k, L.H, L.F, T)
@@ -318,20 +344,22 @@ def main():
             else:
                 r, _ = bench_layer(lib, synth, shape, Ts, max(20, a.steps // 2), a.warmup)
             sweep.append(dict(T=Ts, tokens_per_s=round(r["tokens_per_s"], 1), ms_per_step=round(r["ms_per_step"], 5),
-                              distinct_experts=r["distinct_experts"], layer_hbm_frac=round(r["layer_hbm_frac"], 4),
+                              distinct_experts=r["distinct_experts"], close_call_tokens=r["close_call_tokens"],
+                              layer_hbm_frac=round(r["layer_hbm_frac"], 4),
                               gateup_hbm_frac=round(r["gateup_gbs"] / HBM_PEAK_GBS, 4),
                               stage_ms={kk: round(v, 5) for kk, v in r["stage_ms"].items()}))
 
     cpu = None if a.no_cpu else cpu_baseline(L, hidden, out)
     line = dict(
-        metric="MoE layer tokens/s", value=res["tokens_per_s"], unit="tokens/s", n_gpus=1, steps=a.steps,
+        metric="MoE layer tokens/s", value=res["tokens_per_s"], unit="tokens/s", n_gpus=1, steps=res["steps"],
         warmup=a.warmup, ms_per_step=res["ms_per_step"], higher_is_better=True, scaling="weak",
         vs_baseline=None,
         dtype=("mxfp4 x fp6(3-term, block-scaled) -> f32" if prefill else "mxfp4 x bf16(2-term) -> f32"),
         data="synthetic",
         config=dict(workload=f"{a.workload}: E={shape['E']} top-{shape['k']} H={shape['H']} F={shape['F']} "
                              f"MXFP4, T={T}" + (", 8 hot experts" if shape["hot"] else ""),
-                    tokens=T, distinct_experts=res["distinct_experts"], device=dev_name, compute_units=cus),
+                    tokens=T, distinct_experts=res["distinct_experts"], token_batches_in_rotation=res["batches"],
+                    close_call_tokens=res["close_call_tokens"], device=dev_name, compute_units=cus),
         roofline=roof, cpu_baseline=cpu,
         layer=dict(hbm_frac=res["layer_hbm_frac"], fp4_mfma_frac=res["layer_fp4_frac"],
                    algorithmic_bytes=res["layer_bytes"], algorithmic_flops=res["layer_flops"],

@@ -64,6 +64,7 @@ SIGNATURES = {
     "csk_moe_stack_forward": (C.c_int, [C.POINTER(_P), _I64, _P, _I64]),
     "csk_layer_last_dispatch": (C.c_int, [_P, _P, _P]),
     "csk_moe_router": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P]),
+    "csk_moe_router_logits": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _P]),
     "csk_expert_mlp_mxfp4": (C.c_int, [C.c_int, _P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P,
                                        _I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]),
     "csk_expert_token_mxfp4": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, C.c_int]),
@@ -211,6 +212,16 @@ class Library:
         out = np.empty((T, k, 2), np.float32)
         self.check(self.dll.csk_moe_router(_ptr(hidden), T, H, _ptr(gate_w), E, _ptr(gate_b), k,
                                            int(sigmoid), _ptr(out)))
+        return out
+
+    def moe_router_logits(self, hidden, gate_w, gate_b):
+        hidden, gate_w = _f32(hidden), _f32(gate_w)
+        T, H = hidden.shape
+        E = gate_w.shape[0]
+        gb = _f32(gate_b) if gate_b is not None else None
+        out = np.empty((T, E), np.float32)
+        self.check(self.dll.csk_moe_router_logits(_ptr(hidden), T, H, _ptr(gate_w), E,
+                                                  _ptr(gb) if gb is not None else None, _ptr(out)))
         return out
 
     def expert_mlp(self, expert_id, hidden, F, h_up, h_gate, h_down, b_up, b_gate, b_down, pairs,

@@ -299,8 +299,8 @@ int launch_router(const float* x, const float* gate_w, const float* gate_b, int6
   }
   int rc = check_launch("router_logits_kernel");
   if (rc != CSK_OK) return rc;
-  router_topk_kernel<<<dim3((unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(logits, pairs, ids, (int)T,
-                                                                       (int)E, (int)k, sigmoid);
+  router_topk_kernel<<<dim3((unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
+      logits, pairs, ids, (int)T, (int)E, (int)k, sigmoid, x, gate_w, gate_b, (int)H);
   return check_launch("router_topk_kernel");
 }
 
@@ -768,9 +768,10 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
         L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
     if ((rc = check_launch("router_prep_logits_kernel")) != CSK_OK) return rc;
     mark(CSK_STAGE_DISPATCH);
-    route_small_kernel<<<dim3(1), 1024, 0, g_stream>>>(
+    route_small_kernel<<<dim3(1), 512, 0, g_stream>>>(
         ws.logits, ws.pairs, ws.ids, (int)T, (int)L->E, (int)L->k, L->sigmoid, L->ew_dev, ws.counts,
-        ws.offsets, ws.desc, ws.vlist, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w, ws.pos);
+        ws.offsets, ws.desc, ws.vlist, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w, ws.pos,
+        xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, (int)L->H);
     if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
     if (!stream_path(T, L->H, L->F) && !L->wbf) {
       // few tokens but rows too long for the streaming kernel: the GEMM wants the FP6 form
@@ -887,11 +888,30 @@ struct DevBuf {
 };
 }  // namespace
 
+namespace {
+int router_host(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
+                const float* gate_b, int64_t k, int sigmoid, float* out_pairs, float* out_logits);
+}
+
 extern "C" int csk_moe_router(const float* hidden, int64_t T, int64_t H, const float* gate_w,
                               int64_t E, const float* gate_b, int64_t k, int sigmoid,
                               float* out_pairs) {
   REQUIRE_INIT();
-  if (!hidden || !gate_w || !out_pairs || T < 0) return fail(CSK_ERR_ARG, "csk_moe_router: null argument");
+  if (!out_pairs) return fail(CSK_ERR_ARG, "csk_moe_router: null argument");
+  return router_host(hidden, T, H, gate_w, E, gate_b, k, sigmoid, out_pairs, nullptr);
+}
+
+extern "C" int csk_moe_router_logits(const float* hidden, int64_t T, int64_t H, const float* gate_w,
+                                     int64_t E, const float* gate_b, float* out_logits) {
+  REQUIRE_INIT();
+  if (!out_logits) return fail(CSK_ERR_ARG, "csk_moe_router_logits: null argument");
+  return router_host(hidden, T, H, gate_w, E, gate_b, 1, 0, nullptr, out_logits);
+}
+
+namespace {
+int router_host(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
+                const float* gate_b, int64_t k, int sigmoid, float* out_pairs, float* out_logits) {
+  if (!hidden || !gate_w || T < 0) return fail(CSK_ERR_ARG, "csk_moe_router: null argument");
   if (E <= 0 || E > kMaxExperts || k <= 0 || k > kMaxTopK || k > E || H <= 0 || H % 4)
     return fail(CSK_ERR_ARG, "csk_moe_router: need 1 <= top_k <= min(16, E), E <= 256, H a multiple of 4");
   if (T == 0) return CSK_OK;
@@ -906,10 +926,12 @@ extern "C" int csk_moe_router(const float* hidden, int64_t T, int64_t H, const f
   rc = launch_router(dx.as<float>(), dg.as<float>(), gate_b ? db.as<float>() : nullptr, T, E, H, k,
                      sigmoid, dl.as<float>(), dp.as<float>(), di.as<int>());
   if (rc != CSK_OK) return rc;
-  HIP_TRY(hipMemcpyAsync(out_pairs, dp.p, (size_t)T * k * 8, hipMemcpyDeviceToHost, g_stream));
+  if (out_pairs) HIP_TRY(hipMemcpyAsync(out_pairs, dp.p, (size_t)T * k * 8, hipMemcpyDeviceToHost, g_stream));
+  if (out_logits) HIP_TRY(hipMemcpyAsync(out_logits, dl.p, (size_t)T * E * 4, hipMemcpyDeviceToHost, g_stream));
   HIP_TRY(hipStreamSynchronize(g_stream));
   return CSK_OK;
 }
+}  // namespace
 
 namespace {
 __global__ void select_expert_ids_kernel(const float* __restrict__ pairs, int* __restrict__ ids,

@@ -257,30 +257,23 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
   }
 }
 
-// ------------------------------------------------------------------- top-k
-// One wave per token.  Lane l holds the logits of experts l, l+64, l+128,
-// l+192; each of the k rounds finds the wave-wide maximum (ties -> lowest
-// expert index) with a butterfly over (value, index) and retires it.  Weights
-// follow moe_router_node.h:180-202: sigmoid of the raw logit, or softmax over
-// the selected k with max subtraction, sum in slot order, multiply by 1/sum.
-__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits,
-                                                          float* __restrict__ pairs,
-                                                          int* __restrict__ ids, int T, int E,
-                                                          int k, int sigmoid) {
-  const int lane = threadIdx.x & 63;
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (t >= T) return;
+// --------------------------------------------------- per-token selection
+// One wave selects one token's top k.  Lane l holds the logits of experts l, l+64,
+// l+128, l+192; each round finds the wave-wide maximum (ties -> lowest expert index)
+// with a butterfly over (value, index) and retires it.  One round more than k records
+// the runner-up, so that the k+1 largest logits are known: if any two adjacent ones are
+// closer than the difference between this library's tree-ordered fp32 sums and the
+// reference's strictly sequential ones can be (moe_router_node.h:161-167: sum += h*g,
+// multiply and add rounded separately, bias added last), the wave recomputes all E
+// logits of the token in exactly that order and selects again -- so the expert indices
+// and their slot order equal the reference's whenever the inputs are the same, not only
+// when no two logits are close.  Lane s < k returns slot s in (my_val, my_idx).
+__device__ __forceinline__ void select_topk(float (&v)[4], int lane, int E, int k, float& my_val,
+                                            int& my_idx, float& vmax, bool& close_call, float tol,
+                                            float& runner_up) {
   const float NEG = -__builtin_inff();
-  float v[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int e = lane + 64 * j;
-    v[j] = (e < E) ? logits[(size_t)t * E + e] : NEG;
-  }
-  float my_val = 0.0f;  // lane s keeps slot s
-  int my_idx = 0;
-  float vmax = 0.0f;
-  for (int s = 0; s < k; ++s) {
+  my_val = 0.0f, my_idx = 0, vmax = 0.0f;
+  for (int s = 0; s <= k; ++s) {
     float bv = v[0];
     int bi = lane;
 #pragma unroll
@@ -304,11 +297,121 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restric
       my_val = bv;
       my_idx = bi;
     }
-    if ((bi & 63) == lane) {
+    if (s < k && (bi & 63) == lane) {
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         if ((bi >> 6) == j) v[j] = NEG;
     }
+  }
+  // lanes 0..k hold the k+1 largest in descending order (fewer when E == k)
+  const float below = __shfl_down(my_val, 1, 64);
+  const bool close = lane < k && lane + 1 < E && (my_val - below) <= tol * fmaxf(1.0f, fabsf(my_val));
+  close_call = __any(close);
+  runner_up = __shfl(my_val, min(k, E - 1), 64);
+}
+
+// One logit in the reference's order: a strictly sequential fp32 sum, multiply and add
+// rounded separately (moe_router_node.h:161-167).  The chain of additions cannot be
+// shortened (about ten cycles per element), so the loads are kept out of its way: both
+// rows are fetched two groups of eight float4 (64 elements) ahead of their use, three
+// rotating register sets.  H is a multiple of 32, so the groups need no guards.
+__device__ __forceinline__ float dot_reference_order(const float* __restrict__ xrow,
+                                                     const float* __restrict__ grow, int H) {
+#pragma clang fp contract(off)
+  const CSK_GLOBAL floatx4* x4 = as_global(reinterpret_cast<const floatx4*>(xrow));
+  const CSK_GLOBAL floatx4* g4 = as_global(reinterpret_cast<const floatx4*>(grow));
+  const int ngrp = H >> 5;  // groups of 8 float4
+  floatx4 gq[3][8], xq[3][8];
+  auto fetch = [&](int u, int grp) {
+    const int c = 8 * min(grp, ngrp - 1);  // fetches past the end re-read the last group
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      gq[u][i] = g4[c + i];
+      xq[u][i] = x4[c + i];
+    }
+  };
+  fetch(0, 0);
+  fetch(1, 1);
+  float sum = 0.0f;
+  for (int grp = 0; grp < ngrp; grp += 3) {
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      if (grp + u < ngrp) {
+        fetch((u + 2) % 3, grp + u + 2);
+        // the products do not depend on the running sum: all 32 first, so that only
+        // the additions sit in the dependent chain
+        floatx4 pr[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pr[i] = xq[u][i] * gq[u][i];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          sum = sum + pr[i][0];
+          sum = sum + pr[i][1];
+          sum = sum + pr[i][2];
+          sum = sum + pr[i][3];
+        }
+      }
+    }
+  }
+  return sum;
+}
+
+// Recomputes, in the reference's order, the logits that can take part in a close call:
+// those not more than 2 * tol below the (k+1)-th largest (thr).  The others keep their
+// tree-ordered values, which the bound keeps on their side of thr.
+__device__ __forceinline__ void logits_reference_order(const float* __restrict__ x,
+                                                       const float* __restrict__ g,
+                                                       const float* __restrict__ b, int lane, int E,
+                                                       int H, float thr, float (&v)[4]) {
+#pragma clang fp contract(off)
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = lane + 64 * j;
+    if (e < E && v[j] >= thr) v[j] = dot_reference_order(x, g + (size_t)e * H, H) + (b ? b[e] : 0.0f);
+  }
+}
+
+// How close is a close call.  Measured over 1.3 million logits (six shapes, H from 256 to
+// 2880): |tree-ordered sum - sequential sum| / max(1, |logit|) has an rms of 0.28 and a
+// maximum of 2.3 in units of 2^-24 * sqrt(H) (the random-walk size of the sequential
+// sum's rounding error); the tests hold the maximum below 3.  Two logits can change rank
+// only if they are closer than the sum of their two differences; the threshold is 8 units,
+// twice the largest pair of differences seen.  At gpt-oss shapes about one token in 2500
+// is recomputed.
+__device__ __forceinline__ float close_call_tolerance(int H) { return 8.0f * 5.96e-8f * sqrtf((float)H); }
+
+// ------------------------------------------------------------------- top-k
+// One wave per token (select_topk).  Weights
+// follow moe_router_node.h:180-202: sigmoid of the raw logit, or softmax over
+// the selected k with max subtraction, sum in slot order, multiply by 1/sum.
+__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits,
+                                                          float* __restrict__ pairs,
+                                                          int* __restrict__ ids, int T, int E,
+                                                          int k, int sigmoid,
+                                                          const float* __restrict__ x,
+                                                          const float* __restrict__ g,
+                                                          const float* __restrict__ b, int H) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;
+  const float NEG = -__builtin_inff();
+  float v[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = lane + 64 * j;
+    v[j] = (e < E) ? logits[(size_t)t * E + e] : NEG;
+  }
+  float my_val, vmax, runner_up;  // lane s keeps slot s
+  int my_idx;
+  bool close_call;
+  float v0[4] = {v[0], v[1], v[2], v[3]};
+  const float tol = close_call_tolerance(H);
+  select_topk(v, lane, E, k, my_val, my_idx, vmax, close_call, tol, runner_up);
+  if (close_call) {
+    logits_reference_order(x + (size_t)t * H, g, b, lane, E, H,
+                           runner_up - 2.0f * tol * fmaxf(1.0f, fabsf(runner_up)), v0);
+    select_topk(v0, lane, E, k, my_val, my_idx, vmax, close_call, 0.0f, runner_up);
   }
   float w;
   if (sigmoid) {
@@ -482,17 +585,19 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
 }
 
 // ------------------------------------- small batches: top-k + dispatch, fused
-// One workgroup of 16 waves does, for P = T * k <= 1024 assignments, what
+// One workgroup of eight waves (so that a wave may use 256 registers for the
+// reference-order recomputation) does, for P = T * k <= 1024 assignments, what
 // router_topk_kernel and dispatch_scatter_kernel do in
 // three launches: top-k and weights per token (one wave per token), histogram,
 // exclusive scan, ordered scatter, work descriptors and token groups -- all
 // through LDS.
-__global__ __launch_bounds__(1024) void route_small_kernel(
+__global__ __launch_bounds__(512) void route_small_kernel(
     const float* __restrict__ logits, float* __restrict__ pairs, int* __restrict__ ids_out, int T,
     int E, int k, int sigmoid, const ExpertW* __restrict__ ew, int* __restrict__ counts,
     int* __restrict__ offsets, WorkDesc* __restrict__ desc, int* __restrict__ vlist,
     int* __restrict__ nv, int* __restrict__ mtiles, int* __restrict__ n_mtiles,
-    int* __restrict__ list_tok, float* __restrict__ list_w, int* __restrict__ pos_of_slot) {
+    int* __restrict__ list_tok, float* __restrict__ list_w, int* __restrict__ pos_of_slot,
+    const float* __restrict__ x, const float* __restrict__ g, const float* __restrict__ b, int H) {
   __shared__ int ids[1024];
   __shared__ float wts[1024];
   __shared__ int cnt[kMaxExperts], off[kMaxExperts], act_e[kMaxExperts];
@@ -500,44 +605,23 @@ __global__ __launch_bounds__(1024) void route_small_kernel(
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int P = T * k;
   const float NEG = -__builtin_inff();
-  for (int t = wv; t < T; t += 16) {
+  for (int t = wv; t < T; t += 8) {
     float v[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int e = lane + 64 * j;
       v[j] = (e < E) ? logits[(size_t)t * E + e] : NEG;
     }
-    float my_val = 0.0f, vmax = 0.0f;
-    int my_idx = 0;
-    for (int s = 0; s < k; ++s) {
-      float bv = v[0];
-      int bi = lane;
-#pragma unroll
-      for (int j = 1; j < 4; ++j) {
-        if (v[j] > bv) {
-          bv = v[j];
-          bi = lane + 64 * j;
-        }
-      }
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(bv, o, 64);
-        const int oi = __shfl_xor(bi, o, 64);
-        if (ov > bv || (ov == bv && oi < bi)) {
-          bv = ov;
-          bi = oi;
-        }
-      }
-      if (s == 0) vmax = bv;
-      if (lane == s) {
-        my_val = bv;
-        my_idx = bi;
-      }
-      if ((bi & 63) == lane) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if ((bi >> 6) == j) v[j] = NEG;
-      }
+    float my_val, vmax, runner_up;
+    int my_idx;
+    bool close_call;
+    float v0[4] = {v[0], v[1], v[2], v[3]};
+    const float tol = close_call_tolerance(H);
+    select_topk(v, lane, E, k, my_val, my_idx, vmax, close_call, tol, runner_up);
+    if (close_call) {
+      logits_reference_order(x + (size_t)t * H, g, b, lane, E, H,
+                             runner_up - 2.0f * tol * fmaxf(1.0f, fabsf(runner_up)), v0);
+      select_topk(v0, lane, E, k, my_val, my_idx, vmax, close_call, 0.0f, runner_up);
     }
     float w;
     if (sigmoid) {
@@ -558,7 +642,7 @@ __global__ __launch_bounds__(1024) void route_small_kernel(
   }
   __syncthreads();
   // histogram: wave wv counts experts wv, wv + 16, ... with ballots over the assignments
-  for (int e = wv; e < E; e += 16) {
+  for (int e = wv; e < E; e += 8) {
     int c = 0;
     for (int p0 = 0; p0 < P; p0 += 64) {
       const int p = p0 + lane;
@@ -627,7 +711,7 @@ __global__ __launch_bounds__(1024) void route_small_kernel(
   }
   __syncthreads();
   // ordered scatter: rank of an assignment = matches before it (ballot prefix)
-  for (int e = wv; e < E; e += 16) {
+  for (int e = wv; e < E; e += 8) {
     if (cnt[e] == 0) continue;
     int basep = off[e];
     for (int p0 = 0; p0 < P; p0 += 64) {

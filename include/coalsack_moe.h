@@ -186,6 +186,12 @@ int csk_layer_last_dispatch(csk_layer* L, int32_t* counts_host, int32_t* tokens_
  * weight). */
 int csk_moe_router(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
                    const float* gate_b, int64_t k, int sigmoid_gating, float* out_pairs);
+/* The logits of that router as this library first computes them (fp32, tree-ordered
+ * sums; [T,E]), before any recomputation in the reference's summation order -- a
+ * diagnostic: the tests bound their distance from the reference's sequential sums,
+ * which is what the close-call threshold of the top-k selection rests on. */
+int csk_moe_router_logits(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
+                          const float* gate_b_or_null, float* out_logits);
 /* expert_mlp_node::compute_with_mxfp4 for one expert (expert_mlp_node.h:392-530):
  * out [T,H]; *is_empty = 1 and out untouched when no token selected expert_id
  * (:441-443); rows of unselected tokens are zero (:509-512). */

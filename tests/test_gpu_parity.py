@@ -95,6 +95,74 @@ def test_router_matches_oracle(lib, oracle, T, H, E, k, bias, sigmoid):
     assert np.all(got[..., 1] > 0) and np.allclose(got[..., 1].sum(axis=1), 1.0, atol=1e-5) or sigmoid
 
 
+@pytest.mark.parametrize("T,E,H,sg", [(2048, 32, 2880, 0.02), (1024, 128, 2880, 0.02), (16, 32, 2880, 0.02),
+                                      (2048, 32, 512, 0.05), (300, 200, 256, 0.05)])
+def test_router_logits_distance_from_sequential_sums(lib, oracle, T, E, H, sg):
+    """The close-call threshold of the top-k selection (8 units of 2^-24 sqrt(H)) assumes
+    that no tree-ordered logit is further than 3 units from the reference's sequential sum."""
+    rng = np.random.default_rng(T + E)
+    h = rng.normal(0, 1, (T, H)).astype(np.float32)
+    g = rng.normal(0, sg, (E, H)).astype(np.float32)
+    b = rng.normal(0, 0.01, E).astype(np.float32)
+    got, want = lib.moe_router_logits(h, g, b), oracle.router_logits(h, g, b)
+    rel = np.abs(got.astype(np.float64) - want) / np.maximum(1.0, np.abs(want))
+    assert rel.max() <= 3.0 * 5.96e-8 * np.sqrt(H), rel.max() / (5.96e-8 * np.sqrt(H))
+
+
+def _near_tie_gate(E, H, seed):
+    """Gate rows in near-identical pairs: experts 2i and 2i+1 differ by a few 1e-7 relative,
+    so their logits sit within an ulp or two of each other and the order of the fp32
+    additions decides which one ranks first."""
+    rng = np.random.default_rng(seed)
+    g = rng.normal(0, 0.05, (E, H)).astype(np.float32)
+    for e in range(0, E - 1, 2):
+        g[e + 1] = g[e] * np.float32(1.0 + rng.choice([-3e-7, -1e-7, 1e-7, 3e-7]))
+        g[e + 1, rng.integers(0, H, 8)] += np.float32(1e-7)
+    return g
+
+
+def _no_exact_tie_rows(logits, k):
+    srt = -np.sort(-logits, axis=1)[:, :k + 1]
+    return np.all(srt[:, :-1] != srt[:, 1:], axis=1)
+
+
+@pytest.mark.parametrize("T,E,k,H", [(48, 16, 4, 2880), (300, 32, 4, 2880), (200, 10, 3, 96)])
+def test_router_near_ties_follow_reference_order(lib, oracle, T, E, k, H):
+    """Logits closer than summation-order noise: the indices and their slot order must
+    still be the reference's (sequential-order recomputation of close calls); only exact
+    ties of the reference's own logits are exempt."""
+    rng = np.random.default_rng(T + E)
+    h = rng.normal(0, 1, (T, H)).astype(np.float32)
+    g = _near_tie_gate(E, H, seed=E * 7 + k)
+    b = rng.normal(0, 0.01, E).astype(np.float32)
+    b[1::2] = b[0:E - 1:2][:len(b[1::2])]  # same bias within a pair
+    got = lib.moe_router(h, g, b, k)
+    want = oracle.router(h, g, b, k)
+    ok = _no_exact_tie_rows(oracle.router_logits(h, g, b), k)
+    assert ok.sum() > T // 2
+    # the pairs really are close calls: a float64 ranking disagrees with the reference's on some tokens
+    l64 = h.astype(np.float64) @ g.astype(np.float64).T + b
+    top64 = np.argsort(-l64, axis=1)[:, :k]
+    assert np.any(top64[ok] != want[ok, :, 0].astype(int))
+    assert np.array_equal(got[ok, :, 0], want[ok, :, 0])
+    assert np.max(np.abs(got[ok, :, 1] - want[ok, :, 1])) <= 1e-5
+
+
+def test_layer_small_batch_near_ties_follow_reference_order(lib, oracle):
+    """The same through the fused small-batch routing kernel of the layer forward."""
+    E, k, H, F, T = 8, 2, 2880, 32, 16
+    L = synth.LayerInputs(E, k, H, F, seed=4)
+    L.gate_w = _near_tie_gate(E, H, seed=5)
+    L.gate_b[1::2] = L.gate_b[0::2]
+    hidden = synth.hidden_states(T, H, seed=6)
+    with build_layer(lib, L) as layer:
+        _, pairs = layer.forward(hidden, want_pairs=True)
+    want = oracle.router(hidden, L.gate_w, L.gate_b, k)
+    ok = _no_exact_tie_rows(oracle.router_logits(hidden, L.gate_w, L.gate_b), k)
+    assert ok.sum() >= T // 2
+    assert np.array_equal(pairs[ok, :, 0], want[ok, :, 0])
+
+
 # ------------------------------------------------------------- expert MLP
 
 def _const_matrix(rows, K, code_diag=None):
