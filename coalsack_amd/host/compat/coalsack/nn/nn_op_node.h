@@ -1,7 +1,7 @@
-// Stand-in for include/coalsack/nn/nn_op_node.h:222-315 (variadic_op_node): the
-// base that unpacks named tensor fields from a result_message, calls
-// compute(), and sends the result -- or the caught exception as an error
-// result with a null field -- downstream.
+// Stand-in for include/coalsack/nn/nn_op_node.h:137-220 (binary_op_node) and :222-315
+// (variadic_op_node): the bases that unpack named tensor fields from a
+// result_message, call compute(), and send the result -- or the caught exception
+// as an error result with a null field -- downstream.
 #pragma once
 #include <exception>
 #include <memory>
@@ -23,6 +23,51 @@ inline dynamic_tensor get_tensor_from_result_message(const std::shared_ptr<resul
   if (!t) throw std::runtime_error("Field '" + field_name + "' is not a dynamic_tensor_message");
   return t->get_tensor();
 }
+
+class binary_op_node : public graph_node {
+ protected:
+  graph_edge_ptr output_;
+  std::string node_name_, op_type_, input_a_name_, input_b_name_, output_name_;
+  virtual dynamic_tensor compute(const dynamic_tensor& a, const dynamic_tensor& b) = 0;
+
+ public:
+  explicit binary_op_node(const std::string& op_type)
+      : output_(std::make_shared<graph_edge>(this)), op_type_(op_type) {
+    set_output(output_);
+  }
+  std::string get_proc_name() const override { return "nn_" + op_type_; }
+  void set_input_names(const std::string& a, const std::string& b) {
+    input_a_name_ = a;
+    input_b_name_ = b;
+  }
+  void set_output_name(const std::string& name) { output_name_ = name; }
+  void set_node_name(const std::string& name) { node_name_ = name; }
+  std::vector<std::string> get_input_names() const { return {input_a_name_, input_b_name_}; }
+
+  void process(std::string /*input_name*/, graph_message_ptr message) override {
+    auto in = std::dynamic_pointer_cast<result_message>(message);
+    const uint64_t frame = in ? in->get_frame_number() : 0;
+    std::shared_ptr<result_message> out;
+    if (in && !in->is_ok()) {
+      out = result_message::error({{output_name_, nullptr}}, "Input error");
+    } else {
+      try {
+        dynamic_tensor a, b;
+        if (in) {
+          if (input_a_name_.empty() || input_b_name_.empty())
+            throw std::runtime_error(op_type_ + ": input names not set");
+          a = get_tensor_from_result_message(in, input_a_name_);
+          b = get_tensor_from_result_message(in, input_b_name_);
+        }
+        out = result_message::ok({{output_name_, std::make_shared<dynamic_tensor_message>(compute(a, b))}});
+      } catch (const std::exception& e) {
+        out = result_message::error({{output_name_, nullptr}}, e.what());
+      }
+    }
+    out->set_frame_number(frame);
+    output_->send(out);
+  }
+};
 
 class variadic_op_node : public graph_node {
  protected:

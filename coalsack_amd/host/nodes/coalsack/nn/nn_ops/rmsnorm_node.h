@@ -1,0 +1,51 @@
+// rmsnorm_node backed by the gfx950 library: same class name, setter, test wrapper
+// and error texts as include/coalsack/nn/nn_ops/rmsnorm_node.h of the reference
+// (cited by line below); the normalisation runs in csk_rmsnorm.
+#pragma once
+
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "coalsack/nn/nn_op_node.h"
+#include "coalsack_moe.h"
+
+namespace coalsack {
+
+// input: any shape, normalised over the last dimension; weight: [hidden_dim].
+// out = (x / sqrt(mean(x^2) + epsilon)) * weight   (:62-83)
+class rmsnorm_node : public binary_op_node {
+ public:
+  rmsnorm_node() : binary_op_node("rmsnorm"), epsilon_(1e-5f) {}  // :12
+  void set_epsilon(float epsilon) { epsilon_ = epsilon; }          // :14
+  dynamic_tensor compute_test(const dynamic_tensor& input, const dynamic_tensor& weight) {  // :17-19
+    return compute(input, weight);
+  }
+
+ protected:
+  dynamic_tensor compute(const dynamic_tensor& input, const dynamic_tensor& weight) override {  // :22-57
+    const auto& shape = input.shape();
+    if (shape.empty()) throw std::runtime_error("rmsnorm: input must have at least 1 dimension");
+    int64_t outer_size = 1;
+    for (size_t i = 0; i + 1 < shape.size(); ++i) outer_size *= shape[i];
+    const int64_t hidden_dim = shape.back();
+    if (weight.ndim() != 1 || weight.dim(0) != hidden_dim)
+      throw std::runtime_error("rmsnorm: weight shape must be [hidden_dim]");
+    // the reference also has a float64 branch; this build computes in float32 only
+    if (input.get_dtype() != dtype::float32 || weight.get_dtype() != dtype::float32)
+      throw std::runtime_error("rmsnorm: only float32 supported on this build");
+    dynamic_tensor output(dtype::float32, shape);
+    if (outer_size == 0 || hidden_dim == 0) return output;
+    const int rc = csk_rmsnorm(input.data_ptr<float>(), weight.data_ptr<float>(), output.data_ptr<float>(),
+                               outer_size, hidden_dim, epsilon_);
+    if (rc != CSK_OK) throw std::runtime_error(std::string("rmsnorm: ") + csk_last_error());
+    return output;
+  }
+
+ private:
+  float epsilon_;
+};
+
+}  // namespace coalsack
+
+COALSACK_REGISTER_NODE(coalsack::rmsnorm_node, coalsack::graph_node)

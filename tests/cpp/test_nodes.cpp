@@ -11,9 +11,11 @@
 #include <string>
 #include <vector>
 
+#include "coalsack/nn/nn_ops/add_node.h"
 #include "coalsack/nn/nn_ops/expert_merge_node.h"
 #include "coalsack/nn/nn_ops/expert_mlp_node.h"
 #include "coalsack/nn/nn_ops/moe_router_node.h"
+#include "coalsack/nn/nn_ops/rmsnorm_node.h"
 
 using namespace coalsack;
 
@@ -25,6 +27,8 @@ int orc_expert_mlp_mxfp4(int, const float*, int64_t, int64_t, int64_t, const uin
                          const uint8_t*, const float*, const float*, const float*, const float*, int64_t,
                          int, int, float*, int*);
 int orc_expert_merge(const float*, int64_t, int64_t, int64_t, int64_t, const float* const*, int, float*);
+void orc_rmsnorm(const float*, const float*, float*, int64_t, int64_t, float);
+void orc_add(const float*, const float*, float*, int64_t);
 }
 
 static int g_failed = 0, g_checks = 0;
@@ -164,6 +168,73 @@ static void cpu_merge_argument_errors() {
 }
 
 // ------------------------------------------------------------------ GPU mode
+
+static void cpu_norm_add_argument_errors() {
+  std::mt19937 gen(5);
+  rmsnorm_node norm;
+  add_node add;
+  CHECK(norm.get_proc_name() == "nn_rmsnorm" && add.get_proc_name() == "nn_add");
+  auto x = random_tensor({2, 3, 8}, gen, -1, 1), w = random_tensor({8}, gen, 0.5f, 1.5f);
+  auto w_bad = random_tensor({7}, gen, 0.5f, 1.5f), w2 = random_tensor({1, 8}, gen, 0.5f, 1.5f);
+  CHECK(throws_with([&] { norm.compute_test(dynamic_tensor(dtype::float32, {}), w); },
+                    "rmsnorm: input must have at least 1 dimension"));
+  CHECK(throws_with([&] { norm.compute_test(x, w_bad); }, "rmsnorm: weight shape must be [hidden_dim]"));
+  CHECK(throws_with([&] { norm.compute_test(x, w2); }, "rmsnorm: weight shape must be [hidden_dim]"));
+  CHECK(throws_with([&] { norm.compute_test(dynamic_tensor(dtype::float64, {2, 8}), w); }, "rmsnorm: only float32"));
+  CHECK(throws_with([&] { add.compute_test(x, dynamic_tensor(dtype::float64, {2, 3, 8})); }, "add: input dtype mismatch"));
+  CHECK(throws_with([&] { add.compute_test(x, w); }, "add: broadcasting is not supported"));
+  // through process(): missing input names and upstream errors (nn_op_node.h:172-219)
+  capture_node cap;
+  cap.set_input(norm.get_output());
+  norm.set_output_name("y");
+  auto msg = result_message::ok({{"x", std::make_shared<dynamic_tensor_message>(x)},
+                                 {"w", std::make_shared<dynamic_tensor_message>(w)}});
+  msg->set_frame_number(11);
+  norm.process("default", msg);
+  CHECK(cap.got.size() == 1 && cap.got[0]->is_error() && cap.got[0]->get_frame_number() == 11 &&
+        cap.got[0]->get_error_message() == "rmsnorm: input names not set" && cap.got[0]->get_field("y") == nullptr);
+  norm.set_input_names("x", "w");
+  auto err = result_message::error({{"x", nullptr}}, "upstream");
+  norm.process("default", err);
+  CHECK(cap.got.size() == 2 && cap.got[1]->is_error() && cap.got[1]->get_error_message() == "Input error");
+  CHECK((norm.get_input_names() == std::vector<std::string>{"x", "w"}));
+}
+
+static void gpu_norm_add_tests() {
+  std::mt19937 gen(77);
+  const int64_t B = 2, S = 5, H = 2880;
+  rmsnorm_node norm;
+  add_node add;
+  auto x = random_tensor({B, S, H}, gen, -2, 2), w = random_tensor({H}, gen, 0.5f, 1.5f);
+  // the reference's test values (test_rmsnorm.cpp:74-115): ones with unit weight stay ones
+  dynamic_tensor ones(dtype::float32, {1, 4}), w1(dtype::float32, {4});
+  for (int i = 0; i < 4; ++i) ones.data_ptr<float>()[i] = 1.0f, w1.data_ptr<float>()[i] = 1.0f;
+  auto o1 = norm.compute_test(ones, w1);
+  for (int i = 0; i < 4; ++i) CHECK(std::fabs(o1.data_ptr<float>()[i] - 1.0f) < 1e-4f);
+  norm.set_epsilon(1e-6f);
+  auto y = norm.compute_test(x, w);
+  std::vector<float> want((size_t)(B * S * H));
+  orc_rmsnorm(x.data_ptr<float>(), w.data_ptr<float>(), want.data(), B * S, H, 1e-6f);
+  CHECK(y.shape() == x.shape());
+  float worst = 0;
+  for (size_t i = 0; i < want.size(); ++i) worst = std::fmax(worst, std::fabs(y.data_ptr<float>()[i] - want[i]));
+  CHECK(worst <= 2e-6f);
+  auto z = add.compute_test(x, y);
+  orc_add(x.data_ptr<float>(), y.data_ptr<float>(), want.data(), B * S * H);
+  CHECK(std::memcmp(z.data_ptr<float>(), want.data(), want.size() * sizeof(float)) == 0);
+  // h <- h + f(rmsnorm(h)) wiring through messages (llm_engine.cpp:714-719, 773-777)
+  capture_node cap;
+  cap.set_input(add.get_output());
+  add.set_input_names("h", "moe_out");
+  add.set_output_name("h_next");
+  auto msg = result_message::ok({{"h", std::make_shared<dynamic_tensor_message>(x)},
+                                 {"moe_out", std::make_shared<dynamic_tensor_message>(y)}});
+  msg->set_frame_number(4);
+  add.process("default", msg);
+  CHECK(cap.got.size() == 1 && cap.got[0]->is_ok() && cap.got[0]->get_frame_number() == 4);
+  auto hn = std::dynamic_pointer_cast<dynamic_tensor_message>(cap.got[0]->get_field("h_next"));
+  CHECK(hn && std::memcmp(hn->get_tensor().data_ptr<float>(), want.data(), want.size() * sizeof(float)) == 0);
+}
 
 static void gpu_router_tests() {
   std::printf("router: Basic / TopKSelection / GptOssScale / WeightNormalization\n");
@@ -331,10 +402,12 @@ int main(int argc, char** argv) {
     gpu_router_tests();
     gpu_expert_known_answer();
     gpu_node_chain();
+    gpu_norm_add_tests();
   } else {
     cpu_router_argument_errors();
     cpu_expert_node_paths();
     cpu_merge_argument_errors();
+    cpu_norm_add_argument_errors();
   }
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
   return g_failed ? 1 : 0;
