@@ -60,6 +60,7 @@ constexpr int kMxStageChunks = kGemmBM * 4 * kMx3ChunksPerBlock;  // 1536 x 16 B
 constexpr int kMxRowChunks = 4 * kMx3ChunksPerBlock;              // 24 chunks per token per step
 constexpr int kMxWaves = 4;                                       // waves per workgroup
 constexpr int kMxCopies = kMxStageChunks / 64 / kMxWaves;         // copy instructions per wave per step
+constexpr int kStepLoads = kMxCopies + 2 * 2 * 2;                 // load instructions per wave per step
 
 template <int MODE>
 __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_kernel(ExpertGemmMxArgs a) {
@@ -121,33 +122,48 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
     arow[c] = a.A + (size_t)row * nblk * kMx3ChunksPerBlock + (lc - bs * kMx3ChunksPerBlock);
     ablk[c] = bs;
   }
-  auto copy_a = [&](int stage, int j) {
-#pragma unroll
-    for (int c = 0; c < kMxCopies; ++c) {
+  struct BSet {
+    u32x4 q[2][2];     // [64-wide K chunk of the step][row group]
+    uint32_t s[2][2];  // byte 0 = the block's scale byte (the matrix instruction reads only that byte)
+  };
+  // The kStepLoads load instructions of step j, one at a time: n < kMxCopies copies a part
+  // of the activation tile into LDS, the next four fetch the weight entries, the last four
+  // the scale bytes.
+  auto issue_load = [&](int n, int stage, BSet& b, int j) {
+    if (n < kMxCopies) {
+      const int c = n;
       const int kb = min(4 * j + ablk[c], nblk - 1);  // a block past K re-reads the last one (its weights are zeroed)
       __builtin_amdgcn_global_load_lds(
           arow[c] + (size_t)kb * kMx3ChunksPerBlock,
           reinterpret_cast<__attribute__((address_space(3))) uint4*>(
               reinterpret_cast<uintptr_t>(As + stage * kMxStageChunks + (kMxCopies * wv + c) * 64)),
           16, 0, 0);
+    } else {
+      const int m = (n - kMxCopies) & 3, kc = m >> 1, s = m & 1;
+      const int kb = min(4 * j + 2 * kc + kg, nblk - 1);
+      // Issued as inline assembly: the compiler's wait insertion does not see these as
+      // pending register writes, so it adds no waits of its own for them (it otherwise
+      // drains the whole queue once per loop iteration over a register it reuses); the
+      // explicit count at the step boundary is what guarantees their arrival.
+      if (n < kMxCopies + 4) {
+        const CSK_GLOBAL u32x4* ptr = qp[s] + kb * 16;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(b.q[kc][s]) : "v"(ptr) : "memory");
+      } else {
+        // a dword load at the byte's own (unaligned) address: the matrix instruction reads
+        // only byte 0 of its scale operand, so no widening instruction is needed
+        const CSK_GLOBAL uint8_t* ptr = sp[s] + scale_index(0, kb, 0, slots);
+        asm volatile("global_load_dword %0, %1, off" : "=v"(b.s[kc][s]) : "v"(ptr) : "memory");
+      }
     }
   };
-  struct BSet {
-    u32x4 q[2][2];     // [64-wide K chunk of the step][row group]
-    uint32_t s[2][2];  // byte 0 = the block's scale byte (the matrix instruction reads only that byte)
+  auto copy_a = [&](int stage, int j) {
+    BSet unused;
+#pragma unroll
+    for (int c = 0; c < kMxCopies; ++c) issue_load(c, stage, unused, j);
   };
   auto load_b = [&](BSet& b, int j) {
 #pragma unroll
-    for (int kc = 0; kc < 2; ++kc) {
-      const int kb = min(4 * j + 2 * kc + kg, nblk - 1);
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        b.q[kc][s] = qp[s][kb * 16];
-        // a dword load at the byte's own (unaligned) address: no widening instruction, so
-        // nothing waits for the value before the matrix instruction that uses it
-        b.s[kc][s] = *reinterpret_cast<const CSK_GLOBAL u32_unaligned*>(sp[s] + scale_index(0, kb, 0, slots));
-      }
-    }
+    for (int n = kMxCopies; n < kMxCopies + 8; ++n) issue_load(n, 0, b, j);
   };
 
   floatx16 acc[2][2];  // [32-token sub-tile][row group]
@@ -162,7 +178,12 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
   // Fragment i = (kc, term, 32-token sub-tile) of a step feeds two matrix instructions
   // (the two row groups).  Fragments are requested from LDS two ahead of their use, so
   // the LDS latency is covered by the four matrix instructions in between.
-  auto compute = [&](const BSet& b, int stage, int j) {
+  // The loads of the step after next are issued one per fragment between the matrix
+  // instructions rather than in a burst at the step boundary: the texture address unit
+  // takes 16 cycles per 64-lane 128-bit load, and a burst of 14 per wave, 8 waves per
+  // compute unit, held every wave at the start of the step for longer than the step's
+  // matrix work.
+  auto compute = [&](const BSet& b, int stage, int j, BSet& bn, int stage_n, int jn) {
     const u32x4* at = reinterpret_cast<const u32x4*>(As) + stage * kMxStageChunks;
     i32x8 bw[2][2];
 #pragma unroll
@@ -188,6 +209,8 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
     for (int i = 0; i < 12; ++i) {
       const int kc = i / 6, ms = i & 1;
       if (i + 2 < 12) read_frag(i + 2);
+      issue_load(i, stage_n, bn, jn);
+      if (i + 12 < kStepLoads) issue_load(i + 12, stage_n, bn, jn);
       __builtin_amdgcn_sched_barrier(0);
       // FP6 reads the first six registers; fhi[2] (register 6) is the term's scale byte
       const i32x8 aw = (i32x8)__builtin_shufflevector(flo[i % 3], fhi[i % 3], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -205,7 +228,6 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
   // step j+1, memory counters retire in order, so vmcnt(kStepLoads) means "my part of
   // step j has landed", and the barrier extends that to the other waves' parts and
   // tells that every wave is done reading the stage about to be overwritten.
-  constexpr int kStepLoads = kMxCopies + 2 * 2 * 2;  // copy_a + load_b instructions per step
   constexpr int kWaitStep = (kStepLoads & 15) | (7 << 4) | (15 << 8) | ((kStepLoads >> 4) << 14);
   // The first two steps are requested and awaited in full before the loop, so that the
   // loop is entered with nothing in flight and its body is the steady state from the
@@ -229,10 +251,7 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
     __builtin_amdgcn_s_waitcnt(kWaitStep);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    copy_a((u + 2) % 3, min(jj + 2, nsteps - 1));
-    load_b(bs[(u + 2) % 3], min(jj + 2, nsteps - 1));
-    __builtin_amdgcn_sched_barrier(0);
-    compute(bs[u], u, jj);
+    compute(bs[u], u, jj, bs[(u + 2) % 3], (u + 2) % 3, min(jj + 2, nsteps - 1));
     __builtin_amdgcn_sched_barrier(0);
   };
   // no control-flow joins between the steps of the steady state
@@ -244,6 +263,11 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
     step(2, j + 2);
     if (j + 3 >= nsteps) break;
   }
+  // The re-reads requested past the last step are still in flight and the compiler does
+  // not know it (those loads are inline assembly): nothing may follow the loop before
+  // they have landed, or a register they are about to overwrite could be given a new role.
+  __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0)
+  __builtin_amdgcn_sched_barrier(0);
 
   // epilogue: lane holds weight row n32 of each group; accumulator register r is token
   // (r % 4) + 8 * (r / 4) + 4 * kg of the 32-token sub-tile
