@@ -62,6 +62,7 @@ inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 // Above this many token-expert assignments the token-group list of the
 // weight-streaming kernel is not built.
 constexpr int64_t kStreamMaxP = 2048;
+constexpr size_t kWeightSlack = 4096;  // bytes of mapped memory kept behind weight planes
 constexpr int kStreamWgPerCu = 2;  // resident workgroups of the streaming kernel per compute unit
 
 // ---- workspace shared by every layer (single stream, one call at a time) --
@@ -105,8 +106,15 @@ struct Workspace {
 #define WS_ALLOC(ptr, cnt) \
   if ((rc = dev_alloc(&ptr, (cnt))) != CSK_OK) return rc
     WS_ALLOC(xn, (size_t)nT * nH);
-    WS_ALLOC(xs, (size_t)nT * nH * 2);
-    if (need_xg || had_xg) WS_ALLOC(xg, P * nH * 2);
+    // activation rows: two bf16 terms (128 B per block) or three FP6 terms padded to whole
+    // K steps (96 B per block), whichever is larger; counts are in uint16
+    auto act_elems = [](size_t rows, int64_t dim) {
+      const size_t bf = rows * (size_t)dim * 2;
+      const size_t mx = rows * (size_t)mx3_row_blocks((int)(dim / 32)) * 48;
+      return std::max(bf, mx);
+    };
+    WS_ALLOC(xs, act_elems((size_t)nT, nH));
+    if (need_xg || had_xg) WS_ALLOC(xg, act_elems(P, nH));
     WS_ALLOC(logits, (size_t)nT * nE);
     WS_ALLOC(pairs, P * 2);
     WS_ALLOC(ids, P);
@@ -118,7 +126,7 @@ struct Workspace {
     WS_ALLOC(list_tok, P);
     WS_ALLOC(list_w, P);
     WS_ALLOC(pos, P);
-    WS_ALLOC(act, P * nF * 2);
+    WS_ALLOC(act, act_elems(P, nF));
     WS_ALLOC(y, P * nH);
     WS_ALLOC(tiles, (size_t)4 * (P / 16 + nE + 1));
     WS_ALLOC(n_tiles, 1);
@@ -272,7 +280,7 @@ int launch_prep(const float* src, const float* norm_w, float eps, float* xn, uin
 int launch_mx3(const float* x, uint16_t* x3, int64_t rows, int64_t H, const int* gather_tok,
                const float* gather_w) {
   if (rows == 0) return CSK_OK;
-  const int64_t nb = rows * (H / 32);
+  const int64_t nb = rows * mx3_row_blocks((int)(H / 32));
   mx3_rows_kernel<<<dim3((unsigned)cdiv(nb, 256)), 256, 0, g_stream>>>(
       x, reinterpret_cast<u32x4*>(x3), rows, (int)(H / 32), gather_tok, gather_w);
   return check_launch("mx3_rows_kernel");
@@ -343,6 +351,11 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
   ga.act_out = reinterpret_cast<u32x4*>(a.act_out);
   ga.y_out = a.y_out;
   ga.n_ntiles = (int)cdiv(a.ntile, (NMAT == 2 ? 2 : 4) * kMxWaves);
+  // per-lane offsets into the activation rows and the weight planes are 32-bit
+  const int64_t a_rows = a.list_row ? T : P;
+  if (a_rows * mx3_row_blocks(a.nblk) * 96 >= ((int64_t)1 << 32) ||
+      (int64_t)a.ntile * a.nblk * 256 >= ((int64_t)1 << 32))
+    return fail(CSK_ERR_ARG, "batch too large for the grouped GEMM (activation rows or a weight plane exceed 4 GiB)");
   const int64_t max_mtiles = P / kGemmBM + std::min<int64_t>(E, P);
   const dim3 grid((unsigned)(cdiv(max_mtiles * ga.n_ntiles, kDies) * kDies));
   expert_gemm_mx_kernel<NMAT == 2 ? 0 : 1><<<grid, 64 * kMxWaves, 3 * kMxStageChunks * 16, g_stream>>>(ga);
@@ -543,8 +556,8 @@ extern "C" int csk_mxfp4_upload(const uint8_t* blocks, int64_t rows, int64_t K, 
   m->K = K;
   m->nblk = K / 32;
   m->ntile = cdiv(rows, 16);
-  int rc = dev_alloc(&m->q, (size_t)m->entries());
-  if (rc == CSK_OK) rc = dev_alloc(&m->s, (size_t)m->scale_bytes());
+  int rc = dev_alloc(&m->q, (size_t)m->entries() + kWeightSlack / sizeof(uint4));
+  if (rc == CSK_OK) rc = dev_alloc(&m->s, (size_t)m->scale_bytes() + kWeightSlack);
   if (rc == CSK_OK && hipMemset(m->s, 127, (size_t)m->scale_bytes()) != hipSuccess) rc = fail(CSK_ERR_HIP, "hipMemset failed");
   if (rc == CSK_OK) rc = pack_into(blocks, *m);
   if (rc != CSK_OK) {
@@ -588,8 +601,10 @@ extern "C" int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_
   L->ew_host.assign((size_t)E, ExpertW{});
   rc = dev_alloc(&L->gate_w, (size_t)E * H);
   if (rc == CSK_OK) rc = dev_alloc(&L->gate_b, (size_t)E);
-  if (rc == CSK_OK) rc = dev_alloc(&L->q_all, (size_t)E * L->ent_expert());
-  if (rc == CSK_OK) rc = dev_alloc(&L->s_all, (size_t)E * L->sc_expert());
+  // kWeightSlack: the grouped GEMM reads up to three blocks (and the scale loads three
+  // bytes) past the end of a plane; behind the last plane that must still be mapped memory
+  if (rc == CSK_OK) rc = dev_alloc(&L->q_all, (size_t)E * L->ent_expert() + kWeightSlack / sizeof(uint4));
+  if (rc == CSK_OK) rc = dev_alloc(&L->s_all, (size_t)E * L->sc_expert() + kWeightSlack);
   if (rc == CSK_OK && hipMemset(L->s_all, 127, (size_t)E * L->sc_expert()) != hipSuccess) rc = fail(CSK_ERR_HIP, "hipMemset failed");
   if (rc == CSK_OK) rc = dev_alloc(&L->bias_all, (size_t)E * (2 * F + H));
   if (rc == CSK_OK) rc = dev_alloc(&L->ew_dev, (size_t)E);

@@ -43,13 +43,13 @@ struct ExpertGemmMxArgs {
   const int* mtiles;     // [2 * n]: (expert slot, first token) of each M tile
   const int* n_mtiles;
   const int* list_row;   // packed position -> row of A; null: row = packed position
-  const uint4* A;        // [rows][nblk][6] x 16 B (mx3.h)
+  const uint4* A;        // [rows][mx3_row_blocks(nblk)][6] x 16 B (mx3.h); blocks past nblk are zeros
   int nblk;              // K / 32
   int ntile;             // ceil(N / 16) weight row tiles
   int n_ntiles;          // N tiles per M tile: ceil(ntile / 16) (MODE 0) or ceil(ntile / 32)
   int N;
   int act_type;
-  u32x4* act_out;        // MODE 0: [P][N / 32][6] x 16 B
+  u32x4* act_out;        // MODE 0: [P][mx3_row_blocks(N / 32)][6] x 16 B
   float* y_out;          // MODE 1: [P][N]
 };
 
@@ -89,10 +89,16 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
   const int nsteps = (nblk + 3) >> 2;
   const int slots = scale_slots(nblk);
 
-  // this wave's two 32-row groups (each a pair of packed tiles)
+  // this wave's two 32-row groups (each a pair of packed tiles).  Every address of the main
+  // loop is a wave-uniform base (advanced per step on the scalar unit) plus a 32-bit per-lane
+  // byte offset that never changes, so the loads cost no vector instructions.  Nothing is
+  // clamped: activation rows are padded with zero blocks to a whole number of steps, so the
+  // weight blocks read past K (the next tile's, or the slack behind the last plane) and the
+  // scale bytes read past K (slot padding, 127) are multiplied by exact zeros.
   int tiles[2];  // this lane's packed tile in each group
-  const CSK_GLOBAL u32x4* qp[2];
-  const CSK_GLOBAL uint8_t* sp[2];
+  const char* qbase[2];
+  const char* sbase[2];
+  uint32_t qoff[2], soff[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
     int t;
@@ -102,26 +108,29 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
     const int tc = min(t, a.ntile - 1);
     const uint4* qb = MODE == 0 ? (s == 0 ? wd->w.q_gate : wd->w.q_up) : wd->w.q_down;
     const uint8_t* sb = MODE == 0 ? (s == 0 ? wd->w.s_gate : wd->w.s_up) : wd->w.s_down;
-    qp[s] = as_global(reinterpret_cast<const u32x4*>(qb)) + (size_t)tc * nblk * 16 + n16;
-    sp[s] = as_global(sb) + scale_index(tc, 0, n16, slots);
+    qbase[s] = reinterpret_cast<const char*>(qb);
+    sbase[s] = reinterpret_cast<const char*>(sb);
+    qoff[s] = (uint32_t)((((size_t)tc * nblk + kg) * 16 + n16) * 16);  // entry (tile, block kg, row)
+    soff[s] = (uint32_t)scale_index(tc, kg, n16, slots);
   }
+  const int rowblk = mx3_row_blocks(nblk);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
   // Copy instruction c of wave wv fills chunks [(kMxCopies wv + c) * 64, +64) of the
   // stage, in token-major order; the lane's chunk is physical position pc of token tl
   // and holds logical chunk lc (XOR swizzle on the low three bits).
-  const uint4* arow[kMxCopies];  // source of this lane's chunk at step 0, minus the block term
-  int ablk[kMxCopies];           // block of the step the chunk belongs to
+  uint32_t aoff[kMxCopies];  // byte offset of this lane's chunk at step 0 from a.A
 #pragma unroll
   for (int c = 0; c < kMxCopies; ++c) {
     const int lin = (kMxCopies * wv + c) * 64 + lane;
     const int tl = lin / kMxRowChunks, pc = lin - tl * kMxRowChunks;
     const int lc = (pc & ~7) | ((pc & 7) ^ ((tl >> 1) & 7));
-    const int bs = lc / kMx3ChunksPerBlock;
     const int tlc = min(tl, mcount - 1);  // tokens past the tile re-read its last one
     const int row = a.list_row ? a.list_row[base + tlc] : base + tlc;
-    arow[c] = a.A + (size_t)row * nblk * kMx3ChunksPerBlock + (lc - bs * kMx3ChunksPerBlock);
-    ablk[c] = bs;
+    aoff[c] = (uint32_t)(((size_t)row * rowblk * kMx3ChunksPerBlock + lc) * 16);
   }
+  // LDS destination of copy c of this wave within a stage (wave-uniform)
+  const uint32_t lds_wave = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(kMxCopies * wv * 64 * 16);
   struct BSet {
     u32x4 q[2][2];     // [64-wide K chunk of the step][row group]
     uint32_t s[2][2];  // byte 0 = the block's scale byte (the matrix instruction reads only that byte)
@@ -129,30 +138,28 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
   // The kStepLoads load instructions of step j, one at a time: n < kMxCopies copies a part
   // of the activation tile into LDS, the next four fetch the weight entries, the last four
   // the scale bytes.
+  // All loads are inline assembly in the scalar-base form.  Besides saving the address
+  // arithmetic this keeps them out of the compiler's wait tracking, which otherwise drains
+  // the whole queue once per loop iteration over a register it reuses; the explicit count at
+  // the step boundary is what guarantees their arrival.
   auto issue_load = [&](int n, int stage, BSet& b, int j) {
     if (n < kMxCopies) {
-      const int c = n;
-      const int kb = min(4 * j + ablk[c], nblk - 1);  // a block past K re-reads the last one (its weights are zeroed)
-      __builtin_amdgcn_global_load_lds(
-          arow[c] + (size_t)kb * kMx3ChunksPerBlock,
-          reinterpret_cast<__attribute__((address_space(3))) uint4*>(
-              reinterpret_cast<uintptr_t>(As + stage * kMxStageChunks + (kMxCopies * wv + c) * 64)),
-          16, 0, 0);
+      const char* abase = reinterpret_cast<const char*>(a.A) + (size_t)j * (4 * kMx3ChunksPerBlock * 16);
+      const uint32_t lds = lds_wave + (uint32_t)((stage * kMxStageChunks + n * 64) * 16);
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :
+                   : "v"(aoff[n]), "s"(abase), "s"(lds)
+                   : "memory");
     } else {
       const int m = (n - kMxCopies) & 3, kc = m >> 1, s = m & 1;
-      const int kb = min(4 * j + 2 * kc + kg, nblk - 1);
-      // Issued as inline assembly: the compiler's wait insertion does not see these as
-      // pending register writes, so it adds no waits of its own for them (it otherwise
-      // drains the whole queue once per loop iteration over a register it reuses); the
-      // explicit count at the step boundary is what guarantees their arrival.
       if (n < kMxCopies + 4) {
-        const CSK_GLOBAL u32x4* ptr = qp[s] + kb * 16;
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(b.q[kc][s]) : "v"(ptr) : "memory");
+        const char* base_q = qbase[s] + (size_t)j * 1024 + kc * 512;
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(b.q[kc][s]) : "v"(qoff[s]), "s"(base_q) : "memory");
       } else {
         // a dword load at the byte's own (unaligned) address: the matrix instruction reads
         // only byte 0 of its scale operand, so no widening instruction is needed
-        const CSK_GLOBAL uint8_t* ptr = sp[s] + scale_index(0, kb, 0, slots);
-        asm volatile("global_load_dword %0, %1, off" : "=v"(b.s[kc][s]) : "v"(ptr) : "memory");
+        const char* base_s = sbase[s] + (size_t)((j & 3) * 64 + 32 * kc) * slots + (j >> 2);
+        asm volatile("global_load_dword %0, %1, %2" : "=v"(b.s[kc][s]) : "v"(soff[s]), "s"(base_s) : "memory");
       }
     }
   };
@@ -187,14 +194,10 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
     const u32x4* at = reinterpret_cast<const u32x4*>(As) + stage * kMxStageChunks;
     i32x8 bw[2][2];
 #pragma unroll
-    for (int kc = 0; kc < 2; ++kc) {
-      const bool kv = 4 * j + 2 * kc + kg < nblk;
+    for (int kc = 0; kc < 2; ++kc)
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const u32x4 q = kv ? b.q[kc][s] : u32x4{0u, 0u, 0u, 0u};
-        bw[kc][s] = (i32x8)__builtin_shufflevector(q, q, 0, 1, 2, 3, -1, -1, -1, -1);  // FP4 reads four registers
-      }
-    }
+      for (int s = 0; s < 2; ++s)  // FP4 reads four registers
+        bw[kc][s] = (i32x8)__builtin_shufflevector(b.q[kc][s], b.q[kc][s], 0, 1, 2, 3, -1, -1, -1, -1);
     u32x4 flo[3], fhi[3];
     auto read_frag = [&](int i) {
       const int kc = i / 6, t = (i % 6) >> 1, ms = i & 1;
@@ -285,19 +288,22 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int tl = ms * 32 + (r & 3) + 8 * (r >> 2) + 4 * kg;
-        stage[(tl * kMxWaves + wv) * 33 + n32] = moe_activation(acc[ms][0][r] + bg, acc[ms][1][r] + bu, a.act_type);
+        // features past N belong to the zero padding of the output rows
+        stage[(tl * kMxWaves + wv) * 33 + n32] =
+            rv ? moe_activation(acc[ms][0][r] + bg, acc[ms][1][r] + bu, a.act_type) : 0.0f;
       }
     }
     __syncthreads();
     const int tl = threadIdx.x / kMxWaves, blk = threadIdx.x % kMxWaves;
     const int kb = nt * kMxWaves + blk;
-    if (tl < mcount && kb * 32 < a.N) {
+    const int out_rowblk = mx3_row_blocks(a.N >> 5);  // the down GEMM reads rows padded to whole steps
+    if (tl < mcount && kb < out_rowblk) {
       float v[32];
 #pragma unroll
       for (int i = 0; i < 32; ++i) v[i] = stage[(tl * kMxWaves + blk) * 33 + i];
       u32x4 out[kMx3ChunksPerBlock];
       mx3_quantize_block(v, out);
-      u32x4* o = a.act_out + ((size_t)(base + tl) * (a.N >> 5) + kb) * kMx3ChunksPerBlock;
+      u32x4* o = a.act_out + ((size_t)(base + tl) * out_rowblk + kb) * kMx3ChunksPerBlock;
 #pragma unroll
       for (int c = 0; c < kMx3ChunksPerBlock; ++c) o[c] = out[c];
     }

@@ -25,6 +25,10 @@ namespace csk {
 constexpr int kMx3Terms = 3;
 constexpr int kMx3ChunksPerBlock = 2 * kMx3Terms;  // 16-byte chunks per 32-value block
 
+// Rows are padded with all-zero blocks (codes 0, scale byte 127) to a whole number of the
+// GEMM's four-block K steps, so that the GEMM never has to clamp or mask at the end of K.
+__host__ __device__ inline int mx3_row_blocks(int nblk) { return (nblk + 3) & ~3; }
+
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x32 __attribute__((ext_vector_type(32)));
 typedef uint32_t u32x6 __attribute__((ext_vector_type(6)));
@@ -60,33 +64,42 @@ __device__ __forceinline__ void mx3_quantize_block(float (&r)[32], u32x4 (&out)[
   }
 }
 
-// rows of fp32 -> three-term FP6 blocks, one thread per block:
-//   x3[(row * nblk + kb) * 6 + c] <- quantise(x[src(row)][32 kb .. 32 kb + 31] * w(row))
+// rows of fp32 -> three-term FP6 blocks, one thread per block (padding blocks included):
+//   x3[(row * mx3_row_blocks(nblk) + kb) * 6 + c] <- quantise(x[src(row)][32 kb .. 32 kb + 31] * w(row))
 // src(row) = gather_tok[row] and w(row) = gather_w[row] when given (rows gathered and
 // pre-scaled per dispatch position, expert_mlp_node.h:515-522), else row and 1.
 __global__ __launch_bounds__(256) void mx3_rows_kernel(const float* __restrict__ x,
                                                        u32x4* __restrict__ x3, long rows, int nblk,
                                                        const int* __restrict__ gather_tok,
                                                        const float* __restrict__ gather_w) {
+  const int rowblk = mx3_row_blocks(nblk);
   const long b = (long)blockIdx.x * 256 + threadIdx.x;
-  if (b >= rows * nblk) return;
-  const long row = b / nblk;
-  const int kb = (int)(b - row * nblk);
-  const long srow = gather_tok ? gather_tok[row] : row;
-  const float gw = gather_w ? gather_w[row] : 1.0f;
-  float r[32];
-  const float4* src = reinterpret_cast<const float4*>(x + (srow * nblk + kb) * 32);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float4 v = src[i];
-    r[4 * i] = v.x, r[4 * i + 1] = v.y, r[4 * i + 2] = v.z, r[4 * i + 3] = v.w;
-  }
-  if (gather_w) {
-#pragma unroll
-    for (int i = 0; i < 32; ++i) r[i] = r[i] * gw;
-  }
+  if (b >= rows * rowblk) return;
+  const long row = b / rowblk;
+  const int kb = (int)(b - row * rowblk);
   u32x4 out[kMx3ChunksPerBlock];
-  mx3_quantize_block(r, out);
+  if (kb >= nblk) {
+#pragma unroll
+    for (int t = 0; t < kMx3Terms; ++t) {
+      out[2 * t] = u32x4{0u, 0u, 0u, 0u};
+      out[2 * t + 1] = u32x4{0u, 0u, 127u, 0u};
+    }
+  } else {
+    const long srow = gather_tok ? gather_tok[row] : row;
+    const float gw = gather_w ? gather_w[row] : 1.0f;
+    float r[32];
+    const float4* src = reinterpret_cast<const float4*>(x + (srow * nblk + kb) * 32);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float4 v = src[i];
+      r[4 * i] = v.x, r[4 * i + 1] = v.y, r[4 * i + 2] = v.z, r[4 * i + 3] = v.w;
+    }
+    if (gather_w) {
+#pragma unroll
+      for (int i = 0; i < 32; ++i) r[i] = r[i] * gw;
+    }
+    mx3_quantize_block(r, out);
+  }
 #pragma unroll
   for (int c = 0; c < kMx3ChunksPerBlock; ++c) x3[b * kMx3ChunksPerBlock + c] = out[c];
 }
