@@ -783,7 +783,7 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
         L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
     if ((rc = check_launch("router_prep_logits_kernel")) != CSK_OK) return rc;
     mark(CSK_STAGE_DISPATCH);
-    route_small_kernel<<<dim3(1), 512, 0, g_stream>>>(
+    route_small_kernel<<<dim3(1), kRouteSmallThreads, 0, g_stream>>>(
         ws.logits, ws.pairs, ws.ids, (int)T, (int)L->E, (int)L->k, L->sigmoid, L->ew_dev, ws.counts,
         ws.offsets, ws.desc, ws.vlist, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w, ws.pos,
         xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, (int)L->H);
