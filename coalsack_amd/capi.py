@@ -40,7 +40,13 @@ SIGNATURES = {
     "csk_mxfp4_free": (None, [_P]),
     "csk_mxfp4_dequant": (C.c_int, [_P, _P]),
     "csk_mxfp4_export": (C.c_int, [_P, _P]),
+    "csk_f16_upload": (C.c_int, [_P, _I64, _I64, C.POINTER(_P)]),
+    "csk_f16_free": (None, [_P]),
+    "csk_f16_export": (C.c_int, [_P, _P]),
     "csk_layer_create": (C.c_int, [_I64, _I64, _I64, _I64, C.POINTER(_P)]),
+    "csk_layer_create_f16": (C.c_int, [_I64, _I64, _I64, _I64, C.POINTER(_P)]),
+    "csk_layer_set_expert_f16": (C.c_int, [_P, _I64, _P, _P, _P, _P, _P, _P]),
+    "csk_layer_export_f16": (C.c_int, [_P, _I64, C.c_int, _P]),
     "csk_layer_destroy": (None, [_P]),
     "csk_layer_set_options": (C.c_int, [_P, C.c_int, C.c_int, C.c_int]),
     "csk_layer_set_router": (C.c_int, [_P, _P, _P]),
@@ -67,6 +73,8 @@ SIGNATURES = {
     "csk_moe_router_logits": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _P]),
     "csk_expert_mlp_mxfp4": (C.c_int, [C.c_int, _P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P,
                                        _I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]),
+    "csk_expert_mlp_f16": (C.c_int, [C.c_int, _P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P,
+                                     _I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]),
     "csk_expert_token_mxfp4": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, C.c_int]),
     "csk_expert_merge": (C.c_int, [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]),
     "csk_rmsnorm": (C.c_int, [_P, _P, _P, _I64, _I64, C.c_float]),
@@ -204,6 +212,44 @@ class Library:
         self.check(self.dll.csk_mxfp4_export(h, _ptr(out)))
         return out
 
+    # -- fp16 matrices
+    def f16_upload(self, w):
+        """w: float16 [rows, K], row-major."""
+        w = np.ascontiguousarray(w, dtype=np.float16)
+        rows, K = w.shape
+        h = _P()
+        self.check(self.dll.csk_f16_upload(_ptr(w), rows, K, C.byref(h)))
+        return h
+
+    def f16_free(self, h):
+        self.dll.csk_f16_free(h)
+
+    def f16_export(self, h, rows, K):
+        out = np.empty((rows, K), np.float16)
+        self.check(self.dll.csk_f16_export(h, _ptr(out)))
+        return out
+
+    def expert_mlp_f16(self, expert_id, hidden, w_up, w_gate, w_down, b_up, b_gate, b_down, pairs,
+                       act=ACT_MODIFIED_SWIGLU, weight_before_ffn=False):
+        """w_*: float16 arrays [F,H], [F,H], [H,F]; uploads them, runs the node, frees them."""
+        hidden, pairs = _f32(hidden), _f32(pairs)
+        b_up, b_gate, b_down = _f32(b_up), _f32(b_gate), _f32(b_down)
+        T, H = hidden.shape
+        F = w_up.shape[0]
+        k = pairs.shape[1]
+        hs = [self.f16_upload(w) for w in (w_up, w_gate, w_down)]
+        try:
+            out = np.empty((T, H), np.float32)
+            empty = C.c_int()
+            self.check(self.dll.csk_expert_mlp_f16(
+                expert_id, _ptr(hidden), T, H, F, hs[0], hs[1], hs[2], _ptr(b_up), _ptr(b_gate),
+                _ptr(b_down), _ptr(pairs), k, act, int(weight_before_ffn), _ptr(out),
+                C.byref(empty)))
+        finally:
+            for h in hs:
+                self.f16_free(h)
+        return None if empty.value else out
+
     # -- node-level ops
     def moe_router(self, hidden, gate_w, gate_b, k, sigmoid=False):
         hidden, gate_w, gate_b = _f32(hidden), _f32(gate_w), _f32(gate_b)
@@ -272,8 +318,8 @@ class Library:
         return out
 
     # -- layer
-    def layer(self, E, k, H, F):
-        return Layer(self, E, k, H, F)
+    def layer(self, E, k, H, F, f16=False):
+        return Layer(self, E, k, H, F, f16=f16)
 
     def gguf(self, path):
         return Gguf(self, path)
@@ -339,16 +385,17 @@ class Gguf:
 class Layer:
     """One resident MoE layer (csk_layer_*)."""
 
-    def __init__(self, lib, E, k, H, F):
-        self.lib, self.E, self.k, self.H, self.F = lib, E, k, H, F
+    def __init__(self, lib, E, k, H, F, f16=False):
+        self.lib, self.E, self.k, self.H, self.F, self.f16 = lib, E, k, H, F, f16
         self.h = _P()
-        lib.check(lib.dll.csk_layer_create(E, k, H, F, C.byref(self.h)))
+        create = lib.dll.csk_layer_create_f16 if f16 else lib.dll.csk_layer_create
+        lib.check(create(E, k, H, F, C.byref(self.h)))
 
     @classmethod
-    def adopt(cls, lib, handle, E, k, H, F):
+    def adopt(cls, lib, handle, E, k, H, F, f16=False):
         """Wraps a layer handle the library created itself."""
         self = cls.__new__(cls)
-        self.lib, self.E, self.k, self.H, self.F, self.h = lib, E, k, H, F, handle
+        self.lib, self.E, self.k, self.H, self.F, self.h, self.f16 = lib, E, k, H, F, handle, f16
         return self
 
     def close(self):
@@ -377,6 +424,24 @@ class Layer:
         self.lib.check(self.lib.dll.csk_layer_set_expert(
             self.h, e, _ptr(w_up), _ptr(w_gate), _ptr(w_down), _ptr(b_up), _ptr(b_gate),
             _ptr(b_down)))
+
+    def set_expert_f16(self, e, w_up, w_gate, w_down, b_up=None, b_gate=None, b_down=None):
+        """w_*: float16 arrays [F,H], [F,H], [H,F]."""
+        if w_up is not None:
+            w_up, w_gate, w_down = (np.ascontiguousarray(w, dtype=np.float16)
+                                    for w in (w_up, w_gate, w_down))
+            assert w_up.shape == (self.F, self.H) and w_gate.shape == (self.F, self.H)
+            assert w_down.shape == (self.H, self.F)
+        b_up, b_gate, b_down = _f32(b_up), _f32(b_gate), _f32(b_down)
+        self.lib.check(self.lib.dll.csk_layer_set_expert_f16(
+            self.h, e, _ptr(w_up), _ptr(w_gate), _ptr(w_down), _ptr(b_up), _ptr(b_gate),
+            _ptr(b_down)))
+
+    def export_f16(self, e, which):
+        rows, K = (self.H, self.F) if which == W_DOWN else (self.F, self.H)
+        out = np.empty((rows, K), np.float16)
+        self.lib.check(self.lib.dll.csk_layer_export_f16(self.h, e, which, _ptr(out)))
+        return out
 
     def set_norm(self, w, eps):
         w = _f32(w)

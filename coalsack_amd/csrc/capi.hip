@@ -13,6 +13,7 @@
 #include "common.h"
 #include "expert_stream_kernel.h"
 #include "expert_prefill_kernel.h"
+#include "expert_f16_kernel.h"
 #include "mxfp4_kernels.h"
 #include "router_kernels.h"
 
@@ -136,6 +137,16 @@ struct Workspace {
   }
 };
 Workspace g_ws;
+
+// extra buffers of the fp16 expert path
+struct F16Scratch {
+  size_t rows = 0, width = 0;
+  float* actf = nullptr;  // [P, F] activations before they are split
+  float* rs_x = nullptr;  // scale per input row
+  float* rs_a = nullptr;  // scale per activation row
+  int ensure(size_t rows_, size_t width_);
+};
+F16Scratch g_f16;
 float* g_zero = nullptr;  // zero vector standing in for absent biases
 constexpr size_t kZeroLen = 1 << 16;
 
@@ -171,6 +182,15 @@ struct csk_layer {
   bool has_gate = false, has_gate_b = false;
   uint4* q_all = nullptr;    // [E][gate | up | down] entries
   uint8_t* s_all = nullptr;
+  bool f16 = false;          // fp16 experts: h_all holds [E][gate | up | down] tiles instead
+  u32x4* h_all = nullptr;
+  long ent16_gu() const { return f16_entries(F, H); }
+  long ent16_d() const { return f16_entries(H, F); }
+  long ent16_expert() const { return 2 * ent16_gu() + ent16_d(); }
+  u32x4* view16(int64_t e, int which) const {
+    return h_all + (long)e * ent16_expert() +
+           (which == CSK_W_GATE ? 0 : (which == CSK_W_UP ? ent16_gu() : 2 * ent16_gu()));
+  }
   float* bias_all = nullptr;  // [E][F gate | F up | H down]
   ExpertW* ew_dev = nullptr;
   std::vector<ExpertW> ew_host;
@@ -404,6 +424,78 @@ int launch_combine(const float* y, const float* pairs, const int* pos, const flo
   return check_launch("combine_kernel");
 }
 
+int F16Scratch::ensure(size_t rows_, size_t width_) {
+  if (rows_ <= rows && width_ <= width) return CSK_OK;
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  const size_t nr = std::max(rows, rows_), nw = std::max(width, width_);
+  for (void* p : {(void*)actf, (void*)rs_x, (void*)rs_a})
+    if (p) (void)hipFree(p);
+  actf = nullptr, rs_x = nullptr, rs_a = nullptr, rows = 0, width = 0;
+  int rc = dev_alloc(&actf, nr * nw);
+  if (rc == CSK_OK) rc = dev_alloc(&rs_x, nr);
+  if (rc == CSK_OK) rc = dev_alloc(&rs_a, nr);
+  if (rc != CSK_OK) return rc;
+  rows = nr, width = nw;
+  return CSK_OK;
+}
+
+int launch_f16_split(const float* x, int64_t rows, int64_t K, const int* gather_tok,
+                     const float* gather_w, uint16_t* out, float* rscale) {
+  if (rows == 0) return CSK_OK;
+  f16_split_rows_kernel<<<dim3((unsigned)rows), 256, 0, g_stream>>>(
+      x, (long)K, gather_tok, gather_w, reinterpret_cast<u32x4*>(out), rscale);
+  return check_launch("f16_split_rows_kernel");
+}
+
+// Experts with fp16 weights over the dispatched tokens: ws.y[P,H] <- down(act(gate, up)).
+// x is [T,H] fp32.  Up to 64 tokens every expert's tokens form groups of 16 (one pass over
+// the weights per group, HBM-bound); beyond that groups of 64.
+int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int act_type,
+                    const float* x, bool weight_before_ffn, int64_t gather_rows, Workspace& ws,
+                    bool timed = false) {
+  const int64_t P = T * k;
+  int rc = g_f16.ensure((size_t)P, (size_t)F);
+  if (rc != CSK_OK) return rc;
+  ExpertF16Args a{};
+  a.desc = ws.desc;
+  a.n_slots = (int)E;
+  a.act_type = act_type;
+  if (weight_before_ffn) {
+    // rows gathered per dispatch position and scaled by the routing weight first
+    rc = launch_f16_split(x, gather_rows, H, ws.list_tok, ws.list_w, ws.xg, g_f16.rs_x);
+    a.list_row = nullptr;
+    a.B = reinterpret_cast<const u32x4*>(ws.xg);
+  } else {
+    rc = launch_f16_split(x, T, H, nullptr, nullptr, ws.xs, g_f16.rs_x);
+    a.list_row = ws.list_tok;
+    a.B = reinterpret_cast<const u32x4*>(ws.xs);
+  }
+  if (rc != CSK_OK) return rc;
+  const bool small = T <= 64;
+  const dim3 grid((unsigned)(4 * std::max(g_cus, 1)));
+  a.rscale = g_f16.rs_x;
+  a.nkb = (int)f16_block_count(H);
+  a.N = (int)F;
+  a.ntile = (int)f16_tile_count(F);
+  a.out = g_f16.actf;
+  if (timed) mark(CSK_STAGE_GATEUP);
+  if (small) expert_f16_kernel<0, 1><<<grid, 256, 0, g_stream>>>(a);
+  else expert_f16_kernel<0, 4><<<grid, 256, 0, g_stream>>>(a);
+  if ((rc = check_launch("expert_f16_kernel<0>")) != CSK_OK) return rc;
+  if (timed) mark(CSK_STAGE_DOWN);
+  if ((rc = launch_f16_split(g_f16.actf, P, F, nullptr, nullptr, ws.act, g_f16.rs_a)) != CSK_OK) return rc;
+  a.list_row = nullptr;
+  a.B = reinterpret_cast<const u32x4*>(ws.act);
+  a.rscale = g_f16.rs_a;
+  a.nkb = (int)f16_block_count(F);
+  a.N = (int)H;
+  a.ntile = (int)f16_tile_count(H);
+  a.out = ws.y;
+  if (small) expert_f16_kernel<1, 1><<<grid, 256, 0, g_stream>>>(a);
+  else expert_f16_kernel<1, 4><<<grid, 256, 0, g_stream>>>(a);
+  return check_launch("expert_f16_kernel<1>");
+}
+
 int check_dims(int64_t E, int64_t k, int64_t H, int64_t F) {
   if (E <= 0 || E > kMaxExperts) return fail(CSK_ERR_ARG, "num_experts must be in 1..256");
   if (k <= 0 || k > kMaxTopK || k > E) return fail(CSK_ERR_ARG, "top_k must be in 1..min(16, E)");
@@ -588,13 +680,14 @@ extern "C" int csk_mxfp4_export(const csk_mxfp4* m, uint8_t* host_out) {
 
 // ============================================================ layer
 
-extern "C" int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_layer** out) {
+static int layer_create(int64_t E, int64_t k, int64_t H, int64_t F, bool f16, csk_layer** out) {
   REQUIRE_INIT();
   if (!out) return fail(CSK_ERR_ARG, "csk_layer_create: null out");
   int rc = check_dims(E, k, H, F);
   if (rc != CSK_OK) return rc;
   csk_layer* L = new csk_layer;
   L->E = E, L->k = k, L->H = H, L->F = F;
+  L->f16 = f16;
   L->nblkH = H / 32, L->nblkF = F / 32, L->ntF = cdiv(F, 16), L->ntH = cdiv(H, 16);
   L->expert_set.assign((size_t)E, 0);
   L->expert_bias.assign((size_t)E, 0);
@@ -603,9 +696,13 @@ extern "C" int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_
   if (rc == CSK_OK) rc = dev_alloc(&L->gate_b, (size_t)E);
   // kWeightSlack: the grouped GEMM reads up to three blocks (and the scale loads three
   // bytes) past the end of a plane; behind the last plane that must still be mapped memory
-  if (rc == CSK_OK) rc = dev_alloc(&L->q_all, (size_t)E * L->ent_expert() + kWeightSlack / sizeof(uint4));
-  if (rc == CSK_OK) rc = dev_alloc(&L->s_all, (size_t)E * L->sc_expert() + kWeightSlack);
-  if (rc == CSK_OK && hipMemset(L->s_all, 127, (size_t)E * L->sc_expert()) != hipSuccess) rc = fail(CSK_ERR_HIP, "hipMemset failed");
+  if (f16) {
+    if (rc == CSK_OK) rc = dev_alloc(&L->h_all, (size_t)E * L->ent16_expert());
+  } else {
+    if (rc == CSK_OK) rc = dev_alloc(&L->q_all, (size_t)E * L->ent_expert() + kWeightSlack / sizeof(uint4));
+    if (rc == CSK_OK) rc = dev_alloc(&L->s_all, (size_t)E * L->sc_expert() + kWeightSlack);
+    if (rc == CSK_OK && hipMemset(L->s_all, 127, (size_t)E * L->sc_expert()) != hipSuccess) rc = fail(CSK_ERR_HIP, "hipMemset failed");
+  }
   if (rc == CSK_OK) rc = dev_alloc(&L->bias_all, (size_t)E * (2 * F + H));
   if (rc == CSK_OK) rc = dev_alloc(&L->ew_dev, (size_t)E);
   if (rc == CSK_OK) rc = dev_alloc(&L->norm_w, (size_t)H);
@@ -615,8 +712,15 @@ extern "C" int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_
   }
   for (int64_t e = 0; e < E; ++e) {
     ExpertW& w = L->ew_host[(size_t)e];
-    const csk_mxfp4 g = L->view(e, CSK_W_GATE), u = L->view(e, CSK_W_UP), d = L->view(e, CSK_W_DOWN);
-    w.q_gate = g.q, w.s_gate = g.s, w.q_up = u.q, w.s_up = u.s, w.q_down = d.q, w.s_down = d.s;
+    if (f16) {
+      w.q_gate = reinterpret_cast<const uint4*>(L->view16(e, CSK_W_GATE));
+      w.q_up = reinterpret_cast<const uint4*>(L->view16(e, CSK_W_UP));
+      w.q_down = reinterpret_cast<const uint4*>(L->view16(e, CSK_W_DOWN));
+      w.s_gate = w.s_up = w.s_down = nullptr;
+    } else {
+      const csk_mxfp4 g = L->view(e, CSK_W_GATE), u = L->view(e, CSK_W_UP), d = L->view(e, CSK_W_DOWN);
+      w.q_gate = g.q, w.s_gate = g.s, w.q_up = u.q, w.s_up = u.s, w.q_down = d.q, w.s_down = d.s;
+    }
     w.b_gate = w.b_up = w.b_down = g_zero;
   }
   hipError_t e1 = hipMemcpy(L->ew_dev, L->ew_host.data(), (size_t)E * sizeof(ExpertW), hipMemcpyHostToDevice);
@@ -628,10 +732,17 @@ extern "C" int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_
   return CSK_OK;
 }
 
+extern "C" int csk_layer_create(int64_t E, int64_t k, int64_t H, int64_t F, csk_layer** out) {
+  return layer_create(E, k, H, F, false, out);
+}
+extern "C" int csk_layer_create_f16(int64_t E, int64_t k, int64_t H, int64_t F, csk_layer** out) {
+  return layer_create(E, k, H, F, true, out);
+}
+
 extern "C" void csk_layer_destroy(csk_layer* L) {
   if (!L) return;
   if (g_stream) (void)hipStreamSynchronize(g_stream);
-  void* ps[] = {L->gate_w, L->gate_b, L->q_all, L->s_all, L->bias_all, L->ew_dev, L->norm_w};
+  void* ps[] = {L->gate_w, L->gate_b, L->q_all, L->s_all, L->h_all, L->bias_all, L->ew_dev, L->norm_w};
   for (void* p : ps)
     if (p) (void)hipFree(p);
   delete L;
@@ -685,6 +796,7 @@ extern "C" int csk_layer_set_expert(csk_layer* L, int64_t e, const uint8_t* w_up
                                     const float* b_up, const float* b_gate, const float* b_down) {
   REQUIRE_INIT();
   if (!L || e < 0 || e >= L->E) return fail(CSK_ERR_RANGE, "csk_layer_set_expert: expert index out of range");
+  if (L->f16 && w_up) return fail(CSK_ERR_STATE, "csk_layer_set_expert: this layer holds fp16 experts (csk_layer_set_expert_f16)");
   if ((w_up == nullptr) != (w_gate == nullptr) || (w_up == nullptr) != (w_down == nullptr))
     return fail(CSK_ERR_ARG, "weights must be all present or all absent");
   if (w_up) {
@@ -716,6 +828,23 @@ extern "C" int csk_layer_fill_synthetic(csk_layer* L, uint64_t seed, int64_t lay
   if (!L) return fail(CSK_ERR_ARG, "null layer");
   if (scale_lo < 2 || scale_span < 1 || scale_lo + scale_span - 1 > 254)
     return fail(CSK_ERR_SCALE, "synthetic scale bytes must stay within 2..254");
+  if (L->f16) {
+    // halves j / 2^14 with j uniform in [-2048, 2047] (exact in fp16), zero in the padding
+    for (int64_t e = 0; e < L->E; ++e) {
+      for (int which = 0; which < 3; ++which) {
+        const bool down = which == CSK_W_DOWN;
+        const long rows = down ? L->H : L->F, K = down ? L->F : L->H, ent = f16_entries(rows, K);
+        synth_f16_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(
+            L->view16(e, which), rows, K, ent,
+            seed ^ ((uint64_t)layer_index * 1000003ull + (uint64_t)e * 16ull + (uint64_t)which) * 0x9E3779B97F4A7C15ull);
+      }
+      L->expert_set[(size_t)e] = 1;
+    }
+    int rc = check_launch("synth_f16_kernel");
+    if (rc != CSK_OK) return rc;
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return CSK_OK;
+  }
   for (int64_t e = 0; e < L->E; ++e) {
     for (int which = 0; which < 3; ++which) {
       const csk_mxfp4 m = L->view(e, which);
@@ -743,13 +872,112 @@ extern "C" int csk_layer_dequant(const csk_layer* L, int64_t e, int which, float
   REQUIRE_INIT();
   if (!L || !host_out || e < 0 || e >= L->E || which < 0 || which > 2)
     return fail(CSK_ERR_ARG, "csk_layer_dequant: bad argument");
+  if (L->f16) return fail(CSK_ERR_STATE, "csk_layer_dequant: this layer holds fp16 experts (csk_layer_export_f16)");
   return dequant_to_host(L->view(e, which), host_out);
 }
 extern "C" int csk_layer_export(const csk_layer* L, int64_t e, int which, uint8_t* host_out) {
   REQUIRE_INIT();
   if (!L || !host_out || e < 0 || e >= L->E || which < 0 || which > 2)
     return fail(CSK_ERR_ARG, "csk_layer_export: bad argument");
+  if (L->f16) return fail(CSK_ERR_STATE, "csk_layer_export: this layer holds fp16 experts (csk_layer_export_f16)");
   return export_to_host(L->view(e, which), host_out);
+}
+
+// ------------------------------------------------------------ fp16 matrices
+
+struct csk_f16 {
+  u32x4* w = nullptr;
+  int64_t rows = 0, K = 0;
+};
+
+namespace {
+// row-major halves on the host -> tiles at dst
+int f16_pack_into(const uint16_t* halves, int64_t rows, int64_t K, u32x4* dst) {
+  uint16_t* stage = nullptr;
+  const size_t n = (size_t)rows * K;
+  HIP_TRY(hipMalloc((void**)&stage, n * sizeof(uint16_t)));
+  hipError_t e = hipMemcpyAsync(stage, halves, n * sizeof(uint16_t), hipMemcpyHostToDevice, g_stream);
+  int rc = CSK_OK;
+  if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("hipMemcpy: ") + hipGetErrorString(e));
+  if (rc == CSK_OK) {
+    const long ent = f16_entries(rows, K);
+    f16_pack_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(stage, dst, rows, K, ent);
+    rc = check_launch("f16_pack_kernel");
+  }
+  (void)hipStreamSynchronize(g_stream);
+  (void)hipFree(stage);
+  return rc;
+}
+int f16_export_from(const u32x4* src, int64_t rows, int64_t K, uint16_t* halves) {
+  uint16_t* stage = nullptr;
+  const size_t n = (size_t)rows * K;
+  HIP_TRY(hipMalloc((void**)&stage, n * sizeof(uint16_t)));
+  const long ent = f16_entries(rows, K);
+  f16_unpack_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(src, stage, rows, K, ent);
+  int rc = check_launch("f16_unpack_kernel");
+  if (rc == CSK_OK) {
+    hipError_t e = hipMemcpyAsync(halves, stage, n * sizeof(uint16_t), hipMemcpyDeviceToHost, g_stream);
+    if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("hipMemcpy: ") + hipGetErrorString(e));
+  }
+  (void)hipStreamSynchronize(g_stream);
+  (void)hipFree(stage);
+  return rc;
+}
+}  // namespace
+
+extern "C" int csk_f16_upload(const uint16_t* halves, int64_t rows, int64_t K, csk_f16** out) {
+  REQUIRE_INIT();
+  if (!halves || !out || rows <= 0 || K <= 0)
+    return fail(CSK_ERR_ARG, "csk_f16_upload: need a matrix with rows > 0 and K > 0");
+  if (rows > (int64_t)kZeroLen || K > (int64_t)kZeroLen)
+    return fail(CSK_ERR_ARG, "csk_f16_upload: dimensions above 65536 are not supported");
+  csk_f16* m = new csk_f16;
+  m->rows = rows, m->K = K;
+  int rc = dev_alloc(&m->w, (size_t)f16_entries(rows, K));
+  if (rc == CSK_OK) rc = f16_pack_into(halves, rows, K, m->w);
+  if (rc != CSK_OK) {
+    csk_f16_free(m);
+    return rc;
+  }
+  *out = m;
+  return CSK_OK;
+}
+extern "C" void csk_f16_free(csk_f16* m) {
+  if (!m) return;
+  if (m->w) (void)hipFree(m->w);
+  delete m;
+}
+extern "C" int csk_f16_export(const csk_f16* m, uint16_t* halves_out) {
+  REQUIRE_INIT();
+  if (!m || !halves_out) return fail(CSK_ERR_ARG, "csk_f16_export: null argument");
+  return f16_export_from(m->w, m->rows, m->K, halves_out);
+}
+
+extern "C" int csk_layer_set_expert_f16(csk_layer* L, int64_t e, const uint16_t* w_up,
+                                        const uint16_t* w_gate, const uint16_t* w_down,
+                                        const float* b_up, const float* b_gate,
+                                        const float* b_down) {
+  REQUIRE_INIT();
+  if (!L || e < 0 || e >= L->E) return fail(CSK_ERR_RANGE, "csk_layer_set_expert_f16: expert index out of range");
+  if (!L->f16) return fail(CSK_ERR_STATE, "csk_layer_set_expert_f16: this layer holds MXFP4 experts (csk_layer_create_f16 makes an fp16 one)");
+  if ((w_up == nullptr) != (w_gate == nullptr) || (w_up == nullptr) != (w_down == nullptr))
+    return fail(CSK_ERR_ARG, "weights must be all present or all absent");
+  if (w_up) {
+    int rc = f16_pack_into(w_up, L->F, L->H, L->view16(e, CSK_W_UP));
+    if (rc == CSK_OK) rc = f16_pack_into(w_gate, L->F, L->H, L->view16(e, CSK_W_GATE));
+    if (rc == CSK_OK) rc = f16_pack_into(w_down, L->H, L->F, L->view16(e, CSK_W_DOWN));
+    if (rc != CSK_OK) return rc;
+    L->expert_set[(size_t)e] = 1;
+  }
+  return upload_biases(L, e, b_up, b_gate, b_down);
+}
+extern "C" int csk_layer_export_f16(const csk_layer* L, int64_t e, int which, uint16_t* halves_out) {
+  REQUIRE_INIT();
+  if (!L || !halves_out || e < 0 || e >= L->E || which < 0 || which > 2)
+    return fail(CSK_ERR_ARG, "csk_layer_export_f16: bad argument");
+  if (!L->f16) return fail(CSK_ERR_STATE, "csk_layer_export_f16: this layer holds MXFP4 experts");
+  const bool down = which == CSK_W_DOWN;
+  return f16_export_from(L->view16(e, which), down ? L->H : L->F, down ? L->F : L->H, halves_out);
 }
 
 static int layer_ready(const csk_layer* L, int flags) {
@@ -788,19 +1016,19 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
         ws.offsets, ws.desc, ws.vlist, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w, ws.pos,
         xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, (int)L->H);
     if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
-    if (!stream_path(T, L->H, L->F) && !L->wbf) {
+    if (!L->f16 && !stream_path(T, L->H, L->F) && !L->wbf) {
       // few tokens but rows too long for the streaming kernel: the GEMM wants the FP6 form
       if ((rc = launch_mx3(xr, ws.xs, T, L->H, nullptr, nullptr)) != CSK_OK) return rc;
     }
   } else {
     mark(CSK_STAGE_PREP);
-    const bool stream = stream_path(T, L->H, L->F);
+    const bool stream = !L->f16 && stream_path(T, L->H, L->F);
     if (norm || stream) {
       rc = launch_prep(hidden, norm ? L->norm_w : nullptr, L->eps, norm ? ws.xn : nullptr,
                        stream ? ws.xs : nullptr, T, L->H, nullptr, nullptr);
       if (rc != CSK_OK) return rc;
     }
-    if (!stream && !L->wbf) {
+    if (!L->f16 && !stream && !L->wbf) {
       rc = launch_mx3(xr, ws.xs, T, L->H, nullptr, nullptr);
       if (rc != CSK_OK) return rc;
     }
@@ -811,6 +1039,16 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
     mark(CSK_STAGE_DISPATCH);
     rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, L->ew_dev, ws);
     if (rc != CSK_OK) return rc;
+  }
+  if (L->f16) {
+    rc = run_experts_f16(L->E, T, L->k, L->H, L->F, L->act, xr, L->wbf != 0, P, ws, true);
+    if (rc != CSK_OK) return rc;
+    mark(CSK_STAGE_COMBINE);
+    rc = launch_combine(ws.y, ws.pairs, ws.pos, (flags & CSK_FWD_RESIDUAL) ? hidden : nullptr, out,
+                        T, L->k, L->H, L->wbf);
+    mark(CSK_N_STAGES);
+    g_stage_valid = g_timing;
+    return rc;
   }
   const uint16_t* xa = ws.xs;
   const int* list_row = ws.list_tok;
@@ -1026,6 +1264,71 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
     list_row = ws.list_tok;
   }
   rc = run_experts(1, T, k, H, F, activation, xa, list_row, ws);
+  if (rc != CSK_OK) return rc;
+  expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)T), 256, 0, g_stream>>>(
+      ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
+  if ((rc = check_launch("expand_expert_rows_kernel")) != CSK_OK) return rc;
+  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+extern "C" int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T, int64_t H, int64_t F,
+                                  const csk_f16* w_up, const csk_f16* w_gate, const csk_f16* w_down,
+                                  const float* b_up, const float* b_gate, const float* b_down,
+                                  const float* pairs, int64_t k, int activation,
+                                  int weight_before_ffn, float* out, int* is_empty) {
+  REQUIRE_INIT();
+  if (!hidden || !w_up || !w_gate || !w_down || !pairs || !out || !is_empty || T < 0)
+    return fail(CSK_ERR_ARG, "csk_expert_mlp_f16: null argument");
+  // the router scan comes before the shape checks (expert_mlp_node.h:297-306)
+  bool any = false;
+  for (int64_t p = 0; p < T * k && !any; ++p) any = (int)pairs[2 * p] == expert_id;
+  *is_empty = !any;
+  if (!any) return CSK_OK;
+  if (w_up->rows != F || w_up->K != H)
+    return fail(CSK_ERR_ARG, "expert_mlp: w_up must be [" + std::to_string(F) + ", " + std::to_string(H) + "], got [" +
+                                 std::to_string(w_up->rows) + ", " + std::to_string(w_up->K) + "]");
+  if (w_gate->rows != F || w_gate->K != H)
+    return fail(CSK_ERR_ARG, "expert_mlp: w_gate must be [" + std::to_string(F) + ", " + std::to_string(H) + "], got [" +
+                                 std::to_string(w_gate->rows) + ", " + std::to_string(w_gate->K) + "]");
+  if (w_down->rows != H || w_down->K != F)
+    return fail(CSK_ERR_ARG, "expert_mlp: w_down must be [" + std::to_string(H) + ", " + std::to_string(F) + "], got [" +
+                                 std::to_string(w_down->rows) + ", " + std::to_string(w_down->K) + "]");
+  if (k <= 0 || k > kMaxTopK) return fail(CSK_ERR_ARG, "expert_mlp: top_k must be in 1..16");
+  const int nb = (b_up != nullptr) + (b_gate != nullptr) + (b_down != nullptr);
+  if (nb != 0 && nb != 3) return fail(CSK_ERR_ARG, "expert_mlp: biases must be all present or all absent");
+  Workspace& ws = g_ws;
+  const int64_t Hp = cdiv(H, 32) * 32, Fp = cdiv(F, 32) * 32;  // activation rows are whole blocks
+  int rc = ws.ensure(T, 1, k, Hp, Fp, weight_before_ffn != 0);
+  if (rc != CSK_OK) return rc;
+  const int64_t P = T * k;
+  DevBuf dx, dpairs, dbu, dbg, dbd, dew, dout;
+  if ((rc = dx.upload(hidden, (size_t)T * H * 4)) != CSK_OK) return rc;
+  if ((rc = dpairs.upload(pairs, (size_t)P * 8)) != CSK_OK) return rc;
+  if (nb == 3) {
+    if ((rc = dbu.upload(b_up, (size_t)F * 4)) != CSK_OK) return rc;
+    if ((rc = dbg.upload(b_gate, (size_t)F * 4)) != CSK_OK) return rc;
+    if ((rc = dbd.upload(b_down, (size_t)H * 4)) != CSK_OK) return rc;
+  }
+  ExpertW w{};
+  w.q_gate = reinterpret_cast<const uint4*>(w_gate->w);
+  w.q_up = reinterpret_cast<const uint4*>(w_up->w);
+  w.q_down = reinterpret_cast<const uint4*>(w_down->w);
+  w.b_gate = nb ? dbg.as<float>() : g_zero;
+  w.b_up = nb ? dbu.as<float>() : g_zero;
+  w.b_down = nb ? dbd.as<float>() : g_zero;
+  if ((rc = dew.upload(&w, sizeof w)) != CSK_OK) return rc;
+  if ((rc = dout.alloc((size_t)T * H * 4)) != CSK_OK) return rc;
+  select_expert_ids_kernel<<<dim3((unsigned)cdiv(P, 256)), 256, 0, g_stream>>>(
+      dpairs.as<float>(), ws.ids, (int)P, expert_id);
+  if ((rc = check_launch("select_expert_ids_kernel")) != CSK_OK) return rc;
+  HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
+  HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
+  if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
+  // with weight_before_ffn at most T tokens can select the expert: T rows are gathered; the
+  // ones past its count read the zeroed tail of the lists and are never consumed
+  rc = run_experts_f16(1, T, k, H, F, activation, dx.as<float>(), weight_before_ffn != 0, T, ws);
   if (rc != CSK_OK) return rc;
   expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)T), 256, 0, g_stream>>>(
       ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);

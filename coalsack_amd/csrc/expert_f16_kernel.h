@@ -1,0 +1,314 @@
+// Expert MLP with fp16 weights (include/coalsack/nn/nn_ops/expert_mlp_node.h:269-389,
+// compute_token :533-647): the branch the reference takes when the expert tensors arrive
+// as float16 (dense checkpoints, or Q4_K / Q6_K experts widened at load,
+// src/llm/moe_weight_provider.cpp:134-159).
+//
+// Weights [rows, K] are kept as tiles of 16 rows x 32 columns in matrix-instruction
+// order,
+//     w : [ceil(rows/16)][ceil(K/32)][64 lanes] x 16 B,
+//     lane (n = lane % 16, g = lane / 16) = row 16*tile + n, columns 32*kb + 8*g .. + 7,
+// zero beyond rows and K, so that a wave fetches one operand of v_mfma_f32_16x16x32_f16
+// as 1 KiB of contiguous memory and no dimension needs to be a multiple of anything.
+// The values are the checkpoint's own halves; nothing is rounded.
+//
+// Activations are fp32 in the reference.  Here a row is written as two fp16 terms of the
+// row divided by a power of two chosen so that the row maximum lands in [2^14, 2^15):
+//     x = 2^s * (hi + lo),  hi = fp16(x / 2^s),  lo = fp16(x / 2^s - hi),
+// 22 significant bits for every element within 2^-14 of the row maximum (smaller ones keep
+// an absolute error below 2^-25 of it).  Products of halves are exact in fp32, sums are
+// fp32.  Storage [row][ceil(K/32)][hi: 32 halves | lo: 32 halves] (128 B per block) plus
+// one fp32 scale per row.
+#pragma once
+#include "common.h"
+#include "expert_stream_kernel.h"  // moe_activation
+
+namespace csk {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+
+__host__ __device__ inline long f16_tile_count(long rows) { return (rows + 15) / 16; }
+__host__ __device__ inline long f16_block_count(long K) { return (K + 31) / 32; }
+// 16-byte entries of one packed matrix
+__host__ __device__ inline long f16_entries(long rows, long K) {
+  return f16_tile_count(rows) * f16_block_count(K) * 64;
+}
+
+// row-major halves [rows, K] -> tiles; one thread per 16-byte entry
+__global__ __launch_bounds__(256) void f16_pack_kernel(const uint16_t* __restrict__ src,
+                                                       u32x4* __restrict__ dst, long rows, long K,
+                                                       long entries) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= entries) return;
+  const long nkb = f16_block_count(K);
+  const int lane = (int)(idx & 63);
+  const long kb = (idx >> 6) % nkb, tile = (idx >> 6) / nkb;
+  const long row = tile * 16 + (lane & 15), k0 = kb * 32 + 8 * (lane >> 4);
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  if (row < rows) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const long k = k0 + j;
+      const uint32_t h = k < K ? src[row * K + k] : 0u;
+      w[j >> 1] |= h << (16 * (j & 1));
+    }
+  }
+  dst[idx] = u32x4{w[0], w[1], w[2], w[3]};
+}
+
+// tiles -> row-major halves (the export used to check that packing changed no bit)
+__global__ __launch_bounds__(256) void f16_unpack_kernel(const u32x4* __restrict__ src,
+                                                         uint16_t* __restrict__ dst, long rows,
+                                                         long K, long entries) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= entries) return;
+  const long nkb = f16_block_count(K);
+  const int lane = (int)(idx & 63);
+  const long kb = (idx >> 6) % nkb, tile = (idx >> 6) / nkb;
+  const long row = tile * 16 + (lane & 15), k0 = kb * 32 + 8 * (lane >> 4);
+  if (row >= rows) return;
+  const u32x4 v = src[idx];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const long k = k0 + j;
+    if (k < K) dst[row * K + k] = (uint16_t)(v[j >> 1] >> (16 * (j & 1)));
+  }
+}
+
+// synthetic weights straight into the tiles: halves j / 2^14, j uniform in [-2048, 2047]
+// (every value exact in fp16), a function of (key, row, column) only; zero in the padding
+__global__ __launch_bounds__(256) void synth_f16_kernel(u32x4* __restrict__ dst, long rows, long K,
+                                                        long entries, uint64_t key) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= entries) return;
+  const long nkb = f16_block_count(K);
+  const int lane = (int)(idx & 63);
+  const long kb = (idx >> 6) % nkb, tile = (idx >> 6) / nkb;
+  const long row = tile * 16 + (lane & 15), k0 = kb * 32 + 8 * (lane >> 4);
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  if (row < rows) {
+    const uint64_t r = mix64(key ^ (uint64_t)(row * nkb * 4 + kb * 4 + (lane >> 4)));
+    const uint64_t r2 = mix64(r);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int v = (int)(((j < 4 ? r : r2) >> (16 * (j & 3))) & 0xfff) - 2048;
+      const _Float16 h = (_Float16)((float)v * (1.0f / 16384.0f));
+      if (k0 + j < K) w[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * (j & 1));
+    }
+  }
+  dst[idx] = u32x4{w[0], w[1], w[2], w[3]};
+}
+
+// fp32 rows -> scaled two-term fp16 rows.  One workgroup per output row; the source row is
+// gather_tok[row] scaled by gather_w[row] when given (weight_before_ffn: the reference
+// multiplies the token by its routing weight in fp32 first, expert_mlp_node.h:766-772).
+__global__ __launch_bounds__(256) void f16_split_rows_kernel(const float* __restrict__ x, long K,
+                                                             const int* __restrict__ gather_tok,
+                                                             const float* __restrict__ gather_w,
+                                                             u32x4* __restrict__ out,
+                                                             float* __restrict__ rscale) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  const long srow = gather_tok ? gather_tok[row] : row;
+  const float gw = gather_w ? gather_w[row] : 1.0f;
+  const float* xr = x + srow * K;
+  float m = 0.0f;
+  for (long i = threadIdx.x; i < K; i += 256) m = fmaxf(m, fabsf(xr[i] * gw));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  // 2^s with the row maximum / 2^s in [2^14, 2^15); rows of zeros (or of non-finite
+  // values, which then propagate as they would in fp32) keep s = 0
+  const int eb = (int)((__float_as_uint(m) >> 23) & 0xffu);
+  int s = (eb == 0 || eb == 255) ? 0 : eb - 127 - 14;
+  s = max(-100, min(100, s));
+  const float inv = __uint_as_float((uint32_t)(127 - s) << 23);
+  if (threadIdx.x == 0) rscale[row] = __uint_as_float((uint32_t)(127 + s) << 23);
+  const long nkb = f16_block_count(K);
+  // one thread per 8 consecutive elements: chunk c of block kb
+  for (long i = threadIdx.x; i < nkb * 4; i += 256) {
+    const long kb = i >> 2;
+    const int c = (int)(i & 3);
+    uint32_t hi[4] = {0u, 0u, 0u, 0u}, lo[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const long k = kb * 32 + c * 8 + j;
+      const float v = k < K ? (xr[k] * gw) * inv : 0.0f;
+      const _Float16 h = (_Float16)v;
+      const _Float16 l = (_Float16)(v - (float)h);
+      hi[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * (j & 1));
+      lo[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, l) << (16 * (j & 1));
+    }
+    u32x4* dst = out + (row * nkb + kb) * 8;
+    dst[c] = u32x4{hi[0], hi[1], hi[2], hi[3]};
+    dst[4 + c] = u32x4{lo[0], lo[1], lo[2], lo[3]};
+  }
+}
+
+struct ExpertF16Args {
+  const WorkDesc* desc;  // [n_slots]: active experts first, the rest with Te = 0
+  int n_slots;
+  const int* list_row;   // activation row of a packed position, or null: the position itself
+  const u32x4* B;        // two-term fp16 activation rows
+  const float* rscale;   // their scales
+  int nkb;               // ceil(K / 32)
+  int N;                 // output features: F (gate/up) or H (down)
+  int ntile;             // ceil(N / 16)
+  int act_type;
+  float* out;            // MODE 0: activations [P, N] fp32; MODE 1: y [P, N]
+};
+
+constexpr int kF16Depth = 4;  // K blocks in flight per wave
+
+// MODE 0: act = activation(W_gate x + b_gate, W_up x + b_up); MODE 1: y = W_down act + b_down.
+// A workgroup of four waves takes one work unit at a time: (expert, pair of 16-row weight
+// tiles -- gate and up tile p, or down tiles 2p and 2p+1 --, group of up to 16 * MT dispatched
+// tokens).  Units are numbered expert-major, then pair, then group, so the groups of one
+// expert meet their weight tiles in cache at the same time.  The four waves split K; each
+// keeps kF16Depth blocks of loads in flight in a rotating register set; the partial sums
+// meet in LDS and are added in a fixed order.  The weights are the A operand (rows 4g..4g+3
+// of the tile end up in one lane), the tokens the B operand (lane % 16).
+template <int MODE, int MT>
+__global__ __launch_bounds__(256) void expert_f16_kernel(ExpertF16Args a) {
+  __shared__ int prefix[kMaxExperts + 1];
+  __shared__ floatx4 red[4][2][MT][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int n16 = lane & 15, g = lane >> 4;
+  const int npair = MODE == 0 ? a.ntile : (a.ntile + 1) / 2;
+  constexpr int GT = 16 * MT;  // tokens per group
+  // units per slot, exclusive prefix over slots (wave 0; four consecutive slots per lane)
+  if (wv == 0) {
+    int c[4], tot = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int s = lane * 4 + j;
+      const int te = s < a.n_slots ? a.desc[s].Te : 0;
+      c[j] = ((te + GT - 1) / GT) * npair;
+      tot += c[j];
+    }
+    int inc = tot;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_up(inc, o, 64);
+      if (lane >= o) inc += t;
+    }
+    int run = inc - tot;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      prefix[lane * 4 + j] = run;
+      run += c[j];
+    }
+    if (lane == 63) prefix[kMaxExperts] = inc;
+  }
+  __syncthreads();
+  const int n_units = prefix[kMaxExperts];
+  const int kq = (a.nkb + 3) / 4;
+  const int kb_lo = min(wv * kq, a.nkb), kb_hi = min(kb_lo + kq, a.nkb);
+
+  for (int u = blockIdx.x; u < n_units; u += gridDim.x) {
+    // slot of unit u: last slot whose prefix is <= u (binary search over 256 entries)
+    int s = 0;
+#pragma unroll
+    for (int step = kMaxExperts / 2; step > 0; step >>= 1)
+      if (prefix[s + step] <= u) s += step;
+    const WorkDesc* wd = a.desc + s;
+    const int te = wd->Te, base = wd->base;
+    const int ngrp = (te + GT - 1) / GT;
+    const int r = u - prefix[s];
+    const int p = r / ngrp, m0 = (r - p * ngrp) * GT;
+    const int cnt = min(GT, te - m0);
+    // weight tiles of the pair
+    const int t0 = MODE == 0 ? p : 2 * p;
+    const int t1 = MODE == 0 ? p : min(2 * p + 1, a.ntile - 1);
+    const CSK_GLOBAL u32x4* A0 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_gate : wd->w.q_down)) + (long)t0 * a.nkb * 64 + lane;
+    const CSK_GLOBAL u32x4* A1 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_up : wd->w.q_down)) + (long)t1 * a.nkb * 64 + lane;
+    // activation rows of the lane's token slots (slots past the group re-read its last row)
+    const CSK_GLOBAL u32x4* Brow[MT];
+    float rs[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int pos = base + m0 + min(n16 + 16 * mt, cnt - 1);
+      const long row = a.list_row ? a.list_row[pos] : pos;
+      Brow[mt] = as_global(a.B) + row * a.nkb * 8 + g;
+      rs[mt] = a.rscale[row];
+    }
+    floatx4 acc[2][MT];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    u32x4 qa[kF16Depth][2], qh[kF16Depth][MT], ql[kF16Depth][MT];
+    auto fetch = [&](int slot, int kb) {
+      const int kc = min(kb, kb_hi - 1);  // past the wave's range: re-read its last block
+      qa[slot][0] = A0[(long)kc * 64];
+      qa[slot][1] = A1[(long)kc * 64];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        qh[slot][mt] = Brow[mt][(long)kc * 8];
+        ql[slot][mt] = Brow[mt][(long)kc * 8 + 4];
+      }
+    };
+    auto fma_block = [&](int slot) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const half8 wa = __builtin_bit_cast(half8, qa[slot][t]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, __builtin_bit_cast(half8, qh[slot][mt]), acc[t][mt], 0, 0, 0);
+          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, __builtin_bit_cast(half8, ql[slot][mt]), acc[t][mt], 0, 0, 0);
+        }
+      }
+    };
+    if (kb_lo < kb_hi) {
+#pragma unroll
+      for (int j = 0; j < kF16Depth; ++j) fetch(j, kb_lo + j);
+      for (int kb = kb_lo; kb < kb_hi; kb += kF16Depth) {
+#pragma unroll
+        for (int j = 0; j < kF16Depth; ++j) {
+          if (kb + j < kb_hi) fma_block(j);
+          fetch(j, kb + j + kF16Depth);
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) red[wv][t][mt][lane] = acc[t][mt];
+    __syncthreads();
+    // wave w finishes token sub-groups w, w + 4, ...: partial sums in wave order, scale,
+    // bias, activation
+    for (int mt = wv; mt < MT; mt += 4) {
+      floatx4 v[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        v[t] = ((red[0][t][mt][lane] + red[1][t][mt][lane]) + red[2][t][mt][lane]) + red[3][t][mt][lane];
+      const int slot = n16 + 16 * mt;
+      if (slot < cnt) {
+        const long pos = base + m0 + slot;
+        float scale = 1.0f;
+#pragma unroll
+        for (int q = 0; q < MT; ++q)
+          if (q == mt) scale = rs[q];
+        const CSK_GLOBAL float* b0 = as_global(MODE == 0 ? wd->w.b_gate : wd->w.b_down);
+        const CSK_GLOBAL float* b1 = as_global(MODE == 0 ? wd->w.b_up : wd->w.b_down);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (MODE == 0) {
+            const int f = 16 * p + 4 * g + i;
+            if (f < a.N)
+              a.out[pos * a.N + f] = moe_activation(v[0][i] * scale + b0[f], v[1][i] * scale + b1[f], a.act_type);
+          } else {
+            const int h0 = 16 * (2 * p) + 4 * g + i, h1 = h0 + 16;
+            if (h0 < a.N) a.out[pos * a.N + h0] = v[0][i] * scale + b0[h0];
+            if (h1 < a.N) a.out[pos * a.N + h1] = v[1][i] * scale + b1[h1];
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace csk

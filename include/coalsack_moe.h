@@ -102,6 +102,20 @@ int csk_mxfp4_dequant(const csk_mxfp4* m, float* host_out);
 /* Recover the 17-byte blocks from the resident copy (round-trip check). */
 int csk_mxfp4_export(const csk_mxfp4* m, uint8_t* blocks17_host);
 
+/* ---- resident fp16 matrices ---------------------------------------------- */
+
+/* A [rows, K] row-major matrix of IEEE halves, as expert_mlp_node::compute_fp16
+ * receives w_up / w_gate / w_down (expert_mlp_node.h:269-389: dtype::float16,
+ * 2-D) and as moe_weight_provider::get produces them from F16, Q4_K or Q6_K
+ * checkpoints (src/llm/moe_weight_provider.cpp:134-159).  Kept in HBM as
+ * 16 x 32 tiles in matrix-instruction order; no value changes.  Any rows, K
+ * in 1..65536. */
+typedef struct csk_f16 csk_f16;
+int csk_f16_upload(const uint16_t* halves_host, int64_t rows, int64_t K, csk_f16** out);
+void csk_f16_free(csk_f16* m);
+/* Recover the row-major halves from the resident copy (round-trip check). */
+int csk_f16_export(const csk_f16* m, uint16_t* halves_host);
+
 /* ---- one MoE layer, weights resident ------------------------------------ */
 
 /* E experts, top-k, hidden size H, expert intermediate size F.  H and F must
@@ -132,6 +146,19 @@ int csk_layer_fill_synthetic(csk_layer* L, uint64_t seed, int64_t layer_index, i
                              int scale_span);
 int csk_layer_dequant(const csk_layer* L, int64_t e, int which, float* host_out);
 int csk_layer_export(const csk_layer* L, int64_t e, int which, uint8_t* blocks17_host);
+
+/* The same layer with fp16 experts: the other branch of expert_mlp_node::process
+ * (expert_mlp_node.h:269-389, compute_token :533-647), which the engine takes for
+ * checkpoints whose expert tensors are F16, Q4_K or Q6_K
+ * (src/llm/moe_weight_provider.cpp:134-159).  Router, options, norm, forward and
+ * csk_layer_fill_synthetic (halves j / 2^14, j uniform in [-2048, 2047]) work as
+ * for an MXFP4 layer; the weights come in through csk_layer_set_expert_f16:
+ * row-major halves w_up/w_gate [F,H], w_down [H,F]; biases f32 or all NULL. */
+int csk_layer_create_f16(int64_t E, int64_t k, int64_t H, int64_t F, csk_layer** out);
+int csk_layer_set_expert_f16(csk_layer* L, int64_t e, const uint16_t* w_up, const uint16_t* w_gate,
+                             const uint16_t* w_down, const float* b_up, const float* b_gate,
+                             const float* b_down);
+int csk_layer_export_f16(const csk_layer* L, int64_t e, int which, uint16_t* halves_host);
 
 /* ---------------------------------------------------------------- GGUF ingest
  * Reads a GGUF file's key/value section and tensor table (no tensor data) --
@@ -200,6 +227,15 @@ int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t T, int64_t 
                          const float* b_up, const float* b_gate, const float* b_down,
                          const float* router_pairs, int64_t k, int activation,
                          int weight_before_ffn, float* out, int* is_empty);
+/* expert_mlp_node::compute_fp16 for one expert (expert_mlp_node.h:269-389,
+ * token loop :740-780): conventions of csk_expert_mlp_mxfp4; H and F need not be
+ * multiples of anything (the reference's rows end in a scalar remainder loop,
+ * :578-585). */
+int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T, int64_t H, int64_t F,
+                       const csk_f16* w_up, const csk_f16* w_gate, const csk_f16* w_down,
+                       const float* b_up, const float* b_gate, const float* b_down,
+                       const float* router_pairs, int64_t k, int activation,
+                       int weight_before_ffn, float* out, int* is_empty);
 /* expert_mlp_node::compute_test_mxfp4 (expert_mlp_node.h:63-70): one token,
  * raw 17-byte-block weights in host memory. */
 int csk_expert_token_mxfp4(const float* hidden_vec, const uint8_t* w_up, const uint8_t* w_gate,

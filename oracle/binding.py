@@ -32,12 +32,17 @@ def _u8(a):
     return None if a is None else np.ascontiguousarray(a, dtype=np.uint8)
 
 
+def _f16(a):
+    return None if a is None else np.ascontiguousarray(a, dtype=np.float16)
+
+
 class _LayerStruct(C.Structure):
     _fields_ = [("E", _I64), ("k", _I64), ("H", _I64), ("F", _I64),
                 ("gate_w", _P), ("gate_b", _P), ("w_up", _P), ("w_gate", _P), ("w_down", _P),
                 ("b_up", _P), ("b_gate", _P), ("b_down", _P), ("norm_w", _P),
                 ("norm_eps", C.c_float), ("residual", C.c_int), ("sigmoid", C.c_int),
-                ("act", C.c_int), ("weight_before_ffn", C.c_int)]
+                ("act", C.c_int), ("weight_before_ffn", C.c_int),
+                ("w_up16", _P), ("w_gate16", _P), ("w_down16", _P)]
 
 
 class Oracle:
@@ -58,6 +63,11 @@ class Oracle:
         d.orc_expert_token_mxfp4.argtypes = [_P] * 8 + [_I64, _I64, C.c_int]
         d.orc_expert_mlp_mxfp4.restype = C.c_int
         d.orc_expert_mlp_mxfp4.argtypes = [C.c_int, _P, _I64, _I64, _I64] + [_P] * 7 + \
+            [_I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]
+        d.orc_expert_token_f16.restype = C.c_int
+        d.orc_expert_token_f16.argtypes = [_P] * 8 + [_I64, _I64, C.c_int]
+        d.orc_expert_mlp_f16.restype = C.c_int
+        d.orc_expert_mlp_f16.argtypes = [C.c_int, _P, _I64, _I64, _I64] + [_P] * 7 + \
             [_I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]
         d.orc_expert_merge.restype = C.c_int
         d.orc_expert_merge.argtypes = [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]
@@ -122,6 +132,36 @@ class Oracle:
             raise ValueError(f"orc_expert_mlp_mxfp4 rc={rc}")
         return None if empty.value else out
 
+    def expert_token_f16(self, x, w_up, w_gate, w_down, b_up, b_gate, b_down, act=0):
+        """w_* are float16 arrays, row-major [F,H], [F,H], [H,F]."""
+        x = _f32(x)
+        w_up, w_gate, w_down = _f16(w_up), _f16(w_gate), _f16(w_down)
+        b_up, b_gate, b_down = _f32(b_up), _f32(b_gate), _f32(b_down)
+        F, H = w_up.shape
+        out = np.empty(H, np.float32)
+        rc = self.dll.orc_expert_token_f16(_p(x), _p(w_up), _p(w_gate), _p(w_down), _p(b_up),
+                                           _p(b_gate), _p(b_down), _p(out), H, F, act)
+        if rc:
+            raise ValueError(f"orc_expert_token_f16 rc={rc}")
+        return out
+
+    def expert_mlp_f16(self, expert_id, hidden, w_up, w_gate, w_down, b_up, b_gate, b_down, pairs,
+                       act=0, weight_before_ffn=False):
+        hidden, pairs = _f32(hidden), _f32(pairs)
+        w_up, w_gate, w_down = _f16(w_up), _f16(w_gate), _f16(w_down)
+        b_up, b_gate, b_down = _f32(b_up), _f32(b_gate), _f32(b_down)
+        T, H = hidden.shape
+        F = w_up.shape[0]
+        k = pairs.shape[1]
+        out = np.empty((T, H), np.float32)
+        empty = C.c_int()
+        rc = self.dll.orc_expert_mlp_f16(expert_id, _p(hidden), T, H, F, _p(w_up), _p(w_gate),
+                                         _p(w_down), _p(b_up), _p(b_gate), _p(b_down), _p(pairs),
+                                         k, act, int(weight_before_ffn), _p(out), C.byref(empty))
+        if rc:
+            raise ValueError(f"orc_expert_mlp_f16 rc={rc}")
+        return None if empty.value else out
+
     def expert_merge(self, pairs, expert_outs, H, pre_weighted=False):
         pairs = _f32(pairs)
         T, k = pairs.shape[:2]
@@ -148,12 +188,19 @@ class Oracle:
     def moe_layer(self, hidden, E, k, H, F, gate_w, gate_b, w_up, w_gate, w_down, b_up, b_gate,
                   b_down, norm_w=None, norm_eps=1e-5, residual=False, sigmoid=False, act=0,
                   weight_before_ffn=False, max_tokens=-1):
-        """w_up/w_gate/w_down: uint8 arrays holding all E experts back to back."""
+        """w_up/w_gate/w_down: uint8 arrays holding all E experts back to back (MXFP4 blocks),
+        or float16 arrays [E,F,H], [E,F,H], [E,H,F] (fp16 experts)."""
         hidden = _f32(hidden)
-        keep = [_f32(gate_w), _f32(gate_b), _u8(w_up), _u8(w_gate), _u8(w_down), _f32(b_up),
+        f16 = getattr(w_up, "dtype", None) == np.float16
+        wconv = _f16 if f16 else _u8
+        keep = [_f32(gate_w), _f32(gate_b), wconv(w_up), wconv(w_gate), wconv(w_down), _f32(b_up),
                 _f32(b_gate), _f32(b_down), _f32(norm_w)]
-        L = _LayerStruct(E, k, H, F, *[_p(a) for a in keep], norm_eps, int(residual), int(sigmoid),
-                         act, int(weight_before_ffn))
+        ptrs = [_p(a) for a in keep]
+        w16 = ptrs[2:5] if f16 else [None, None, None]
+        if f16:
+            ptrs[2:5] = [None, None, None]
+        L = _LayerStruct(E, k, H, F, *ptrs, norm_eps, int(residual), int(sigmoid),
+                         act, int(weight_before_ffn), *w16)
         T = hidden.shape[0]
         out = np.zeros((T, H), np.float32)
         pairs = np.empty((T, k, 2), np.float32)

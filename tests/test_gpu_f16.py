@@ -1,0 +1,169 @@
+"""GPU parity of the fp16 expert path (csk_f16_*, csk_expert_mlp_f16, fp16 layers) against
+the CPU restatement, through the C ABI.  Tolerance: 1e-3 of the output scale, as for the
+MXFP4 path; measured differences are ~1e-6."""
+import numpy as np
+import pytest
+
+from coalsack_amd import capi, synth
+from tests.helpers import assert_layer_close
+from tests.test_oracle_expert import modified_swiglu_ref
+from tests.test_oracle_expert_f16 import random_f16_expert
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("rows,K", [(16, 32), (37, 45), (1, 1), (200, 2880), (2880, 96)])
+def test_f16_upload_export_round_trip(lib, rows, K):
+    rng = np.random.default_rng([rows, K])
+    w = rng.standard_normal((rows, K)).astype(np.float16)
+    w.reshape(-1)[:4] = np.array([0.0, -0.0, 65504.0, 6e-8], np.float16)[:min(4, w.size)]
+    h = lib.f16_upload(w)
+    try:
+        back = lib.f16_export(h, rows, K)
+    finally:
+        lib.f16_free(h)
+    assert np.array_equal(back.view(np.uint16), w.view(np.uint16))
+
+
+def test_reference_known_answer_two_by_two(lib):
+    # test/test_expert_mlp.cpp:118-200
+    x = np.array([[1.0, 0.5]], np.float32)
+    w_up = np.zeros((2, 2), np.float16)
+    w_gate = np.zeros((2, 2), np.float16)
+    w_down = np.zeros((2, 2), np.float16)
+    w_up[0, 0] = 1.0
+    w_gate[0, 0] = 1.0
+    w_down.reshape(-1)[0] = 1.0
+    w_down.reshape(-1)[2] = 1.0
+    b_up = np.array([0.5, 0.0], np.float32)
+    zero = np.zeros(2, np.float32)
+    pairs = np.array([[[0, 1.0], [1, 0.0], [2, 0.0], [3, 0.0]]], np.float32)
+    out = lib.expert_mlp_f16(0, x, w_up, w_gate, w_down, b_up, zero, zero, pairs)
+    assert abs(out[0, 0] - modified_swiglu_ref(1.0, 1.5)) < 1e-3  # the reference's own tolerance
+    assert abs(out[0, 0] - modified_swiglu_ref(1.0, 1.5)) < 1e-6
+
+
+@pytest.mark.parametrize("T,H,F", [(5, 64, 96), (7, 37, 29), (3, 2880, 2880), (150, 96, 160),
+                                   (70, 45, 50)])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("act,wbf", [(0, False), (1, False), (0, True)])
+def test_expert_node_matches_oracle(lib, oracle, T, H, F, bias, act, wbf):
+    if H == 2880 and (bias or act or wbf):
+        pytest.skip("large shape: one variant is enough")
+    rng = np.random.default_rng([T, H, F, act])
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    w = random_f16_expert(rng, H, F, 0.1)
+    b = [rng.standard_normal(n).astype(np.float32) * 0.1 for n in (F, F, H)] if bias else [None] * 3
+    k = 2
+    pairs = np.zeros((T, k, 2), np.float32)
+    sel = rng.random(T) < 0.6
+    sel[0] = True
+    pairs[:, 0, 0] = np.where(sel, 4, 1)
+    pairs[:, 1, 0] = 2
+    pairs[..., 1] = rng.random((T, k)).astype(np.float32)
+    got = lib.expert_mlp_f16(4, hidden, *w, *b, pairs, act=act, weight_before_ffn=wbf)
+    want = oracle.expert_mlp_f16(4, hidden, *w, *b, pairs, act=act, weight_before_ffn=wbf)
+    assert_layer_close(got, want)
+    assert not got[~sel].any()
+    assert lib.expert_mlp_f16(9, hidden, *w, *b, pairs, act=act, weight_before_ffn=wbf) is None
+
+
+def test_expert_node_shape_errors(lib):
+    hidden = np.zeros((2, 8), np.float32)
+    pairs = np.zeros((2, 1, 2), np.float32)
+    good = np.zeros((4, 8), np.float16), np.zeros((4, 8), np.float16), np.zeros((8, 4), np.float16)
+    with pytest.raises(capi.CskError, match="w_down must be"):
+        lib.expert_mlp_f16(0, hidden, good[0], good[1], np.zeros((8, 5), np.float16), None, None, None, pairs)
+    with pytest.raises(capi.CskError, match="w_gate must be"):
+        lib.expert_mlp_f16(0, hidden, good[0], np.zeros((4, 7), np.float16), good[2], None, None, None, pairs)
+    with pytest.raises(capi.CskError, match="biases"):
+        lib.expert_mlp_f16(0, hidden, *good, np.zeros(4, np.float32), None, None, pairs)
+
+
+def _f16_layer(lib, L, ws, bias=True, norm=False, **opts):
+    layer = lib.layer(L.E, L.k, L.H, L.F, f16=True)
+    layer.set_router(L.gate_w, L.gate_b)
+    for e in range(L.E):
+        b = (L.b_up[e], L.b_gate[e], L.b_down[e]) if bias else (None, None, None)
+        layer.set_expert_f16(e, *ws[e], *b)
+    if norm:
+        layer.set_norm(L.norm_w, 1e-5)
+    if opts:
+        layer.set_options(**opts)
+    return layer
+
+
+def _oracle_f16_layer(oracle, L, ws, hidden, bias=True, norm=False, residual=False, **opts):
+    w_up = np.stack([w[0] for w in ws])
+    w_gate = np.stack([w[1] for w in ws])
+    w_down = np.stack([w[2] for w in ws])
+    return oracle.moe_layer(hidden, L.E, L.k, L.H, L.F, L.gate_w, L.gate_b, w_up, w_gate, w_down,
+                            L.b_up if bias else None, L.b_gate if bias else None,
+                            L.b_down if bias else None, norm_w=L.norm_w if norm else None,
+                            norm_eps=1e-5, residual=residual, **opts)
+
+
+@pytest.mark.parametrize("T", [1, 5, 33, 64, 65, 200])
+def test_f16_layer_matches_oracle(lib, oracle, T):
+    L = synth.LayerInputs(8, 2, 96, 160, seed=17, with_norm=True)
+    rng = np.random.default_rng(17)
+    ws = [random_f16_expert(rng, L.H, L.F, 0.1) for _ in range(L.E)]
+    hidden = synth.hidden_states(T, L.H)
+    with _f16_layer(lib, L, ws, norm=True) as layer:
+        for flags in (0, capi.FWD_RMSNORM | capi.FWD_RESIDUAL):
+            got, pairs = layer.forward(hidden, flags=flags, want_pairs=True)
+            want, wpairs = _oracle_f16_layer(oracle, L, ws, hidden, norm=bool(flags),
+                                             residual=bool(flags))
+            assert np.array_equal(pairs[..., 0], wpairs[..., 0])
+            assert_layer_close(got, want)
+            counts, _ = layer.last_dispatch(T)
+            assert counts.sum() == T * L.k
+
+
+@pytest.mark.parametrize("opts", [dict(sigmoid=True), dict(act=1), dict(weight_before_ffn=True),
+                                  dict(sigmoid=True, act=1, weight_before_ffn=True)])
+@pytest.mark.parametrize("T", [6, 130])
+def test_f16_layer_variants(lib, oracle, opts, T):
+    L = synth.LayerInputs(6, 3, 64, 96, seed=23)
+    rng = np.random.default_rng(23)
+    ws = [random_f16_expert(rng, L.H, L.F, 0.1) for _ in range(L.E)]
+    hidden = synth.hidden_states(T, L.H)
+    with _f16_layer(lib, L, ws, **opts) as layer:
+        got = layer.forward(hidden)
+        want, _ = _oracle_f16_layer(oracle, L, ws, hidden, **opts)
+        assert_layer_close(got, want)
+
+
+def test_f16_layer_20b_shape_device_weights(lib, oracle):
+    """20b-shaped layer (32 experts, top-4, 2880 x 2880) with weights generated on the GPU;
+    the oracle gets them back through the export, only for the experts the tokens select."""
+    L = synth.LayerInputs(32, 4, 2880, 2880, seed=31)
+    T = 4
+    hidden = synth.hidden_states(T, L.H)
+    with lib.layer(L.E, L.k, L.H, L.F, f16=True) as layer:
+        layer.set_router(L.gate_w, L.gate_b)
+        layer.fill_synthetic(31, 0)
+        for e in range(L.E):
+            layer.set_expert_f16(e, None, None, None, L.b_up[e], L.b_gate[e], L.b_down[e])
+        got, pairs = layer.forward(hidden, want_pairs=True)
+        want_pairs = oracle.router(hidden, L.gate_w, L.gate_b, L.k)
+        assert np.array_equal(pairs[..., 0], want_pairs[..., 0])
+        want = np.zeros_like(got)
+        for t in range(T):
+            for j in range(L.k):
+                e = int(want_pairs[t, j, 0])
+                w = [layer.export_f16(e, which) for which in (capi.W_UP, capi.W_GATE, capi.W_DOWN)]
+                assert np.abs(w[0].astype(np.float32)).max() <= 0.125
+                y = oracle.expert_token_f16(hidden[t], *w, L.b_up[e], L.b_gate[e], L.b_down[e])
+                want[t] += want_pairs[t, j, 1] * y
+        assert_layer_close(got, want)
+
+
+def test_layer_kinds_do_not_mix(lib):
+    with lib.layer(2, 1, 32, 32, f16=True) as layer:
+        with pytest.raises(capi.CskError, match="fp16 experts"):
+            layer.set_expert(0, np.zeros(32 * 17, np.uint8), np.zeros(32 * 17, np.uint8),
+                             np.zeros(32 * 17, np.uint8))
+    with lib.layer(2, 1, 32, 32) as layer:
+        with pytest.raises(capi.CskError, match="MXFP4 experts"):
+            layer.set_expert_f16(0, *[np.zeros((32, 32), np.float16)] * 3)
