@@ -16,6 +16,10 @@ Workloads (BASELINE.json configs):
   c3_20b_prefill  same layer, T = 2048
   c4_120b         128 experts, 8 hot experts (+2.0 router bias), T in {1,16,4096}
   c5_stack        36 layers of the 120b shape with RMSNorm + residual, T in {1,8,64}
+Neighbouring paths (not the headline):
+  gguf_ingest     one 20b-shaped block from a GGUF file into a resident layer
+  f16_20b_decode  the 20b-shaped layer with fp16 experts (the reference's other expert branch), T = 16
+  f16_20b_prefill same, T = 2048
 """
 import argparse
 import json
@@ -30,7 +34,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP4_PEAK_TFLOPS = 10100.0  # dense MXFP4, published
-MAT_BYTES = 2880 * 90 * 17      # one [2880, 2880] MXFP4 matrix in 17-byte blocks
+MFMA_F16_PEAK_TFLOPS = 2500.0   # dense fp16, published
 
 SHAPES = {
     "c2_20b_decode": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=16, sweep=[1, 2, 4, 8, 16, 32]),
@@ -39,22 +43,30 @@ SHAPES = {
     "c5_stack": dict(E=128, k=4, H=2880, F=2880, hot=8, default_T=8, sweep=[1, 8, 64], layers=36),
     # next-row workload: one 20b-shaped block read from a GGUF file into a resident layer
     "gguf_ingest": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=4, sweep=[]),
+    # next-row workloads: the same layer with fp16 experts
+    "f16_20b_decode": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=16, sweep=[1, 4, 16, 64], f16=True),
+    "f16_20b_prefill": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=2048, sweep=[], f16=True),
 }
 
 
-def layer_bytes(E, k, H, F, T, U):
+def matrix_bytes(rows, K, f16=False):
+    """One expert matrix: fp16, or MXFP4 in 17-byte blocks of 32."""
+    return rows * K * 2 if f16 else rows * (K // 32) * 17
+
+
+def layer_bytes(E, k, H, F, T, U, f16=False):
     """Algorithmic HBM bytes of one layer forward: every distinct expert's three
     matrices and biases once, the router weights, activations in and out, router
     output."""
-    mat_gu = F * (H // 32) * 17
-    mat_d = H * (F // 32) * 17
+    mat_gu = matrix_bytes(F, H, f16)
+    mat_d = matrix_bytes(H, F, f16)
     return U * (2 * mat_gu + mat_d + (2 * F + H) * 4) + E * H * 4 + E * 4 + 2 * T * H * 4 + T * k * 8
 
 
-def gateup_bytes(H, F, T, k, U):
+def gateup_bytes(H, F, T, k, U, f16=False):
     """Algorithmic bytes of the gate/up kernel: both matrices and biases of every
     distinct expert once, the fp32 activations in, the fp32 activations out."""
-    return U * (2 * F * (H // 32) * 17 + 2 * F * 4) + T * H * 4 + T * k * F * 4
+    return U * (2 * matrix_bytes(F, H, f16) + 2 * F * 4) + T * H * 4 + T * k * F * 4
 
 
 def layer_flops(E, k, H, F, T):
@@ -64,11 +76,15 @@ def layer_flops(E, k, H, F, T):
 def make_layer(lib, synth, shape, seed, layer_index=0, norm=False):
     L = synth.LayerInputs(shape["E"], shape["k"], shape["H"], shape["F"], seed=seed, layer=layer_index,
                           hot_experts=shape["hot"], with_norm=norm)
-    layer = lib.layer(L.E, L.k, L.H, L.F)
+    f16 = bool(shape.get("f16"))
+    layer = lib.layer(L.E, L.k, L.H, L.F, f16=f16)
     layer.set_router(L.gate_w, L.gate_b)
     layer.fill_synthetic(L.seed, L.layer)
     for e in range(L.E):
-        layer.set_expert(e, None, None, None, L.b_up[e], L.b_gate[e], L.b_down[e])
+        if f16:
+            layer.set_expert_f16(e, None, None, None, L.b_up[e], L.b_gate[e], L.b_down[e])
+        else:
+            layer.set_expert(e, None, None, None, L.b_up[e], L.b_gate[e], L.b_down[e])
     if norm:
         layer.set_norm(L.norm_w, 1e-5)
     return L, layer
@@ -163,6 +179,16 @@ def bench_layer(lib, synth, shape, T, steps, warmup, seed=1234):
     U = float(np.mean(Us))
     hidden = hiddens[0]
     out = lib.to_host(d_out, (T, L.H))
+    f16 = bool(shape.get("f16"))
+    L.f16_weights = None
+    if f16:
+        # the CPU leg needs the generated halves of the experts its token sample selects
+        from coalsack_amd import capi
+        ns = min(T, 2)
+        _, pairs = layer.forward(hidden[:ns], want_pairs=True)
+        L.f16_weights = {int(e): [layer.export_f16(int(e), w) for w in (capi.W_UP, capi.W_GATE, capi.W_DOWN)]
+                         for e in sorted(set(pairs[..., 0].astype(int).ravel().tolist()))}
+        L.f16_sample = ns
     for d in d_ins:
         lib.dev_free(d)
     lib.dev_free(d_out)
@@ -171,11 +197,11 @@ def bench_layer(lib, synth, shape, T, steps, warmup, seed=1234):
                stage_ms=stages, finite=bool(np.all(np.isfinite(out))),
                max_tokens_per_expert=tmax, batches=nb, steps=steps,
                close_call_tokens=sum(close_calls(L, h, L.k) for h in hiddens))
-    res["layer_bytes"] = layer_bytes(L.E, L.k, L.H, L.F, T, U)
+    res["layer_bytes"] = layer_bytes(L.E, L.k, L.H, L.F, T, U, f16)
     res["layer_hbm_frac"] = res["layer_bytes"] / (ms * 1e-3) / (HBM_PEAK_GBS * 1e9)
     res["layer_flops"] = layer_flops(L.E, L.k, L.H, L.F, T)
     res["layer_fp4_frac"] = res["layer_flops"] / (ms * 1e-3) / (MFMA_FP4_PEAK_TFLOPS * 1e12)
-    gu = gateup_bytes(L.H, L.F, T, L.k, U)
+    gu = gateup_bytes(L.H, L.F, T, L.k, U, f16)
     res["gateup_bytes"] = gu
     res["gateup_gbs"] = gu / (stages["gateup"] * 1e-3) / 1e9
     return res, (L, hidden, out)
@@ -277,6 +303,34 @@ def cpu_baseline(L, hidden, gpu_out, budget_s=12.0):
                 gpu_vs_cpu_max_rel_err=err)
 
 
+def cpu_baseline_f16(L, hidden, gpu_out, budget_s=12.0):
+    """The CPU checker's fp16 expert path on the first tokens of the batch (the ones whose
+    experts' generated weights were read back), one thread."""
+    from oracle.binding import Oracle
+    orc = Oracle()
+    ns = L.f16_sample
+    E, H, F = L.E, L.H, L.F
+    w_up = np.zeros((E, F, H), np.float16)
+    w_gate = np.zeros((E, F, H), np.float16)
+    w_down = np.zeros((E, H, F), np.float16)
+    for e, (u, g, d) in L.f16_weights.items():
+        w_up[e], w_gate[e], w_down[e] = u, g, d
+    args = (hidden[:ns], E, L.k, H, F, L.gate_w, L.gate_b, w_up, w_gate, w_down, L.b_up, L.b_gate, L.b_down)
+    t0 = time.perf_counter()
+    ref, _ = orc.moe_layer(*args)
+    first = time.perf_counter() - t0
+    reps = int(max(1, min(50, budget_s / max(first, 1e-6))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        ref, _ = orc.moe_layer(*args)
+    dt = time.perf_counter() - t0
+    err = float(np.max(np.abs(gpu_out[:ns] - ref)) / max(1e-6, np.max(np.abs(ref))))
+    return dict(value=ns * reps / dt, unit="tokens/s", cores=1, kind="port", all_cores=None,
+                sample=f"first {ns} of {hidden.shape[0]} tokens x {reps} repeats, {dt:.1f} s on one host core "
+                       f"(CPU cost is linear in tokens x top_k)",
+                gpu_vs_cpu_max_rel_err=err)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -340,7 +394,16 @@ def main():
         lib.dev_free(dst)
     res, (L, hidden, out) = bench_layer(lib, synth, shape, T, a.steps, a.warmup)
     prefill = T >= 512
-    if prefill:
+    f16 = bool(shape.get("f16"))
+    if f16 and prefill:
+        st = res["stage_ms"]
+        fl = T * shape["k"] * 4 * shape["H"] * shape["F"]
+        roof = dict(bound="mfma", kernel="expert_f16_gemm_kernel<0> (gate/up + SwiGLU)", achieved=fl / (st["gateup"] * 1e-3) / 1e12,
+                    peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s", traffic=None)
+    elif f16:
+        roof = dict(bound="hbm", kernel="expert_f16_kernel<0,1> (gate/up + SwiGLU)",
+                    achieved=res["gateup_gbs"], peak=HBM_PEAK_GBS, unit="GB/s", traffic=None)
+    elif prefill:
         st = res["stage_ms"]
         fl = T * shape["k"] * 4 * shape["H"] * shape["F"]  # gate + up flops
         roof = dict(bound="mfma", kernel="expert_gemm_mx_kernel<0> (gate/up + SwiGLU)", achieved=fl / (st["gateup"] * 1e-3) / 1e12,
@@ -373,15 +436,16 @@ def main():
                               gateup_hbm_frac=round(r["gateup_gbs"] / HBM_PEAK_GBS, 4),
                               stage_ms={kk: round(v, 5) for kk, v in r["stage_ms"].items()}))
 
-    cpu = None if a.no_cpu else cpu_baseline(L, hidden, out)
+    cpu = None if a.no_cpu else (cpu_baseline_f16(L, hidden, out) if f16 else cpu_baseline(L, hidden, out))
     line = dict(
         metric="MoE layer tokens/s", value=res["tokens_per_s"], unit="tokens/s", n_gpus=1, steps=res["steps"],
         warmup=a.warmup, ms_per_step=res["ms_per_step"], higher_is_better=True, scaling="weak",
         vs_baseline=None,
-        dtype=("mxfp4 x fp6(3-term, block-scaled) -> f32" if prefill else "mxfp4 x bf16(2-term) -> f32"),
+        dtype=("f16 x f16(2-term) -> f32" if f16 else
+               "mxfp4 x fp6(3-term, block-scaled) -> f32" if prefill else "mxfp4 x bf16(2-term) -> f32"),
         data="synthetic",
         config=dict(workload=f"{a.workload}: E={shape['E']} top-{shape['k']} H={shape['H']} F={shape['F']} "
-                             f"MXFP4, T={T}" + (", 8 hot experts" if shape["hot"] else ""),
+                             f"{'fp16' if f16 else 'MXFP4'}, T={T}" + (", 8 hot experts" if shape["hot"] else ""),
                     tokens=T, distinct_experts=res["distinct_experts"], token_batches_in_rotation=res["batches"],
                     close_call_tokens=res["close_call_tokens"], device=dev_name, compute_units=cus),
         roofline=roof, cpu_baseline=cpu,

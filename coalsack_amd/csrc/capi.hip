@@ -473,14 +473,27 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   if (rc != CSK_OK) return rc;
   const bool small = T <= 64;
   const dim3 grid((unsigned)(4 * std::max(g_cus, 1)));
+  ExpertF16GemmArgs ga{};
+  ga.desc = ws.desc;
+  ga.mtiles = ws.tiles;
+  ga.n_mtiles = ws.n_tiles;
+  ga.act_type = act_type;
+  const int64_t max_mtiles = P / 64 + std::min<int64_t>(E, P);
+  auto gemm_grid = [&](int n_ntiles) { return dim3((unsigned)(cdiv(max_mtiles * n_ntiles, kF16Dies) * kF16Dies)); };
   a.rscale = g_f16.rs_x;
   a.nkb = (int)f16_block_count(H);
   a.N = (int)F;
   a.ntile = (int)f16_tile_count(F);
   a.out = g_f16.actf;
   if (timed) mark(CSK_STAGE_GATEUP);
-  if (small) expert_f16_kernel<0, 1><<<grid, 256, 0, g_stream>>>(a);
-  else expert_f16_kernel<0, 4><<<grid, 256, 0, g_stream>>>(a);
+  if (small) {
+    expert_f16_kernel<0, 1><<<grid, 256, 0, g_stream>>>(a);
+  } else {
+    ga.list_row = a.list_row, ga.B = a.B, ga.rscale = a.rscale, ga.nkb = a.nkb, ga.N = a.N;
+    ga.ntile = a.ntile, ga.out = a.out;
+    ga.n_ntiles = (int)cdiv(F, 128);
+    expert_f16_gemm_kernel<0><<<gemm_grid(ga.n_ntiles), 256, 0, g_stream>>>(ga);
+  }
   if ((rc = check_launch("expert_f16_kernel<0>")) != CSK_OK) return rc;
   if (timed) mark(CSK_STAGE_DOWN);
   if ((rc = launch_f16_split(g_f16.actf, P, F, nullptr, nullptr, ws.act, g_f16.rs_a)) != CSK_OK) return rc;
@@ -491,8 +504,14 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   a.N = (int)H;
   a.ntile = (int)f16_tile_count(H);
   a.out = ws.y;
-  if (small) expert_f16_kernel<1, 1><<<grid, 256, 0, g_stream>>>(a);
-  else expert_f16_kernel<1, 4><<<grid, 256, 0, g_stream>>>(a);
+  if (small) {
+    expert_f16_kernel<1, 1><<<grid, 256, 0, g_stream>>>(a);
+  } else {
+    ga.list_row = a.list_row, ga.B = a.B, ga.rscale = a.rscale, ga.nkb = a.nkb, ga.N = a.N;
+    ga.ntile = a.ntile, ga.out = a.out;
+    ga.n_ntiles = (int)cdiv(H, 256);
+    expert_f16_gemm_kernel<1><<<gemm_grid(ga.n_ntiles), 256, 0, g_stream>>>(ga);
+  }
   return check_launch("expert_f16_kernel<1>");
 }
 

@@ -311,4 +311,165 @@ __global__ __launch_bounds__(256) void expert_f16_kernel(ExpertF16Args a) {
   }
 }
 
+// ---------------------------------------------------------------- many tokens
+// Grouped GEMM for batches in which an expert sees tens to hundreds of tokens.  A
+// workgroup (4 waves) owns 64 dispatched tokens x 256 weight rows (128 features of gate
+// and up, or 256 rows of down) on v_mfma_f32_32x32x16_f16: tokens are the A operand
+// (accumulator register <-> token), weight rows the B operand (lane % 32 <-> row), so a
+// wave's stores are 128 contiguous bytes per token.  Per K step of 64 the token panel
+// (64 tokens x [hi | lo] = 16 KB) goes through LDS, double buffered, 16-byte chunks
+// XOR-swizzled by token so that the 32 lanes of a fragment read hit distinct banks; the
+// weights go from memory straight to registers, one step ahead, each slice reloaded into
+// the registers it has just been consumed from.  Work units (M tile, N
+// tile) are numbered M-tile major and dealt to the eight dies in contiguous eighths.
+struct ExpertF16GemmArgs {
+  const WorkDesc* desc;
+  const int* mtiles;    // (slot, first token) per 64-token M tile
+  const int* n_mtiles;
+  const int* list_row;  // activation row of a packed position, or null: the position itself
+  const u32x4* B;       // two-term fp16 activation rows
+  const float* rscale;
+  int nkb, N, ntile, n_ntiles, act_type;
+  float* out;
+};
+
+constexpr int kF16Dies = 8;
+
+template <int MODE>
+__global__ __launch_bounds__(256, 3) void expert_f16_gemm_kernel(ExpertF16GemmArgs a) {
+  __shared__ u32x4 panel[2][64 * 16];  // [buffer][token][16 chunks: block 0 hi 0-3, lo 0-3, block 1 ...]
+  __shared__ float rs_sh[64];
+  const int n_units = *a.n_mtiles * a.n_ntiles;
+  const int per_die = (n_units + kF16Dies - 1) / kF16Dies;
+  const int slot_i = blockIdx.x / kF16Dies;
+  const int unit = (blockIdx.x % kF16Dies) * per_die + slot_i;
+  if (slot_i >= per_die || unit >= n_units) return;
+  const int mt = unit / a.n_ntiles, nt = unit - mt * a.n_ntiles;
+  const WorkDesc* wd = a.desc + a.mtiles[2 * mt];
+  const int m0 = a.mtiles[2 * mt + 1];
+  const int base = wd->base + m0;
+  const int mcount = min(64, wd->Te - m0);
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int n32 = lane & 31, kg = lane >> 5;
+  const int n16 = n32 & 15, th = n32 >> 4;
+  const int nkb = a.nkb, nsteps = (nkb + 1) >> 1;
+
+  // this lane's weight entries: row n32 of the wave's two 32-row groups
+  int rows[2];
+  const CSK_GLOBAL u32x4* W[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int t = MODE == 0 ? nt * 8 + wv * 2 + th : nt * 16 + wv * 4 + 2 * s + th;
+    rows[s] = t * 16 + n16;
+    const uint4* q = MODE == 0 ? (s == 0 ? wd->w.q_gate : wd->w.q_up) : wd->w.q_down;
+    W[s] = as_global(reinterpret_cast<const u32x4*>(q)) + (long)min(t, a.ntile - 1) * nkb * 64 + n16 + 16 * kg;
+  }
+  // staging: thread copies chunk sc of tokens st + 16 i
+  const int sc = threadIdx.x & 15, st = threadIdx.x >> 4;
+  const CSK_GLOBAL u32x4* Arow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int pos = base + min(st + 16 * i, mcount - 1);  // tokens past the tile re-read its last
+    const long row = a.list_row ? a.list_row[pos] : pos;
+    Arow[i] = as_global(a.B) + row * nkb * 8 + (sc & 7);
+    if (sc == 0) rs_sh[st + 16 * i] = a.rscale[row];
+  }
+  const int sblk = sc >> 3;  // block of the step this thread's chunk belongs to
+
+  floatx16 acc[2][2];  // [32-token half][row group]
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[ms][s][r] = 0.0f;
+
+  u32x4 wq[2][4];  // [row group][16-wide K slice of the step]
+  u32x4 aq[4];
+  auto load_w = [&](int s, int sl, int j) {
+    const int kb = 2 * j + (sl >> 1);
+    // a block past K (odd block count) contributes nothing
+    wq[s][sl] = kb < nkb ? W[s][(long)kb * 64 + 32 * (sl & 1)] : u32x4{0u, 0u, 0u, 0u};
+  };
+  auto load_a = [&](int j) {
+    const int kbs = min(2 * j + sblk, nkb - 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) aq[i] = Arow[i][(long)kbs * 8];
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int tok = st + 16 * i;
+      panel[buf][tok * 16 + (sc ^ (tok & 15))] = aq[i];
+    }
+  };
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) load_w(s, sl, 0);
+  load_a(0);
+  stash(0);
+  __syncthreads();
+  for (int j = 0; j < nsteps; ++j) {
+    const int buf = j & 1;
+    const bool more = j + 1 < nsteps;
+    if (more) load_a(j + 1);
+#pragma unroll
+    for (int sl = 0; sl < 4; ++sl) {
+      // logical chunk of this lane's 8 halves: block sl / 2, [hi | lo], quarter 2 (sl % 2) + kg
+      const int c_hi = (sl >> 1) * 8 + 2 * (sl & 1) + kg, c_lo = c_hi + 4;
+      half8 hi[2], lo[2];
+#pragma unroll
+      for (int ms = 0; ms < 2; ++ms) {
+        const int tok = ms * 32 + n32;
+        hi[ms] = __builtin_bit_cast(half8, panel[buf][tok * 16 + (c_hi ^ n16)]);
+        lo[ms] = __builtin_bit_cast(half8, panel[buf][tok * 16 + (c_lo ^ n16)]);
+      }
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const half8 w = __builtin_bit_cast(half8, wq[s][sl]);
+#pragma unroll
+        for (int ms = 0; ms < 2; ++ms) {
+          acc[ms][s] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi[ms], w, acc[ms][s], 0, 0, 0);
+          acc[ms][s] = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo[ms], w, acc[ms][s], 0, 0, 0);
+        }
+        // the slice's registers are free as soon as its matrix instructions have issued:
+        // the next step's weights go straight back into them (one register set in rotation)
+        if (more) load_w(s, sl, j + 1);
+      }
+    }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+  // accumulator register r is token (r % 4) + 8 (r / 4) + 4 kg of its 32-token half
+  const CSK_GLOBAL float* b0 = as_global(MODE == 0 ? wd->w.b_gate : wd->w.b_down);
+  const CSK_GLOBAL float* b1 = as_global(MODE == 0 ? wd->w.b_up : wd->w.b_down);
+  float bias[2];
+  bool rv[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    rv[s] = rows[s] < a.N;
+    bias[s] = rv[s] ? (s == 0 ? b0 : b1)[rows[s]] : 0.0f;
+  }
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int tl = ms * 32 + (r & 3) + 8 * (r >> 2) + 4 * kg;
+      if (tl >= mcount) continue;
+      const float sc_t = rs_sh[tl];
+      float* o = a.out + (long)(base + tl) * a.N;
+      if (MODE == 0) {
+        if (rv[0])
+          o[rows[0]] = moe_activation(acc[ms][0][r] * sc_t + bias[0], acc[ms][1][r] * sc_t + bias[1], a.act_type);
+      } else {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+          if (rv[s]) o[rows[s]] = acc[ms][s][r] * sc_t + bias[s];
+      }
+    }
+  }
+}
+
 }  // namespace csk
