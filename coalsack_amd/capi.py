@@ -379,7 +379,7 @@ class Gguf:
         gi = self.tensor_info(f"blk.{block}.ffn_gate_inp.weight")
         up = self.tensor_info(f"blk.{block}.ffn_up_exps.weight")
         return Layer.adopt(self.lib, h, gi["dims"][1], self.get_u32(arch + ".expert_used_count"),
-                           gi["dims"][0], up["dims"][1])
+                           gi["dims"][0], up["dims"][1], f16=up["type"] == 1)
 
 
 class Layer:

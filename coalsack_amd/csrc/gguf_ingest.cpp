@@ -1,5 +1,5 @@
 // GGUF ingest for the MoE path: parses a GGUF file's metadata and tensor table and
-// builds a resident MoE layer (router, MXFP4 experts, biases, FFN norm) for one
+// builds a resident MoE layer (router, MXFP4 or F16 experts, biases, FFN norm) for one
 // transformer block through the public C ABI.  Host-only code.
 //
 // Follows the reference's reader and weight provider:
@@ -296,8 +296,10 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
   for (int i = 0; i < 3; ++i) {
     tw[i] = find(g, p + wn[i]);
     if (!tw[i]) return fail(CSK_ERR_ARG, "Tensor not found: " + p + wn[i]);
-    if (tw[i]->type != kGgmlMxfp4)
-      return fail(CSK_ERR_ARG, p + wn[i] + ": only MXFP4 expert weights are supported on this path");
+    if (tw[i]->type != kGgmlMxfp4 && tw[i]->type != kGgmlF16)
+      return fail(CSK_ERR_ARG, p + wn[i] + ": only MXFP4 and F16 expert weights are supported on this path");
+    if (tw[i]->type != tw[0]->type)
+      return fail(CSK_ERR_ARG, p + ": the three expert tensors must be of one type (all MXFP4 or all F16)");
     if (tw[i]->dims.size() != 3 || tw[i]->dims[2] != E)
       return fail(CSK_ERR_ARG, p + wn[i] + ": expected [K, rows, experts]");
     tb[i] = find(g, p + bn[i]);
@@ -312,16 +314,22 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
   if ((tb[0] != nullptr) != (tb[1] != nullptr) || (tb[0] != nullptr) != (tb[2] != nullptr))
     return fail(CSK_ERR_ARG, p + ": expert biases must be all present or all absent");
 
+  // F16 expert tensors take the node's float16 branch (expert_mlp_node.h:269-389)
+  const bool f16 = tw[0]->type == kGgmlF16;
   csk_layer* L = nullptr;
-  int rc = csk_layer_create(E, k, (int64_t)H, (int64_t)F, &L);
+  int rc = f16 ? csk_layer_create_f16(E, k, (int64_t)H, (int64_t)F, &L)
+               : csk_layer_create(E, k, (int64_t)H, (int64_t)F, &L);
   if (rc != CSK_OK) return rc;
   auto bail = [&](int code, const std::string& msg) {
     csk_layer_destroy(L);
     return msg.empty() ? code : fail(code, msg);
   };
   // gpt-oss: softmax gating, modified SwiGLU, weights applied at the merge;
-  // llama4: sigmoid gating, routing weight applied before the FFN (llm_engine.cpp:145-161)
-  rc = csk_layer_set_options(L, llama4 ? 1 : 0, CSK_ACT_MODIFIED_SWIGLU, llama4 ? 1 : 0);
+  // llama4: sigmoid gating, routing weight applied before the FFN (llm_engine.cpp:145-161);
+  // every architecture but gpt-oss gets the standard SwiGLU (llm_engine.cpp:738-740)
+  rc = csk_layer_set_options(L, llama4 ? 1 : 0,
+                             arch == "gpt-oss" ? CSK_ACT_MODIFIED_SWIGLU : CSK_ACT_STANDARD_SWIGLU,
+                             llama4 ? 1 : 0);
   if (rc != CSK_OK) return bail(rc, "");
 
   std::vector<float> gw((size_t)E * H), gb;
@@ -337,7 +345,9 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
   if (rc != CSK_OK) return bail(rc, "");
 
   // expert e of a stacked tensor starts at offset + e * slice bytes (moe_weight_provider.cpp:160-188)
-  const size_t sl[3] = {(size_t)(F * (H / 32) * 17), (size_t)(F * (H / 32) * 17), (size_t)(H * (F / 32) * 17)};
+  const size_t sl[3] = {f16 ? (size_t)(F * H * 2) : (size_t)(F * (H / 32) * 17),
+                        f16 ? (size_t)(F * H * 2) : (size_t)(F * (H / 32) * 17),
+                        f16 ? (size_t)(H * F * 2) : (size_t)(H * (F / 32) * 17)};
   const size_t bl[3] = {(size_t)F, (size_t)F, (size_t)H};
   std::vector<uint8_t> w[3];
   std::vector<float> b[3];
@@ -352,8 +362,12 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
       if (tb[i] && !read_at(g, tb[i]->offset + (uint64_t)e * bl[i] * 4, b[i].data(), bl[i] * 4))
         return bail(CSK_ERR_ARG, "short read: " + p + bn[i]);
     }
-    rc = csk_layer_set_expert(L, e, w[0].data(), w[1].data(), w[2].data(), tb[0] ? b[0].data() : nullptr,
-                              tb[1] ? b[1].data() : nullptr, tb[2] ? b[2].data() : nullptr);
+    const float* bp[3] = {tb[0] ? b[0].data() : nullptr, tb[1] ? b[1].data() : nullptr,
+                          tb[2] ? b[2].data() : nullptr};
+    rc = f16 ? csk_layer_set_expert_f16(L, e, reinterpret_cast<const uint16_t*>(w[0].data()),
+                                        reinterpret_cast<const uint16_t*>(w[1].data()),
+                                        reinterpret_cast<const uint16_t*>(w[2].data()), bp[0], bp[1], bp[2])
+             : csk_layer_set_expert(L, e, w[0].data(), w[1].data(), w[2].data(), bp[0], bp[1], bp[2]);
     if (rc != CSK_OK) return bail(rc, "");
   }
   const TensorInfo* tn = find(g, p + "." + norm_name);

@@ -52,9 +52,12 @@ def write_gguf(path, metadata, tensors, alignment=32, version=3):
     return len(head) + pad  # start of the tensor data
 
 
-def moe_block_tensors(L, block, bias=True, norm=True, router_bias=True, norm_name="post_attention_norm.weight"):
+def moe_block_tensors(L, block, bias=True, norm=True, router_bias=True, norm_name="post_attention_norm.weight",
+                      f16_weights=None):
     """Tensors of one transformer block's MoE part from synth.LayerInputs, stacked over
-    experts the way the reference's provider slices them (moe_weight_provider.cpp:97-188)."""
+    experts the way the reference's provider slices them (moe_weight_provider.cpp:97-188).
+    f16_weights: per expert (w_up [F,H], w_gate [F,H], w_down [H,F]) float16 arrays, written
+    as F16 tensors instead of the MXFP4 blocks."""
     p = f"blk.{block}"
     t = [(p + ".ffn_gate_inp.weight", GGML_F32, [L.H, L.E], np.ascontiguousarray(L.gate_w, np.float32).tobytes())]
     if router_bias:
@@ -62,8 +65,12 @@ def moe_block_tensors(L, block, bias=True, norm=True, router_bias=True, norm_nam
     names = ["ffn_up_exps", "ffn_gate_exps", "ffn_down_exps"]
     for which, nm in enumerate(names):
         rows, K = (L.F, L.H) if which < 2 else (L.H, L.F)
-        data = b"".join(L.blocks(e, which).tobytes() for e in range(L.E))
-        t.append((f"{p}.{nm}.weight", GGML_MXFP4, [K, rows, L.E], data))
+        if f16_weights is not None:
+            data = b"".join(np.ascontiguousarray(f16_weights[e][which], np.float16).tobytes() for e in range(L.E))
+            t.append((f"{p}.{nm}.weight", GGML_F16, [K, rows, L.E], data))
+        else:
+            data = b"".join(L.blocks(e, which).tobytes() for e in range(L.E))
+            t.append((f"{p}.{nm}.weight", GGML_MXFP4, [K, rows, L.E], data))
         if bias:
             b = (L.b_up, L.b_gate, L.b_down)[which]
             t.append((f"{p}.{nm}.bias", GGML_F32, [rows, L.E], np.ascontiguousarray(b, np.float32).tobytes()))

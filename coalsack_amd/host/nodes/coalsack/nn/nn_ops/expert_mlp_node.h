@@ -1,14 +1,14 @@
 // expert_mlp_node backed by the gfx950 library: same class name, constructor,
 // setters, test wrapper, input order, output conventions and error texts as
 // include/coalsack/nn/nn_ops/expert_mlp_node.h of the reference (cited by line
-// below) for MXFP4 weights; the body calls csk_expert_mlp_mxfp4.
+// below), for both kinds of weights process() distinguishes (:113-136): MXFP4
+// messages go to csk_expert_mlp_mxfp4, float16 tensors to csk_expert_mlp_f16.
 //
 // Weights are uploaded (repacked into the resident device layout) the first
 // time a storage pointer is seen and cached per node: moe_weight_provider
 // hands out the same storage from its own cache on every frame
 // (src/llm/moe_weight_provider.cpp:75-225), so a layer's experts become
-// resident after the first token.  The FP16 branch of the reference node
-// (:269-389) is not part of this path and reports an error.
+// resident after the first token.
 #pragma once
 
 #include <memory>
@@ -36,6 +36,7 @@ class expert_mlp_node : public graph_node {
   }
   ~expert_mlp_node() override {
     for (auto& kv : resident_) csk_mxfp4_free(kv.second.handle);
+    for (auto& kv : resident16_) csk_f16_free(kv.second.handle);
   }
   expert_mlp_node(const expert_mlp_node&) = delete;
   expert_mlp_node& operator=(const expert_mlp_node&) = delete;
@@ -48,6 +49,11 @@ class expert_mlp_node : public graph_node {
   void set_activation_type(activation_type t) { activation_type_ = t; }
   activation_type get_activation_type() const { return activation_type_; }
   void set_weight_before_ffn(bool v) { weight_before_ffn_ = v; }  // :52
+  std::vector<std::string> get_input_names() const { return input_names_; }
+  std::string get_output_name() const { return output_name_; }
+
+  // Public wrapper for testing (:57-60): the float16 branch on plain tensors.
+  dynamic_tensor compute_test(const std::vector<dynamic_tensor>& inputs) { return compute_fp16(inputs); }
 
   // One token through raw 17-byte-block weights (:63-70).
   void compute_test_mxfp4(const float* hidden_vec, const uint8_t* w_up_data, const uint8_t* w_gate_data,
@@ -82,10 +88,19 @@ class expert_mlp_node : public graph_node {
           if (!f) throw std::runtime_error("expert_mlp: missing field " + name);
           fields.push_back(f);
         }
-        if (fields.size() < 2 || !std::dynamic_pointer_cast<dynamic_mx_tensor_message>(fields[1]))
-          throw std::runtime_error("expert_mlp: only MXFP4 weights are supported on the GPU path");
-        out = result_message::ok(
-            {{output_name_, std::make_shared<dynamic_tensor_message>(compute_with_mxfp4(fields))}});
+        dynamic_tensor result;
+        if (fields.size() > 1 && std::dynamic_pointer_cast<dynamic_mx_tensor_message>(fields[1])) {
+          result = compute_with_mxfp4(fields);
+        } else {  // :120-130
+          std::vector<dynamic_tensor> inputs;
+          for (const auto& f : fields) {
+            auto t = std::dynamic_pointer_cast<dynamic_tensor_message>(f);
+            if (!t) throw std::runtime_error("expert_mlp: expected dynamic_tensor_message");
+            inputs.push_back(t->get_tensor());
+          }
+          result = compute_fp16(inputs);
+        }
+        out = result_message::ok({{output_name_, std::make_shared<dynamic_tensor_message>(result)}});
       } catch (const std::exception& e) {
         out = result_message::error({{output_name_, nullptr}}, e.what());
       }
@@ -120,6 +135,104 @@ class expert_mlp_node : public graph_node {
       throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
     resident_[key] = resident{h, t.dim(0), t.dim(1)};
     return h;
+  }
+
+  struct resident16 {
+    csk_f16* handle;
+    int64_t rows, cols;
+  };
+
+  csk_f16* resident_copy16(const dynamic_tensor& t) {
+    const uint16_t* key = t.data_ptr<uint16_t>();
+    auto it = resident16_.find(key);
+    if (it != resident16_.end() && it->second.rows == t.dim(0) && it->second.cols == t.dim(1))
+      return it->second.handle;
+    if (it != resident16_.end()) {
+      csk_f16_free(it->second.handle);
+      resident16_.erase(it);
+    }
+    csk_f16* h = nullptr;
+    if (csk_f16_upload(key, t.dim(0), t.dim(1), &h) != CSK_OK)
+      throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
+    resident16_[key] = resident16{h, t.dim(0), t.dim(1)};
+    return h;
+  }
+
+  static std::string dims2(int64_t a, int64_t b) {
+    return "[" + std::to_string(a) + ", " + std::to_string(b) + "]";
+  }
+
+  dynamic_tensor compute_fp16(const std::vector<dynamic_tensor>& inputs) {  // :269-389
+    if (inputs.size() != 5 && inputs.size() != 8)
+      throw std::runtime_error(
+          "expert_mlp: expected 5 or 8 inputs (hidden, w_up, w_gate, w_down[, b_up, b_gate, "
+          "b_down], router_output), got " +
+          std::to_string(inputs.size()));
+    const bool has_bias = inputs.size() == 8;
+    const dynamic_tensor& hidden = inputs[0];
+    const dynamic_tensor& w_up = inputs[1];
+    const dynamic_tensor& w_gate = inputs[2];
+    const dynamic_tensor& w_down = inputs[3];
+    const dynamic_tensor& router = inputs[has_bias ? 7 : 4];
+    if (router.ndim() != 4 || router.dim(3) != 2)
+      throw std::runtime_error("expert_mlp: router_output must be 4D [batch, seq_len, top_k, 2], got " +
+                               std::to_string(router.ndim()) + "D");
+    if (router.get_dtype() != dtype::float32)
+      throw std::runtime_error("expert_mlp: router_output must be float32");
+    // not selected by any token: a {0}-shaped tensor, before anything else is looked at (:297-306)
+    const int64_t top_k = router.dim(2);
+    const float* rp = router.data_ptr<float>();
+    bool any = false;
+    for (int64_t p = 0; p < router.dim(0) * router.dim(1) * top_k && !any; ++p)
+      any = static_cast<int>(rp[2 * p]) == expert_id_;
+    if (!any) return dynamic_tensor(dtype::float32, {0});
+    if (hidden.ndim() != 3)
+      throw std::runtime_error("expert_mlp: hidden_states must be 3D [batch, seq_len, hidden_dim], got " +
+                               std::to_string(hidden.ndim()) + "D");
+    const int64_t tokens = hidden.dim(0) * hidden.dim(1), hidden_dim = hidden.dim(2);
+    if (w_up.ndim() != 2 || w_gate.ndim() != 2 || w_down.ndim() != 2)
+      throw std::runtime_error(
+          "expert_mlp: all weights must be 2D [expert_ffn_dim, hidden_dim] or [hidden_dim, "
+          "expert_ffn_dim]");
+    const int64_t ffn = w_up.dim(0);
+    if (w_up.dim(1) != hidden_dim)
+      throw std::runtime_error("expert_mlp: w_up must be " + dims2(ffn, hidden_dim) + ", got " +
+                               dims2(w_up.dim(0), w_up.dim(1)));
+    if (w_gate.dim(0) != ffn || w_gate.dim(1) != hidden_dim)
+      throw std::runtime_error("expert_mlp: w_gate must be " + dims2(ffn, hidden_dim) + ", got " +
+                               dims2(w_gate.dim(0), w_gate.dim(1)));
+    if (w_down.dim(0) != hidden_dim || w_down.dim(1) != ffn)
+      throw std::runtime_error("expert_mlp: w_down must be " + dims2(hidden_dim, ffn) + ", got " +
+                               dims2(w_down.dim(0), w_down.dim(1)));
+    if (has_bias) {
+      const dynamic_tensor &b_up = inputs[4], &b_gate = inputs[5], &b_down = inputs[6];
+      if (b_up.ndim() != 1 || b_up.dim(0) != ffn)
+        throw std::runtime_error("expert_mlp: b_up must be [expert_ffn_dim=" + std::to_string(ffn) +
+                                 "], got [" + std::to_string(b_up.dim(0)) + "]");
+      if (b_gate.ndim() != 1 || b_gate.dim(0) != ffn)
+        throw std::runtime_error("expert_mlp: b_gate must be [expert_ffn_dim=" + std::to_string(ffn) +
+                                 "], got [" + std::to_string(b_gate.dim(0)) + "]");
+      if (b_down.ndim() != 1 || b_down.dim(0) != hidden_dim)
+        throw std::runtime_error("expert_mlp: b_down must be [hidden_dim=" + std::to_string(hidden_dim) +
+                                 "], got [" + std::to_string(b_down.dim(0)) + "]");
+    }
+    if (w_up.get_dtype() != dtype::float16 || w_gate.get_dtype() != dtype::float16 ||
+        w_down.get_dtype() != dtype::float16)
+      throw std::runtime_error("expert_mlp: all weights must be FLOAT16");
+    if (hidden.get_dtype() != dtype::float32)
+      throw std::runtime_error("expert_mlp: hidden_states must be FLOAT32");
+
+    dynamic_tensor output(dtype::float32, hidden.shape());
+    int is_empty = 0;
+    const int rc = csk_expert_mlp_f16(
+        expert_id_, hidden.data_ptr<float>(), tokens, hidden_dim, ffn, resident_copy16(w_up),
+        resident_copy16(w_gate), resident_copy16(w_down),
+        has_bias ? inputs[4].data_ptr<float>() : nullptr, has_bias ? inputs[5].data_ptr<float>() : nullptr,
+        has_bias ? inputs[6].data_ptr<float>() : nullptr, rp, top_k, act_code(),
+        weight_before_ffn_ ? 1 : 0, output.data_ptr<float>(), &is_empty);
+    if (rc != CSK_OK) throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
+    if (is_empty) return dynamic_tensor(dtype::float32, {0});
+    return output;
   }
 
   dynamic_tensor compute_with_mxfp4(const std::vector<graph_message_ptr>& msgs) {  // :392-485
@@ -195,6 +308,7 @@ class expert_mlp_node : public graph_node {
   activation_type activation_type_ = activation_type::MODIFIED_SWIGLU;
   bool weight_before_ffn_ = false;
   std::unordered_map<const uint8_t*, resident> resident_;
+  std::unordered_map<const uint16_t*, resident16> resident16_;
 };
 
 }  // namespace coalsack

@@ -27,6 +27,9 @@ int orc_expert_mlp_mxfp4(int, const float*, int64_t, int64_t, int64_t, const uin
                          const uint8_t*, const float*, const float*, const float*, const float*, int64_t,
                          int, int, float*, int*);
 int orc_expert_merge(const float*, int64_t, int64_t, int64_t, int64_t, const float* const*, int, float*);
+int orc_expert_mlp_f16(int, const float*, int64_t, int64_t, int64_t, const uint16_t*, const uint16_t*,
+                       const uint16_t*, const float*, const float*, const float*, const float*, int64_t, int,
+                       int, float*, int*);
 void orc_rmsnorm(const float*, const float*, float*, int64_t, int64_t, float);
 void orc_add(const float*, const float*, float*, int64_t);
 }
@@ -149,6 +152,80 @@ static void cpu_expert_node_paths() {
   node.set_input_names({"hidden", "w_up", "w_gate", "w_down"});
   node.process("default", msg);
   CHECK(cap.got[4]->is_error() && cap.got[4]->get_error_message() == "expert_mlp: expected 5 or 8 inputs for MXFP4, got 4");
+}
+
+// float32 -> IEEE half bits, round to nearest even (test data only)
+static uint16_t half_bits(float f) {
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  const int32_t e = (int32_t)((x >> 23) & 0xff) - 127 + 15;
+  uint32_t m = x & 0x7fffffu;
+  if (e >= 31) return (uint16_t)(sign | 0x7c00u);
+  if (e <= 0) {
+    if (e < -10) return (uint16_t)sign;
+    m |= 0x800000u;
+    const int sh = 14 - e;
+    uint32_t h = m >> sh;
+    const uint32_t rem = m & ((1u << sh) - 1), half = 1u << (sh - 1);
+    if (rem > half || (rem == half && (h & 1))) ++h;
+    return (uint16_t)(sign | h);
+  }
+  uint32_t h = ((uint32_t)e << 10) | (m >> 13);
+  const uint32_t rem = m & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1))) ++h;
+  return (uint16_t)(sign | h);
+}
+
+static dynamic_tensor random_half_tensor(const std::vector<int64_t>& shape, std::mt19937& gen, float lo, float hi) {
+  dynamic_tensor t(dtype::float16, shape);
+  std::uniform_real_distribution<float> d(lo, hi);
+  uint16_t* p = t.data_ptr<uint16_t>();
+  for (int64_t i = 0; i < t.numel(); ++i) p[i] = half_bits(d(gen));
+  return t;
+}
+
+static dynamic_tensor router_first_slot(int64_t B, int64_t S, int64_t K, int first_expert) {
+  // test/test_expert_mlp.cpp:84-95: slot 0 names first_expert, slot k names expert k, weights 1 / top_k
+  dynamic_tensor r(dtype::float32, {B, S, K, 2});
+  float* p = r.data_ptr<float>();
+  for (int64_t t = 0; t < B * S; ++t)
+    for (int64_t k = 0; k < K; ++k) {
+      p[(t * K + k) * 2] = k == 0 ? (float)first_expert : (float)k;
+      p[(t * K + k) * 2 + 1] = 1.0f / (float)K;
+    }
+  return r;
+}
+
+static void cpu_expert_fp16_argument_errors() {
+  std::printf("expert_mlp (float16 weights): argument errors, unselected expert\n");
+  std::mt19937 gen(3);
+  expert_mlp_node node(0);
+  auto hidden = random_tensor({1, 2, 8}, gen, -1, 1);
+  auto w_up = random_half_tensor({16, 8}, gen, -0.1f, 0.1f), w_gate = random_half_tensor({16, 8}, gen, -0.1f, 0.1f);
+  auto w_down = random_half_tensor({8, 16}, gen, -0.1f, 0.1f);
+  auto router = router_first_slot(1, 2, 4, 0);
+  CHECK(throws_with([&] { node.compute_test({hidden, w_up, w_gate, router}); },
+                    "expert_mlp: expected 5 or 8 inputs (hidden, w_up, w_gate, w_down[, b_up, b_gate, b_down], router_output), got 4"));
+  CHECK(throws_with([&] { node.compute_test({hidden, w_up, w_gate, w_down, dynamic_tensor(dtype::float32, {1, 2, 8})}); },
+                    "expert_mlp: router_output must be 4D [batch, seq_len, top_k, 2], got 3D"));
+  CHECK(throws_with([&] { node.compute_test({dynamic_tensor(dtype::float32, {2, 8}), w_up, w_gate, w_down, router}); },
+                    "expert_mlp: hidden_states must be 3D [batch, seq_len, hidden_dim], got 2D"));
+  CHECK(throws_with([&] { node.compute_test({hidden, random_half_tensor({16, 7}, gen, -1, 1), w_gate, w_down, router}); },
+                    "expert_mlp: w_up must be [16, 8], got [16, 7]"));
+  CHECK(throws_with([&] { node.compute_test({hidden, w_up, random_half_tensor({15, 8}, gen, -1, 1), w_down, router}); },
+                    "expert_mlp: w_gate must be [16, 8], got [15, 8]"));
+  CHECK(throws_with([&] { node.compute_test({hidden, w_up, w_gate, random_half_tensor({8, 15}, gen, -1, 1), router}); },
+                    "expert_mlp: w_down must be [8, 16], got [8, 15]"));
+  CHECK(throws_with([&] { node.compute_test({hidden, w_up, w_gate, w_down, random_tensor({15}, gen, 0, 1),
+                                             random_tensor({16}, gen, 0, 1), random_tensor({8}, gen, 0, 1), router}); },
+                    "expert_mlp: b_up must be [expert_ffn_dim=16], got [15]"));
+  CHECK(throws_with([&] { node.compute_test({hidden, random_tensor({16, 8}, gen, -1, 1), w_gate, w_down, router}); },
+                    "expert_mlp: all weights must be FLOAT16"));
+  // an expert no token selected returns the {0}-shaped tensor before any shape is looked at (:297-306)
+  expert_mlp_node other(9);
+  auto out = other.compute_test({dynamic_tensor(dtype::float32, {2, 8}), w_up, w_gate, w_down, router});
+  CHECK(out.ndim() == 1 && out.dim(0) == 0);
 }
 
 static void cpu_merge_argument_errors() {
@@ -309,6 +386,78 @@ static void gpu_expert_known_answer() {
   for (int i = 0; i < H; ++i) CHECK(std::fabs(out[i] - want2) < 1e-3f);
 }
 
+// The reference's four float16 tests (test/test_expert_mlp.cpp) on the GPU node, each
+// also compared with the CPU checker.
+static void gpu_expert_fp16_tests() {
+  std::printf("expert_mlp (float16 weights): Basic, ModifiedSwigluActivation, MultipleExperts, GptOssScale\n");
+  std::mt19937 gen(42);
+  auto run_case = [&](int expert_id, int64_t B, int64_t S, int64_t H, int64_t F, int64_t K, bool through_messages) {
+    auto hidden = random_tensor({B, S, H}, gen, -0.5f, 0.5f);
+    auto w_up = random_half_tensor({F, H}, gen, -0.1f, 0.1f), w_gate = random_half_tensor({F, H}, gen, -0.1f, 0.1f);
+    auto w_down = random_half_tensor({H, F}, gen, -0.1f, 0.1f);
+    auto b_up = random_tensor({F}, gen, -0.05f, 0.05f), b_gate = random_tensor({F}, gen, -0.05f, 0.05f);
+    auto b_down = random_tensor({H}, gen, -0.05f, 0.05f);
+    auto router = router_first_slot(B, S, K, expert_id);
+    expert_mlp_node node(expert_id);
+    CHECK(node.get_expert_id() == expert_id);
+    dynamic_tensor out;
+    if (through_messages) {
+      node.set_input_names({"hidden", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "router"});
+      node.set_output_name("out");
+      capture_node cap;
+      cap.set_input(node.get_output());
+      auto mk = [](const dynamic_tensor& t) { return std::make_shared<dynamic_tensor_message>(t); };
+      node.process("default", result_message::ok({{"hidden", mk(hidden)}, {"w_up", mk(w_up)}, {"w_gate", mk(w_gate)},
+                                                  {"w_down", mk(w_down)}, {"b_up", mk(b_up)}, {"b_gate", mk(b_gate)},
+                                                  {"b_down", mk(b_down)}, {"router", mk(router)}}));
+      CHECK(cap.got.size() == 1 && cap.got[0]->is_ok());
+      out = std::dynamic_pointer_cast<dynamic_tensor_message>(cap.got[0]->get_field("out"))->get_tensor();
+    } else {
+      out = node.compute_test({hidden, w_up, w_gate, w_down, b_up, b_gate, b_down, router});
+    }
+    CHECK(out.shape() == hidden.shape());
+    bool nonzero = false, nan = false;
+    for (int64_t i = 0; i < out.numel(); ++i) {
+      nonzero |= std::fabs(out.data_ptr<float>()[i]) > 1e-6f;
+      nan |= std::isnan(out.data_ptr<float>()[i]);
+    }
+    CHECK(nonzero && !nan);
+    std::vector<float> want(B * S * H);
+    int empty = 0;
+    orc_expert_mlp_f16(expert_id, hidden.data_ptr<float>(), B * S, H, F, w_up.data_ptr<uint16_t>(),
+                       w_gate.data_ptr<uint16_t>(), w_down.data_ptr<uint16_t>(), b_up.data_ptr<float>(),
+                       b_gate.data_ptr<float>(), b_down.data_ptr<float>(), router.data_ptr<float>(), K, 0, 0,
+                       want.data(), &empty);
+    float worst = 0;
+    for (int64_t i = 0; i < out.numel(); ++i)
+      worst = std::fmax(worst, std::fabs(out.data_ptr<float>()[i] - want[i]) / std::fmax(1.0f, std::fabs(want[i])));
+    CHECK(!empty && worst <= 1e-3f);
+    return worst;
+  };
+  run_case(0, 1, 2, 8, 16, 4, false);                                  // Basic (:49-115)
+  for (int e : {0, 5, 15, 31}) run_case(e, 1, 1, 8, 16, 4, e == 5);     // MultipleExperts (:203-276)
+  const float w = run_case(0, 2, 4, 128, 128, 4, true);                 // GptOssScale (:279-354)
+  std::printf("  GptOssScale: max rel err against the CPU path %.3g\n", w);
+  // ModifiedSwigluActivation (:118-200): hidden_dim = expert_ffn_dim = 2
+  dynamic_tensor hidden(dtype::float32, {1, 1, 2});
+  hidden.data_ptr<float>()[0] = 1.0f, hidden.data_ptr<float>()[1] = 0.5f;
+  dynamic_tensor w_up(dtype::float16, {2, 2}), w_gate(dtype::float16, {2, 2}), w_down(dtype::float16, {2, 2});
+  dynamic_tensor b_up(dtype::float32, {2}), b_gate(dtype::float32, {2}), b_down(dtype::float32, {2});
+  for (auto* t : {&w_up, &w_gate, &w_down}) std::memset(t->data_ptr<uint16_t>(), 0, 8);
+  for (auto* t : {&b_up, &b_gate, &b_down}) std::memset(t->data_ptr<float>(), 0, 8);
+  w_up.data_ptr<uint16_t>()[0] = half_bits(1.0f);
+  b_up.data_ptr<float>()[0] = 0.5f;
+  w_gate.data_ptr<uint16_t>()[0] = half_bits(1.0f);
+  w_down.data_ptr<uint16_t>()[0] = half_bits(1.0f);
+  w_down.data_ptr<uint16_t>()[2] = half_bits(1.0f);
+  dynamic_tensor router(dtype::float32, {1, 1, 4, 2});
+  for (int k = 0; k < 4; ++k) router.data_ptr<float>()[2 * k] = (float)k, router.data_ptr<float>()[2 * k + 1] = k == 0;
+  expert_mlp_node node(0);
+  auto out = node.compute_test({hidden, w_up, w_gate, w_down, b_up, b_gate, b_down, router});
+  const float want = 1.0f / (1.0f + std::exp(1.702f * -1.0f)) * (1.5f + 1.0f);
+  CHECK(std::fabs(out.data_ptr<float>()[0] - want) < 1e-3f);
+}
+
 // router -> E expert nodes -> merge, wired with edges and result messages the way
 // llm_engine builds the block (src/llm/llm_engine.cpp:721-753), against the CPU checker.
 static void gpu_node_chain() {
@@ -401,11 +550,13 @@ int main(int argc, char** argv) {
     }
     gpu_router_tests();
     gpu_expert_known_answer();
+    gpu_expert_fp16_tests();
     gpu_node_chain();
     gpu_norm_add_tests();
   } else {
     cpu_router_argument_errors();
     cpu_expert_node_paths();
+    cpu_expert_fp16_argument_errors();
     cpu_merge_argument_errors();
     cpu_norm_add_argument_errors();
   }

@@ -108,15 +108,56 @@ def test_layer_from_gguf_llama4_switches_and_errors(lib, oracle, tmp_path):
     with lib.gguf(path) as g, g.layer(0) as layer:
         got = layer.forward(hidden, capi.FWD_RMSNORM)
     L.gate_b = np.zeros(E, np.float32)
-    want, _ = oracle_layer(oracle, L, hidden, bias=False, norm=True, sigmoid=True, weight_before_ffn=True)
+    # llama4: sigmoid gating, weight before the FFN, standard SwiGLU (llm_engine.cpp:145-161, 738-740)
+    want, _ = oracle_layer(oracle, L, hidden, bias=False, norm=True, sigmoid=True, weight_before_ffn=True,
+                           act=1)
     assert_layer_close(got, want)
-    # an F16 expert tensor is refused, not misread
-    bad = [(n, (gw.GGML_F16 if n.endswith("ffn_up_exps.weight") else t), d, b)
-           for n, t, d, b in gw.moe_block_tensors(L, 0, bias=False, router_bias=False)]
-    bad[1] = (bad[1][0], gw.GGML_F16, bad[1][2], np.zeros(E * F * H, np.float16).tobytes())
-    gw.write_gguf(str(tmp_path / "f16.gguf"), _meta(E=E, k=k), bad)
-    with lib.gguf(str(tmp_path / "f16.gguf")) as g:
-        with pytest.raises(capi.CskError, match="only MXFP4"):
+    # expert tensors of mixed or unsupported types are refused, not misread
+    mixed = gw.moe_block_tensors(L, 0, bias=False, router_bias=False)
+    mixed[1] = (mixed[1][0], gw.GGML_F16, mixed[1][2], np.zeros(E * F * H, np.float16).tobytes())
+    gw.write_gguf(str(tmp_path / "mixed.gguf"), _meta(E=E, k=k), mixed)
+    # Q4_K: 144 bytes per 256 elements
+    q4 = [(n, 12, d, bytes(int(np.prod(d)) // 256 * 144)) if "_exps.weight" in n else (n, t, d, b)
+          for n, t, d, b in gw.moe_block_tensors(L, 0, bias=False, router_bias=False)]
+    gw.write_gguf(str(tmp_path / "q4k.gguf"), _meta(E=E, k=k), q4)
+    with lib.gguf(str(tmp_path / "mixed.gguf")) as g:
+        with pytest.raises(capi.CskError, match="must be of one type"):
             g.layer(0)
         with pytest.raises(capi.CskError, match="Tensor not found"):
             g.layer(3)
+    with lib.gguf(str(tmp_path / "q4k.gguf")) as g:
+        with pytest.raises(capi.CskError, match="only MXFP4 and F16"):
+            g.layer(0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T", [5, 90])
+def test_layer_from_gguf_f16_experts(lib, oracle, tmp_path, T):
+    """A block whose expert tensors are F16: the file-built layer holds the file's halves,
+    equals a layer built through csk_layer_set_expert_f16 bit for bit, and matches the CPU
+    path's float16 branch."""
+    from tests.test_oracle_expert_f16 import random_f16_expert
+    E, k, H, F = 6, 2, 96, 160
+    L = synth.LayerInputs(E, k, H, F, seed=41, with_norm=True)
+    rng = np.random.default_rng(41)
+    ws = [random_f16_expert(rng, H, F, 0.1) for _ in range(E)]
+    path = str(tmp_path / "f16.gguf")
+    gw.write_gguf(path, _meta(E=E, k=k), gw.moe_block_tensors(L, 0, f16_weights=ws))
+    hidden = synth.hidden_states(T, H, seed=5)
+    flags = capi.FWD_RMSNORM | capi.FWD_RESIDUAL
+    with lib.gguf(path) as g:
+        with g.layer(0) as layer, lib.layer(E, k, H, F, f16=True) as hand:
+            assert layer.f16 and (layer.E, layer.k, layer.H, layer.F) == (E, k, H, F)
+            hand.set_router(L.gate_w, L.gate_b)
+            hand.set_norm(L.norm_w, 1e-5)
+            for e in range(E):
+                hand.set_expert_f16(e, *ws[e], L.b_up[e], L.b_gate[e], L.b_down[e])
+                for which in range(3):
+                    assert np.array_equal(layer.export_f16(e, which).view(np.uint16),
+                                          ws[e][which].view(np.uint16))
+            got = layer.forward(hidden, flags)
+            assert nbits_differ(got, hand.forward(hidden, flags)) == 0
+    want, _ = oracle.moe_layer(hidden, E, k, H, F, L.gate_w, L.gate_b, np.stack([w[0] for w in ws]),
+                               np.stack([w[1] for w in ws]), np.stack([w[2] for w in ws]), L.b_up,
+                               L.b_gate, L.b_down, norm_w=L.norm_w, norm_eps=1e-5, residual=True)
+    assert_layer_close(got, want)
