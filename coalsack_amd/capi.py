@@ -41,11 +41,13 @@ SIGNATURES = {
     "csk_mxfp4_dequant": (C.c_int, [_P, _P]),
     "csk_mxfp4_export": (C.c_int, [_P, _P]),
     "csk_f16_upload": (C.c_int, [_P, _I64, _I64, C.POINTER(_P)]),
+    "csk_f16_upload_ggml": (C.c_int, [C.c_int, _P, _I64, _I64, C.POINTER(_P)]),
     "csk_f16_free": (None, [_P]),
     "csk_f16_export": (C.c_int, [_P, _P]),
     "csk_layer_create": (C.c_int, [_I64, _I64, _I64, _I64, C.POINTER(_P)]),
     "csk_layer_create_f16": (C.c_int, [_I64, _I64, _I64, _I64, C.POINTER(_P)]),
     "csk_layer_set_expert_f16": (C.c_int, [_P, _I64, _P, _P, _P, _P, _P, _P]),
+    "csk_layer_set_expert_matrix": (C.c_int, [_P, _I64, C.c_int, C.c_int, _P]),
     "csk_layer_export_f16": (C.c_int, [_P, _I64, C.c_int, _P]),
     "csk_layer_destroy": (None, [_P]),
     "csk_layer_set_options": (C.c_int, [_P, C.c_int, C.c_int, C.c_int]),
@@ -221,6 +223,13 @@ class Library:
         self.check(self.dll.csk_f16_upload(_ptr(w), rows, K, C.byref(h)))
         return h
 
+    def f16_upload_ggml(self, ggml_type, data, rows, K):
+        """data: uint8 stream of a [rows, K] matrix stored as ggml F16 (1), Q4_K (12) or Q6_K (14)."""
+        data = _u8(data)
+        h = _P()
+        self.check(self.dll.csk_f16_upload_ggml(ggml_type, _ptr(data), rows, K, C.byref(h)))
+        return h
+
     def f16_free(self, h):
         self.dll.csk_f16_free(h)
 
@@ -379,7 +388,7 @@ class Gguf:
         gi = self.tensor_info(f"blk.{block}.ffn_gate_inp.weight")
         up = self.tensor_info(f"blk.{block}.ffn_up_exps.weight")
         return Layer.adopt(self.lib, h, gi["dims"][1], self.get_u32(arch + ".expert_used_count"),
-                           gi["dims"][0], up["dims"][1], f16=up["type"] == 1)
+                           gi["dims"][0], up["dims"][1], f16=up["type"] != 39)
 
 
 class Layer:
@@ -436,6 +445,10 @@ class Layer:
         self.lib.check(self.lib.dll.csk_layer_set_expert_f16(
             self.h, e, _ptr(w_up), _ptr(w_gate), _ptr(w_down), _ptr(b_up), _ptr(b_gate),
             _ptr(b_down)))
+
+    def set_expert_matrix(self, e, which, ggml_type, data):
+        data = _u8(data)
+        self.lib.check(self.lib.dll.csk_layer_set_expert_matrix(self.h, e, which, ggml_type, _ptr(data)))
 
     def export_f16(self, e, which):
         rows, K = (self.H, self.F) if which == W_DOWN else (self.F, self.H)

@@ -194,7 +194,7 @@ struct csk_layer {
   float* bias_all = nullptr;  // [E][F gate | F up | H down]
   ExpertW* ew_dev = nullptr;
   std::vector<ExpertW> ew_host;
-  std::vector<char> expert_set, expert_bias;
+  std::vector<char> expert_set, expert_bias, matrix_set;
   float* norm_w = nullptr;
   float eps = 1e-5f;
   bool has_norm = false;
@@ -710,6 +710,7 @@ static int layer_create(int64_t E, int64_t k, int64_t H, int64_t F, bool f16, cs
   L->nblkH = H / 32, L->nblkF = F / 32, L->ntF = cdiv(F, 16), L->ntH = cdiv(H, 16);
   L->expert_set.assign((size_t)E, 0);
   L->expert_bias.assign((size_t)E, 0);
+  L->matrix_set.assign((size_t)E, 0);
   L->ew_host.assign((size_t)E, ExpertW{});
   rc = dev_alloc(&L->gate_w, (size_t)E * H);
   if (rc == CSK_OK) rc = dev_alloc(&L->gate_b, (size_t)E);
@@ -910,17 +911,34 @@ struct csk_f16 {
 };
 
 namespace {
-// row-major halves on the host -> tiles at dst
-int f16_pack_into(const uint16_t* halves, int64_t rows, int64_t K, u32x4* dst) {
-  uint16_t* stage = nullptr;
+constexpr int kGgmlF16Type = 1;
+// bytes of a row-major [rows, K] matrix stored as ggml type F16, Q4_K or Q6_K; 0 = unsupported
+size_t ggml_matrix_bytes(int type, int64_t rows, int64_t K) {
   const size_t n = (size_t)rows * K;
-  HIP_TRY(hipMalloc((void**)&stage, n * sizeof(uint16_t)));
-  hipError_t e = hipMemcpyAsync(stage, halves, n * sizeof(uint16_t), hipMemcpyHostToDevice, g_stream);
+  if (type == kGgmlF16Type) return n * 2;
+  if (type == kGgmlQ4K) return n % 256 ? 0 : n / 256 * 144;
+  if (type == kGgmlQ6K) return n % 256 ? 0 : n / 256 * 210;
+  return 0;
+}
+// row-major matrix on the host (halves, or a Q4_K / Q6_K stream) -> fp16 tiles at dst
+int f16_pack_into(const void* data, int type, int64_t rows, int64_t K, u32x4* dst) {
+  const size_t bytes = ggml_matrix_bytes(type, rows, K);
+  if (!bytes)
+    return fail(CSK_ERR_ARG, "fp16 experts take ggml types F16 (1), Q4_K (12) and Q6_K (14), K-quants with rows * K a multiple of 256");
+  uint8_t* stage = nullptr;
+  HIP_TRY(hipMalloc((void**)&stage, bytes));
+  hipError_t e = hipMemcpyAsync(stage, data, bytes, hipMemcpyHostToDevice, g_stream);
   int rc = CSK_OK;
   if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("hipMemcpy: ") + hipGetErrorString(e));
   if (rc == CSK_OK) {
     const long ent = f16_entries(rows, K);
-    f16_pack_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(stage, dst, rows, K, ent);
+    const dim3 grid((unsigned)cdiv(ent, 256));
+    if (type == kGgmlF16Type)
+      f16_pack_kernel<<<grid, 256, 0, g_stream>>>(reinterpret_cast<const uint16_t*>(stage), dst, rows, K, ent);
+    else if (type == kGgmlQ4K)
+      kquant_pack_kernel<kGgmlQ4K><<<grid, 256, 0, g_stream>>>(stage, dst, rows, K, ent);
+    else
+      kquant_pack_kernel<kGgmlQ6K><<<grid, 256, 0, g_stream>>>(stage, dst, rows, K, ent);
     rc = check_launch("f16_pack_kernel");
   }
   (void)hipStreamSynchronize(g_stream);
@@ -953,7 +971,24 @@ extern "C" int csk_f16_upload(const uint16_t* halves, int64_t rows, int64_t K, c
   csk_f16* m = new csk_f16;
   m->rows = rows, m->K = K;
   int rc = dev_alloc(&m->w, (size_t)f16_entries(rows, K));
-  if (rc == CSK_OK) rc = f16_pack_into(halves, rows, K, m->w);
+  if (rc == CSK_OK) rc = f16_pack_into(halves, kGgmlF16Type, rows, K, m->w);
+  if (rc != CSK_OK) {
+    csk_f16_free(m);
+    return rc;
+  }
+  *out = m;
+  return CSK_OK;
+}
+extern "C" int csk_f16_upload_ggml(int ggml_type, const void* data, int64_t rows, int64_t K, csk_f16** out) {
+  REQUIRE_INIT();
+  if (!data || !out || rows <= 0 || K <= 0)
+    return fail(CSK_ERR_ARG, "csk_f16_upload_ggml: need a matrix with rows > 0 and K > 0");
+  if (rows > (int64_t)kZeroLen || K > (int64_t)kZeroLen)
+    return fail(CSK_ERR_ARG, "csk_f16_upload_ggml: dimensions above 65536 are not supported");
+  csk_f16* m = new csk_f16;
+  m->rows = rows, m->K = K;
+  int rc = dev_alloc(&m->w, (size_t)f16_entries(rows, K));
+  if (rc == CSK_OK) rc = f16_pack_into(data, ggml_type, rows, K, m->w);
   if (rc != CSK_OK) {
     csk_f16_free(m);
     return rc;
@@ -982,13 +1017,27 @@ extern "C" int csk_layer_set_expert_f16(csk_layer* L, int64_t e, const uint16_t*
   if ((w_up == nullptr) != (w_gate == nullptr) || (w_up == nullptr) != (w_down == nullptr))
     return fail(CSK_ERR_ARG, "weights must be all present or all absent");
   if (w_up) {
-    int rc = f16_pack_into(w_up, L->F, L->H, L->view16(e, CSK_W_UP));
-    if (rc == CSK_OK) rc = f16_pack_into(w_gate, L->F, L->H, L->view16(e, CSK_W_GATE));
-    if (rc == CSK_OK) rc = f16_pack_into(w_down, L->H, L->F, L->view16(e, CSK_W_DOWN));
+    int rc = f16_pack_into(w_up, kGgmlF16Type, L->F, L->H, L->view16(e, CSK_W_UP));
+    if (rc == CSK_OK) rc = f16_pack_into(w_gate, kGgmlF16Type, L->F, L->H, L->view16(e, CSK_W_GATE));
+    if (rc == CSK_OK) rc = f16_pack_into(w_down, kGgmlF16Type, L->H, L->F, L->view16(e, CSK_W_DOWN));
     if (rc != CSK_OK) return rc;
+    L->matrix_set[(size_t)e] = 7;
     L->expert_set[(size_t)e] = 1;
   }
   return upload_biases(L, e, b_up, b_gate, b_down);
+}
+extern "C" int csk_layer_set_expert_matrix(csk_layer* L, int64_t e, int which, int ggml_type,
+                                           const void* data) {
+  REQUIRE_INIT();
+  if (!L || !data || e < 0 || e >= L->E || which < 0 || which > 2)
+    return fail(CSK_ERR_ARG, "csk_layer_set_expert_matrix: bad argument");
+  if (!L->f16) return fail(CSK_ERR_STATE, "csk_layer_set_expert_matrix: this layer holds MXFP4 experts (csk_layer_create_f16 makes an fp16 one)");
+  const bool down = which == CSK_W_DOWN;
+  int rc = f16_pack_into(data, ggml_type, down ? L->H : L->F, down ? L->F : L->H, L->view16(e, which));
+  if (rc != CSK_OK) return rc;
+  L->matrix_set[(size_t)e] |= (char)(1 << which);
+  if (L->matrix_set[(size_t)e] == 7) L->expert_set[(size_t)e] = 1;
+  return CSK_OK;
 }
 extern "C" int csk_layer_export_f16(const csk_layer* L, int64_t e, int which, uint16_t* halves_out) {
   REQUIRE_INIT();

@@ -74,6 +74,99 @@ __global__ __launch_bounds__(256) void f16_unpack_kernel(const u32x4* __restrict
   }
 }
 
+// ---- K-quant expert tensors widened to fp16 at load
+// (src/llm/moe_weight_provider.cpp:17-33, 134-159: dequantize_block_q4_K / q6_K to fp32,
+// then fp32_to_fp16; include/coalsack/gguf/gguf_dequant.h:149-258, 458-487).  The
+// arithmetic is the reference's operation by operation -- every product and difference
+// rounded separately, and the conversion of a build without F16C, which truncates the
+// mantissa -- so the resident halves equal the ones its provider would hand to the node.
+constexpr int kGgmlQ4K = 12, kGgmlQ6K = 14;
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+// gguf_dequant.h:463-487
+__device__ __forceinline__ uint32_t f32_to_f16_truncating(float f) {
+  const uint32_t bits = __float_as_uint(f);
+  const uint32_t sign = (bits >> 16) & 0x8000u;
+  const int e = (int)((bits >> 23) & 0xffu) - 127 + 15;
+  uint32_t m = (bits >> 13) & 0x3ffu;
+  if (e <= 0) {
+    if (e < -10) return sign;
+    m |= 0x400u;
+    m >>= (1 - e);
+    return sign | m;
+  }
+  if (e >= 31) return sign | 0x7c00u;
+  return sign | ((uint32_t)e << 10) | m;
+}
+
+// value idx of a Q4_K stream (144-byte super-blocks of 256; gguf_dequant.h:149-204)
+__device__ __forceinline__ float q4k_value(const uint8_t* __restrict__ src, long idx) {
+#pragma clang fp contract(off)
+  const uint8_t* blk = src + (idx >> 8) * 144;
+  const int w = (int)(idx & 255), j = w >> 5, l = w & 31;
+  const float d = half_bits_to_float(blk[0] | (blk[1] << 8));
+  const float dmin = half_bits_to_float(blk[2] | (blk[3] << 8));
+  const uint8_t* sc = blk + 4;
+  uint32_t s6, m6;
+  if (j < 4) {
+    s6 = sc[j] & 0x3F;
+    m6 = sc[j + 4] & 0x3F;
+  } else {
+    s6 = (sc[j + 4] & 0x0F) | ((sc[j - 4] >> 6) << 4);
+    m6 = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4);
+  }
+  const float dj = d * (float)s6;
+  const float mj = dmin * (float)m6;
+  const uint32_t qb = blk[16 + 32 * (j >> 1) + l];
+  const float prod = dj * (float)((j & 1) ? (qb >> 4) : (qb & 0x0F));
+  return prod - mj;
+}
+
+// value idx of a Q6_K stream (210-byte super-blocks of 256; gguf_dequant.h:220-258)
+__device__ __forceinline__ float q6k_value(const uint8_t* __restrict__ src, long idx) {
+#pragma clang fp contract(off)
+  const uint8_t* blk = src + (idx >> 8) * 210;
+  const int w = (int)(idx & 255), n = w >> 7, r = w & 127, g = r >> 5, l = r & 31;
+  const uint8_t* ql = blk + 64 * n;
+  const uint8_t* qh = blk + 128 + 32 * n;
+  const int8_t* sc = reinterpret_cast<const int8_t*>(blk + 192) + 8 * n;
+  const uint32_t lb = ql[l + 32 * (g & 1)];
+  const uint32_t low = g >= 2 ? (lb >> 4) : (lb & 0xF);
+  const uint32_t high = (qh[l] >> (2 * g)) & 3;
+  const int q = (int)(int8_t)(low | (high << 4)) - 32;
+  const float d = half_bits_to_float(blk[208] | (blk[209] << 8));
+  const float ds = d * (float)sc[(l >> 4) + 2 * g];
+  return ds * (float)q;
+}
+
+// K-quant stream of a row-major [rows, K] matrix -> fp16 tiles; one thread per 16-byte entry
+template <int TYPE>
+__global__ __launch_bounds__(256) void kquant_pack_kernel(const uint8_t* __restrict__ src,
+                                                          u32x4* __restrict__ dst, long rows, long K,
+                                                          long entries) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= entries) return;
+  const long nkb = f16_block_count(K);
+  const int lane = (int)(idx & 63);
+  const long kb = (idx >> 6) % nkb, tile = (idx >> 6) / nkb;
+  const long row = tile * 16 + (lane & 15), k0 = kb * 32 + 8 * (lane >> 4);
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  if (row < rows) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const long k = k0 + j;
+      if (k < K) {
+        const float v = TYPE == kGgmlQ4K ? q4k_value(src, row * K + k) : q6k_value(src, row * K + k);
+        w[j >> 1] |= f32_to_f16_truncating(v) << (16 * (j & 1));
+      }
+    }
+  }
+  dst[idx] = u32x4{w[0], w[1], w[2], w[3]};
+}
+
 // synthetic weights straight into the tiles: halves j / 2^14, j uniform in [-2048, 2047]
 // (every value exact in fp16), a function of (key, row, column) only; zero in the padding
 __global__ __launch_bounds__(256) void synth_f16_kernel(u32x4* __restrict__ dst, long rows, long K,

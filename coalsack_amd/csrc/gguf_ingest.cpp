@@ -1,5 +1,5 @@
 // GGUF ingest for the MoE path: parses a GGUF file's metadata and tensor table and
-// builds a resident MoE layer (router, MXFP4 or F16 experts, biases, FFN norm) for one
+// builds a resident MoE layer (router, MXFP4 or F16 / Q4_K / Q6_K experts, biases, FFN norm) for one
 // transformer block through the public C ABI.  Host-only code.
 //
 // Follows the reference's reader and weight provider:
@@ -26,7 +26,7 @@ namespace {
 
 constexpr uint32_t kMagic = 0x46554747u;  // "GGUF"
 enum : uint32_t { T_U8, T_I8, T_U16, T_I16, T_U32, T_I32, T_F32, T_BOOL, T_STR, T_ARR, T_U64, T_I64, T_F64 };
-constexpr uint32_t kGgmlF32 = 0, kGgmlF16 = 1, kGgmlMxfp4 = 39;
+constexpr uint32_t kGgmlF32 = 0, kGgmlF16 = 1, kGgmlQ4K = 12, kGgmlQ6K = 14, kGgmlMxfp4 = 39;
 
 int fail(int code, const std::string& msg) {
   csk_set_error_(msg.c_str());
@@ -296,10 +296,13 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
   for (int i = 0; i < 3; ++i) {
     tw[i] = find(g, p + wn[i]);
     if (!tw[i]) return fail(CSK_ERR_ARG, "Tensor not found: " + p + wn[i]);
-    if (tw[i]->type != kGgmlMxfp4 && tw[i]->type != kGgmlF16)
-      return fail(CSK_ERR_ARG, p + wn[i] + ": only MXFP4 and F16 expert weights are supported on this path");
-    if (tw[i]->type != tw[0]->type)
-      return fail(CSK_ERR_ARG, p + ": the three expert tensors must be of one type (all MXFP4 or all F16)");
+    const uint32_t ty = tw[i]->type;
+    if (ty != kGgmlMxfp4 && ty != kGgmlF16 && ty != kGgmlQ4K && ty != kGgmlQ6K)
+      return fail(CSK_ERR_ARG, p + wn[i] + ": only MXFP4, F16, Q4_K and Q6_K expert weights are supported on this path");
+    // the node decides between its two branches by the kind of w_up alone
+    // (expert_mlp_node.h:113-117), so MXFP4 cannot be mixed with the fp16 kinds
+    if ((ty == kGgmlMxfp4) != (tw[0]->type == kGgmlMxfp4))
+      return fail(CSK_ERR_ARG, p + ": expert tensors must be all MXFP4, or each of F16 / Q4_K / Q6_K");
     if (tw[i]->dims.size() != 3 || tw[i]->dims[2] != E)
       return fail(CSK_ERR_ARG, p + wn[i] + ": expected [K, rows, experts]");
     tb[i] = find(g, p + bn[i]);
@@ -315,7 +318,7 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
     return fail(CSK_ERR_ARG, p + ": expert biases must be all present or all absent");
 
   // F16 expert tensors take the node's float16 branch (expert_mlp_node.h:269-389)
-  const bool f16 = tw[0]->type == kGgmlF16;
+  const bool f16 = tw[0]->type != kGgmlMxfp4;
   csk_layer* L = nullptr;
   int rc = f16 ? csk_layer_create_f16(E, k, (int64_t)H, (int64_t)F, &L)
                : csk_layer_create(E, k, (int64_t)H, (int64_t)F, &L);
@@ -345,9 +348,22 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
   if (rc != CSK_OK) return bail(rc, "");
 
   // expert e of a stacked tensor starts at offset + e * slice bytes (moe_weight_provider.cpp:160-188)
-  const size_t sl[3] = {f16 ? (size_t)(F * H * 2) : (size_t)(F * (H / 32) * 17),
-                        f16 ? (size_t)(F * H * 2) : (size_t)(F * (H / 32) * 17),
-                        f16 ? (size_t)(H * F * 2) : (size_t)(H * (F / 32) * 17)};
+  // (one expert's K-quant slice is a whole number of super-blocks: moe_weight_provider.cpp:136-141)
+  auto slice_bytes = [&](uint32_t ty, uint64_t rows, uint64_t K) -> size_t {
+    const uint64_t n = rows * K;
+    switch (ty) {
+      case kGgmlF16: return (size_t)(n * 2);
+      case kGgmlQ4K: return (size_t)((n + 255) / 256 * 144);
+      case kGgmlQ6K: return (size_t)((n + 255) / 256 * 210);
+      default: return (size_t)(rows * (K / 32) * 17);
+    }
+  };
+  const size_t sl[3] = {slice_bytes(tw[0]->type, F, H), slice_bytes(tw[1]->type, F, H),
+                        slice_bytes(tw[2]->type, H, F)};
+  if (f16 && (F * H) % 256 != 0)
+    for (int i = 0; i < 3; ++i)
+      if (tw[i]->type == kGgmlQ4K || tw[i]->type == kGgmlQ6K)
+        return bail(CSK_ERR_ARG, p + wn[i] + ": a K-quant expert slice must be a multiple of 256 values");
   const size_t bl[3] = {(size_t)F, (size_t)F, (size_t)H};
   std::vector<uint8_t> w[3];
   std::vector<float> b[3];
@@ -364,10 +380,14 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
     }
     const float* bp[3] = {tb[0] ? b[0].data() : nullptr, tb[1] ? b[1].data() : nullptr,
                           tb[2] ? b[2].data() : nullptr};
-    rc = f16 ? csk_layer_set_expert_f16(L, e, reinterpret_cast<const uint16_t*>(w[0].data()),
-                                        reinterpret_cast<const uint16_t*>(w[1].data()),
-                                        reinterpret_cast<const uint16_t*>(w[2].data()), bp[0], bp[1], bp[2])
-             : csk_layer_set_expert(L, e, w[0].data(), w[1].data(), w[2].data(), bp[0], bp[1], bp[2]);
+    if (f16) {
+      const int which[3] = {CSK_W_UP, CSK_W_GATE, CSK_W_DOWN};
+      for (int i = 0; i < 3 && rc == CSK_OK; ++i)
+        rc = csk_layer_set_expert_matrix(L, e, which[i], (int)tw[i]->type, w[i].data());
+      if (rc == CSK_OK) rc = csk_layer_set_expert_f16(L, e, nullptr, nullptr, nullptr, bp[0], bp[1], bp[2]);
+    } else {
+      rc = csk_layer_set_expert(L, e, w[0].data(), w[1].data(), w[2].data(), bp[0], bp[1], bp[2]);
+    }
     if (rc != CSK_OK) return bail(rc, "");
   }
   const TensorInfo* tn = find(g, p + "." + norm_name);

@@ -53,11 +53,12 @@ def write_gguf(path, metadata, tensors, alignment=32, version=3):
 
 
 def moe_block_tensors(L, block, bias=True, norm=True, router_bias=True, norm_name="post_attention_norm.weight",
-                      f16_weights=None):
+                      f16_weights=None, raw_weights=None):
     """Tensors of one transformer block's MoE part from synth.LayerInputs, stacked over
     experts the way the reference's provider slices them (moe_weight_provider.cpp:97-188).
     f16_weights: per expert (w_up [F,H], w_gate [F,H], w_down [H,F]) float16 arrays, written
-    as F16 tensors instead of the MXFP4 blocks."""
+    as F16 tensors instead of the MXFP4 blocks.  raw_weights: per matrix kind a pair
+    (ggml_type, [bytes of expert 0, bytes of expert 1, ...]) written as they are."""
     p = f"blk.{block}"
     t = [(p + ".ffn_gate_inp.weight", GGML_F32, [L.H, L.E], np.ascontiguousarray(L.gate_w, np.float32).tobytes())]
     if router_bias:
@@ -65,7 +66,10 @@ def moe_block_tensors(L, block, bias=True, norm=True, router_bias=True, norm_nam
     names = ["ffn_up_exps", "ffn_gate_exps", "ffn_down_exps"]
     for which, nm in enumerate(names):
         rows, K = (L.F, L.H) if which < 2 else (L.H, L.F)
-        if f16_weights is not None:
+        if raw_weights is not None:
+            ty, per_expert = raw_weights[which]
+            t.append((f"{p}.{nm}.weight", ty, [K, rows, L.E], b"".join(bytes(x) for x in per_expert)))
+        elif f16_weights is not None:
             data = b"".join(np.ascontiguousarray(f16_weights[e][which], np.float16).tobytes() for e in range(L.E))
             t.append((f"{p}.{nm}.weight", GGML_F16, [K, rows, L.E], data))
         else:

@@ -113,6 +113,13 @@ int csk_mxfp4_export(const csk_mxfp4* m, uint8_t* blocks17_host);
 typedef struct csk_f16 csk_f16;
 int csk_f16_upload(const uint16_t* halves_host, int64_t rows, int64_t K, csk_f16** out);
 void csk_f16_free(csk_f16* m);
+/* The same from a matrix stored as ggml type F16 (1), Q4_K (12) or Q6_K (14): K-quant
+ * streams are widened to fp16 exactly as moe_weight_provider::get does
+ * (src/llm/moe_weight_provider.cpp:17-33, 134-159: dequantize_block_q4_K / q6_K, then
+ * fp32_to_fp16 -- the truncating conversion of a build without F16C,
+ * include/coalsack/gguf/gguf_dequant.h:149-258, 458-487).  rows * K must be a multiple
+ * of 256 for the K-quants. */
+int csk_f16_upload_ggml(int ggml_type, const void* data_host, int64_t rows, int64_t K, csk_f16** out);
 /* Recover the row-major halves from the resident copy (round-trip check). */
 int csk_f16_export(const csk_f16* m, uint16_t* halves_host);
 
@@ -158,6 +165,9 @@ int csk_layer_create_f16(int64_t E, int64_t k, int64_t H, int64_t F, csk_layer**
 int csk_layer_set_expert_f16(csk_layer* L, int64_t e, const uint16_t* w_up, const uint16_t* w_gate,
                              const uint16_t* w_down, const float* b_up, const float* b_gate,
                              const float* b_down);
+/* One matrix of expert e (which = CSK_W_UP / CSK_W_GATE / CSK_W_DOWN) from ggml type
+ * F16, Q4_K or Q6_K data, as csk_f16_upload_ggml; a checkpoint may mix the three. */
+int csk_layer_set_expert_matrix(csk_layer* L, int64_t e, int which, int ggml_type, const void* data_host);
 int csk_layer_export_f16(const csk_layer* L, int64_t e, int which, uint16_t* halves_host);
 
 /* ---------------------------------------------------------------- GGUF ingest

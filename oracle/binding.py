@@ -55,6 +55,14 @@ class Oracle:
         d.orc_e8m0_to_fp32_half.argtypes = [C.c_uint8]
         d.orc_dequant_mxfp4.restype = None
         d.orc_dequant_mxfp4.argtypes = [_P, _P, _I64]
+        for name in ("orc_dequant_q4_k", "orc_dequant_q6_k"):
+            getattr(d, name).restype = None
+            getattr(d, name).argtypes = [_P, _P, _I64]
+        for name in ("orc_q4k_to_fp16", "orc_q6k_to_fp16"):
+            getattr(d, name).restype = C.c_int
+            getattr(d, name).argtypes = [_P, _P, _I64]
+        d.orc_fp32_to_fp16.restype = C.c_uint16
+        d.orc_fp32_to_fp16.argtypes = [C.c_float]
         d.orc_router.restype = C.c_int
         d.orc_router.argtypes = [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P]
         d.orc_router_logits.restype = None
@@ -86,6 +94,26 @@ class Oracle:
         out = np.empty(k, np.float32)
         self.dll.orc_dequant_mxfp4(_p(blocks), _p(out), k)
         return out
+
+    def dequant_kquant(self, kind, blocks, k):
+        """kind: "q4_k" (144-byte super-blocks) or "q6_k" (210-byte); k values, fp32."""
+        blocks = _u8(blocks)
+        out = np.empty(k, np.float32)
+        getattr(self.dll, "orc_dequant_" + kind)(_p(blocks), _p(out), k)
+        return out
+
+    def kquant_to_fp16(self, kind, blocks, k):
+        """The weight provider's widening of a K-quant slice: uint16 bit patterns."""
+        blocks = _u8(blocks)
+        out = np.empty(k, np.uint16)
+        rc = getattr(self.dll, {"q4_k": "orc_q4k_to_fp16", "q6_k": "orc_q6k_to_fp16"}[kind])(_p(blocks), _p(out), k)
+        if rc:
+            raise ValueError(f"kquant_to_fp16 rc={rc}")
+        return out
+
+    def fp32_to_fp16(self, x):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        return np.array([self.dll.orc_fp32_to_fp16(float(v)) for v in x], np.uint16)
 
     def router(self, hidden, gate_w, gate_b, k, sigmoid=False):
         hidden, gate_w, gate_b = _f32(hidden), _f32(gate_w), _f32(gate_b)
@@ -222,6 +250,14 @@ class RefCodec:
         d.ref_e8m0_to_fp32_half.argtypes = [C.c_uint8]
         d.ref_dequantize_block_mxfp4.restype = None
         d.ref_dequantize_block_mxfp4.argtypes = [_P, _P, _I64]
+        self.has_kquant = hasattr(d, "ref_q4k_to_fp16")
+        if self.has_kquant:
+            for name in ("ref_dequantize_block_q4_K", "ref_dequantize_block_q6_K", "ref_q4k_to_fp16",
+                         "ref_q6k_to_fp16"):
+                getattr(d, name).restype = None
+                getattr(d, name).argtypes = [_P, _P, _I64]
+            d.ref_fp32_to_fp16.restype = C.c_uint16
+            d.ref_fp32_to_fp16.argtypes = [C.c_float]
 
     def e8m0(self, x):
         return self.dll.ref_e8m0_to_fp32_half(int(x))
@@ -231,3 +267,20 @@ class RefCodec:
         out = np.empty(k, np.float32)
         self.dll.ref_dequantize_block_mxfp4(_p(blocks), _p(out), k)
         return out
+
+    def dequant_kquant(self, kind, blocks, k):
+        blocks = _u8(blocks)
+        out = np.empty(k, np.float32)
+        getattr(self.dll, {"q4_k": "ref_dequantize_block_q4_K", "q6_k": "ref_dequantize_block_q6_K"}[kind])(
+            _p(blocks), _p(out), k)
+        return out
+
+    def kquant_to_fp16(self, kind, blocks, k):
+        blocks = _u8(blocks)
+        out = np.empty(k, np.uint16)
+        getattr(self.dll, {"q4_k": "ref_q4k_to_fp16", "q6_k": "ref_q6k_to_fp16"}[kind])(_p(blocks), _p(out), k)
+        return out
+
+    def fp32_to_fp16(self, x):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1)
+        return np.array([self.dll.ref_fp32_to_fp16(float(v)) for v in x], np.uint16)

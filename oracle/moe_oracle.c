@@ -16,6 +16,12 @@
  *          256 scale bytes x 16 codes), the reference's known answers
  *          (test/test_gguf_dequant.cpp:244-279) and the closed form
  *          lut[c] * 2^(e-128) via ldexp.
+ *   orc_dequant_q4_k / orc_dequant_q6_k / orc_fp32_to_fp16 / orc_q4k_to_fp16 /
+ *   orc_q6k_to_fp16 (the weight provider's widening of K-quant experts to fp16)
+ *        - the reference's own header compiled as oracle/_ref, bit-exact on
+ *          random super-blocks and on every fp32 exponent / rounding pattern,
+ *          and the committed fixture tests/golden/kquant_codec.npz written from
+ *          that build.
  *   orc_router
  *        - known answer {5,4,3} (test/test_moe_router.cpp:82-138), invariants
  *          (:62-78,:178-201), brute-force argsort + float64 softmax on random
@@ -92,6 +98,111 @@ void orc_dequant_mxfp4(const uint8_t* src, float* dst, int64_t k) {
       dst[i * 32 + j + 16] = (float)k_lut[blk[1 + j] >> 4] * scale;
     }
   }
+}
+
+/* ------------------------------------------------- K-quant experts -> fp16 */
+
+static float half_to_float(uint16_t h);
+
+/* gguf_dequant.h:149-204: Q4_K, super-blocks of 256 values in 144 bytes: fp16 d,
+ * fp16 dmin, 12 bytes of packed 6-bit scales and mins, 128 bytes of nibbles.
+ * value = (d * scale) * q - (dmin * min), each operation rounded (no FMA). */
+void orc_dequant_q4_k(const uint8_t* src, float* dst, int64_t k) {
+  const int64_t nb = k / 256;
+  for (int64_t i = 0; i < nb; ++i, src += 144) {
+    uint16_t dh, mh;
+    memcpy(&dh, src, 2);
+    memcpy(&mh, src + 2, 2);
+    const float d = half_to_float(dh), dmin = half_to_float(mh);
+    const uint8_t* sc = src + 4;
+    const uint8_t* q = src + 16;
+    for (int j = 0; j < 8; ++j) { /* sub-block j: 32 values */
+      uint8_t s6, m6;
+      if (j < 4) {
+        s6 = sc[j] & 0x3F;
+        m6 = sc[j + 4] & 0x3F;
+      } else {
+        s6 = (uint8_t)((sc[j + 4] & 0x0F) | ((sc[j - 4] >> 6) << 4));
+        m6 = (uint8_t)((sc[j + 4] >> 4) | ((sc[j] >> 6) << 4));
+      }
+      const float dj = d * (float)s6;
+      const float mj = dmin * (float)m6;
+      const uint8_t* qp = q + 32 * (j / 2); /* a pair of sub-blocks shares 32 bytes */
+      for (int l = 0; l < 32; ++l) {
+        const int nib = (j & 1) ? (qp[l] >> 4) : (qp[l] & 0x0F);
+        volatile float prod = dj * (float)nib;
+        dst[i * 256 + j * 32 + l] = prod - mj;
+      }
+    }
+  }
+}
+
+/* gguf_dequant.h:220-258: Q6_K, super-blocks of 256 values in 210 bytes: 128 bytes
+ * of low nibbles, 64 bytes of high bit pairs, 16 int8 scales, fp16 d.
+ * value = (d * scale) * q with q in -32..31. */
+void orc_dequant_q6_k(const uint8_t* src, float* dst, int64_t k) {
+  const int64_t nb = k / 256;
+  for (int64_t i = 0; i < nb; ++i, src += 210) {
+    const uint8_t* ql = src;
+    const uint8_t* qh = src + 128;
+    const int8_t* sc = (const int8_t*)(src + 192);
+    uint16_t dh;
+    memcpy(&dh, src + 208, 2);
+    const float d = half_to_float(dh);
+    float* y = dst + i * 256;
+    for (int n = 0; n < 2; ++n, y += 128, ql += 64, qh += 32, sc += 8) {
+      for (int l = 0; l < 32; ++l) {
+        const int is = l / 16;
+        const int q[4] = {
+            (int)(int8_t)((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32,
+            (int)(int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32,
+            (int)(int8_t)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32,
+            (int)(int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32};
+        for (int g = 0; g < 4; ++g) {
+          volatile float ds = d * (float)sc[is + 2 * g];
+          y[l + 32 * g] = ds * (float)q[g];
+        }
+      }
+    }
+  }
+}
+
+/* gguf_dequant.h:458-487, the branch a build without -mf16c takes (the reference's
+ * Release build has no -march): the mantissa is truncated, not rounded; values
+ * below the smallest subnormal give zero; anything with an exponent of 16 or more,
+ * NaN included, gives infinity. */
+uint16_t orc_fp32_to_fp16(float f) {
+  uint32_t bits;
+  memcpy(&bits, &f, 4);
+  const uint32_t sign = (bits >> 16) & 0x8000u;
+  const int32_t e = (int32_t)((bits >> 23) & 0xFF) - 127 + 15;
+  uint32_t m = (bits >> 13) & 0x3FFu;
+  if (e <= 0) {
+    if (e < -10) return (uint16_t)sign;
+    m |= 0x400u;
+    m >>= (1 - e);
+    return (uint16_t)(sign | m);
+  }
+  if (e >= 31) return (uint16_t)(sign | 0x7C00u);
+  return (uint16_t)(sign | ((uint32_t)e << 10) | m);
+}
+
+/* src/llm/moe_weight_provider.cpp:17-33: one expert's slice widened to fp16 */
+int orc_q4k_to_fp16(const uint8_t* src, uint16_t* dst, int64_t k) {
+  float* tmp = (float*)malloc((size_t)k * sizeof(float));
+  if (!tmp) return ORC_ERR_ARG;
+  orc_dequant_q4_k(src, tmp, k);
+  for (int64_t i = 0; i < k; ++i) dst[i] = orc_fp32_to_fp16(tmp[i]);
+  free(tmp);
+  return ORC_OK;
+}
+int orc_q6k_to_fp16(const uint8_t* src, uint16_t* dst, int64_t k) {
+  float* tmp = (float*)malloc((size_t)k * sizeof(float));
+  if (!tmp) return ORC_ERR_ARG;
+  orc_dequant_q6_k(src, tmp, k);
+  for (int64_t i = 0; i < k; ++i) dst[i] = orc_fp32_to_fp16(tmp[i]);
+  free(tmp);
+  return ORC_OK;
 }
 
 /* ----------------------------------------------------------------- router */
@@ -364,7 +475,7 @@ int orc_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t T, int64_t 
 /* ------------------------------------------------- expert MLP, fp16 weights */
 
 /* IEEE binary16 -> binary32, exact (what _cvtsh_ss / _mm256_cvtph_ps return). */
-static inline float half_to_float(uint16_t h) {
+static float half_to_float(uint16_t h) {
   const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
   uint32_t exp = (h >> 10) & 0x1fu, man = h & 0x3ffu, bits;
   if (exp == 0) {

@@ -116,17 +116,17 @@ def test_layer_from_gguf_llama4_switches_and_errors(lib, oracle, tmp_path):
     mixed = gw.moe_block_tensors(L, 0, bias=False, router_bias=False)
     mixed[1] = (mixed[1][0], gw.GGML_F16, mixed[1][2], np.zeros(E * F * H, np.float16).tobytes())
     gw.write_gguf(str(tmp_path / "mixed.gguf"), _meta(E=E, k=k), mixed)
-    # Q4_K: 144 bytes per 256 elements
-    q4 = [(n, 12, d, bytes(int(np.prod(d)) // 256 * 144)) if "_exps.weight" in n else (n, t, d, b)
+    # Q5_K (type 13): 176 bytes per 256 elements
+    q4 = [(n, 13, d, bytes(int(np.prod(d)) // 256 * 176)) if "_exps.weight" in n else (n, t, d, b)
           for n, t, d, b in gw.moe_block_tensors(L, 0, bias=False, router_bias=False)]
     gw.write_gguf(str(tmp_path / "q4k.gguf"), _meta(E=E, k=k), q4)
     with lib.gguf(str(tmp_path / "mixed.gguf")) as g:
-        with pytest.raises(capi.CskError, match="must be of one type"):
+        with pytest.raises(capi.CskError, match="must be all MXFP4"):
             g.layer(0)
         with pytest.raises(capi.CskError, match="Tensor not found"):
             g.layer(3)
     with lib.gguf(str(tmp_path / "q4k.gguf")) as g:
-        with pytest.raises(capi.CskError, match="only MXFP4 and F16"):
+        with pytest.raises(capi.CskError, match="only MXFP4, F16, Q4_K and Q6_K"):
             g.layer(0)
 
 
@@ -160,4 +160,37 @@ def test_layer_from_gguf_f16_experts(lib, oracle, tmp_path, T):
     want, _ = oracle.moe_layer(hidden, E, k, H, F, L.gate_w, L.gate_b, np.stack([w[0] for w in ws]),
                                np.stack([w[1] for w in ws]), np.stack([w[2] for w in ws]), L.b_up,
                                L.b_gate, L.b_down, norm_w=L.norm_w, norm_eps=1e-5, residual=True)
+    assert_layer_close(got, want)
+
+
+@pytest.mark.gpu
+def test_layer_from_gguf_kquant_experts(lib, oracle, tmp_path):
+    """A block in the style of a Q4_K_M checkpoint: gate and up experts Q4_K, down experts
+    Q6_K.  The resident halves equal what the reference's weight provider hands to the node
+    (K-quant -> fp32 -> truncating fp16), and the forward matches the CPU path's float16
+    branch over those halves."""
+    from tests.golden.make_kquant_golden import random_blocks
+    E, k, H, F = 4, 2, 128, 256
+    L = synth.LayerInputs(E, k, H, F, seed=51, with_norm=True)
+    rng = np.random.default_rng(51)
+    nsb = H * F // 256
+    raw = [(12, [random_blocks(rng, "q4_k", nsb).tobytes() for _ in range(E)]),
+           (12, [random_blocks(rng, "q4_k", nsb).tobytes() for _ in range(E)]),
+           (14, [random_blocks(rng, "q6_k", nsb).tobytes() for _ in range(E)])]
+    path = str(tmp_path / "q4km.gguf")
+    gw.write_gguf(path, _meta(E=E, k=k), gw.moe_block_tensors(L, 0, raw_weights=raw))
+    halves = [[oracle.kquant_to_fp16("q4_k" if raw[w][0] == 12 else "q6_k",
+                                     np.frombuffer(raw[w][1][e], np.uint8), H * F)
+               .reshape((H, F) if w == 2 else (F, H)) for w in range(3)] for e in range(E)]
+    hidden = synth.hidden_states(9, H, seed=6)
+    with lib.gguf(path) as g, g.layer(0) as layer:
+        assert layer.f16
+        for e in range(E):
+            for w in range(3):
+                assert np.array_equal(layer.export_f16(e, w).view(np.uint16), halves[e][w])
+        got = layer.forward(hidden, capi.FWD_RMSNORM)
+    stack = lambda w: np.stack([halves[e][w] for e in range(E)]).view(np.float16)
+    want, _ = oracle.moe_layer(hidden, E, k, H, F, L.gate_w, L.gate_b, stack(0), stack(1), stack(2), L.b_up,
+                               L.b_gate, L.b_down, norm_w=L.norm_w, norm_eps=1e-5)
+    assert np.all(np.isfinite(want))
     assert_layer_close(got, want)

@@ -25,6 +25,40 @@ def test_f16_upload_export_round_trip(lib, rows, K):
     assert np.array_equal(back.view(np.uint16), w.view(np.uint16))
 
 
+@pytest.mark.parametrize("kind,ty", [("q4_k", 12), ("q6_k", 14)])
+@pytest.mark.parametrize("rows,K", [(16, 256), (48, 160), (37, 256), (2880, 512)])
+def test_kquant_upload_equals_weight_provider_halves(lib, oracle, kind, ty, rows, K):
+    """csk_f16_upload_ggml on a Q4_K / Q6_K stream leaves exactly the halves the reference's
+    provider computes (dequantize, then the truncating fp32 -> fp16), also when super-blocks
+    straddle rows (K = 160)."""
+    from tests.golden.make_kquant_golden import random_blocks
+    rng = np.random.default_rng([rows, K, ty])
+    blocks = random_blocks(rng, kind, rows * K // 256).reshape(-1)
+    want = oracle.kquant_to_fp16(kind, blocks, rows * K).reshape(rows, K)
+    h = lib.f16_upload_ggml(ty, blocks, rows, K)
+    try:
+        got = lib.f16_export(h, rows, K)
+    finally:
+        lib.f16_free(h)
+    assert np.array_equal(got.view(np.uint16), want)
+
+
+def test_kquant_upload_fixture_and_errors(lib):
+    import os
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "kquant_codec.npz"))
+    for tag, ty in (("q4", 12), ("q6", 14)):
+        b = gold[tag + "_blocks"]
+        h = lib.f16_upload_ggml(ty, b.reshape(-1), 48, 256)
+        try:
+            assert np.array_equal(lib.f16_export(h, 48, 256).view(np.uint16).reshape(-1), gold[tag + "_f16"])
+        finally:
+            lib.f16_free(h)
+    with pytest.raises(capi.CskError, match="multiple of 256"):
+        lib.f16_upload_ggml(12, np.zeros(144, np.uint8), 3, 100)
+    with pytest.raises(capi.CskError, match="ggml types"):
+        lib.f16_upload_ggml(13, np.zeros(176, np.uint8), 16, 16)
+
+
 def test_reference_known_answer_two_by_two(lib):
     # test/test_expert_mlp.cpp:118-200
     x = np.array([[1.0, 0.5]], np.float32)
