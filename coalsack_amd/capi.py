@@ -77,6 +77,7 @@ SIGNATURES = {
                                        _I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]),
     "csk_expert_mlp_f16": (C.c_int, [C.c_int, _P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P,
                                      _I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]),
+    "csk_dense_ffn_f16": (C.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]),
     "csk_expert_token_mxfp4": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, C.c_int]),
     "csk_expert_merge": (C.c_int, [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]),
     "csk_rmsnorm": (C.c_int, [_P, _P, _P, _I64, _I64, C.c_float]),
@@ -258,6 +259,22 @@ class Library:
             for h in hs:
                 self.f16_free(h)
         return None if empty.value else out
+
+    def dense_ffn_f16(self, hidden, w_gate, w_up, w_down, b_gate=None, b_up=None, b_down=None):
+        """dense_ffn_node with float16 weights [F,H], [F,H], [H,F]; uploads them for the call."""
+        hidden = _f32(hidden)
+        b_gate, b_up, b_down = _f32(b_gate), _f32(b_up), _f32(b_down)
+        T, H = hidden.shape
+        F = w_gate.shape[0]
+        hs = [self.f16_upload(w) for w in (w_gate, w_up, w_down)]
+        try:
+            out = np.empty((T, H), np.float32)
+            self.check(self.dll.csk_dense_ffn_f16(_ptr(hidden), T, H, F, hs[0], hs[1], hs[2], _ptr(b_gate),
+                                                  _ptr(b_up), _ptr(b_down), _ptr(out)))
+        finally:
+            for h in hs:
+                self.f16_free(h)
+        return out
 
     # -- node-level ops
     def moe_router(self, hidden, gate_w, gate_b, k, sigmoid=False):

@@ -452,7 +452,7 @@ int launch_f16_split(const float* x, int64_t rows, int64_t K, const int* gather_
 // the weights per group, HBM-bound); beyond that groups of 64.
 int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int act_type,
                     const float* x, bool weight_before_ffn, int64_t gather_rows, Workspace& ws,
-                    bool timed = false) {
+                    bool timed = false, bool identity_rows = false) {
   const int64_t P = T * k;
   int rc = g_f16.ensure((size_t)P, (size_t)F);
   if (rc != CSK_OK) return rc;
@@ -467,7 +467,7 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
     a.B = reinterpret_cast<const u32x4*>(ws.xg);
   } else {
     rc = launch_f16_split(x, T, H, nullptr, nullptr, ws.xs, g_f16.rs_x);
-    a.list_row = ws.list_tok;
+    a.list_row = identity_rows ? nullptr : ws.list_tok;  // identity: position p is token p
     a.B = reinterpret_cast<const u32x4*>(ws.xs);
   }
   if (rc != CSK_OK) return rc;
@@ -1402,6 +1402,61 @@ extern "C" int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T,
       ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
   if ((rc = check_launch("expand_expert_rows_kernel")) != CSK_OK) return rc;
   HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+namespace {
+// One work descriptor holding every token (position p = token p) and its 64-token tiles.
+__global__ void dense_desc_kernel(WorkDesc* desc, const ExpertW* ew, int T, int* mtiles, int* n_mtiles) {
+  if (threadIdx.x == 0) {
+    write_work_desc(desc, true, 0, T, 0, ew);
+    *n_mtiles = (T + 63) / 64;
+  }
+  for (int i = threadIdx.x; i < (T + 63) / 64; i += blockDim.x) {
+    mtiles[2 * i] = 0;
+    mtiles[2 * i + 1] = 64 * i;
+  }
+}
+}  // namespace
+
+extern "C" int csk_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int64_t F,
+                                 const csk_f16* w_gate, const csk_f16* w_up, const csk_f16* w_down,
+                                 const float* b_gate, const float* b_up, const float* b_down,
+                                 float* out) {
+  REQUIRE_INIT();
+  if (!hidden || !w_gate || !w_up || !w_down || !out || T < 0)
+    return fail(CSK_ERR_ARG, "csk_dense_ffn_f16: null argument");
+  if (w_gate->rows != F || w_gate->K != H || w_up->rows != F || w_up->K != H)
+    return fail(CSK_ERR_ARG, "dense_ffn: gate_w/up_w shape mismatch");
+  if (w_down->rows != H || w_down->K != F)
+    return fail(CSK_ERR_ARG, "dense_ffn: down_w shape mismatch, expected [" + std::to_string(H) + ", " +
+                                 std::to_string(F) + "], got [" + std::to_string(w_down->rows) + ", " +
+                                 std::to_string(w_down->K) + "]");
+  if (T == 0) return CSK_OK;
+  if (T > (int64_t)1 << 24) return fail(CSK_ERR_ARG, "dense_ffn: more than 2^24 tokens");
+  Workspace& ws = g_ws;
+  int rc = ws.ensure(T, 1, 1, cdiv(H, 32) * 32, cdiv(F, 32) * 32, false);
+  if (rc != CSK_OK) return rc;
+  DevBuf dx, dbg, dbu, dbd, dew;
+  if ((rc = dx.upload(hidden, (size_t)T * H * 4)) != CSK_OK) return rc;
+  // each bias is optional on its own (dense_ffn_node.h:196-197, 213)
+  if (b_gate && (rc = dbg.upload(b_gate, (size_t)F * 4)) != CSK_OK) return rc;
+  if (b_up && (rc = dbu.upload(b_up, (size_t)F * 4)) != CSK_OK) return rc;
+  if (b_down && (rc = dbd.upload(b_down, (size_t)H * 4)) != CSK_OK) return rc;
+  ExpertW w{};
+  w.q_gate = reinterpret_cast<const uint4*>(w_gate->w);
+  w.q_up = reinterpret_cast<const uint4*>(w_up->w);
+  w.q_down = reinterpret_cast<const uint4*>(w_down->w);
+  w.b_gate = b_gate ? dbg.as<float>() : g_zero;
+  w.b_up = b_up ? dbu.as<float>() : g_zero;
+  w.b_down = b_down ? dbd.as<float>() : g_zero;
+  if ((rc = dew.upload(&w, sizeof w)) != CSK_OK) return rc;
+  dense_desc_kernel<<<1, 256, 0, g_stream>>>(ws.desc, dew.as<ExpertW>(), (int)T, ws.tiles, ws.n_tiles);
+  if ((rc = check_launch("dense_desc_kernel")) != CSK_OK) return rc;
+  rc = run_experts_f16(1, T, 1, H, F, CSK_ACT_STANDARD_SWIGLU, dx.as<float>(), false, T, ws, false, true);
+  if (rc != CSK_OK) return rc;
+  HIP_TRY(hipMemcpyAsync(out, ws.y, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
   HIP_TRY(hipStreamSynchronize(g_stream));
   return CSK_OK;
 }

@@ -1,0 +1,102 @@
+// dense_ffn_node backed by the gfx950 library: same class name, input order, output
+// and error texts as include/coalsack/nn/nn_ops/dense_ffn_node.h of the reference (cited
+// by line below); float16 weights run in csk_dense_ffn_f16.  Weights are uploaded at the
+// first sight of their storage pointer and cached per node (the engine feeds the same
+// weight tensors every frame, src/llm/llm_engine.cpp:755-771).
+#pragma once
+
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "coalsack/nn/nn_op_node.h"
+#include "coalsack_moe.h"
+
+namespace coalsack {
+
+// output = down_proj(silu(gate_proj(x)) * up_proj(x)) for every token (:14-27).
+// Inputs: hidden [B, S, D] f32, gate_w / up_w [ffn, D], down_w [D, ffn] float16,
+// optionally gate_b, up_b [ffn], down_b [D] f32.
+class dense_ffn_node : public variadic_op_node {
+ public:
+  dense_ffn_node() : variadic_op_node("dense_ffn", 4) {}  // :30
+  ~dense_ffn_node() override {
+    for (auto& kv : resident_) csk_f16_free(kv.second.handle);
+  }
+  dense_ffn_node(const dense_ffn_node&) = delete;
+  dense_ffn_node& operator=(const dense_ffn_node&) = delete;
+  std::string get_proc_name() const override { return "dense_ffn"; }  // :32
+  // not in the reference (its compute is reached through process only): for tests
+  dynamic_tensor compute_test(const std::vector<dynamic_tensor>& inputs) { return compute(inputs); }
+
+ protected:
+  dynamic_tensor compute(const std::vector<dynamic_tensor>& inputs) override {  // :35-118
+    if (inputs.size() != 4 && inputs.size() != 7)
+      throw std::runtime_error(
+          "dense_ffn: expected 4 or 7 inputs (hidden, gate_w, up_w, down_w[, gate_b, up_b, "
+          "down_b]), got " +
+          std::to_string(inputs.size()));
+    const dynamic_tensor& hidden = inputs[0];
+    const dynamic_tensor& gate_w = inputs[1];
+    const dynamic_tensor& up_w = inputs[2];
+    const dynamic_tensor& down_w = inputs[3];
+    const bool has_bias = inputs.size() == 7;
+    if (hidden.ndim() != 3)
+      throw std::runtime_error("dense_ffn: hidden_states must be 3D [B, S, D], got " +
+                               std::to_string(hidden.ndim()) + "D");
+    if (gate_w.ndim() != 2 || up_w.ndim() != 2 || down_w.ndim() != 2)
+      throw std::runtime_error("dense_ffn: weight tensors must be 2D");
+    const dtype wt = gate_w.get_dtype();
+    if ((wt != dtype::float16 && wt != dtype::float32) || up_w.get_dtype() != wt || down_w.get_dtype() != wt)
+      throw std::runtime_error("dense_ffn: weight tensors must all be FLOAT16 or all FLOAT32");
+    if (hidden.get_dtype() != dtype::float32)
+      throw std::runtime_error("dense_ffn: hidden_states must be FLOAT32");
+    const int64_t tokens = hidden.dim(0) * hidden.dim(1), hidden_dim = hidden.dim(2), ffn_dim = gate_w.dim(0);
+    if (gate_w.dim(1) != hidden_dim || up_w.dim(0) != ffn_dim || up_w.dim(1) != hidden_dim)
+      throw std::runtime_error("dense_ffn: gate_w/up_w shape mismatch");
+    if (down_w.dim(0) != hidden_dim || down_w.dim(1) != ffn_dim)
+      throw std::runtime_error("dense_ffn: down_w shape mismatch, expected [" + std::to_string(hidden_dim) +
+                               ", " + std::to_string(ffn_dim) + "], got [" + std::to_string(down_w.dim(0)) +
+                               ", " + std::to_string(down_w.dim(1)) + "]");
+    // the reference also has a scalar branch for FLOAT32 weights (:101-114); the engine
+    // hands this node float16 ones unless the checkpoint stores them as F32
+    if (wt != dtype::float16)
+      throw std::runtime_error("dense_ffn: FLOAT32 weights are not supported on this build");
+    dynamic_tensor output(dtype::float32, {hidden.dim(0), hidden.dim(1), hidden_dim});
+    if (tokens == 0) return output;
+    const int rc = csk_dense_ffn_f16(hidden.data_ptr<float>(), tokens, hidden_dim, ffn_dim, resident_copy(gate_w),
+                                     resident_copy(up_w), resident_copy(down_w),
+                                     has_bias ? inputs[4].data_ptr<float>() : nullptr,
+                                     has_bias ? inputs[5].data_ptr<float>() : nullptr,
+                                     has_bias ? inputs[6].data_ptr<float>() : nullptr, output.data_ptr<float>());
+    if (rc != CSK_OK) throw std::runtime_error(std::string("dense_ffn: ") + csk_last_error());
+    return output;
+  }
+
+ private:
+  struct resident {
+    csk_f16* handle;
+    int64_t rows, cols;
+  };
+  csk_f16* resident_copy(const dynamic_tensor& t) {
+    const uint16_t* key = t.data_ptr<uint16_t>();
+    auto it = resident_.find(key);
+    if (it != resident_.end() && it->second.rows == t.dim(0) && it->second.cols == t.dim(1))
+      return it->second.handle;
+    if (it != resident_.end()) {
+      csk_f16_free(it->second.handle);
+      resident_.erase(it);
+    }
+    csk_f16* h = nullptr;
+    if (csk_f16_upload(key, t.dim(0), t.dim(1), &h) != CSK_OK)
+      throw std::runtime_error(std::string("dense_ffn: ") + csk_last_error());
+    resident_[key] = resident{h, t.dim(0), t.dim(1)};
+    return h;
+  }
+  std::unordered_map<const uint16_t*, resident> resident_;
+};
+
+}  // namespace coalsack
+
+COALSACK_REGISTER_NODE(coalsack::dense_ffn_node, coalsack::graph_node)

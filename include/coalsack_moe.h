@@ -246,6 +246,13 @@ int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T, int64_t H,
                        const float* b_up, const float* b_gate, const float* b_down,
                        const float* router_pairs, int64_t k, int activation,
                        int weight_before_ffn, float* out, int* is_empty);
+/* dense_ffn_node::compute with float16 weights (include/coalsack/nn/nn_ops/dense_ffn_node.h:
+ * 36-118, compute_token :163-218): the shared expert of llama4-style blocks
+ * (src/llm/llm_engine.cpp:755-771) -- every token through one gated MLP with the standard
+ * SwiGLU.  out [T,H]; w_gate/w_up [F,H], w_down [H,F]; each bias f32 or NULL.  Any H, F. */
+int csk_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int64_t F, const csk_f16* w_gate,
+                      const csk_f16* w_up, const csk_f16* w_down, const float* b_gate,
+                      const float* b_up, const float* b_down, float* out);
 /* expert_mlp_node::compute_test_mxfp4 (expert_mlp_node.h:63-70): one token,
  * raw 17-byte-block weights in host memory. */
 int csk_expert_token_mxfp4(const float* hidden_vec, const uint8_t* w_up, const uint8_t* w_gate,

@@ -77,6 +77,8 @@ class Oracle:
         d.orc_expert_mlp_f16.restype = C.c_int
         d.orc_expert_mlp_f16.argtypes = [C.c_int, _P, _I64, _I64, _I64] + [_P] * 7 + \
             [_I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]
+        d.orc_dense_ffn_f16.restype = C.c_int
+        d.orc_dense_ffn_f16.argtypes = [_P, _I64, _I64, _I64] + [_P] * 7
         d.orc_expert_merge.restype = C.c_int
         d.orc_expert_merge.argtypes = [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]
         d.orc_rmsnorm.restype = None
@@ -189,6 +191,20 @@ class Oracle:
         if rc:
             raise ValueError(f"orc_expert_mlp_f16 rc={rc}")
         return None if empty.value else out
+
+    def dense_ffn_f16(self, hidden, w_gate, w_up, w_down, b_gate=None, b_up=None, b_down=None):
+        """dense_ffn_node: hidden [T,H]; float16 w_gate/w_up [F,H], w_down [H,F]."""
+        hidden = _f32(hidden)
+        w_gate, w_up, w_down = _f16(w_gate), _f16(w_up), _f16(w_down)
+        b_gate, b_up, b_down = _f32(b_gate), _f32(b_up), _f32(b_down)
+        T, H = hidden.shape
+        F = w_gate.shape[0]
+        out = np.empty((T, H), np.float32)
+        rc = self.dll.orc_dense_ffn_f16(_p(hidden), T, H, F, _p(w_gate), _p(w_up), _p(w_down), _p(b_gate),
+                                        _p(b_up), _p(b_down), _p(out))
+        if rc:
+            raise ValueError(f"orc_dense_ffn_f16 rc={rc}")
+        return out
 
     def expert_merge(self, pairs, expert_outs, H, pre_weighted=False):
         pairs = _f32(pairs)

@@ -42,6 +42,9 @@
  *          remainder loop), dimensions that are not multiples of 8, and
  *          agreement with the MXFP4 functions on weights that both formats
  *          hold exactly.  PARITY UNPINNED at the last ulp, as above.
+ *   orc_dense_ffn_f16
+ *        - the fp16 expert function it is built from (pinned above) and an
+ *          independent float64 evaluation with the standard SwiGLU.
  *   orc_expert_merge
  *        - definition sum_k w_k * y_{e_k}; one-hot weights reduce to a copy;
  *          linearity; error cases.
@@ -579,6 +582,25 @@ int orc_expert_mlp_f16(int expert_id, const float* hidden, int64_t T, int64_t H,
     }
     rc = expert_token_f16(x, w_up, w_gate, w_down, b_up, b_gate, b_down, o, H, F, act, scratch);
   }
+  free(scratch);
+  return rc;
+}
+
+/* include/coalsack/nn/nn_ops/dense_ffn_node.h:28-219: the shared expert of llama4-style
+ * blocks.  Every token goes through one gated MLP with float16 weights and the standard
+ * SwiGLU; compute_token (:163-218) is the expert's float16 loop (same accumulator lanes,
+ * horizontal sum and remainder), the bias is added to the sum afterwards, which gives the
+ * same value.  Weight order gate, up, down as the node's inputs. */
+int orc_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int64_t F, const uint16_t* w_gate,
+                      const uint16_t* w_up, const uint16_t* w_down, const float* b_gate,
+                      const float* b_up, const float* b_down, float* out) {
+  if (T < 0 || H <= 0 || F <= 0) return ORC_ERR_ARG;
+  float* scratch = (float*)malloc((size_t)F * sizeof(float));
+  if (!scratch) return ORC_ERR_ARG;
+  int rc = ORC_OK;
+  for (int64_t t = 0; t < T && rc == ORC_OK; ++t)
+    rc = expert_token_f16(hidden + t * H, w_up, w_gate, w_down, b_up, b_gate, b_down, out + t * H, H, F,
+                          ORC_ACT_STANDARD_SWIGLU, scratch);
   free(scratch);
   return rc;
 }

@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "coalsack/nn/nn_ops/add_node.h"
+#include "coalsack/nn/nn_ops/dense_ffn_node.h"
 #include "coalsack/nn/nn_ops/expert_merge_node.h"
 #include "coalsack/nn/nn_ops/expert_mlp_node.h"
 #include "coalsack/nn/nn_ops/moe_router_node.h"
@@ -30,6 +31,8 @@ int orc_expert_merge(const float*, int64_t, int64_t, int64_t, int64_t, const flo
 int orc_expert_mlp_f16(int, const float*, int64_t, int64_t, int64_t, const uint16_t*, const uint16_t*,
                        const uint16_t*, const float*, const float*, const float*, const float*, int64_t, int,
                        int, float*, int*);
+int orc_dense_ffn_f16(const float*, int64_t, int64_t, int64_t, const uint16_t*, const uint16_t*, const uint16_t*,
+                      const float*, const float*, const float*, float*);
 void orc_rmsnorm(const float*, const float*, float*, int64_t, int64_t, float);
 void orc_add(const float*, const float*, float*, int64_t);
 }
@@ -226,6 +229,31 @@ static void cpu_expert_fp16_argument_errors() {
   expert_mlp_node other(9);
   auto out = other.compute_test({dynamic_tensor(dtype::float32, {2, 8}), w_up, w_gate, w_down, router});
   CHECK(out.ndim() == 1 && out.dim(0) == 0);
+}
+
+static void cpu_dense_ffn_argument_errors() {
+  std::printf("dense_ffn: argument errors\n");
+  std::mt19937 gen(5);
+  dense_ffn_node node;
+  CHECK(node.get_proc_name() == "dense_ffn");
+  auto hidden = random_tensor({1, 3, 8}, gen, -1, 1);
+  auto gate = random_half_tensor({16, 8}, gen, -0.1f, 0.1f), up = random_half_tensor({16, 8}, gen, -0.1f, 0.1f);
+  auto down = random_half_tensor({8, 16}, gen, -0.1f, 0.1f);
+  CHECK(throws_with([&] { node.compute_test({hidden, gate, up}); },
+                    "dense_ffn: expected 4 or 7 inputs (hidden, gate_w, up_w, down_w[, gate_b, up_b, down_b]), got 3"));
+  CHECK(throws_with([&] { node.compute_test({dynamic_tensor(dtype::float32, {3, 8}), gate, up, down}); },
+                    "dense_ffn: hidden_states must be 3D [B, S, D], got 2D"));
+  CHECK(throws_with([&] { node.compute_test({hidden, dynamic_tensor(dtype::float16, {16}), up, down}); },
+                    "dense_ffn: weight tensors must be 2D"));
+  CHECK(throws_with([&] { node.compute_test({hidden, gate, random_tensor({16, 8}, gen, -1, 1), down}); },
+                    "dense_ffn: weight tensors must all be FLOAT16 or all FLOAT32"));
+  CHECK(throws_with([&] { node.compute_test({hidden, gate, random_half_tensor({15, 8}, gen, -1, 1), down}); },
+                    "dense_ffn: gate_w/up_w shape mismatch"));
+  CHECK(throws_with([&] { node.compute_test({hidden, gate, up, random_half_tensor({8, 15}, gen, -1, 1)}); },
+                    "dense_ffn: down_w shape mismatch, expected [8, 16], got [8, 15]"));
+  CHECK(throws_with([&] { node.compute_test({hidden, random_tensor({16, 8}, gen, -1, 1), random_tensor({16, 8}, gen, -1, 1),
+                                             random_tensor({8, 16}, gen, -1, 1)}); },
+                    "dense_ffn: FLOAT32 weights are not supported on this build"));
 }
 
 static void cpu_merge_argument_errors() {
@@ -458,6 +486,46 @@ static void gpu_expert_fp16_tests() {
   CHECK(std::fabs(out.data_ptr<float>()[0] - want) < 1e-3f);
 }
 
+static void gpu_dense_ffn_tests() {
+  std::printf("dense_ffn: shared expert through result messages, against the CPU path\n");
+  std::mt19937 gen(9);
+  for (const auto& dims : std::vector<std::vector<int64_t>>{{1, 5, 64, 96}, {2, 40, 72, 130}, {1, 3, 30, 20}}) {
+    const int64_t B = dims[0], S = dims[1], H = dims[2], F = dims[3];
+    for (bool bias : {false, true}) {
+      auto hidden = random_tensor({B, S, H}, gen, -1, 1);
+      auto gate = random_half_tensor({F, H}, gen, -0.2f, 0.2f), up = random_half_tensor({F, H}, gen, -0.2f, 0.2f);
+      auto down = random_half_tensor({H, F}, gen, -0.2f, 0.2f);
+      auto bg = random_tensor({F}, gen, -0.1f, 0.1f), bu = random_tensor({F}, gen, -0.1f, 0.1f);
+      auto bd = random_tensor({H}, gen, -0.1f, 0.1f);
+      dense_ffn_node node;
+      capture_node cap;
+      cap.set_input(node.get_output());
+      node.set_output_name("out");
+      auto mk = [](const dynamic_tensor& t) { return std::make_shared<dynamic_tensor_message>(t); };
+      if (bias) {
+        node.set_input_names({"x", "g", "u", "d", "bg", "bu", "bd"});
+        node.process("default", result_message::ok({{"x", mk(hidden)}, {"g", mk(gate)}, {"u", mk(up)}, {"d", mk(down)},
+                                                    {"bg", mk(bg)}, {"bu", mk(bu)}, {"bd", mk(bd)}}));
+      } else {
+        node.set_input_names({"x", "g", "u", "d"});
+        node.process("default", result_message::ok({{"x", mk(hidden)}, {"g", mk(gate)}, {"u", mk(up)}, {"d", mk(down)}}));
+      }
+      CHECK(cap.got.size() == 1 && cap.got[0]->is_ok());
+      auto out = std::dynamic_pointer_cast<dynamic_tensor_message>(cap.got[0]->get_field("out"))->get_tensor();
+      CHECK(out.shape() == hidden.shape());
+      std::vector<float> want(B * S * H);
+      CHECK(orc_dense_ffn_f16(hidden.data_ptr<float>(), B * S, H, F, gate.data_ptr<uint16_t>(), up.data_ptr<uint16_t>(),
+                              down.data_ptr<uint16_t>(), bias ? bg.data_ptr<float>() : nullptr,
+                              bias ? bu.data_ptr<float>() : nullptr, bias ? bd.data_ptr<float>() : nullptr,
+                              want.data()) == 0);
+      float worst = 0;
+      for (int64_t i = 0; i < out.numel(); ++i)
+        worst = std::fmax(worst, std::fabs(out.data_ptr<float>()[i] - want[i]) / std::fmax(1.0f, std::fabs(want[i])));
+      CHECK(worst <= 1e-3f);
+    }
+  }
+}
+
 // router -> E expert nodes -> merge, wired with edges and result messages the way
 // llm_engine builds the block (src/llm/llm_engine.cpp:721-753), against the CPU checker.
 static void gpu_node_chain() {
@@ -551,12 +619,14 @@ int main(int argc, char** argv) {
     gpu_router_tests();
     gpu_expert_known_answer();
     gpu_expert_fp16_tests();
+    gpu_dense_ffn_tests();
     gpu_node_chain();
     gpu_norm_add_tests();
   } else {
     cpu_router_argument_errors();
     cpu_expert_node_paths();
     cpu_expert_fp16_argument_errors();
+    cpu_dense_ffn_argument_errors();
     cpu_merge_argument_errors();
     cpu_norm_add_argument_errors();
   }

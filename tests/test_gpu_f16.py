@@ -201,3 +201,30 @@ def test_layer_kinds_do_not_mix(lib):
     with lib.layer(2, 1, 32, 32) as layer:
         with pytest.raises(capi.CskError, match="MXFP4 experts"):
             layer.set_expert_f16(0, *[np.zeros((32, 32), np.float16)] * 3)
+
+
+@pytest.mark.parametrize("T,H,F", [(1, 64, 96), (7, 37, 29), (64, 96, 160), (65, 96, 160), (300, 128, 72),
+                                   (3, 1024, 2048)])
+@pytest.mark.parametrize("bias", ["none", "all", "down_only"])
+def test_dense_ffn_matches_oracle(lib, oracle, T, H, F, bias):
+    """The shared expert (dense_ffn_node): every token through one fp16 gated MLP."""
+    rng = np.random.default_rng([T, H, F])
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    w_up, w_gate, w_down = random_f16_expert(rng, H, F, 0.1)
+    bg, bu, bd = [rng.standard_normal(n).astype(np.float32) * 0.1 for n in (F, F, H)]
+    if bias == "none":
+        bg = bu = bd = None
+    elif bias == "down_only":
+        bg = bu = None
+    got = lib.dense_ffn_f16(hidden, w_gate, w_up, w_down, bg, bu, bd)
+    want = oracle.dense_ffn_f16(hidden, w_gate, w_up, w_down, bg, bu, bd)
+    assert_layer_close(got, want)
+
+
+def test_dense_ffn_shape_errors(lib):
+    hidden = np.zeros((2, 8), np.float32)
+    g, u, d = np.zeros((4, 8), np.float16), np.zeros((4, 8), np.float16), np.zeros((8, 4), np.float16)
+    with pytest.raises(capi.CskError, match="gate_w/up_w shape mismatch"):
+        lib.dense_ffn_f16(hidden, g, np.zeros((5, 8), np.float16), d)
+    with pytest.raises(capi.CskError, match="down_w shape mismatch, expected"):
+        lib.dense_ffn_f16(hidden, g, u, np.zeros((8, 5), np.float16))

@@ -126,3 +126,18 @@ def test_layer_with_fp16_experts_equals_node_chain(oracle):
     rc, merged = oracle.expert_merge(pairs, outs, H)
     assert rc == 0
     assert np.array_equal(out, merged)
+
+
+@pytest.mark.parametrize("T,H,F", [(1, 8, 8), (5, 37, 29), (3, 64, 96)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_dense_ffn_against_float64(oracle, T, H, F, bias):
+    """dense_ffn_node.h:163-218: every token, standard SwiGLU, weight order gate, up, down."""
+    rng = np.random.default_rng([T, H, F, bias])
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    w_up, w_gate, w_down = random_f16_expert(rng, H, F, 0.2)
+    b = [rng.standard_normal(n).astype(np.float32) * 0.1 for n in (F, F, H)] if bias else [None] * 3
+    got = oracle.dense_ffn_f16(hidden, w_gate, w_up, w_down, *b)
+    for t in range(T):
+        want = mlp_f64(hidden[t], w_up, w_gate, w_down, b[1], b[0], b[2], act=1)
+        assert np.abs(got[t] - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+        assert np.array_equal(got[t], oracle.expert_token_f16(hidden[t], w_up, w_gate, w_down, b[1], b[0], b[2], act=1))
