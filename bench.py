@@ -401,7 +401,7 @@ def main():
         roof = dict(bound="mfma", kernel="expert_f16_gemm_kernel<0> (gate/up + SwiGLU)", achieved=fl / (st["gateup"] * 1e-3) / 1e12,
                     peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s", traffic=None)
     elif f16:
-        roof = dict(bound="hbm", kernel="expert_f16_kernel<0,1> (gate/up + SwiGLU)",
+        roof = dict(bound="hbm", kernel="expert_f16_kernel<0> (gate/up + SwiGLU)",
                     achieved=res["gateup_gbs"], peak=HBM_PEAK_GBS, unit="GB/s", traffic=None)
     elif prefill:
         st = res["stage_ms"]

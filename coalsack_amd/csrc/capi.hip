@@ -487,7 +487,7 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   a.out = g_f16.actf;
   if (timed) mark(CSK_STAGE_GATEUP);
   if (small) {
-    expert_f16_kernel<0, 1><<<grid, 256, 0, g_stream>>>(a);
+    expert_f16_kernel<0><<<grid, 256, 0, g_stream>>>(a);
   } else {
     ga.list_row = a.list_row, ga.B = a.B, ga.rscale = a.rscale, ga.nkb = a.nkb, ga.N = a.N;
     ga.ntile = a.ntile, ga.out = a.out;
@@ -505,7 +505,7 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   a.ntile = (int)f16_tile_count(H);
   a.out = ws.y;
   if (small) {
-    expert_f16_kernel<1, 1><<<grid, 256, 0, g_stream>>>(a);
+    expert_f16_kernel<1><<<grid, 256, 0, g_stream>>>(a);
   } else {
     ga.list_row = a.list_row, ga.B = a.B, ga.rscale = a.rscale, ga.nkb = a.nkb, ga.N = a.N;
     ga.ntile = a.ntile, ga.out = a.out;

@@ -256,20 +256,22 @@ constexpr int kF16Depth = 4;  // K blocks in flight per wave
 
 // MODE 0: act = activation(W_gate x + b_gate, W_up x + b_up); MODE 1: y = W_down act + b_down.
 // A workgroup of four waves takes one work unit at a time: (expert, pair of 16-row weight
-// tiles -- gate and up tile p, or down tiles 2p and 2p+1 --, group of up to 16 * MT dispatched
+// tiles -- gate and up tile p, or down tiles 2p and 2p+1 --, group of up to 16 dispatched
 // tokens).  Units are numbered expert-major, then pair, then group, so the groups of one
 // expert meet their weight tiles in cache at the same time.  The four waves split K; each
 // keeps kF16Depth blocks of loads in flight in a rotating register set; the partial sums
 // meet in LDS and are added in a fixed order.  The weights are the A operand (rows 4g..4g+3
 // of the tile end up in one lane), the tokens the B operand (lane % 16).
-template <int MODE, int MT>
+constexpr int kF16GroupTokens = 16;
+
+template <int MODE>
 __global__ __launch_bounds__(256) void expert_f16_kernel(ExpertF16Args a) {
   __shared__ int prefix[kMaxExperts + 1];
-  __shared__ floatx4 red[4][2][MT][64];
+  __shared__ floatx4 red[4][2][64];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int n16 = lane & 15, g = lane >> 4;
   const int npair = MODE == 0 ? a.ntile : (a.ntile + 1) / 2;
-  constexpr int GT = 16 * MT;  // tokens per group
+  constexpr int GT = kF16GroupTokens;
   // units per slot, exclusive prefix over slots (wave 0; four consecutive slots per lane)
   if (wv == 0) {
     int c[4], tot = 0;
@@ -316,42 +318,27 @@ __global__ __launch_bounds__(256) void expert_f16_kernel(ExpertF16Args a) {
     const int t1 = MODE == 0 ? p : min(2 * p + 1, a.ntile - 1);
     const CSK_GLOBAL u32x4* A0 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_gate : wd->w.q_down)) + (long)t0 * a.nkb * 64 + lane;
     const CSK_GLOBAL u32x4* A1 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_up : wd->w.q_down)) + (long)t1 * a.nkb * 64 + lane;
-    // activation rows of the lane's token slots (slots past the group re-read its last row)
-    const CSK_GLOBAL u32x4* Brow[MT];
-    float rs[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int pos = base + m0 + min(n16 + 16 * mt, cnt - 1);
-      const long row = a.list_row ? a.list_row[pos] : pos;
-      Brow[mt] = as_global(a.B) + row * a.nkb * 8 + g;
-      rs[mt] = a.rscale[row];
-    }
-    floatx4 acc[2][MT];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[t][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    // activation row of the lane's token slot (slots past the group re-read its last row)
+    const int pos_l = base + m0 + min(n16, cnt - 1);
+    const long row = a.list_row ? a.list_row[pos_l] : pos_l;
+    const CSK_GLOBAL u32x4* Brow = as_global(a.B) + row * a.nkb * 8 + g;
+    const float scale = a.rscale[row];
+    floatx4 acc[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
 
-    u32x4 qa[kF16Depth][2], qh[kF16Depth][MT], ql[kF16Depth][MT];
+    u32x4 qa[kF16Depth][2], qh[kF16Depth], ql[kF16Depth];
     auto fetch = [&](int slot, int kb) {
       const int kc = min(kb, kb_hi - 1);  // past the wave's range: re-read its last block
       qa[slot][0] = A0[(long)kc * 64];
       qa[slot][1] = A1[(long)kc * 64];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        qh[slot][mt] = Brow[mt][(long)kc * 8];
-        ql[slot][mt] = Brow[mt][(long)kc * 8 + 4];
-      }
+      qh[slot] = Brow[(long)kc * 8];
+      ql[slot] = Brow[(long)kc * 8 + 4];
     };
     auto fma_block = [&](int slot) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         const half8 wa = __builtin_bit_cast(half8, qa[slot][t]);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, __builtin_bit_cast(half8, qh[slot][mt]), acc[t][mt], 0, 0, 0);
-          acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, __builtin_bit_cast(half8, ql[slot][mt]), acc[t][mt], 0, 0, 0);
-        }
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, __builtin_bit_cast(half8, qh[slot]), acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wa, __builtin_bit_cast(half8, ql[slot]), acc[t], 0, 0, 0);
       }
     };
     if (kb_lo < kb_hi) {
@@ -365,38 +352,28 @@ __global__ __launch_bounds__(256) void expert_f16_kernel(ExpertF16Args a) {
         }
       }
     }
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) red[wv][t][mt][lane] = acc[t][mt];
+    red[wv][0][lane] = acc[0];
+    red[wv][1][lane] = acc[1];
     __syncthreads();
-    // wave w finishes token sub-groups w, w + 4, ...: partial sums in wave order, scale,
-    // bias, activation
-    for (int mt = wv; mt < MT; mt += 4) {
+    // wave 0 finishes the unit: partial sums in wave order, row scale, bias, activation
+    if (wv == 0 && n16 < cnt) {
       floatx4 v[2];
 #pragma unroll
       for (int t = 0; t < 2; ++t)
-        v[t] = ((red[0][t][mt][lane] + red[1][t][mt][lane]) + red[2][t][mt][lane]) + red[3][t][mt][lane];
-      const int slot = n16 + 16 * mt;
-      if (slot < cnt) {
-        const long pos = base + m0 + slot;
-        float scale = 1.0f;
+        v[t] = ((red[0][t][lane] + red[1][t][lane]) + red[2][t][lane]) + red[3][t][lane];
+      const long pos = base + m0 + n16;
+      const CSK_GLOBAL float* b0 = as_global(MODE == 0 ? wd->w.b_gate : wd->w.b_down);
+      const CSK_GLOBAL float* b1 = as_global(MODE == 0 ? wd->w.b_up : wd->w.b_down);
 #pragma unroll
-        for (int q = 0; q < MT; ++q)
-          if (q == mt) scale = rs[q];
-        const CSK_GLOBAL float* b0 = as_global(MODE == 0 ? wd->w.b_gate : wd->w.b_down);
-        const CSK_GLOBAL float* b1 = as_global(MODE == 0 ? wd->w.b_up : wd->w.b_down);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (MODE == 0) {
-            const int f = 16 * p + 4 * g + i;
-            if (f < a.N)
-              a.out[pos * a.N + f] = moe_activation(v[0][i] * scale + b0[f], v[1][i] * scale + b1[f], a.act_type);
-          } else {
-            const int h0 = 16 * (2 * p) + 4 * g + i, h1 = h0 + 16;
-            if (h0 < a.N) a.out[pos * a.N + h0] = v[0][i] * scale + b0[h0];
-            if (h1 < a.N) a.out[pos * a.N + h1] = v[1][i] * scale + b1[h1];
-          }
+      for (int i = 0; i < 4; ++i) {
+        if (MODE == 0) {
+          const int f = 16 * p + 4 * g + i;
+          if (f < a.N)
+            a.out[pos * a.N + f] = moe_activation(v[0][i] * scale + b0[f], v[1][i] * scale + b1[f], a.act_type);
+        } else {
+          const int h0 = 16 * (2 * p) + 4 * g + i, h1 = h0 + 16;
+          if (h0 < a.N) a.out[pos * a.N + h0] = v[0][i] * scale + b0[h0];
+          if (h1 < a.N) a.out[pos * a.N + h1] = v[1][i] * scale + b1[h1];
         }
       }
     }
