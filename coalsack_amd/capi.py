@@ -78,6 +78,7 @@ SIGNATURES = {
     "csk_expert_mlp_f16": (C.c_int, [C.c_int, _P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P,
                                      _I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]),
     "csk_dense_ffn_f16": (C.c_int, [_P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]),
+    "csk_matmul_transpose_f16": (C.c_int, [_P, _I64, _I64, _P, _P]),
     "csk_expert_token_mxfp4": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, C.c_int]),
     "csk_expert_merge": (C.c_int, [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]),
     "csk_rmsnorm": (C.c_int, [_P, _P, _P, _I64, _I64, C.c_float]),
@@ -274,6 +275,18 @@ class Library:
         finally:
             for h in hs:
                 self.f16_free(h)
+        return out
+
+    def matmul_transpose_f16(self, a, w):
+        """a [M,K] f32 x w [N,K]^T (float16) -> [M,N]; uploads w for the call."""
+        a = _f32(a)
+        M, K = a.shape
+        h = self.f16_upload(w)
+        try:
+            out = np.empty((M, w.shape[0]), np.float32)
+            self.check(self.dll.csk_matmul_transpose_f16(_ptr(a), M, K, h, _ptr(out)))
+        finally:
+            self.f16_free(h)
         return out
 
     # -- node-level ops

@@ -447,6 +447,41 @@ int launch_f16_split(const float* x, int64_t rows, int64_t K, const int* gather_
   return check_launch("f16_split_rows_kernel");
 }
 
+// y[P, N] <- W_down(expert of the position) x rows + b_down over two-term fp16 rows [P, K]:
+// the down projection of the experts, and any plain linear layer (one descriptor).
+int launch_f16_projection(int64_t E, int64_t T, int64_t P, int64_t K, int64_t N, const uint16_t* rows,
+                          const float* rscale, float* y, Workspace& ws) {
+  if (T <= 64) {
+    ExpertF16Args a{};
+    a.desc = ws.desc;
+    a.n_slots = (int)E;
+    a.list_row = nullptr;
+    a.B = reinterpret_cast<const u32x4*>(rows);
+    a.rscale = rscale;
+    a.nkb = (int)f16_block_count(K);
+    a.N = (int)N;
+    a.ntile = (int)f16_tile_count(N);
+    a.out = y;
+    expert_f16_kernel<1><<<dim3((unsigned)(4 * std::max(g_cus, 1))), 256, 0, g_stream>>>(a);
+  } else {
+    ExpertF16GemmArgs ga{};
+    ga.desc = ws.desc;
+    ga.mtiles = ws.tiles;
+    ga.n_mtiles = ws.n_tiles;
+    ga.list_row = nullptr;
+    ga.B = reinterpret_cast<const u32x4*>(rows);
+    ga.rscale = rscale;
+    ga.nkb = (int)f16_block_count(K);
+    ga.N = (int)N;
+    ga.ntile = (int)f16_tile_count(N);
+    ga.n_ntiles = (int)cdiv(N, 256);
+    ga.out = y;
+    const int64_t max_mtiles = P / 64 + std::min<int64_t>(E, P);
+    expert_f16_gemm_kernel<1><<<dim3((unsigned)(cdiv(max_mtiles * ga.n_ntiles, kF16Dies) * kF16Dies)), 256, 0, g_stream>>>(ga);
+  }
+  return check_launch("expert_f16_kernel<1>");
+}
+
 // Experts with fp16 weights over the dispatched tokens: ws.y[P,H] <- down(act(gate, up)).
 // x is [T,H] fp32.  Up to 64 tokens every expert's tokens form groups of 16 (one pass over
 // the weights per group, HBM-bound); beyond that groups of 64.
@@ -497,22 +532,7 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   if ((rc = check_launch("expert_f16_kernel<0>")) != CSK_OK) return rc;
   if (timed) mark(CSK_STAGE_DOWN);
   if ((rc = launch_f16_split(g_f16.actf, P, F, nullptr, nullptr, ws.act, g_f16.rs_a)) != CSK_OK) return rc;
-  a.list_row = nullptr;
-  a.B = reinterpret_cast<const u32x4*>(ws.act);
-  a.rscale = g_f16.rs_a;
-  a.nkb = (int)f16_block_count(F);
-  a.N = (int)H;
-  a.ntile = (int)f16_tile_count(H);
-  a.out = ws.y;
-  if (small) {
-    expert_f16_kernel<1><<<grid, 256, 0, g_stream>>>(a);
-  } else {
-    ga.list_row = a.list_row, ga.B = a.B, ga.rscale = a.rscale, ga.nkb = a.nkb, ga.N = a.N;
-    ga.ntile = a.ntile, ga.out = a.out;
-    ga.n_ntiles = (int)cdiv(H, 256);
-    expert_f16_gemm_kernel<1><<<gemm_grid(ga.n_ntiles), 256, 0, g_stream>>>(ga);
-  }
-  return check_launch("expert_f16_kernel<1>");
+  return launch_f16_projection(E, T, P, F, H, ws.act, g_f16.rs_a, ws.y, ws);
 }
 
 int check_dims(int64_t E, int64_t k, int64_t H, int64_t F) {
@@ -1457,6 +1477,36 @@ extern "C" int csk_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int6
   rc = run_experts_f16(1, T, 1, H, F, CSK_ACT_STANDARD_SWIGLU, dx.as<float>(), false, T, ws, false, true);
   if (rc != CSK_OK) return rc;
   HIP_TRY(hipMemcpyAsync(out, ws.y, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+extern "C" int csk_matmul_transpose_f16(const float* a_host, int64_t M, int64_t K, const csk_f16* w,
+                                       float* out) {
+  REQUIRE_INIT();
+  if (!a_host || !w || !out || M < 0 || K <= 0)
+    return fail(CSK_ERR_ARG, "csk_matmul_transpose_f16: null argument");
+  if (w->K != K) return fail(CSK_ERR_ARG, "matmul_transpose_mixed: incompatible dimensions");
+  if (M == 0) return CSK_OK;
+  if (M > (int64_t)1 << 24) return fail(CSK_ERR_ARG, "matmul_transpose_mixed: more than 2^24 rows");
+  const int64_t N = w->rows;
+  Workspace& ws = g_ws;
+  // rows of A take the place of the activations of a down projection: [M, K] -> [M, N]
+  int rc = ws.ensure(M, 1, 1, cdiv(N, 32) * 32, cdiv(K, 32) * 32, false);
+  if (rc == CSK_OK) rc = g_f16.ensure((size_t)M, 1);
+  if (rc != CSK_OK) return rc;
+  DevBuf da, dew;
+  if ((rc = da.upload(a_host, (size_t)M * K * 4)) != CSK_OK) return rc;
+  ExpertW ew{};
+  ew.q_down = reinterpret_cast<const uint4*>(w->w);
+  ew.b_gate = ew.b_up = ew.b_down = g_zero;
+  if ((rc = dew.upload(&ew, sizeof ew)) != CSK_OK) return rc;
+  dense_desc_kernel<<<1, 256, 0, g_stream>>>(ws.desc, dew.as<ExpertW>(), (int)M, ws.tiles, ws.n_tiles);
+  if ((rc = check_launch("dense_desc_kernel")) != CSK_OK) return rc;
+  if ((rc = launch_f16_split(da.as<float>(), M, K, nullptr, nullptr, ws.act, g_f16.rs_a)) != CSK_OK) return rc;
+  rc = launch_f16_projection(1, M, M, K, N, ws.act, g_f16.rs_a, ws.y, ws);
+  if (rc != CSK_OK) return rc;
+  HIP_TRY(hipMemcpyAsync(out, ws.y, (size_t)M * N * 4, hipMemcpyDeviceToHost, g_stream));
   HIP_TRY(hipStreamSynchronize(g_stream));
   return CSK_OK;
 }

@@ -253,6 +253,11 @@ int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T, int64_t H,
 int csk_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int64_t F, const csk_f16* w_gate,
                       const csk_f16* w_up, const csk_f16* w_down, const float* b_gate,
                       const float* b_up, const float* b_down, float* out);
+/* matmul_transpose_mixed_node::compute with a 2-D float16 weight
+ * (include/coalsack/nn/nn_ops/matmul_transpose_mixed_node.h:25-110, compute_matmul_avx2_fp16b
+ * :198-308): out [M,N] = A [M,K] (fp32, leading dimensions flattened) x W [N,K]^T -- the
+ * engine's linear projections (include/coalsack/llm/graph_builder.h:90-105). */
+int csk_matmul_transpose_f16(const float* a_host, int64_t M, int64_t K, const csk_f16* w, float* out_host);
 /* expert_mlp_node::compute_test_mxfp4 (expert_mlp_node.h:63-70): one token,
  * raw 17-byte-block weights in host memory. */
 int csk_expert_token_mxfp4(const float* hidden_vec, const uint8_t* w_up, const uint8_t* w_gate,

@@ -79,6 +79,8 @@ class Oracle:
             [_I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]
         d.orc_dense_ffn_f16.restype = C.c_int
         d.orc_dense_ffn_f16.argtypes = [_P, _I64, _I64, _I64] + [_P] * 7
+        d.orc_matmul_transpose_f16.restype = None
+        d.orc_matmul_transpose_f16.argtypes = [_P, _P, _P, _I64, _I64, _I64]
         d.orc_expert_merge.restype = C.c_int
         d.orc_expert_merge.argtypes = [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]
         d.orc_rmsnorm.restype = None
@@ -204,6 +206,15 @@ class Oracle:
                                         _p(b_up), _p(b_down), _p(out))
         if rc:
             raise ValueError(f"orc_dense_ffn_f16 rc={rc}")
+        return out
+
+    def matmul_transpose_f16(self, a, b):
+        """matmul_transpose_mixed_node with a float16 weight: a [M,K] f32, b [N,K] f16 -> [M,N]."""
+        a, b = _f32(a), _f16(b)
+        M, K = a.shape
+        N = b.shape[0]
+        out = np.empty((M, N), np.float32)
+        self.dll.orc_matmul_transpose_f16(_p(a), _p(b), _p(out), M, K, N)
         return out
 
     def expert_merge(self, pairs, expert_outs, H, pre_weighted=False):

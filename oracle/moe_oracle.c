@@ -45,6 +45,10 @@
  *   orc_dense_ffn_f16
  *        - the fp16 expert function it is built from (pinned above) and an
  *          independent float64 evaluation with the standard SwiGLU.
+ *   orc_matmul_transpose_f16
+ *        - float64 matrix product over the fp16 weights widened exactly, shapes
+ *          that exercise both column paths and every remainder, identity /
+ *          one-hot weights.  PARITY UNPINNED at the last ulp, as above.
  *   orc_expert_merge
  *        - definition sum_k w_k * y_{e_k}; one-hot weights reduce to a copy;
  *          linearity; error cases.
@@ -603,6 +607,40 @@ int orc_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int64_t F, cons
                           ORC_ACT_STANDARD_SWIGLU, scratch);
   free(scratch);
   return rc;
+}
+
+/* include/coalsack/nn/nn_ops/matmul_transpose_mixed_node.h:198-308 (compute_matmul_avx2_fp16b):
+ * out[M,N] = A[M,K] (fp32) x B[N,K]^T (fp16), the linear projections of the engine
+ * (graph_builder.h:90-105).  Columns in tiles of four: two 8-lane accumulators per column over
+ * K in steps of 16 (fused multiply-adds), merged, an 8-wide remainder step, the horizontal sum,
+ * then the last K % 8 elements one by one (fused, as g++ contracts them in a function compiled
+ * for FMA hardware); the N % 4 remainder columns use one accumulator over steps of 8. */
+__attribute__((target("f16c,avx2,fma"))) void orc_matmul_transpose_f16(const float* a, const uint16_t* b,
+                                                                        float* out, int64_t M, int64_t K,
+                                                                        int64_t N) {
+  for (int64_t i = 0; i < M; ++i) {
+    const float* ar = a + i * K;
+    for (int64_t j = 0; j < N; ++j) {
+      const uint16_t* br = b + j * K;
+      const int tiled = j < (N / 4) * 4;
+      int64_t k = 0;
+      __m256 sum = _mm256_setzero_ps();
+      if (tiled) {
+        __m256 sa = _mm256_setzero_ps(), sb = _mm256_setzero_ps();
+        for (; k + 16 <= K; k += 16) {
+          sa = _mm256_fmadd_ps(_mm256_loadu_ps(ar + k), _mm256_cvtph_ps(_mm_loadu_si128((const __m128i*)(br + k))), sa);
+          sb = _mm256_fmadd_ps(_mm256_loadu_ps(ar + k + 8),
+                               _mm256_cvtph_ps(_mm_loadu_si128((const __m128i*)(br + k + 8))), sb);
+        }
+        sum = _mm256_add_ps(sa, sb);
+      }
+      for (; k + 8 <= K; k += 8)
+        sum = _mm256_fmadd_ps(_mm256_loadu_ps(ar + k), _mm256_cvtph_ps(_mm_loadu_si128((const __m128i*)(br + k))), sum);
+      float r = hsum_avx2(sum);
+      for (; k < K; ++k) r = __builtin_fmaf(ar[k], half_to_float(br[k]), r);
+      out[i * N + j] = r;
+    }
+  }
 }
 
 /* ------------------------------------------------------------------ merge */

@@ -14,6 +14,7 @@
 #include "coalsack/nn/nn_ops/add_node.h"
 #include "coalsack/nn/nn_ops/dense_ffn_node.h"
 #include "coalsack/nn/nn_ops/expert_merge_node.h"
+#include "coalsack/nn/nn_ops/matmul_transpose_mixed_node.h"
 #include "coalsack/nn/nn_ops/expert_mlp_node.h"
 #include "coalsack/nn/nn_ops/moe_router_node.h"
 #include "coalsack/nn/nn_ops/rmsnorm_node.h"
@@ -33,6 +34,7 @@ int orc_expert_mlp_f16(int, const float*, int64_t, int64_t, int64_t, const uint1
                        int, float*, int*);
 int orc_dense_ffn_f16(const float*, int64_t, int64_t, int64_t, const uint16_t*, const uint16_t*, const uint16_t*,
                       const float*, const float*, const float*, float*);
+void orc_matmul_transpose_f16(const float*, const uint16_t*, float*, int64_t, int64_t, int64_t);
 void orc_rmsnorm(const float*, const float*, float*, int64_t, int64_t, float);
 void orc_add(const float*, const float*, float*, int64_t);
 }
@@ -254,6 +256,20 @@ static void cpu_dense_ffn_argument_errors() {
   CHECK(throws_with([&] { node.compute_test({hidden, random_tensor({16, 8}, gen, -1, 1), random_tensor({16, 8}, gen, -1, 1),
                                              random_tensor({8, 16}, gen, -1, 1)}); },
                     "dense_ffn: FLOAT32 weights are not supported on this build"));
+}
+
+static void cpu_matmul_argument_errors() {
+  std::printf("matmul_transpose_mixed: argument errors\n");
+  std::mt19937 gen(6);
+  matmul_transpose_mixed_node node;
+  CHECK(node.get_proc_name() == "nn_matmul_transpose_mixed");
+  auto a = random_tensor({2, 3, 8}, gen, -1, 1);
+  auto w = random_half_tensor({5, 8}, gen, -1, 1);
+  CHECK(throws_with([&] { node.compute_test(dynamic_tensor(dtype::float64, {3, 8}), w); }, "matmul_transpose_mixed: input A must be fp32"));
+  CHECK(throws_with([&] { node.compute_test(a, dynamic_tensor(dtype::int32, {5, 8})); }, "matmul_transpose_mixed: input B must be fp32 or fp16"));
+  CHECK(throws_with([&] { node.compute_test(dynamic_tensor(dtype::float32, {8}), w); }, "matmul_transpose_mixed: inputs must be at least 2D"));
+  CHECK(throws_with([&] { node.compute_test(a, random_half_tensor({5, 7}, gen, -1, 1)); }, "matmul_transpose_mixed: incompatible dimensions"));
+  CHECK(throws_with([&] { node.compute_test(a, random_tensor({5, 8}, gen, -1, 1)); }, "only a 2D fp16 input B is supported"));
 }
 
 static void cpu_merge_argument_errors() {
@@ -486,6 +502,25 @@ static void gpu_expert_fp16_tests() {
   CHECK(std::fabs(out.data_ptr<float>()[0] - want) < 1e-3f);
 }
 
+static void gpu_matmul_tests() {
+  std::printf("matmul_transpose_mixed: projections against the CPU path\n");
+  std::mt19937 gen(10);
+  for (const auto& dims : std::vector<std::vector<int64_t>>{{1, 1, 64, 96}, {2, 40, 72, 130}, {1, 3, 30, 21}}) {
+    const int64_t B = dims[0], S = dims[1], K = dims[2], N = dims[3];
+    auto a = random_tensor({B, S, K}, gen, -1, 1);
+    auto w = random_half_tensor({N, K}, gen, -0.2f, 0.2f);
+    matmul_transpose_mixed_node node;
+    auto out = node.compute_test(a, w);
+    CHECK((out.shape() == std::vector<int64_t>{B, S, N}));
+    std::vector<float> want(B * S * N);
+    orc_matmul_transpose_f16(a.data_ptr<float>(), w.data_ptr<uint16_t>(), want.data(), B * S, K, N);
+    float worst = 0;
+    for (int64_t i = 0; i < out.numel(); ++i)
+      worst = std::fmax(worst, std::fabs(out.data_ptr<float>()[i] - want[i]) / std::fmax(1.0f, std::fabs(want[i])));
+    CHECK(worst <= 1e-3f);
+  }
+}
+
 static void gpu_dense_ffn_tests() {
   std::printf("dense_ffn: shared expert through result messages, against the CPU path\n");
   std::mt19937 gen(9);
@@ -620,6 +655,7 @@ int main(int argc, char** argv) {
     gpu_expert_known_answer();
     gpu_expert_fp16_tests();
     gpu_dense_ffn_tests();
+    gpu_matmul_tests();
     gpu_node_chain();
     gpu_norm_add_tests();
   } else {
@@ -627,6 +663,7 @@ int main(int argc, char** argv) {
     cpu_expert_node_paths();
     cpu_expert_fp16_argument_errors();
     cpu_dense_ffn_argument_errors();
+    cpu_matmul_argument_errors();
     cpu_merge_argument_errors();
     cpu_norm_add_argument_errors();
   }

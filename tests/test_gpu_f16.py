@@ -228,3 +228,18 @@ def test_dense_ffn_shape_errors(lib):
         lib.dense_ffn_f16(hidden, g, np.zeros((5, 8), np.float16), d)
     with pytest.raises(capi.CskError, match="down_w shape mismatch, expected"):
         lib.dense_ffn_f16(hidden, g, u, np.zeros((8, 5), np.float16))
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 64, 96), (7, 37, 29), (64, 2880, 512), (65, 96, 160), (300, 128, 72),
+                                   (2, 5120, 1024)])
+def test_matmul_transpose_matches_oracle(lib, oracle, M, K, N):
+    """matmul_transpose_mixed_node with a float16 weight (the engine's linear projections)."""
+    rng = np.random.default_rng([M, K, N])
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.1).astype(np.float16)
+    got = lib.matmul_transpose_f16(a, w)
+    want = oracle.matmul_transpose_f16(a, w)
+    assert got.shape == (M, N)
+    assert_layer_close(got, want)
+    with pytest.raises(capi.CskError, match="incompatible dimensions"):
+        lib.matmul_transpose_f16(a[:, :K - 1] if K > 1 else a, w)

@@ -141,3 +141,17 @@ def test_dense_ffn_against_float64(oracle, T, H, F, bias):
         want = mlp_f64(hidden[t], w_up, w_gate, w_down, b[1], b[0], b[2], act=1)
         assert np.abs(got[t] - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
         assert np.array_equal(got[t], oracle.expert_token_f16(hidden[t], w_up, w_gate, w_down, b[1], b[0], b[2], act=1))
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 8, 4), (3, 37, 5), (5, 64, 7), (2, 24, 9), (4, 100, 16)])
+def test_matmul_transpose_against_float64(oracle, M, K, N):
+    """matmul_transpose_mixed_node.h:198-308 with a float16 weight: both column paths (tiles of
+    four, remainder columns) and every K remainder."""
+    rng = np.random.default_rng([M, K, N])
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.3).astype(np.float16)
+    got = oracle.matmul_transpose_f16(a, w)
+    want = a.astype(np.float64) @ w.astype(np.float64).T
+    assert np.abs(got - want).max() <= 2e-6 * np.sqrt(K) * max(1.0, np.abs(want).max())
+    eye = np.eye(N, K, dtype=np.float16)
+    assert np.array_equal(oracle.matmul_transpose_f16(a, eye), a[:, :N] if N <= K else np.pad(a, ((0, 0), (0, N - K))))
