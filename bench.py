@@ -12,7 +12,7 @@ projections), timed live with HIP events on the library's stream;
 single-threaded path) timed on this host on a bounded sample.
 
 Workloads (BASELINE.json configs):
-  c2_20b_decode   32 experts, top-4, H = F = 2880, T in {1,2,4,8,16,32} (default, T=16)
+  c2_20b_decode   32 experts, top-4, H = F = 2880, T in {1,2,4,8,16,32,64} (default, T=16)
   c3_20b_prefill  same layer, T = 2048
   c4_120b         128 experts, 8 hot experts (+2.0 router bias), T in {1,16,4096}
   c5_stack        36 layers of the 120b shape with RMSNorm + residual, T in {1,8,64}
@@ -37,7 +37,7 @@ MFMA_FP4_PEAK_TFLOPS = 10100.0  # dense MXFP4, published
 MFMA_F16_PEAK_TFLOPS = 2500.0   # dense fp16, published
 
 SHAPES = {
-    "c2_20b_decode": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=16, sweep=[1, 2, 4, 8, 16, 32]),
+    "c2_20b_decode": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=16, sweep=[1, 2, 4, 8, 16, 32, 64]),
     "c3_20b_prefill": dict(E=32, k=4, H=2880, F=2880, hot=0, default_T=2048, sweep=[]),
     "c4_120b": dict(E=128, k=4, H=2880, F=2880, hot=8, default_T=16, sweep=[1, 16]),
     "c5_stack": dict(E=128, k=4, H=2880, F=2880, hot=8, default_T=8, sweep=[1, 8, 64], layers=36),

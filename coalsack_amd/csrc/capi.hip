@@ -332,32 +332,43 @@ int launch_router(const float* x, const float* gate_w, const float* gate_b, int6
   return check_launch("router_topk_kernel");
 }
 
+// Tokens of an expert contracted per pass over its weights by the streaming kernel.  An
+// expert with more tokens than that is streamed once per group, so larger batches take
+// groups of six (at 32 tokens and top-4 of 32 experts a quarter fewer passes); up to 16
+// tokens few experts see more than four and the four-token kernel, which is the faster of
+// the two per byte, wins (measured at T = 8, 16, 32).
+inline int stream_group_tokens(int64_t T) { return T <= 16 ? kStreamG : kStreamGWide; }
+
 int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, int64_t E,
                     const ExpertW* ew, Workspace& ws) {
   dispatch_scatter_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(
       ids, pairs, (int)P, (int)k, (int)E, ws.counts, ew, ws.offsets, ws.desc,
       P <= kStreamMaxP ? ws.vlist : nullptr, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w,
-      ws.pos);
+      ws.pos, stream_group_tokens(P / std::max<int64_t>(k, 1)));
   return check_launch("dispatch_scatter_kernel");
 }
 
 // Weight-streaming kernel for small batches (every expert sees few tokens, the
 // layer is HBM-bound); grouped GEMM otherwise.
+template <int NMAT, int G>
+int launch_stream(ExpertStreamArgs a, int64_t P, Workspace& ws) {
+  a.vlist = ws.vlist;
+  a.nv = ws.nv;
+  // kStreamWgPerCu workgroups per compute unit in steady state; a batch so small that
+  // every work unit can have a workgroup of its own (three fit a compute unit) gets that
+  const int64_t npair = NMAT == 2 ? a.ntile : (a.ntile + 1) / 2;
+  const int64_t cus = std::max(g_cus, 1);
+  const int64_t nwg = (G == kStreamG && P * npair <= 3 * cus) ? P * npair : kStreamWgPerCu * cus;  // (small P implies G == kStreamG)
+  const size_t lds = (size_t)G * a.nblk * 128 + (size_t)2 * 4 * ((G + 3) / 4) * 8 * 16 * sizeof(float);
+  expert_stream_kernel<NMAT == 2 ? 0 : 1, G><<<dim3((unsigned)nwg), 256, lds, g_stream>>>(a);
+  return check_launch("expert_stream_kernel");
+}
+
 template <int NMAT>
 int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspace& ws, bool stream) {
-  if (stream) {
-    constexpr int G = kStreamG;
-    a.vlist = ws.vlist;
-    a.nv = ws.nv;
-    // kStreamWgPerCu workgroups per compute unit in steady state; a batch so small that
-    // every work unit can have a workgroup of its own (three fit a compute unit) gets that
-    const int64_t npair = NMAT == 2 ? a.ntile : (a.ntile + 1) / 2;
-    const int64_t cus = std::max(g_cus, 1);
-    const int64_t nwg = P * npair <= 3 * cus ? P * npair : kStreamWgPerCu * cus;
-    const size_t lds = (size_t)G * a.nblk * 128 + 2 * 4 * 8 * 16 * sizeof(float);
-    expert_stream_kernel<NMAT == 2 ? 0 : 1, G><<<dim3((unsigned)nwg), 256, lds, g_stream>>>(a);
-    return check_launch("expert_stream_kernel");
-  }
+  if (stream)
+    return stream_group_tokens(T) == kStreamG ? launch_stream<NMAT, kStreamG>(a, P, ws)
+                                              : launch_stream<NMAT, kStreamGWide>(a, P, ws);
   ExpertGemmMxArgs ga{};
   ga.desc = a.desc;
   ga.mtiles = ws.tiles;
@@ -1102,7 +1113,7 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
     route_small_kernel<<<dim3(1), kRouteSmallThreads, 0, g_stream>>>(
         ws.logits, ws.pairs, ws.ids, (int)T, (int)L->E, (int)L->k, L->sigmoid, L->ew_dev, ws.counts,
         ws.offsets, ws.desc, ws.vlist, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w, ws.pos,
-        xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, (int)L->H);
+        xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, (int)L->H, stream_group_tokens(T));
     if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
     if (!L->f16 && !stream_path(T, L->H, L->F) && !L->wbf) {
       // few tokens but rows too long for the streaming kernel: the GEMM wants the FP6 form

@@ -17,7 +17,8 @@ constexpr int kTileRows = 16;   // weight rows per packed tile (= MFMA N)
 constexpr int kBlk = 32;        // MXFP4 block length along K
 constexpr int kMaxTopK = 16;
 constexpr int kMaxExperts = 256;
-constexpr int kStreamG = 4;      // tokens per pass of the weight-streaming expert kernel
+constexpr int kStreamG = 4;      // tokens per pass of the weight-streaming expert kernel: batches of up to four tokens
+constexpr int kStreamGWide = 6;  // ... and larger ones (six rows of activations are what two workgroups per compute unit can hold in LDS)
 
 // Resident weights of one expert.  Each matrix [rows, K] is stored as
 //   q: [rows/16][K/32][16] x 16 bytes -- byte b of an entry holds elements

@@ -31,7 +31,7 @@ struct WorkDesc {
 // unconditional.
 struct ExpertStreamArgs {
   const WorkDesc* desc;
-  const int* vlist;      // [2 * nv]: (expert slot, first token) of each group of kStreamG tokens
+  const int* vlist;      // [2 * nv]: (expert slot, first token) of each group of G tokens
   const int* nv;         // number of such groups
   const int* list_row;   // packed position -> row of A; null: row = packed position
   const uint4* A;        // [rows][nblk][8] x 16 B: 32 bf16 hi then 32 bf16 lo per block
@@ -106,7 +106,8 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
   const int nblk = a.nblk;
   const int row_u4 = nblk * 8;                   // uint4 per activation row
   uint4* As = reinterpret_cast<uint4*>(smem);    // [G][row_u4]
-  float* red = reinterpret_cast<float*>(smem + (size_t)G * row_u4 * 16);  // [2][4][NV][16]: live lanes only
+  constexpr int LG = (G + 3) / 4;  // lane groups g whose accumulator rows 4g..4g+3 hold tokens
+  float* red = reinterpret_cast<float*>(smem + (size_t)G * row_u4 * 16);  // [2][4][LG][NV][16]: live lanes only
 
   const int npair = MODE == 0 ? a.ntile : (a.ntile + 1) >> 1;
   // Teams of W workgroups share one token group and interleave its units
@@ -177,8 +178,8 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
       b0 = bp0[min(ta * 16 + n, a.N - 1)];  // bias pointers are never null (absent bias = zero vector)
       b1 = bp1[min(tb * 16 + n, a.N - 1)];
     };
-    static_assert(G <= 4, "live accumulator rows are those of lanes g == 0");
-    const bool live = g == 0;  // tokens 0..G-1 are accumulator rows 0..3 of lanes 0..15
+    static_assert(G <= 8, "the reduction buffer holds two lane groups");
+    const bool live = g < LG;  // token t is accumulator row t % 4 of lanes 16 (t / 4) .. 16 (t / 4) + 15
 
     // Contracts unit `unit` out of ws and, step by step, refills ws with unit `next`.
     auto compute_unit = [&](WSet& ws, int unit, int next) {
@@ -220,13 +221,13 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
         load_step(ws, next, s);  // this step's registers are free: start the next unit's loads
       }
       load_unit_scalars(ws.sc[0], ws.sc[1], ws.b0, ws.b1, next);
-      float* rbuf = red + (size_t)par * 4 * NV * 16;
+      float* rbuf = red + (size_t)par * 4 * LG * NV * 16;
       par ^= 1;
       if (live) {
 #pragma unroll
         for (int m = 0; m < 2; ++m)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) rbuf[(wv * NV + m * 4 + i) * 16 + n] = acc[m][0][i] + acc[m][1][i];
+          for (int i = 0; i < 4; ++i) rbuf[((wv * LG + g) * NV + m * 4 + i) * 16 + n] = acc[m][0][i] + acc[m][1][i];
       }
       __syncthreads();
       if (wv == (unit & 3) && live) {
@@ -236,8 +237,8 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int o = m * 4 + i;
-            v2[m][i] = ((rbuf[(0 * NV + o) * 16 + n] + rbuf[(1 * NV + o) * 16 + n]) +
-                        rbuf[(2 * NV + o) * 16 + n]) + rbuf[(3 * NV + o) * 16 + n];
+            v2[m][i] = ((rbuf[((0 * LG + g) * NV + o) * 16 + n] + rbuf[((1 * LG + g) * NV + o) * 16 + n]) +
+                        rbuf[((2 * LG + g) * NV + o) * 16 + n]) + rbuf[((3 * LG + g) * NV + o) * 16 + n];
           }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {

@@ -579,7 +579,7 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
     int* __restrict__ counts, const ExpertW* __restrict__ ew, int* __restrict__ offsets,
     WorkDesc* __restrict__ desc, int* __restrict__ vlist, int* __restrict__ nv,
     int* __restrict__ mtiles, int* __restrict__ n_mtiles, int* __restrict__ list_tok,
-    float* __restrict__ list_w, int* __restrict__ pos_of_slot) {
+    float* __restrict__ list_w, int* __restrict__ pos_of_slot, int group_tokens) {
   const int e = blockIdx.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   __shared__ int sh[8];
@@ -624,7 +624,7 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
         cc[j] = ee < E ? cnt[ee] : 0;
         tot += cc[j];
         nact += cc[j] > 0;
-        ngrp += (cc[j] + kStreamG - 1) / kStreamG;
+        ngrp += (cc[j] + group_tokens - 1) / group_tokens;
         nmt += (cc[j] + 63) / 64;
       }
       int s_tot = tot, s_act = nact, s_grp = ngrp, s_mt = nmt;  // inclusive scans over lanes
@@ -648,7 +648,7 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
           offsets[ee] = run;
           if (cc[j] > 0) {
             if (vlist) {
-              for (int gb = 0; gb < cc[j]; gb += kStreamG) {
+              for (int gb = 0; gb < cc[j]; gb += group_tokens) {
                 vlist[2 * gi] = slot;
                 vlist[2 * gi + 1] = gb;
                 ++gi;
@@ -717,7 +717,8 @@ __global__ __launch_bounds__(kRouteSmallThreads) void route_small_kernel(
     int* __restrict__ offsets, WorkDesc* __restrict__ desc, int* __restrict__ vlist,
     int* __restrict__ nv, int* __restrict__ mtiles, int* __restrict__ n_mtiles,
     int* __restrict__ list_tok, float* __restrict__ list_w, int* __restrict__ pos_of_slot,
-    const float* __restrict__ x, const float* __restrict__ g, const float* __restrict__ b, int H) {
+    const float* __restrict__ x, const float* __restrict__ g, const float* __restrict__ b, int H,
+    int group_tokens) {
   constexpr int NW = kRouteSmallThreads / 64;
   __shared__ int ids[1024];
   __shared__ float wts[1024];
@@ -808,7 +809,7 @@ __global__ __launch_bounds__(kRouteSmallThreads) void route_small_kernel(
       c[j] = e < E ? cnt[e] : 0;
       tot += c[j];
       nact += c[j] > 0;
-      ngrp += (c[j] + kStreamG - 1) / kStreamG;
+      ngrp += (c[j] + group_tokens - 1) / group_tokens;
       nmt += (c[j] + 63) / 64;
     }
     int s_tot = tot, s_act = nact, s_grp = ngrp, s_mt = nmt;  // inclusive scans over lanes
@@ -831,7 +832,7 @@ __global__ __launch_bounds__(kRouteSmallThreads) void route_small_kernel(
         off[e] = run;
         offsets[e] = run;
         if (c[j] > 0) {
-          for (int gb = 0; gb < c[j]; gb += kStreamG) {
+          for (int gb = 0; gb < c[j]; gb += group_tokens) {
             vlist[2 * gi] = slot;
             vlist[2 * gi + 1] = gb;
             ++gi;
