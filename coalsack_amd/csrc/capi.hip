@@ -116,7 +116,7 @@ struct Workspace {
     };
     WS_ALLOC(xs, act_elems((size_t)nT, nH));
     if (need_xg || had_xg) WS_ALLOC(xg, act_elems(P, nH));
-    WS_ALLOC(logits, (size_t)nT * nE);
+    WS_ALLOC(logits, (size_t)nT * nE * (1 + kRouterMaxSplits));  // final logits, then partial ones per split of H
     WS_ALLOC(pairs, P * 2);
     WS_ALLOC(ids, P);
     WS_ALLOC(counts, (size_t)nE);
@@ -315,20 +315,31 @@ int launch_router(const float* x, const float* gate_w, const float* gate_b, int6
                   int64_t H, int64_t k, int sigmoid, float* logits, float* pairs, int* ids) {
   if (T == 0) return CSK_OK;
   const unsigned gx = (unsigned)cdiv(E, 4);
+  int nsplit = 0;  // > 0: the logits kernel wrote partial logits behind the [T, E] final ones
   if (T <= 2) {
     router_logits_kernel<1><<<dim3(gx, (unsigned)T), 256, 0, g_stream>>>(x, gate_w, gate_b, logits,
                                                                          (int)T, (int)E, (int)H);
   } else if (T <= 64) {
     router_logits_kernel<4><<<dim3(gx, (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
         x, gate_w, gate_b, logits, (int)T, (int)E, (int)H);
+  } else if (H % 16 == 0 && cdiv(H, 64) <= kRouterChunks * kRouterMaxSplits) {
+    // splits of H: as many as it takes to keep a split's token rows in registers, and to give
+    // the chip two workgroups per compute unit
+    const int64_t nchunk = cdiv(H, 64);
+    int64_t splits = std::max(cdiv(nchunk, kRouterChunks), cdiv(2 * std::max(g_cus, 1), cdiv(T, 32)));
+    splits = std::min<int64_t>(std::min<int64_t>(splits, kRouterMaxSplits), nchunk);
+    const int64_t cps = cdiv(nchunk, splits);
+    nsplit = (int)cdiv(nchunk, cps);
+    router_logits_mfma_kernel<<<dim3((unsigned)cdiv(T, 32), (unsigned)nsplit), 256, 0, g_stream>>>(
+        x, gate_w, logits + T * E, (int)T, (int)E, (int)H, (int)cps);
   } else {
-    router_logits_mfma_kernel<<<dim3((unsigned)cdiv(T, 32), (unsigned)cdiv(E, 32)), 256, 0, g_stream>>>(
+    router_logits_kernel<4><<<dim3(gx, (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
         x, gate_w, gate_b, logits, (int)T, (int)E, (int)H);
   }
   int rc = check_launch("router_logits_kernel");
   if (rc != CSK_OK) return rc;
   router_topk_kernel<<<dim3((unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
-      logits, pairs, ids, (int)T, (int)E, (int)k, sigmoid, x, gate_w, gate_b, (int)H);
+      logits, pairs, ids, (int)T, (int)E, (int)k, sigmoid, x, gate_w, gate_b, (int)H, logits + T * E, nsplit);
   return check_launch("router_topk_kernel");
 }
 
@@ -1272,7 +1283,7 @@ int router_host(const float* hidden, int64_t T, int64_t H, const float* gate_w, 
   if ((rc = dx.upload(hidden, (size_t)T * H * 4)) != CSK_OK) return rc;
   if ((rc = dg.upload(gate_w, (size_t)E * H * 4)) != CSK_OK) return rc;
   if (gate_b && (rc = db.upload(gate_b, (size_t)E * 4)) != CSK_OK) return rc;
-  if ((rc = dl.alloc((size_t)T * E * 4)) != CSK_OK) return rc;
+  if ((rc = dl.alloc((size_t)T * E * 4 * (1 + kRouterMaxSplits))) != CSK_OK) return rc;
   if ((rc = dp.alloc((size_t)T * k * 8)) != CSK_OK) return rc;
   if ((rc = di.alloc((size_t)T * k * 4)) != CSK_OK) return rc;
   rc = launch_router(dx.as<float>(), dg.as<float>(), gate_b ? db.as<float>() : nullptr, T, E, H, k,

@@ -92,67 +92,84 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float* __restr
 
 // ------------------------------------------------- router logits, many tokens
 // The same logits as an fp32 GEMM on the matrix cores (v_mfma_f32_32x32x2_f32: fp32
-// operands, fp32 accumulation, so nothing is rounded to a narrower type).  A workgroup
-// owns 32 tokens x 32 experts; its four waves take interleaved 16-wide slices of H and
-// their partial tiles are added in LDS in a fixed order.  Operand ownership: lane l
-// holds row l%32 (token, or expert) and k index l/32 of the two; each lane loads eight
-// consecutive values of its row per iteration and feeds them to eight instructions --
-// any assignment of k to (instruction, lane half) is valid as long as both operands
-// use the same one.
+// operands, fp32 accumulation, so nothing is rounded to a narrower type).  Workgroup
+// (x, y) owns 32 tokens and split y of H (up to kRouterChunks chunks of 64): it loads its
+// part of the 32 token rows into registers once and walks all the experts, 32 at a time,
+// so the hidden states are read once however many experts there are, and the splits give
+// a batch of a few thousand tokens enough workgroups to fill the chip.  Within a chunk the
+// four waves take 16-wide slices; their partial tiles are added in LDS in a fixed order
+// and written as partial logits [split][T][E], which the top-k kernel sums in split order
+// and completes with the bias.  Operand ownership: lane l holds row l%32 (token, or
+// expert) and k index l/32 of the two; each lane loads eight consecutive values of its
+// row per chunk and feeds them to eight instructions -- any assignment of k to
+// (instruction, lane half) is valid as long as both operands use the same one.
+// H must be a multiple of 16.
+constexpr int kRouterChunks = 12;     // chunks of 64 per split: the token rows of a split stay in registers
+constexpr int kRouterMaxSplits = 8;
+
 __global__ __launch_bounds__(256) void router_logits_mfma_kernel(const float* __restrict__ x,
                                                                  const float* __restrict__ g,
-                                                                 const float* __restrict__ b,
-                                                                 float* __restrict__ logits, int T,
-                                                                 int E, int H) {
+                                                                 float* __restrict__ partial, int T,
+                                                                 int E, int H, int chunks_per_split) {
   __shared__ float part[4][32][33];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int r32 = lane & 31, half = lane >> 5;
-  const int t0 = blockIdx.x * 32, e0 = blockIdx.y * 32;
-  const float* xr = x + (size_t)min(t0 + r32, T - 1) * H + 8 * half;
-  const float* gr = g + (size_t)min(e0 + r32, E - 1) * H + 8 * half;
-  floatx16 acc;
+  const int t0 = blockIdx.x * 32;
+  const int c0 = blockIdx.y * chunks_per_split;
+  const int k_lane = 16 * wv + 8 * half;  // this lane's eight columns within a chunk
+  const float* xr = x + (size_t)min(t0 + r32, T - 1) * H + k_lane;
+  // the split's part of the token rows; columns past H are zeros (they then add nothing)
+  floatx4 xa[kRouterChunks], xb[kRouterChunks];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-  // loads run two iterations ahead of the arithmetic (three rolling register sets)
-  const int nit = (H - 16 * wv + 63) / 64;
-  float4 xa[3], xb[3], ga[3], gb[3];
-  auto load = [&](int u, int i) {
-    const int k0 = 16 * wv + 64 * min(i, nit - 1);
-    xa[u] = *reinterpret_cast<const float4*>(xr + k0);
-    xb[u] = *reinterpret_cast<const float4*>(xr + k0 + 4);
-    ga[u] = *reinterpret_cast<const float4*>(gr + k0);
-    gb[u] = *reinterpret_cast<const float4*>(gr + k0 + 4);
-  };
-  if (nit > 0) {
+  for (int i = 0; i < kRouterChunks; ++i) {
+    const int k0 = 64 * (c0 + i);
+    const bool in = i < chunks_per_split && k0 + k_lane + 8 <= H;
+    xa[i] = in ? *reinterpret_cast<const floatx4*>(xr + k0) : floatx4{0.f, 0.f, 0.f, 0.f};
+    xb[i] = in ? *reinterpret_cast<const floatx4*>(xr + k0 + 4) : floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  // the last chunk this lane may load from the expert rows (clamped loads meet zeros above)
+  const int c_last = max(0, (H - k_lane - 8) / 64);
+  float* out = partial + (size_t)blockIdx.y * T * E;
+  for (int e0 = 0; e0 < E; e0 += 32) {
+    const float* gr = g + (size_t)min(e0 + r32, E - 1) * H + k_lane;
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    // expert rows: loads run two chunks ahead of the arithmetic (three rolling register sets)
+    floatx4 ga[3], gb[3];
+    auto load = [&](int u, int i) {
+      const int k0 = 64 * min(c0 + i, c_last);
+      ga[u] = *reinterpret_cast<const floatx4*>(gr + k0);
+      gb[u] = *reinterpret_cast<const floatx4*>(gr + k0 + 4);
+    };
     load(0, 0);
     load(1, 1);
-  }
-  for (int i = 0; i < nit; i += 3) {
 #pragma unroll
-    for (int u = 0; u < 3; ++u) {
-      if (i + u < nit) {
-        load((u + 2) % 3, i + u + 2);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].x, ga[u].x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].y, ga[u].y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].z, ga[u].z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[u].w, ga[u].w, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[u].x, gb[u].x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[u].y, gb[u].y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[u].z, gb[u].z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[u].w, gb[u].w, acc, 0, 0, 0);
+    for (int i = 0; i < kRouterChunks; ++i) {
+      if (i < chunks_per_split) {
+        const int u = i % 3;
+        load((u + 2) % 3, i + 2);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i][0], ga[u][0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i][1], ga[u][1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i][2], ga[u][2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xa[i][3], ga[u][3], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i][0], gb[u][0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i][1], gb[u][1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i][2], gb[u][2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xb[i][3], gb[u][3], acc, 0, 0, 0);
       }
     }
-  }
-  // accumulator register r of lane (expert column r32, half) is token (r%4) + 8 (r/4) + 4 half
+    // accumulator register r of lane (expert column r32, half) is token (r%4) + 8 (r/4) + 4 half
 #pragma unroll
-  for (int r = 0; r < 16; ++r) part[wv][(r & 3) + 8 * (r >> 2) + 4 * half][r32] = acc[r];
-  __syncthreads();
-  for (int i = threadIdx.x; i < 32 * 32; i += 256) {
-    const int tl = i >> 5, el = i & 31;
-    if (t0 + tl < T && e0 + el < E) {
-      const float s = (part[0][tl][el] + part[1][tl][el]) + (part[2][tl][el] + part[3][tl][el]);
-      logits[(size_t)(t0 + tl) * E + e0 + el] = s + (b ? b[e0 + el] : 0.0f);
+    for (int r = 0; r < 16; ++r) part[wv][(r & 3) + 8 * (r >> 2) + 4 * half][r32] = acc[r];
+    __syncthreads();
+    for (int i = threadIdx.x; i < 32 * 32; i += 256) {
+      const int tl = i >> 5, el = i & 31;
+      if (t0 + tl < T && e0 + el < E)
+        out[(size_t)(t0 + tl) * E + e0 + el] =
+            (part[0][tl][el] + part[1][tl][el]) + (part[2][tl][el] + part[3][tl][el]);
     }
+    __syncthreads();
   }
 }
 
@@ -481,13 +498,15 @@ __device__ __forceinline__ float routing_weight(float my_val, float vmax, int la
 // One wave per token (select_topk).  Weights
 // follow moe_router_node.h:180-202: sigmoid of the raw logit, or softmax over
 // the selected k with max subtraction, sum in slot order, multiply by 1/sum.
-__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits,
+__global__ __launch_bounds__(256) void router_topk_kernel(float* __restrict__ logits,
                                                           float* __restrict__ pairs,
                                                           int* __restrict__ ids, int T, int E,
                                                           int k, int sigmoid,
                                                           const float* __restrict__ x,
                                                           const float* __restrict__ g,
-                                                          const float* __restrict__ b, int H) {
+                                                          const float* __restrict__ b, int H,
+                                                          const float* __restrict__ partial,
+                                                          int nsplit) {
   __shared__ CloseCallLds cc;
   __shared__ float cc_thr[4];
   __shared__ int cc_flag[4];
@@ -499,7 +518,19 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restric
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int e = lane + 64 * j;
-    v[j] = (live && e < E) ? logits[(size_t)t * E + e] : NEG;
+    v[j] = NEG;
+    if (live && e < E) {
+      if (nsplit > 0) {
+        // partial logits of the splits of H, in split order, then the bias; the sum is kept
+        // for the recomputation below and for callers that ask for the logits
+        float sum = partial[(size_t)t * E + e];
+        for (int sp = 1; sp < nsplit; ++sp) sum += partial[((size_t)sp * T + t) * E + e];
+        v[j] = sum + (b ? b[e] : 0.0f);
+        logits[(size_t)t * E + e] = v[j];
+      } else {
+        v[j] = logits[(size_t)t * E + e];
+      }
+    }
   }
   float my_val, vmax, runner_up;  // lane s keeps slot s
   int my_idx;
