@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -26,6 +27,13 @@ hipStream_t g_stream = nullptr;
 bool g_ready = false;
 int g_device = -1;
 int g_cus = 0;
+// The library owns one stream and one workspace, so calls are serialised: an entry point
+// holds this lock from its first line to its return (recursive: entry points call one
+// another).  Callers may therefore come from any thread, e.g. the per-layer worker threads
+// of the reference's scheduler (layer_scheduler_node), without locking of their own.
+std::recursive_mutex g_api;
+thread_local bool t_device_bound = false;  // the current device is a per-thread setting
+#define API_LOCK() std::lock_guard<std::recursive_mutex> csk_api_guard_(g_api)
 
 int fail(int code, const std::string& msg) {
   g_err = msg;
@@ -40,9 +48,12 @@ int fail(int code, const std::string& msg) {
   } while (0)
 
 #define REQUIRE_INIT()                                                          \
-  do {                                                                          \
-    if (!g_ready) return fail(CSK_ERR_STATE, "csk_init has not been called");   \
-  } while (0)
+  API_LOCK();                                                                   \
+  if (!g_ready) return fail(CSK_ERR_STATE, "csk_init has not been called");     \
+  if (!t_device_bound) {                                                        \
+    HIP_TRY(hipSetDevice(g_device));                                            \
+    t_device_bound = true;                                                      \
+  }
 
 int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
@@ -570,6 +581,7 @@ int check_dims(int64_t E, int64_t k, int64_t H, int64_t F) {
 // ============================================================ process-wide
 
 extern "C" int csk_init(int device) {
+  API_LOCK();
   int n = 0;
   HIP_TRY(hipGetDeviceCount(&n));
   if (device < 0 || device >= n) return fail(CSK_ERR_HIP, "no such GPU device");
@@ -586,6 +598,7 @@ extern "C" int csk_init(int device) {
   g_device = device;
   g_cus = prop.multiProcessorCount;
   g_ready = true;
+  t_device_bound = true;
   return CSK_OK;
 }
 
@@ -627,6 +640,7 @@ extern "C" void* csk_dev_alloc(size_t bytes) {
     g_err = "csk_init has not been called";
     return nullptr;
   }
+  if (!t_device_bound && hipSetDevice(g_device) == hipSuccess) t_device_bound = true;
   void* p = nullptr;
   hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
   if (e != hipSuccess) {
@@ -722,6 +736,7 @@ extern "C" int csk_mxfp4_upload(const uint8_t* blocks, int64_t rows, int64_t K, 
 }
 extern "C" void csk_mxfp4_free(csk_mxfp4* m) {
   if (!m) return;
+  API_LOCK();
   if (m->owned) {
     if (m->q) (void)hipFree(m->q);
     if (m->s) (void)hipFree(m->s);
@@ -803,6 +818,7 @@ extern "C" int csk_layer_create_f16(int64_t E, int64_t k, int64_t H, int64_t F, 
 
 extern "C" void csk_layer_destroy(csk_layer* L) {
   if (!L) return;
+  API_LOCK();
   if (g_stream) (void)hipStreamSynchronize(g_stream);
   void* ps[] = {L->gate_w, L->gate_b, L->q_all, L->s_all, L->h_all, L->bias_all, L->ew_dev, L->norm_w};
   for (void* p : ps)
@@ -1040,6 +1056,7 @@ extern "C" int csk_f16_upload_ggml(int ggml_type, const void* data, int64_t rows
 }
 extern "C" void csk_f16_free(csk_f16* m) {
   if (!m) return;
+  API_LOCK();
   if (m->w) (void)hipFree(m->w);
   delete m;
 }

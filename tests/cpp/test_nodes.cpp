@@ -9,6 +9,7 @@
 #include <functional>
 #include <random>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "coalsack/nn/nn_ops/add_node.h"
@@ -644,6 +645,56 @@ static void gpu_node_chain() {
   CHECK(worst <= 1e-3f);
 }
 
+// Nodes of different layers may be driven from different threads (the reference runs each
+// layer's nodes on that layer's scheduler thread, layer_scheduler_node); the library
+// serialises the calls, so results must equal those of the same calls made one after another.
+static void gpu_concurrent_callers() {
+  std::printf("concurrent callers: four threads, each with its own nodes\n");
+  constexpr int kThreads = 4, kRounds = 6;
+  struct Job {
+    dynamic_tensor a, w, hidden, gate, up, down, want_mm, want_ffn;
+    int bad = 0;
+  };
+  std::vector<Job> jobs(kThreads);
+  std::mt19937 gen(77);
+  for (int i = 0; i < kThreads; ++i) {
+    Job& j = jobs[i];
+    const int64_t S = 5 + 9 * i, K = 64 + 32 * i, N = 96 + 16 * i;
+    j.a = random_tensor({1, S, K}, gen, -1, 1);
+    j.w = random_half_tensor({N, K}, gen, -0.2f, 0.2f);
+    j.hidden = random_tensor({1, S, K}, gen, -1, 1);
+    j.gate = random_half_tensor({N, K}, gen, -0.2f, 0.2f);
+    j.up = random_half_tensor({N, K}, gen, -0.2f, 0.2f);
+    j.down = random_half_tensor({K, N}, gen, -0.2f, 0.2f);
+    matmul_transpose_mixed_node mm;
+    dense_ffn_node ffn;
+    j.want_mm = mm.compute_test(j.a, j.w);
+    j.want_ffn = ffn.compute_test({j.hidden, j.gate, j.up, j.down});
+  }
+  auto same = [](const dynamic_tensor& x, const dynamic_tensor& y) {
+    return x.shape() == y.shape() &&
+           std::memcmp(x.data_ptr<float>(), y.data_ptr<float>(), x.numel() * sizeof(float)) == 0;
+  };
+  std::vector<std::thread> pool;
+  for (int i = 0; i < kThreads; ++i)
+    pool.emplace_back([&, i] {
+      Job& j = jobs[i];
+      matmul_transpose_mixed_node mm;
+      dense_ffn_node ffn;
+      for (int r = 0; r < kRounds; ++r) {
+        try {
+          if (!same(mm.compute_test(j.a, j.w), j.want_mm)) ++j.bad;
+          if (!same(ffn.compute_test({j.hidden, j.gate, j.up, j.down}), j.want_ffn)) ++j.bad;
+        } catch (const std::exception& e) {
+          std::printf("  thread %d: %s\n", i, e.what());
+          ++j.bad;
+        }
+      }
+    });
+  for (auto& t : pool) t.join();
+  for (int i = 0; i < kThreads; ++i) CHECK(jobs[i].bad == 0);
+}
+
 int main(int argc, char** argv) {
   const bool gpu = argc > 1 && std::string(argv[1]) == "--gpu";
   if (gpu) {
@@ -658,6 +709,7 @@ int main(int argc, char** argv) {
     gpu_matmul_tests();
     gpu_node_chain();
     gpu_norm_add_tests();
+    gpu_concurrent_callers();
   } else {
     cpu_router_argument_errors();
     cpu_expert_node_paths();

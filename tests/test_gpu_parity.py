@@ -423,3 +423,32 @@ def test_prefill_ragged_small_shape(lib, oracle):
     same = np.all(pairs[..., 0] == wpairs[..., 0], axis=1)
     assert same.mean() > 0.99
     assert_layer_close(got[same], want[same])
+
+
+def test_concurrent_forwards_equal_sequential(lib):
+    """Two threads, each driving its own layer through the C ABI at the same time (ctypes
+    releases the interpreter lock during a call): the library serialises the calls, so every
+    result is bit-identical to the one the same call gives when made alone."""
+    import threading
+    shapes = [(8, 2, 128, 160, 21), (16, 4, 256, 192, 150)]
+    layers, hiddens, wants = [], [], []
+    for i, (E, k, H, F, T) in enumerate(shapes):
+        L = synth.LayerInputs(E, k, H, F, seed=40 + i)
+        layer = build_layer(lib, L)
+        hidden = synth.hidden_states(T, H, seed=i)
+        layers.append(layer), hiddens.append(hidden), wants.append(layer.forward(hidden))
+    bad = [0, 0]
+
+    def work(i):
+        for _ in range(20):
+            if not np.array_equal(layers[i].forward(hiddens[i]), wants[i]):
+                bad[i] += 1
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for layer in layers:
+        layer.close()
+    assert bad == [0, 0]
