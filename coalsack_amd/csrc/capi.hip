@@ -1138,10 +1138,11 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
         L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
     if ((rc = check_launch("router_prep_logits_kernel")) != CSK_OK) return rc;
     mark(CSK_STAGE_DISPATCH);
-    route_small_kernel<<<dim3(1), kRouteSmallThreads, 0, g_stream>>>(
-        ws.logits, ws.pairs, ws.ids, (int)T, (int)L->E, (int)L->k, L->sigmoid, L->ew_dev, ws.counts,
-        ws.offsets, ws.desc, ws.vlist, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w, ws.pos,
-        xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, (int)L->H, stream_group_tokens(T));
+    RouteIn rin{ws.logits, xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, L->ew_dev,
+                (int)T, (int)L->E, (int)L->k, (int)L->H, L->sigmoid, stream_group_tokens(T)};
+    RouteOut rout{ws.pairs, ws.ids, ws.pos, ws.counts, ws.offsets, ws.desc, ws.vlist, ws.nv,
+                  ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w};
+    route_small_kernel<<<dim3(1), kRouteSmallThreads, 0, g_stream>>>(rin, rout);
     if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
     if (!L->f16 && !stream_path(T, L->H, L->F) && !L->wbf) {
       // few tokens but rows too long for the streaming kernel: the GEMM wants the FP6 form

@@ -42,6 +42,13 @@ struct ExpertW {
   const float* b_down;
 };
 
+// One entry per active expert, written by the dispatch kernels; entries past
+// the active count have Te == 0.
+struct WorkDesc {
+  int e, Te, base, pad;
+  ExpertW w;
+};
+
 // Pointers read out of device structures are generic to the compiler, which
 // would then use FLAT loads (tracked by both memory counters and therefore
 // always waited for in full).  These casts pin them to global memory.

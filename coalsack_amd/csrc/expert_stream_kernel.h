@@ -19,13 +19,6 @@
 
 namespace csk {
 
-// One entry per active expert, written by the dispatch kernel; entries past
-// the active count have Te == 0.
-struct WorkDesc {
-  int e, Te, base, pad;
-  ExpertW w;
-};
-
 // Bias pointers inside desc[].w must not be null for expert_stream_kernel: the
 // host substitutes a zero vector for an absent bias, so that the loads are
 // unconditional.

@@ -4,7 +4,7 @@
 #pragma once
 #include "common.h"
 #include "mx3.h"
-#include "expert_stream_kernel.h"
+#include "route_select.h"
 
 namespace csk {
 
@@ -274,226 +274,6 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
   }
 }
 
-// --------------------------------------------------- per-token selection
-// Maximum over the 64 lanes, the same value returned in every lane: four cross-lane steps
-// inside each row of 16 (quad swaps, half-row and row mirrors: ordinary vector-ALU latency,
-// where a shuffle through the LDS crossbar takes ten times as long) and the four row
-// results combined through scalar registers.
-template <int CTRL>
-__device__ __forceinline__ float dpp_max(float a) {
-  const int x = __float_as_int(a);
-  return fmaxf(a, __int_as_float(__builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false)));
-}
-__device__ __forceinline__ float wave_max_all(float v) {
-  v = dpp_max<0xB1>(v);   // quad_perm [1,0,3,2]
-  v = dpp_max<0x4E>(v);   // quad_perm [2,3,0,1]
-  v = dpp_max<0x141>(v);  // row_half_mirror
-  v = dpp_max<0x140>(v);  // row_mirror
-  const int x = __float_as_int(v);
-  const float r0 = __int_as_float(__builtin_amdgcn_readlane(x, 0));
-  const float r1 = __int_as_float(__builtin_amdgcn_readlane(x, 16));
-  const float r2 = __int_as_float(__builtin_amdgcn_readlane(x, 32));
-  const float r3 = __int_as_float(__builtin_amdgcn_readlane(x, 48));
-  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
-}
-
-// One wave selects one token's top k.  Lane l holds the logits of experts l, l+64,
-// l+128, l+192; each round finds the wave-wide maximum, locates its owner with ballots
-// (ties -> lowest expert index) and retires it.  One round more than k records
-// the runner-up, so that the k+1 largest logits are known: if any two adjacent ones are
-// closer than the difference between this library's tree-ordered fp32 sums and the
-// reference's strictly sequential ones can be (moe_router_node.h:161-167: sum += h*g,
-// multiply and add rounded separately, bias added last), the caller recomputes the
-// logits in question in exactly that order and selects again -- so the expert indices
-// and their slot order equal the reference's whenever the inputs are the same, not only
-// when no two logits are close.  Lane s < k returns slot s in (my_val, my_idx).
-__device__ __forceinline__ void select_topk(float (&v)[4], int lane, int E, int k, float& my_val,
-                                            int& my_idx, float& vmax, bool& close_call, float tol,
-                                            float& runner_up) {
-  const float NEG = -__builtin_inff();
-  my_val = 0.0f, my_idx = 0, vmax = 0.0f;
-  for (int s = 0; s <= k; ++s) {
-    const float best = wave_max_all(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
-    // its owner: lowest expert index among equals = lowest register j, then lowest lane
-    int bi = 0;
-    bool found = false;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const unsigned long long m = __ballot(v[j] == best);
-      if (!found && m != 0ull) {
-        bi = (int)__builtin_ctzll(m) + 64 * j;
-        found = true;
-      }
-    }
-    if (s == 0) vmax = best;
-    if (lane == s) {
-      my_val = best;
-      my_idx = bi;
-    }
-    if (s < k && (bi & 63) == lane) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if ((bi >> 6) == j) v[j] = NEG;
-    }
-  }
-  // lanes 0..k hold the k+1 largest in descending order (fewer when E == k)
-  const float below = __shfl_down(my_val, 1, 64);
-  const bool close = lane < k && lane + 1 < E && (my_val - below) <= tol * fmaxf(1.0f, fabsf(my_val));
-  close_call = __any(close);
-  runner_up = __shfl(my_val, min(k, E - 1), 64);
-}
-
-// Logits in the reference's order: a strictly sequential fp32 sum per logit, multiply and
-// add rounded separately (moe_router_node.h:161-167).  The chain of H dependent additions
-// cannot be shortened, everything else can be taken out of its way: the whole workgroup
-// multiplies (coalesced loads, the products do not depend on the running sum) and stages
-// the rounded products of up to kCcBatch logits in LDS, one chunk of K ahead; lane c of
-// wave 0 then only reads row c back and adds, all rows side by side.
-constexpr int kCcBatch = 8;              // logits recomputed side by side
-constexpr int kCcChunk = 768;            // elements of K staged per step
-constexpr int kCcStride = kCcChunk + 4;  // LDS row stride: rows start four banks apart
-
-struct CloseCallLds {
-  alignas(16) float prod[2][kCcBatch][kCcStride];
-  float fixed[kMaxExperts];  // the token's logits, recomputed ones replaced
-  int cand[kMaxExperts];
-  int ncand;
-};
-
-// Called by all NT threads of the workgroup with the same arguments.  Recomputes the
-// logits that can take part in a close call -- those not below thr, which is set a safe
-// margin under the (k+1)-th largest; the others keep their tree-ordered values, which the
-// bound on the difference keeps on their side of thr -- and leaves all E logits of the
-// token in s.fixed.  H must be a multiple of 4.
-template <int NT>
-__device__ __forceinline__ void logits_reference_order_wg(const float* __restrict__ x,
-                                                          const float* __restrict__ g,
-                                                          const float* __restrict__ b,
-                                                          const float* __restrict__ logit_row, int E,
-                                                          int H, float thr, CloseCallLds& s) {
-#pragma clang fp contract(off)
-  constexpr int kC4 = kCcChunk / 4;
-  constexpr int kProducers = NT - 64;  // wave 0 only adds
-  constexpr int kItems = (kCcBatch * kC4 + kProducers - 1) / kProducers;
-  const int tid = threadIdx.x, ptid = tid - 64;
-  if (tid == 0) s.ncand = 0;
-  __syncthreads();
-  for (int e = tid; e < E; e += NT) {
-    const float v = logit_row[e];
-    s.fixed[e] = v;
-    if (v >= thr) s.cand[atomicAdd(&s.ncand, 1)] = e;
-  }
-  __syncthreads();
-  const int m = s.ncand;
-  const CSK_GLOBAL floatx4* x4 = as_global(reinterpret_cast<const floatx4*>(x));
-  const CSK_GLOBAL floatx4* g4 = as_global(reinterpret_cast<const floatx4*>(g));
-  const int H4 = H >> 2;
-  const int nchunk = (H4 + kC4 - 1) / kC4;
-  for (int c0 = 0; c0 < m; c0 += kCcBatch) {
-    const int mb = min(kCcBatch, m - c0);
-    // producers: rounded products of chunk ci of the batch's rows -> LDS buffer ci & 1
-    auto produce = [&](int ci) {
-      const int h4 = ci * kC4, len4 = min(kC4, H4 - h4);
-      floatx4 xq[kItems], gq[kItems];
-#pragma unroll
-      for (int it = 0; it < kItems; ++it) {
-        const int idx = ptid + it * kProducers, c = idx / kC4, i4 = idx - c * kC4;
-        if (c < mb && i4 < len4) {
-          xq[it] = x4[h4 + i4];
-          gq[it] = g4[(size_t)s.cand[c0 + c] * H4 + h4 + i4];
-        }
-      }
-#pragma unroll
-      for (int it = 0; it < kItems; ++it) {
-        const int idx = ptid + it * kProducers, c = idx / kC4, i4 = idx - c * kC4;
-        if (c < mb && i4 < len4)
-          *reinterpret_cast<floatx4*>(&s.prod[ci & 1][c][4 * i4]) = xq[it] * gq[it];
-      }
-    };
-    if (ptid >= 0) produce(0);
-    __syncthreads();
-    float sum = 0.0f;
-    for (int ci = 0; ci < nchunk; ++ci) {
-      if (ptid >= 0) {
-        if (ci + 1 < nchunk) produce(ci + 1);  // while wave 0 adds chunk ci
-      } else if (tid < mb) {
-        const int len4 = min(kC4, H4 - ci * kC4);
-        const floatx4* row = reinterpret_cast<const floatx4*>(&s.prod[ci & 1][tid][0]);
-        floatx4 qa[8], qb[8];
-        // reads run up to 15 entries past the chunk (into the next row: never added)
-        auto rd = [&](floatx4(&q)[8], int i0) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) q[i] = row[i0 + i];
-        };
-        auto add = [&](const floatx4(&q)[8]) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            sum = sum + q[i][0];
-            sum = sum + q[i][1];
-            sum = sum + q[i][2];
-            sum = sum + q[i][3];
-          }
-        };
-        auto add_tail = [&](const floatx4(&q)[8], int n) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            if (i < n) {
-              sum = sum + q[i][0];
-              sum = sum + q[i][1];
-              sum = sum + q[i][2];
-              sum = sum + q[i][3];
-            }
-          }
-        };
-        // two register sets of eight float4 in rotation: the reads of one are in flight
-        // while the other is added; whole groups carry no guards
-        const int full = len4 & ~7;
-        int i0 = 0;
-        rd(qa, 0);
-        for (; i0 + 16 <= full; i0 += 16) {
-          rd(qb, i0 + 8);
-          add(qa);
-          rd(qa, i0 + 16);
-          add(qb);
-        }
-        if (i0 + 8 <= full) {
-          rd(qb, i0 + 8);
-          add(qa);
-          add_tail(qb, len4 - i0 - 8);
-        } else {
-          add_tail(qa, len4 - i0);
-        }
-      }
-      __syncthreads();
-    }
-    if (tid < mb) {
-      const int e = s.cand[c0 + tid];
-      s.fixed[e] = sum + (b ? b[e] : 0.0f);
-    }
-    __syncthreads();
-  }
-}
-
-// How close is a close call.  Measured over 1.3 million logits (six shapes, H from 256 to
-// 2880): |tree-ordered sum - sequential sum| / max(1, |logit|) has an rms of 0.28 and a
-// maximum of 2.3 in units of 2^-24 * sqrt(H) (the random-walk size of the sequential
-// sum's rounding error); the tests hold the maximum below 3.  Two logits can change rank
-// only if they are closer than the sum of their two differences; the threshold is 8 units,
-// twice the largest pair of differences seen.  At gpt-oss shapes about one token in 2500
-// is recomputed.
-__device__ __forceinline__ float close_call_tolerance(int H) { return 8.0f * 5.96e-8f * sqrtf((float)H); }
-
-// Routing weight of slot `lane` (moe_router_node.h:180-202): sigmoid of the raw logit, or
-// softmax over the selected k with max subtraction, sum in slot order, multiply by 1/sum.
-__device__ __forceinline__ float routing_weight(float my_val, float vmax, int lane, int k, int sigmoid) {
-  if (sigmoid) return 1.0f / (1.0f + expf(-my_val));
-  float w = (lane < k) ? expf(my_val - vmax) : 0.0f;
-  float sum = 0.0f;
-  for (int s = 0; s < k; ++s) sum += __shfl(w, s, 64);  // slot order
-  const float inv = (sum > 0.0f) ? (1.0f / sum) : 0.0f;
-  return w * inv;
-}
-
 // ------------------------------------------------------------------- top-k
 // One wave per token (select_topk).  Weights
 // follow moe_router_node.h:180-202: sigmoid of the raw logit, or softmax over
@@ -575,26 +355,6 @@ __global__ __launch_bounds__(256) void router_topk_kernel(float* __restrict__ lo
 __global__ void pairs_to_ids_kernel(const float* __restrict__ pairs, int* __restrict__ ids, int P) {
   const int p = blockIdx.x * blockDim.x + threadIdx.x;
   if (p < P) ids[p] = (int)pairs[2 * (size_t)p];
-}
-
-// Work descriptor of one active-expert slot (all zero when the slot is unused), written
-// field by field: a local copy of the structure would live in scratch memory.
-__device__ __forceinline__ void write_work_desc(WorkDesc* d, bool on, int e, int Te, int base,
-                                                const ExpertW* __restrict__ ew) {
-  const ExpertW* src = ew + e;
-  d->e = e;
-  d->Te = on ? Te : 0;
-  d->base = on ? base : 0;
-  d->pad = 0;
-  d->w.q_gate = on ? src->q_gate : nullptr;
-  d->w.s_gate = on ? src->s_gate : nullptr;
-  d->w.q_up = on ? src->q_up : nullptr;
-  d->w.s_up = on ? src->s_up : nullptr;
-  d->w.q_down = on ? src->q_down : nullptr;
-  d->w.s_down = on ? src->s_down : nullptr;
-  d->w.b_gate = on ? src->b_gate : nullptr;
-  d->w.b_up = on ? src->b_up : nullptr;
-  d->w.b_down = on ? src->b_down : nullptr;
 }
 
 // ----------------------------------------------------------------- dispatch
@@ -735,179 +495,14 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
   }
 }
 
-// ------------------------------------- small batches: top-k + dispatch, fused
-// One workgroup of sixteen waves does, for P = T * k <= 1024 assignments, what
-// router_topk_kernel and dispatch_scatter_kernel do in
-// two launches: top-k and weights per token (one wave per token), histogram,
-// exclusive scan, ordered scatter, work descriptors and token groups -- all
-// through LDS.
+// ------------------------------------- small batches: top-k + dispatch, one launch
+// A single workgroup of sixteen waves routes the batch (route_workgroup) and writes every
+// output.
 constexpr int kRouteSmallThreads = 1024;
-__global__ __launch_bounds__(kRouteSmallThreads) void route_small_kernel(
-    const float* __restrict__ logits, float* __restrict__ pairs, int* __restrict__ ids_out, int T,
-    int E, int k, int sigmoid, const ExpertW* __restrict__ ew, int* __restrict__ counts,
-    int* __restrict__ offsets, WorkDesc* __restrict__ desc, int* __restrict__ vlist,
-    int* __restrict__ nv, int* __restrict__ mtiles, int* __restrict__ n_mtiles,
-    int* __restrict__ list_tok, float* __restrict__ list_w, int* __restrict__ pos_of_slot,
-    const float* __restrict__ x, const float* __restrict__ g, const float* __restrict__ b, int H,
-    int group_tokens) {
-  constexpr int NW = kRouteSmallThreads / 64;
-  __shared__ int ids[1024];
-  __shared__ float wts[1024];
-  __shared__ int cnt[kMaxExperts], off[kMaxExperts], act_e[kMaxExperts];
-  __shared__ int na_sh;
-  __shared__ CloseCallLds cc;
-  __shared__ int cc_tok[64], cc_n;
-  __shared__ float cc_thr[64];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int P = T * k;
-  const float NEG = -__builtin_inff();
-  const float tol = close_call_tolerance(H);
-  if (threadIdx.x == 0) cc_n = 0;
-  __syncthreads();
-  auto publish = [&](int t, float my_val, int my_idx, float vmax) {
-    const float w = routing_weight(my_val, vmax, lane, k, sigmoid);
-    if (lane < k) {
-      reinterpret_cast<float2*>(pairs)[(size_t)t * k + lane] = make_float2((float)my_idx, w);
-      ids_out[t * k + lane] = my_idx;
-      ids[t * k + lane] = my_idx;
-      wts[t * k + lane] = w;
-    }
-  };
-  for (int t = wv; t < T; t += NW) {
-    float v[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int e = lane + 64 * j;
-      v[j] = (e < E) ? logits[(size_t)t * E + e] : NEG;
-    }
-    float my_val, vmax, runner_up;
-    int my_idx;
-    bool close_call;
-    select_topk(v, lane, E, k, my_val, my_idx, vmax, close_call, tol, runner_up);
-    if (close_call) {
-      if (lane == 0) {
-        const int n = atomicAdd(&cc_n, 1);
-        cc_tok[n] = t;
-        cc_thr[n] = runner_up - 2.0f * tol * fmaxf(1.0f, fabsf(runner_up));
-      }
-    } else {
-      publish(t, my_val, my_idx, vmax);
-    }
-  }
-  __syncthreads();
-  // rare: tokens with a close call among their k+1 largest logits are recomputed in the
-  // reference's order by the whole workgroup, one after the other; wave 0 selects again
-  for (int n = 0; n < cc_n; ++n) {
-    const int t = cc_tok[n];
-    logits_reference_order_wg<kRouteSmallThreads>(x + (size_t)t * H, g, b, logits + (size_t)t * E,
-                                                  E, H, cc_thr[n], cc);
-    if (wv == 0) {
-      float v[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int e = lane + 64 * j;
-        v[j] = e < E ? cc.fixed[e] : NEG;
-      }
-      float my_val, vmax, runner_up;
-      int my_idx;
-      bool close_call;
-      select_topk(v, lane, E, k, my_val, my_idx, vmax, close_call, 0.0f, runner_up);
-      publish(t, my_val, my_idx, vmax);
-    }
-    __syncthreads();
-  }
-  __syncthreads();
-  // histogram: wave wv counts experts wv, wv + NW, ... with ballots over the assignments
-  for (int e = wv; e < E; e += NW) {
-    int c = 0;
-    for (int p0 = 0; p0 < P; p0 += 64) {
-      const int p = p0 + lane;
-      c += __popcll(__ballot(p < P && ids[p] == e));
-    }
-    if (lane == 0) {
-      cnt[e] = c;
-      counts[e] = c;
-    }
-  }
-  __syncthreads();
-  // exclusive scan, active experts, token groups, M tiles: wave 0, four consecutive
-  // experts per lane, wave-wide prefix sums
-  if (wv == 0) {
-    int c[4], tot = 0, nact = 0, ngrp = 0, nmt = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int e = lane * 4 + j;
-      c[j] = e < E ? cnt[e] : 0;
-      tot += c[j];
-      nact += c[j] > 0;
-      ngrp += (c[j] + group_tokens - 1) / group_tokens;
-      nmt += (c[j] + 63) / 64;
-    }
-    int s_tot = tot, s_act = nact, s_grp = ngrp, s_mt = nmt;  // inclusive scans over lanes
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int t0 = __shfl_up(s_tot, o, 64), t1 = __shfl_up(s_act, o, 64);
-      const int t2 = __shfl_up(s_grp, o, 64), t3 = __shfl_up(s_mt, o, 64);
-      if (lane >= o) {
-        s_tot += t0;
-        s_act += t1;
-        s_grp += t2;
-        s_mt += t3;
-      }
-    }
-    int run = s_tot - tot, slot = s_act - nact, gi = s_grp - ngrp, mi = s_mt - nmt;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int e = lane * 4 + j;
-      if (e < E) {
-        off[e] = run;
-        offsets[e] = run;
-        if (c[j] > 0) {
-          for (int gb = 0; gb < c[j]; gb += group_tokens) {
-            vlist[2 * gi] = slot;
-            vlist[2 * gi + 1] = gb;
-            ++gi;
-          }
-          for (int m0 = 0; m0 < c[j]; m0 += 64) {
-            mtiles[2 * mi] = slot;
-            mtiles[2 * mi + 1] = m0;
-            ++mi;
-          }
-          act_e[slot++] = e;
-        }
-        run += c[j];
-      }
-    }
-    if (lane == 63) {
-      offsets[E] = s_tot;
-      na_sh = s_act;
-      *nv = s_grp;
-      *n_mtiles = s_mt;
-    }
-  }
-  __syncthreads();
-  // ordered scatter: rank of an assignment = matches before it (ballot prefix)
-  for (int e = wv; e < E; e += NW) {
-    if (cnt[e] == 0) continue;
-    int basep = off[e];
-    for (int p0 = 0; p0 < P; p0 += 64) {
-      const int p = p0 + lane;
-      const bool hit = p < P && ids[p] == e;
-      const unsigned long long m = __ballot(hit);
-      if (hit) {
-        const int pos = basep + __popcll(m & ((1ull << lane) - 1ull));
-        list_tok[pos] = p / k;
-        list_w[pos] = wts[p];
-        pos_of_slot[p] = pos;
-      }
-      basep += __popcll(m);
-    }
-  }
-  if ((int)threadIdx.x < E) {
-    const bool on = (int)threadIdx.x < na_sh;
-    const int e = on ? act_e[threadIdx.x] : 0;
-    write_work_desc(desc + threadIdx.x, on, e, cnt[e], off[e], ew);
-  }
+constexpr int kRouteSmallMaxP = 1024;
+__global__ __launch_bounds__(kRouteSmallThreads) void route_small_kernel(RouteIn in, RouteOut out) {
+  __shared__ RouteLds<kCcBatch, kRouteSmallMaxP> lds;
+  route_workgroup<kRouteSmallThreads, kCcBatch, kRouteSmallMaxP>(in, out, lds);
 }
 
 // ------------------------------------------------------------------ combine
