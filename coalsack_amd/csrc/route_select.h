@@ -282,6 +282,7 @@ struct RouteLds {
   float wts[MAXP];     // its routing weight
   int cnt[kMaxExperts], off[kMaxExperts], act_e[kMaxExperts];
   int na;
+  unsigned long long ew[kMaxExperts * (sizeof(ExpertW) / 8)];  // the experts' weight pointers, staged early
   CloseCallLdsT<CCB> cc;
   int cc_tok[64], cc_n;
   float cc_thr[64];
@@ -296,6 +297,16 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
   const float NEG = -__builtin_inff();
   const float tol = close_call_tolerance(r.H);
   if (threadIdx.x == 0) s.cc_n = 0;
+  // the table of weight pointers is needed last (work descriptors); its load is started
+  // first, so that its latency runs beside that of the logits
+  static_assert(sizeof(ExpertW) % 8 == 0, "copied as 64-bit words");
+  constexpr int kEwWords = kMaxExperts * (int)(sizeof(ExpertW) / 8), kEwPerThread = (kEwWords + NT - 1) / NT;
+  unsigned long long ew_reg[kEwPerThread];
+#pragma unroll
+  for (int i = 0; i < kEwPerThread; ++i) {
+    const int w = threadIdx.x + i * NT;
+    ew_reg[i] = w < E * (int)(sizeof(ExpertW) / 8) ? reinterpret_cast<const unsigned long long*>(r.ew)[w] : 0ull;
+  }
   __syncthreads();
   auto publish_token = [&](int t, float my_val, int my_idx, float vmax) {
     const float w = routing_weight(my_val, vmax, lane, k, r.sigmoid);
@@ -326,6 +337,11 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
     } else {
       publish_token(t, my_val, my_idx, vmax);
     }
+  }
+#pragma unroll
+  for (int i = 0; i < kEwPerThread; ++i) {
+    const int w = threadIdx.x + i * NT;
+    if (w < kEwWords) s.ew[w] = ew_reg[i];
   }
   __syncthreads();
   // rare: tokens with a close call among their k+1 largest logits are recomputed in the
@@ -440,7 +456,7 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
   for (int i = threadIdx.x; i < E; i += NT) {
     const bool on = i < s.na;
     const int e = on ? s.act_e[i] : 0;
-    write_work_desc(o.desc + i, on, e, s.cnt[e], s.off[e], r.ew);
+    write_work_desc(o.desc + i, on, e, s.cnt[e], s.off[e], reinterpret_cast<const ExpertW*>(s.ew));
   }
 }
 }  // namespace csk
