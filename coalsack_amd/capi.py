@@ -130,7 +130,7 @@ class Library:
     # -- helpers
     def check(self, rc):
         if rc != OK:
-            raise CskError(rc, self.dll.csk_last_error().decode())
+            raise CskError(rc, self.dll.csk_last_error().decode(errors="replace"))
 
     def init(self, device=0):
         self.check(self.dll.csk_init(device))
@@ -148,7 +148,7 @@ class Library:
     def dev_alloc(self, nbytes):
         p = self.dll.csk_dev_alloc(nbytes)
         if not p:
-            raise CskError(ERR_HIP, self.dll.csk_last_error().decode())
+            raise CskError(ERR_HIP, self.dll.csk_last_error().decode(errors="replace"))
         return p
 
     def dev_free(self, p):
@@ -390,7 +390,7 @@ class Gguf:
         out = []
         for i in range(n.value):
             self.lib.check(self.lib.dll.csk_gguf_tensor_name(self.h, i, buf, 512))
-            out.append(buf.value.decode())
+            out.append(buf.value.decode(errors="replace"))
         return out
 
     def tensor_info(self, name):
@@ -408,7 +408,7 @@ class Gguf:
     def get_str(self, key):
         buf = C.create_string_buffer(1024)
         self.lib.check(self.lib.dll.csk_gguf_get_str(self.h, key.encode(), buf, 1024))
-        return buf.value.decode()
+        return buf.value.decode(errors="replace")
 
     def layer(self, block):
         """Resident MoE layer of transformer block `block` (csk_layer_from_gguf)."""
