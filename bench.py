@@ -242,6 +242,25 @@ def bench_stack(lib, synth, shape, T, steps, warmup, n_layers, seed=1234):
                 distinct_experts_per_layer=distinct)
 
 
+def measured_copy_gbs(lib, nbytes=256 << 20, reps=10):
+    """What a plain copy kernel reaches on this box (bytes read + bytes written per second):
+    the practical ceiling beside the 8 TB/s on the data sheet."""
+    src, dst = lib.dev_alloc(nbytes), lib.dev_alloc(nbytes)
+    lib.copy_d2d(dst, src, nbytes)  # first touch
+    e0, e1 = lib.event(), lib.event()
+    lib.record(e0)
+    for _ in range(reps):
+        lib.copy_d2d(dst, src, nbytes)
+    lib.record(e1)
+    lib.synchronize()
+    ms = lib.elapsed_ms(e0, e1)
+    lib.dll.csk_event_destroy(e0)
+    lib.dll.csk_event_destroy(e1)
+    lib.dev_free(src)
+    lib.dev_free(dst)
+    return 2 * nbytes * reps / (ms * 1e-3) / 1e9
+
+
 def cpu_baseline(L, hidden, gpu_out, budget_s=12.0):
     """Times the CPU checker (single thread, as the reference's layer runs) on
     the same layer and tokens; repeats the forward until about budget_s of CPU
@@ -420,6 +439,9 @@ def main():
         roof["traffic"] = rec["bytes"]
         roof["traffic_source"] = rec["source"]
     roof["frac"] = roof["achieved"] / roof["peak"]
+    if roof["bound"] == "hbm":
+        roof["measured_copy_gbs"] = round(measured_copy_gbs(lib), 1)
+        roof["frac_of_measured_copy"] = roof["achieved"] / roof["measured_copy_gbs"]
     roof["kernel_ms"] = res["stage_ms"]["gateup"]
     roof["algorithmic_bytes"] = res["gateup_bytes"]
 
