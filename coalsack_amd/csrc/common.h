@@ -87,10 +87,26 @@ __device__ __forceinline__ void split_bf16(float x, uint16_t& hi, uint16_t& lo) 
   lo = (uint16_t)float_to_bf16_bits(x - bf16_bits_to_float(h));
 }
 
+// Sum over the 64 lanes, the same value returned in every lane: four cross-lane steps
+// inside each row of 16 (quad swaps, half-row and row mirrors -- ordinary vector-ALU
+// latency, where a shuffle through the LDS crossbar takes ten times as long), then the four
+// row sums through scalar registers.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float a) {
+  const int x = __float_as_int(a);
+  return a + __int_as_float(__builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+  v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141>(v);  // row_half_mirror
+  v = dpp_add<0x140>(v);  // row_mirror
+  const int x = __float_as_int(v);
+  const float r0 = __int_as_float(__builtin_amdgcn_readlane(x, 0));
+  const float r1 = __int_as_float(__builtin_amdgcn_readlane(x, 16));
+  const float r2 = __int_as_float(__builtin_amdgcn_readlane(x, 32));
+  const float r3 = __int_as_float(__builtin_amdgcn_readlane(x, 48));
+  return (r0 + r1) + (r2 + r3);
 }
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {

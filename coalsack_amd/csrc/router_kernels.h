@@ -222,15 +222,45 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
   const float bias = b ? b[e] : 0.0f;
   {
     const int t0 = blockIdx.y * 4;
+    const int nt = min(4, T - t0);  // tokens of this tile (the same in every thread)
+    // this thread's part of the token rows stays in registers between the two passes
+    constexpr int kMaxIter = 4;     // 256 threads x 4 float4 x 4 = H up to 4096; longer rows are read again
+    float4 xr[4][kMaxIter];
+    const bool held = H4 <= 256 * kMaxIter;
+    if (held) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (i < nt) {
+#pragma unroll
+          for (int j = 0; j < kMaxIter; ++j) {
+            const int c = threadIdx.x + 256 * j;
+            xr[i][j] = c < H4 ? reinterpret_cast<const float4*>(hidden + (size_t)(t0 + i) * H)[c]
+                              : make_float4(0.f, 0.f, 0.f, 0.f);
+          }
+        }
+      }
+    }
+    auto row = [&](int i, int j, int c) -> float4 {
+      return held ? xr[i][j] : reinterpret_cast<const float4*>(hidden + (size_t)(t0 + i) * H)[c];
+    };
     float den[4] = {1.0f, 1.0f, 1.0f, 1.0f};
     if (norm_w) {
       float ss[4] = {0.f, 0.f, 0.f, 0.f};
-      for (int c = threadIdx.x; c < H4; c += 256) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int t = min(t0 + i, T - 1);
-          const float4 xv = reinterpret_cast<const float4*>(hidden + (size_t)t * H)[c];
-          ss[i] += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
+      for (int i = 0; i < 4; ++i) {
+        if (i < nt) {
+          if (held) {
+#pragma unroll
+            for (int j = 0; j < kMaxIter; ++j) {
+              const float4 xv = xr[i][j];  // chunks past H are zeros
+              ss[i] += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
+            }
+          } else {
+            for (int c = threadIdx.x; c < H4; c += 256) {
+              const float4 xv = row(i, 0, c);
+              ss[i] += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
+            }
+          }
         }
       }
 #pragma unroll
@@ -244,21 +274,36 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
         den[i] = sqrtf(((part[0][0][i] + part[0][1][i]) + (part[0][2][i] + part[0][3][i])) / (float)H + eps);
     }
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int c = threadIdx.x; c < H4; c += 256) {
-      const float4 gv = g4[c];
-      float4 wv4 = make_float4(1.f, 1.f, 1.f, 1.f);
-      if (norm_w) wv4 = w4[c];
+    auto dot = [&](int i, float4 xv, const float4& gv, const float4& wv4) {
+      if (norm_w) {
+        xv.x = (xv.x / den[i]) * wv4.x;
+        xv.y = (xv.y / den[i]) * wv4.y;
+        xv.z = (xv.z / den[i]) * wv4.z;
+        xv.w = (xv.w / den[i]) * wv4.w;
+      }
+      acc[i] += xv.x * gv.x + xv.y * gv.y + xv.z * gv.z + xv.w * gv.w;
+    };
+    if (held) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int t = min(t0 + i, T - 1);
-        float4 xv = reinterpret_cast<const float4*>(hidden + (size_t)t * H)[c];
-        if (norm_w) {
-          xv.x = (xv.x / den[i]) * wv4.x;
-          xv.y = (xv.y / den[i]) * wv4.y;
-          xv.z = (xv.z / den[i]) * wv4.z;
-          xv.w = (xv.w / den[i]) * wv4.w;
+      for (int j = 0; j < kMaxIter; ++j) {
+        const int c = threadIdx.x + 256 * j;
+        if (c < H4) {
+          const float4 gv = g4[c];
+          float4 wv4 = make_float4(1.f, 1.f, 1.f, 1.f);
+          if (norm_w) wv4 = w4[c];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (i < nt) dot(i, xr[i][j], gv, wv4);
         }
-        acc[i] += xv.x * gv.x + xv.y * gv.y + xv.z * gv.z + xv.w * gv.w;
+      }
+    } else {
+      for (int c = threadIdx.x; c < H4; c += 256) {
+        const float4 gv = g4[c];
+        float4 wv4 = make_float4(1.f, 1.f, 1.f, 1.f);
+        if (norm_w) wv4 = w4[c];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (i < nt) dot(i, row(i, 0, c), gv, wv4);
       }
     }
 #pragma unroll
