@@ -69,10 +69,13 @@ __device__ __forceinline__ void select_topk(float (&v)[4], int lane, int E, int 
     }
   }
   // lanes 0..k hold the k+1 largest in descending order (fewer when E == k)
-  const float below = __shfl_down(my_val, 1, 64);
+  // the value one lane up (wave_shl:1, a vector-ALU operation) and slot min(k, E - 1) through
+  // a scalar register: no trip through the LDS crossbar
+  const int mv = __float_as_int(my_val);
+  const float below = __int_as_float(__builtin_amdgcn_update_dpp(mv, mv, 0x130, 0xf, 0xf, false));
   const bool close = lane < k && lane + 1 < E && (my_val - below) <= tol * fmaxf(1.0f, fabsf(my_val));
   close_call = __any(close);
-  runner_up = __shfl(my_val, min(k, E - 1), 64);
+  runner_up = __int_as_float(__builtin_amdgcn_readlane(mv, min(k, E - 1)));
 }
 
 // Logits in the reference's order: a strictly sequential fp32 sum per logit, multiply and
@@ -223,7 +226,7 @@ __device__ __forceinline__ float routing_weight(float my_val, float vmax, int la
   if (sigmoid) return 1.0f / (1.0f + expf(-my_val));
   float w = (lane < k) ? expf(my_val - vmax) : 0.0f;
   float sum = 0.0f;
-  for (int s = 0; s < k; ++s) sum += __shfl(w, s, 64);  // slot order
+  for (int s = 0; s < k; ++s) sum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), s));  // slot order
   const float inv = (sum > 0.0f) ? (1.0f / sum) : 0.0f;
   return w * inv;
 }
@@ -276,6 +279,29 @@ struct RouteOut {
   int* list_tok;      // [T * k]
   float* list_w;      // [T * k]
 };
+// Inclusive prefix sum over the 64 lanes: shifts inside each row of 16 on the vector ALU
+// (lanes without a source add zero), then the totals of the rows before through scalar
+// registers.
+template <int CTRL>
+__device__ __forceinline__ int dpp_shr_add(int v) {
+  return v + __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+__device__ __forceinline__ int wave_scan_inclusive(int v, int lane) {
+  v = dpp_shr_add<0x111>(v);  // row_shr:1
+  v = dpp_shr_add<0x112>(v);  // row_shr:2
+  v = dpp_shr_add<0x114>(v);  // row_shr:4
+  v = dpp_shr_add<0x118>(v);  // row_shr:8
+  const int t0 = __builtin_amdgcn_readlane(v, 15), t1 = __builtin_amdgcn_readlane(v, 31);
+  const int t2 = __builtin_amdgcn_readlane(v, 47);
+  const int row = lane >> 4;
+  return v + (row >= 1 ? t0 : 0) + (row >= 2 ? t1 : 0) + (row >= 3 ? t2 : 0);
+}
+
+// ceil(c / g) for the group sizes in use without a run-time integer division
+__device__ __forceinline__ int group_count(int c, int g) {
+  return g == 4 ? (c + 3) >> 2 : g == 6 ? (c + 5) / 6 : (c + g - 1) / g;
+}
+
 template <int CCB, int MAXP>
 struct RouteLds {
   int ids[MAXP];       // expert of assignment p = t * k + slot
@@ -300,6 +326,7 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
   // the table of weight pointers is needed last (work descriptors); its load is started
   // first, so that its latency runs beside that of the logits
   static_assert(sizeof(ExpertW) % 8 == 0, "copied as 64-bit words");
+  static_assert(MAXP < 32768, "counts are scanned as 16-bit halves");
   constexpr int kEwWords = kMaxExperts * (int)(sizeof(ExpertW) / 8), kEwPerThread = (kEwWords + NT - 1) / NT;
   unsigned long long ew_reg[kEwPerThread];
 #pragma unroll
@@ -390,21 +417,12 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
       c[j] = e < E ? s.cnt[e] : 0;
       tot += c[j];
       nact += c[j] > 0;
-      ngrp += (c[j] + group_tokens - 1) / group_tokens;
+      ngrp += group_count(c[j], group_tokens);
       nmt += (c[j] + 63) / 64;
     }
-    int s_tot = tot, s_act = nact, s_grp = ngrp, s_mt = nmt;  // inclusive scans over lanes
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int t0 = __shfl_up(s_tot, d, 64), t1 = __shfl_up(s_act, d, 64);
-      const int t2 = __shfl_up(s_grp, d, 64), t3 = __shfl_up(s_mt, d, 64);
-      if (lane >= d) {
-        s_tot += t0;
-        s_act += t1;
-        s_grp += t2;
-        s_mt += t3;
-      }
-    }
+    // inclusive scans over the lanes, two 16-bit counts to a register (none exceeds MAXP)
+    const int sa = wave_scan_inclusive(tot | (ngrp << 16), lane), sb = wave_scan_inclusive(nact | (nmt << 16), lane);
+    const int s_tot = sa & 0xffff, s_grp = sa >> 16, s_act = sb & 0xffff, s_mt = sb >> 16;
     int run = s_tot - tot, slot = s_act - nact, gi = s_grp - ngrp, mi = s_mt - nmt;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -437,6 +455,7 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
   }
   __syncthreads();
   // ordered scatter: rank of an assignment = matches before it (ballot prefix)
+  const unsigned inv_k = (65536u + (unsigned)k - 1u) / (unsigned)k;  // p / k == p * inv_k >> 16 for p <= 1024, k <= 16
   for (int e = wv; e < E; e += NW) {
     if (s.cnt[e] == 0) continue;
     int basep = s.off[e];
@@ -446,7 +465,7 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
       const unsigned long long m = __ballot(hit);
       if (hit) {
         const int pos = basep + __popcll(m & ((1ull << lane) - 1ull));
-        o.list_tok[pos] = p / k;
+        o.list_tok[pos] = (int)(((unsigned)p * inv_k) >> 16);
         o.list_w[pos] = s.wts[p];
         o.pos_of_slot[p] = pos;
       }
