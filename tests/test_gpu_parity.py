@@ -452,3 +452,39 @@ def test_concurrent_forwards_equal_sequential(lib):
     for layer in layers:
         layer.close()
     assert bad == [0, 0]
+
+
+@pytest.mark.parametrize("E,k,H,F,T,n_layers", [(8, 2, 128, 160, 1, 4), (8, 2, 128, 160, 8, 4), (16, 4, 256, 192, 64, 3),
+                                                (128, 4, 2880, 2880, 1, 2), (128, 4, 2880, 2880, 8, 2)])
+def test_stack_config5(lib, oracle, E, k, H, F, T, n_layers):
+    """BASELINE config 5: h <- h + MoE(RMSNorm(h)) through several layers on the device
+    (csk_moe_stack_forward).  The stack equals the same layers called one at a time bit for
+    bit, and every layer's output matches the CPU path fed with that layer's actual input
+    (so that a routing near-tie in one layer is not carried into the next comparison)."""
+    from coalsack_amd.capi import stack_forward
+    flags = capi.FWD_RMSNORM | capi.FWD_RESIDUAL
+    big = H >= 2048
+    Ls = [synth.LayerInputs(E, k, H, F, seed=77, layer=i, with_norm=True) for i in range(n_layers)]
+    layers = [build_layer(lib, L, norm=True, device_weights=big) for L in Ls]
+    hidden = synth.hidden_states(T, H, seed=3)
+    d_h = lib.to_device(hidden)
+    try:
+        stack_forward(lib, layers, d_h, T)
+        got_stack = lib.to_host(d_h, hidden.shape)
+        h = hidden
+        for L, layer in zip(Ls, layers):
+            nxt, pairs = layer.forward(h, flags, want_pairs=True)
+            n = T if not big else min(T, 3)
+            if big:  # replay only the experts the first tokens select
+                want, wpairs = oracle_layer_subset(oracle, L, h, n, norm=True, residual=True)
+            else:
+                want, wpairs = oracle_layer(oracle, L, h, norm=True, residual=True)
+            same = np.all(pairs[:n, :, 0] == wpairs[:n, :, 0], axis=1)
+            assert same.mean() >= 0.9
+            assert_layer_close(nxt[:n][same], want[:n][same])
+            h = nxt
+        assert np.array_equal(got_stack, h)
+    finally:
+        lib.dev_free(d_h)
+        for layer in layers:
+            layer.close()
