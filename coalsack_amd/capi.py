@@ -70,6 +70,7 @@ SIGNATURES = {
     "csk_moe_forward": (C.c_int, [_P, _P, _I64, _P, C.c_int]),
     "csk_moe_forward_host": (C.c_int, [_P, _P, _I64, _P, _P, C.c_int]),
     "csk_moe_stack_forward": (C.c_int, [C.POINTER(_P), _I64, _P, _I64]),
+    "csk_set_pass_tokens": (C.c_int, [_I64]),
     "csk_layer_last_dispatch": (C.c_int, [_P, _P, _P]),
     "csk_moe_router": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P]),
     "csk_moe_router_logits": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _P]),
@@ -167,6 +168,9 @@ class Library:
 
     def copy_d2d(self, dst, src, nbytes):
         self.check(self.dll.csk_copy_d2d(dst, src, nbytes))
+
+    def set_pass_tokens(self, tokens):
+        self.check(self.dll.csk_set_pass_tokens(tokens))
 
     def synchronize(self):
         self.check(self.dll.csk_synchronize())

@@ -1115,14 +1115,15 @@ static int layer_ready(const csk_layer* L, int flags) {
   return CSK_OK;
 }
 
-extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, float* out, int flags) {
-  REQUIRE_INIT();
-  if (!L || !hidden || !out || T < 0) return fail(CSK_ERR_ARG, "csk_moe_forward: bad argument");
-  int rc = layer_ready(L, flags);
-  if (rc != CSK_OK) return rc;
-  L->last_T = T;
-  if (T == 0) return CSK_OK;
-  if (T * L->k > (int64_t)1 << 24) return fail(CSK_ERR_ARG, "T * top_k exceeds 2^24");
+namespace {
+// Tokens are independent of one another, so a long batch is processed in passes of at most
+// g_pass_tokens tokens: the workspace stays bounded and the 32-bit offsets of the grouped
+// GEMM always fit.  Passes are of (nearly) equal size, so that all of them take the same
+// kernels.
+int64_t g_pass_tokens = 32768;
+
+int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int flags) {
+  int rc = CSK_OK;
   Workspace& ws = g_ws;
   rc = ws.ensure(T, L->E, L->k, L->H, L->F, L->wbf);
   if (rc != CSK_OK) return rc;
@@ -1198,6 +1199,37 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
   return rc;
 }
 
+// sizes of the passes a batch of T tokens is processed in: n passes of `each` tokens (the last one shorter)
+void pass_plan(int64_t T, int64_t& n, int64_t& each) {
+  n = std::max<int64_t>(1, cdiv(T, g_pass_tokens));
+  each = cdiv(T, n);
+}
+}  // namespace
+
+extern "C" int csk_set_pass_tokens(int64_t tokens) {
+  API_LOCK();
+  if (tokens < 1 || tokens > 65536) return fail(CSK_ERR_ARG, "csk_set_pass_tokens: need 1 <= tokens <= 65536");
+  g_pass_tokens = tokens;
+  return CSK_OK;
+}
+
+extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, float* out, int flags) {
+  REQUIRE_INIT();
+  if (!L || !hidden || !out || T < 0) return fail(CSK_ERR_ARG, "csk_moe_forward: bad argument");
+  int rc = layer_ready(L, flags);
+  if (rc != CSK_OK) return rc;
+  L->last_T = T;
+  if (T == 0) return CSK_OK;
+  int64_t n, each;
+  pass_plan(T, n, each);
+  L->last_T = n == 1 ? T : -1;  // the dispatch lists of a batch taken in several passes are those of its last pass only
+  for (int64_t t0 = 0; t0 < T; t0 += each) {
+    rc = forward_pass(L, hidden + t0 * L->H, std::min(each, T - t0), out + t0 * L->H, flags);
+    if (rc != CSK_OK) return rc;
+  }
+  return CSK_OK;
+}
+
 extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T, float* out,
                                     float* pairs_out, int flags) {
   REQUIRE_INIT();
@@ -1210,10 +1242,21 @@ extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T
   int rc = CSK_OK;
   if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("hipMalloc: ") + hipGetErrorString(e));
   if (rc == CSK_OK) rc = csk_copy_h2d(dh, hidden, n * sizeof(float));
-  if (rc == CSK_OK) rc = csk_moe_forward(L, dh, T, dout, flags);
+  if (rc == CSK_OK && !pairs_out) rc = csk_moe_forward(L, dh, T, dout, flags);
+  if (rc == CSK_OK && pairs_out) {
+    // pass by pass, as csk_moe_forward does: the router output lives in the workspace of a pass
+    rc = layer_ready(L, flags);
+    int64_t np, each;
+    pass_plan(T, np, each);
+    L->last_T = np == 1 ? T : -1;
+    for (int64_t t0 = 0; t0 < T && rc == CSK_OK; t0 += each) {
+      const int64_t tn = std::min(each, T - t0);
+      rc = forward_pass(L, dh + t0 * L->H, tn, dout + t0 * L->H, flags);
+      if (rc == CSK_OK)
+        rc = csk_copy_d2h(pairs_out + t0 * L->k * 2, g_ws.pairs, (size_t)tn * L->k * 2 * sizeof(float));
+    }
+  }
   if (rc == CSK_OK) rc = csk_copy_d2h(out, dout, n * sizeof(float));
-  if (rc == CSK_OK && pairs_out)
-    rc = csk_copy_d2h(pairs_out, g_ws.pairs, (size_t)T * L->k * 2 * sizeof(float));
   (void)hipStreamSynchronize(g_stream);
   (void)hipFree(dh);
   if (dout) (void)hipFree(dout);
@@ -1234,7 +1277,9 @@ extern "C" int csk_moe_stack_forward(csk_layer* const* layers, int64_t n_layers,
 extern "C" int csk_layer_last_dispatch(csk_layer* L, int32_t* counts_host, int32_t* tokens_host) {
   REQUIRE_INIT();
   if (!L) return fail(CSK_ERR_ARG, "null layer");
-  if (L->last_T <= 0) return fail(CSK_ERR_STATE, "no forward has run on this layer");
+  if (L->last_T < 0)
+    return fail(CSK_ERR_STATE, "the last forward took its batch in several passes: there is no single dispatch to report");
+  if (L->last_T == 0) return fail(CSK_ERR_STATE, "no forward has run on this layer");
   if (counts_host) {
     int rc = csk_copy_d2h(counts_host, g_ws.counts, (size_t)L->E * sizeof(int));
     if (rc != CSK_OK) return rc;

@@ -194,15 +194,21 @@ int csk_gguf_get_str(const csk_gguf* g, const char* key, char* buf, size_t cap);
  * of a stacked tensor is the slice at offset + e * rows * (K/32) * 17 --
  * moe_weight_provider::get, src/llm/moe_weight_provider.cpp:160-188; it takes
  * the place of that provider and its LRU cache: all experts stay in HBM.
- * MXFP4 expert tensors only. */
+ * Expert tensors are MXFP4, or F16 / Q4_K / Q6_K (a layer with fp16 experts,
+ * as moe_weight_provider.cpp:134-159 hands them to the node). */
 int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out);
 
 /* Router -> dispatch -> expert MLPs -> merge for T tokens, everything on the
- * GPU: hidden and out are device pointers [T,H] f32 (out may not alias
- * hidden).  Stands in for the node chain llm_engine wires per layer
- * (src/llm/llm_engine.cpp:714-777).  Asynchronous on the library's stream. */
+ * GPU: hidden and out are device pointers [T,H] f32 (out may be hidden itself:
+ * the layer then updates the rows in place).  Stands in for the node chain
+ * llm_engine wires per layer (src/llm/llm_engine.cpp:714-777).  Asynchronous on
+ * the library's stream.  Any T: a batch longer than the pass size (32768 tokens
+ * unless csk_set_pass_tokens changed it) is taken in several passes of equal
+ * size -- tokens do not depend on one another -- so the workspace stays bounded. */
 int csk_moe_forward(csk_layer* L, const float* hidden_device, int64_t T, float* out_device,
                     int flags);
+/* Largest number of tokens one pass of csk_moe_forward takes (1..65536). */
+int csk_set_pass_tokens(int64_t tokens);
 /* Same through host buffers; also returns the router output [T,k,2] when
  * pairs_out is not NULL.  Synchronous. */
 int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T, float* out, float* pairs_out,

@@ -488,3 +488,36 @@ def test_stack_config5(lib, oracle, E, k, H, F, T, n_layers):
         lib.dev_free(d_h)
         for layer in layers:
             layer.close()
+
+
+def test_long_batch_in_passes(lib, oracle):
+    """A batch longer than the pass size is taken in passes of equal size (tokens are
+    independent): same result bit for bit while the passes use the kernels the whole batch
+    would, same router output, and the CPU path's result in any case."""
+    L = synth.LayerInputs(8, 2, 128, 160, seed=21, with_norm=True)
+    T = 333
+    hidden = synth.hidden_states(T, L.H, seed=9)
+    flags = capi.FWD_RMSNORM | capi.FWD_RESIDUAL
+    with build_layer(lib, L, norm=True) as layer:
+        whole, pairs = layer.forward(hidden, flags, want_pairs=True)
+        layer.last_dispatch(T)
+        try:
+            lib.set_pass_tokens(100)  # four passes of 84, 84, 84, 81 tokens: grouped GEMM, as the whole batch
+            got, gpairs = layer.forward(hidden, flags, want_pairs=True)
+            assert np.array_equal(got, whole) and np.array_equal(gpairs, pairs)
+            assert np.array_equal(layer.forward(hidden, flags), whole)
+            with pytest.raises(capi.CskError, match="several passes"):
+                layer.last_dispatch(T)
+            lib.set_pass_tokens(50)   # seven passes of 48 tokens: the streaming kernels
+            small, spairs = layer.forward(hidden, flags, want_pairs=True)
+        finally:
+            lib.set_pass_tokens(32768)
+        with pytest.raises(capi.CskError):
+            lib.set_pass_tokens(0)
+    # other kernels, another summation order: the same experts (no near-tie in this batch), weights to rounding
+    assert np.array_equal(spairs[..., 0], pairs[..., 0]) and np.max(np.abs(spairs[..., 1] - pairs[..., 1])) < 1e-5
+    want, wpairs = oracle_layer(oracle, L, hidden, norm=True, residual=True)
+    same = np.all(pairs[..., 0] == wpairs[..., 0], axis=1)
+    assert same.mean() > 0.99
+    assert_layer_close(small[same], want[same])
+    assert_layer_close(whole[same], want[same])
