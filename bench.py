@@ -173,9 +173,12 @@ def bench_layer(lib, synth, shape, T, steps, warmup, seed=1234):
     Us, tmax = [], 0
     for i in range(nb - 1, -1, -1):  # batch 0 last: its output is the one checked
         layer.forward_device(d_ins[i], T, d_out)
-        counts, _ = layer.last_dispatch(T)
-        Us.append(int(np.count_nonzero(counts)))
-        tmax = max(tmax, int(counts.max()))
+        if T <= 32768:
+            counts, _ = layer.last_dispatch(T)
+            Us.append(int(np.count_nonzero(counts)))
+            tmax = max(tmax, int(counts.max()))
+        else:  # taken in several passes: no single dispatch to read back; every expert is in use
+            Us.append(shape["E"])
     U = float(np.mean(Us))
     hidden = hiddens[0]
     out = lib.to_host(d_out, (T, L.H))
