@@ -1134,9 +1134,15 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
     // small batch: prologue + logits in one launch, top-k + dispatch in another
     mark(CSK_STAGE_PREP);
     mark(CSK_STAGE_ROUTER);
-    router_prep_logits_kernel<<<dim3((unsigned)(L->E + 4), (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
-        hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, ws.xs, L->gate_w,
-        L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
+    // a workgroup takes one expert (latency) as long as all of them are resident at once, four beyond
+    if (cdiv(T, 4) * (L->E + 4) <= 5 * std::max(g_cus, 1))  // five of these workgroups fit a compute unit
+      router_prep_logits_kernel<1><<<dim3((unsigned)(L->E + 4), (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
+          hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, ws.xs, L->gate_w,
+          L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
+    else
+      router_prep_logits_kernel<4><<<dim3((unsigned)(cdiv(L->E, 4) + 4), (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
+          hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, ws.xs, L->gate_w,
+          L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
     if ((rc = check_launch("router_prep_logits_kernel")) != CSK_OK) return rc;
     mark(CSK_STAGE_DISPATCH);
     RouteIn rin{ws.logits, xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, L->ew_dev,

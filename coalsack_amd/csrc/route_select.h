@@ -344,25 +344,39 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
       s.wts[t * k + lane] = w;
     }
   };
-  for (int t = wv; t < T; t += NW) {
-    float v[4];
+  // a wave's tokens four at a time: their logits are requested together, so that a wave
+  // with several tokens waits for memory once
+  for (int t0 = wv; t0 < T; t0 += 4 * NW) {
+    float v[4][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int e = lane + 64 * j;
-      v[j] = (e < E) ? r.logits[(size_t)t * E + e] : NEG;
-    }
-    float my_val, vmax, runner_up;
-    int my_idx;
-    bool close_call;
-    select_topk(v, lane, E, k, my_val, my_idx, vmax, close_call, tol, runner_up);
-    if (close_call) {
-      if (lane == 0) {
-        const int n = atomicAdd(&s.cc_n, 1);
-        s.cc_tok[n] = t;
-        s.cc_thr[n] = runner_up - 2.0f * tol * fmaxf(1.0f, fabsf(runner_up));
+    for (int q = 0; q < 4; ++q) {
+      const int t = t0 + q * NW;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int e = lane + 64 * j;
+        v[q][j] = (t < T && e < E) ? r.logits[(size_t)t * E + e] : NEG;
       }
-    } else {
-      publish_token(t, my_val, my_idx, vmax);
+    }
+#pragma unroll 1  // one copy of the selection code: the token in turn sits in v[0], the others move up
+    for (int q = 0; q < 4; ++q) {
+      const int t = t0 + q * NW;
+      if (t < T) {
+        float my_val, vmax, runner_up;
+        int my_idx;
+        bool close_call;
+        select_topk(v[0], lane, E, k, my_val, my_idx, vmax, close_call, tol, runner_up);
+        if (close_call) {
+          if (lane == 0) {
+            const int n = atomicAdd(&s.cc_n, 1);
+            s.cc_tok[n] = t;
+            s.cc_thr[n] = runner_up - 2.0f * tol * fmaxf(1.0f, fabsf(runner_up));
+          }
+        } else {
+          publish_token(t, my_val, my_idx, vmax);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[0][j] = v[1][j], v[1][j] = v[2][j], v[2][j] = v[3][j];
     }
   }
 #pragma unroll

@@ -174,148 +174,227 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(const float* __
 }
 
 // --------------------------------------------- small batches: prologue + logits
-// One launch for small T: workgroups x in [0, E) compute the logits of one expert for
-// the four tokens of tile y (the four waves split H, so all loads of a row are in flight at
-// once); workgroups x in [E, E + 4) run the prologue of one token of tile y (RMSNorm, f32 copy,
-// bf16 hi/lo split).  With RMSNorm the expert workgroups recompute each token's
-// normalisation themselves -- 2 H flops per token -- instead of waiting for the
-// prologue.  Restates moe_router_node.h:161-167 and rmsnorm_node.h:62-83.
+// One launch for small T: workgroups x in [0, ceil(E / EPW)) compute the logits of EPW experts
+// for the four tokens of tile y (the four waves split H, so all loads of a row are in flight
+// at once; the token rows stay in registers across the experts); the next four workgroups
+// run the prologue of one token of tile y each (RMSNorm, f32 copy, bf16 hi/lo split).  With
+// RMSNorm the expert workgroups recompute each token's normalisation themselves -- 2 H flops
+// per token -- instead of waiting for the prologue.  EPW = 1 spreads a handful of tokens
+// over as many workgroups as there are experts (latency); EPW = 4 is for batches whose
+// one-expert workgroups would not all be resident at once (64 tokens, 128 experts: 2112 of
+// them, 18.6 us; a quarter as many read the token rows a quarter as often).
+// Restates moe_router_node.h:161-167 and rmsnorm_node.h:62-83.
+template <int EPW>
 __global__ __launch_bounds__(256) void router_prep_logits_kernel(
     const float* __restrict__ hidden, const float* __restrict__ norm_w, float eps,
     float* __restrict__ xn, uint16_t* __restrict__ xs, const float* __restrict__ g,
     const float* __restrict__ b, float* __restrict__ logits, int T, int E, int H) {
-  __shared__ float part[2][4][4];
+  __shared__ float part[4][4];
+  __shared__ float dots[EPW][4][4];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  if ((int)blockIdx.x >= E) {  // ---- prologue of token t (one of four per token tile)
-    const int t = (blockIdx.x - E) + 4 * blockIdx.y;
-    if (blockIdx.x - E >= 4 || t >= T) return;
-    const float* x = hidden + (size_t)t * H;
+  const int n_ewg = (E + EPW - 1) / EPW;  // workgroups that compute logits
+  if ((int)blockIdx.x >= n_ewg) {  // ---- prologue of token t (one of four per token tile)
+    const int t = (blockIdx.x - n_ewg) + 4 * blockIdx.y;
+    if (blockIdx.x - n_ewg >= 4 || t >= T) return;
+    // four columns per thread, the row's loads all in flight at once and kept in registers
+    // between the two passes (rows longer than 4096 take further rounds of the same)
+    const float4* x4 = reinterpret_cast<const float4*>(hidden + (size_t)t * H);
+    const int H4p = H >> 2;
+    constexpr int kIter = 4;
     float den = 1.0f;
     if (norm_w) {
       float ss = 0.0f;
-      for (int d = threadIdx.x; d < H; d += 256) ss += x[d] * x[d];
+      for (int c0 = 0; c0 < H4p; c0 += 256 * kIter) {
+        float4 xv[kIter];
+#pragma unroll
+        for (int j = 0; j < kIter; ++j) {
+          const int c = c0 + threadIdx.x + 256 * j;
+          xv[j] = c < H4p ? x4[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < kIter; ++j) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
+      }
       ss = wave_sum(ss);
-      if (lane == 0) part[0][wv][0] = ss;
+      if (lane == 0) part[wv][0] = ss;
       __syncthreads();
-      ss = (part[0][0][0] + part[0][1][0]) + (part[0][2][0] + part[0][3][0]);
+      ss = (part[0][0] + part[1][0]) + (part[2][0] + part[3][0]);
       den = sqrtf(ss / (float)H + eps);
     }
-    for (int d = threadIdx.x; d < H; d += 256) {
-      float v = x[d];
-      if (norm_w) {
-        v = (v / den) * norm_w[d];
-        xn[(size_t)t * H + d] = v;
+    const float4* nw4 = reinterpret_cast<const float4*>(norm_w);
+    for (int c0 = 0; c0 < H4p; c0 += 256 * kIter) {
+      float4 xv[kIter], wv4[kIter];
+#pragma unroll
+      for (int j = 0; j < kIter; ++j) {
+        const int c = c0 + threadIdx.x + 256 * j;
+        if (c < H4p) {
+          xv[j] = x4[c];
+          if (norm_w) wv4[j] = nw4[c];
+        }
       }
-      uint16_t hi, lo;
-      split_bf16(v, hi, lo);
-      uint16_t* o = xs + ((size_t)t * (H / 32) + (d >> 5)) * 64 + (d & 31);
-      o[0] = hi;
-      o[32] = lo;
+#pragma unroll
+      for (int j = 0; j < kIter; ++j) {
+        const int c = c0 + threadIdx.x + 256 * j;
+        if (c < H4p) {
+          float4 v = xv[j];
+          if (norm_w) {
+            v.x = (v.x / den) * wv4[j].x, v.y = (v.y / den) * wv4[j].y;
+            v.z = (v.z / den) * wv4[j].z, v.w = (v.w / den) * wv4[j].w;
+            reinterpret_cast<float4*>(xn + (size_t)t * H)[c] = v;
+          }
+          uint16_t hi[4], lo[4];
+          split_bf16(v.x, hi[0], lo[0]);
+          split_bf16(v.y, hi[1], lo[1]);
+          split_bf16(v.z, hi[2], lo[2]);
+          split_bf16(v.w, hi[3], lo[3]);
+          const int d = 4 * c;  // four columns of one 32-column block
+          uint16_t* o = xs + ((size_t)t * (H / 32) + (d >> 5)) * 64 + (d & 31);
+          *reinterpret_cast<uint2*>(o) = make_uint2(hi[0] | ((uint32_t)hi[1] << 16), hi[2] | ((uint32_t)hi[3] << 16));
+          *reinterpret_cast<uint2*>(o + 32) = make_uint2(lo[0] | ((uint32_t)lo[1] << 16), lo[2] | ((uint32_t)lo[3] << 16));
+        }
+      }
     }
     return;
   }
-  // ---- logits of expert e for four tokens (token tile blockIdx.y)
-  const int e = blockIdx.x;
+  // ---- logits of experts e0 .. e0 + EPW - 1 for four tokens (token tile blockIdx.y)
+  const int e0 = blockIdx.x * EPW;
   const int H4 = H >> 2;
-  const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)e * H);
   const float4* w4 = reinterpret_cast<const float4*>(norm_w);
-  const float bias = b ? b[e] : 0.0f;
-  {
-    const int t0 = blockIdx.y * 4;
-    const int nt = min(4, T - t0);  // tokens of this tile (the same in every thread)
-    // this thread's part of the token rows stays in registers between the two passes
-    constexpr int kMaxIter = 4;     // 256 threads x 4 float4 x 4 = H up to 4096; longer rows are read again
-    float4 xr[4][kMaxIter];
-    const bool held = H4 <= 256 * kMaxIter;
-    if (held) {
+  const int t0 = blockIdx.y * 4;
+  const int nt = min(4, T - t0);  // tokens of this tile (the same in every thread)
+  // this thread's part of the token rows stays in registers between the passes
+  constexpr int kMaxIter = 4;     // 256 threads x 4 float4 x 4 = H up to 4096; longer rows are read again
+  float4 xr[4][kMaxIter];
+  const bool held = H4 <= 256 * kMaxIter;
+  if (held) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (i < nt) {
+    for (int i = 0; i < 4; ++i) {
+      if (i < nt) {
+#pragma unroll
+        for (int j = 0; j < kMaxIter; ++j) {
+          const int c = threadIdx.x + 256 * j;
+          xr[i][j] = c < H4 ? reinterpret_cast<const float4*>(hidden + (size_t)(t0 + i) * H)[c]
+                            : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+      }
+    }
+  }
+  auto row = [&](int i, int c) -> float4 {
+    return reinterpret_cast<const float4*>(hidden + (size_t)(t0 + i) * H)[c];
+  };
+  // 1 / rms per token: the logits only have to be within the close-call tolerance of the
+  // reference's (a token inside it is recomputed from the exactly normalised row the
+  // prologue workgroups write), so the rows are scaled by a reciprocal here, one
+  // multiplication per element where the exact form is a correctly rounded division; the
+  // difference, 1 ulp per element, moves a logit by about a hundredth of the tolerance's unit
+  float inv[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+  if (norm_w) {
+    float ss[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (i < nt) {
+        if (held) {
 #pragma unroll
           for (int j = 0; j < kMaxIter; ++j) {
-            const int c = threadIdx.x + 256 * j;
-            xr[i][j] = c < H4 ? reinterpret_cast<const float4*>(hidden + (size_t)(t0 + i) * H)[c]
-                              : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 xv = xr[i][j];  // chunks past H are zeros
+            ss[i] += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
+          }
+        } else {
+          for (int c = threadIdx.x; c < H4; c += 256) {
+            const float4 xv = row(i, c);
+            ss[i] += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
           }
         }
       }
     }
-    auto row = [&](int i, int j, int c) -> float4 {
-      return held ? xr[i][j] : reinterpret_cast<const float4*>(hidden + (size_t)(t0 + i) * H)[c];
-    };
-    float den[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-    if (norm_w) {
-      float ss[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (i < nt) {
-          if (held) {
-#pragma unroll
-            for (int j = 0; j < kMaxIter; ++j) {
-              const float4 xv = xr[i][j];  // chunks past H are zeros
-              ss[i] += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
-            }
-          } else {
-            for (int c = threadIdx.x; c < H4; c += 256) {
-              const float4 xv = row(i, 0, c);
-              ss[i] += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
-            }
-          }
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float s = wave_sum(ss[i]);
-        if (lane == 0) part[0][wv][i] = s;
-      }
-      __syncthreads();
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        den[i] = sqrtf(((part[0][0][i] + part[0][1][i]) + (part[0][2][i] + part[0][3][i])) / (float)H + eps);
+    for (int i = 0; i < 4; ++i) {
+      const float sum = wave_sum(ss[i]);
+      if (lane == 0) part[wv][i] = sum;
     }
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    auto dot = [&](int i, float4 xv, const float4& gv, const float4& wv4) {
-      if (norm_w) {
-        xv.x = (xv.x / den[i]) * wv4.x;
-        xv.y = (xv.y / den[i]) * wv4.y;
-        xv.z = (xv.z / den[i]) * wv4.z;
-        xv.w = (xv.w / den[i]) * wv4.w;
-      }
-      acc[i] += xv.x * gv.x + xv.y * gv.y + xv.z * gv.z + xv.w * gv.w;
-    };
-    if (held) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      inv[i] = 1.0f / sqrtf(((part[0][i] + part[1][i]) + (part[2][i] + part[3][i])) / (float)H + eps);
+    if (held) {  // normalise the held rows once, for all the experts of this workgroup
 #pragma unroll
       for (int j = 0; j < kMaxIter; ++j) {
         const int c = threadIdx.x + 256 * j;
         if (c < H4) {
-          const float4 gv = g4[c];
-          float4 wv4 = make_float4(1.f, 1.f, 1.f, 1.f);
-          if (norm_w) wv4 = w4[c];
+          const float4 wv4 = w4[c];
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (i < nt) dot(i, xr[i][j], gv, wv4);
+          for (int i = 0; i < 4; ++i) {
+            if (i < nt) {
+              xr[i][j].x = (xr[i][j].x * inv[i]) * wv4.x;
+              xr[i][j].y = (xr[i][j].y * inv[i]) * wv4.y;
+              xr[i][j].z = (xr[i][j].z * inv[i]) * wv4.z;
+              xr[i][j].w = (xr[i][j].w * inv[i]) * wv4.w;
+            }
+          }
+        }
+      }
+    }
+  }
+  // the gate row of the next expert is requested before the current one is used
+  float4 gq[2][kMaxIter];
+  auto load_gate = [&](float4(&q)[kMaxIter], int ee) {
+    const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)min(e0 + ee, E - 1) * H);
+#pragma unroll
+    for (int j = 0; j < kMaxIter; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      q[j] = c < H4 ? g4[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
+  if (held) load_gate(gq[0], 0);
+#pragma unroll
+  for (int ee = 0; ee < EPW; ++ee) {
+    const int e = min(e0 + ee, E - 1);  // a workgroup past the last expert repeats it; nothing is stored
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (held) {
+      if (ee + 1 < EPW) load_gate(gq[(ee + 1) & 1], ee + 1);
+#pragma unroll
+      for (int j = 0; j < kMaxIter; ++j) {
+        const float4 gv = gq[ee & 1][j];  // chunks past H are zeros on both sides
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (i < nt) {
+            const float4 xv = xr[i][j];
+            acc[i] += xv.x * gv.x + xv.y * gv.y + xv.z * gv.z + xv.w * gv.w;
+          }
         }
       }
     } else {
+      const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)e * H);
       for (int c = threadIdx.x; c < H4; c += 256) {
         const float4 gv = g4[c];
         float4 wv4 = make_float4(1.f, 1.f, 1.f, 1.f);
         if (norm_w) wv4 = w4[c];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (i < nt) dot(i, row(i, 0, c), gv, wv4);
+        for (int i = 0; i < 4; ++i) {
+          if (i < nt) {
+            float4 xv = row(i, c);
+            if (norm_w) {
+              xv.x = (xv.x * inv[i]) * wv4.x;
+              xv.y = (xv.y * inv[i]) * wv4.y;
+              xv.z = (xv.z * inv[i]) * wv4.z;
+              xv.w = (xv.w * inv[i]) * wv4.w;
+            }
+            acc[i] += xv.x * gv.x + xv.y * gv.y + xv.z * gv.z + xv.w * gv.w;
+          }
+        }
       }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float s = wave_sum(acc[i]);
-      if (lane == 0) part[1][wv][i] = s;
+      const float sum = wave_sum(acc[i]);
+      if (lane == 0) dots[ee][wv][i] = sum;
     }
-    __syncthreads();
-    if (threadIdx.x < 4 && t0 + (int)threadIdx.x < T) {
-      const int i = threadIdx.x;
-      logits[(size_t)(t0 + i) * E + e] = ((part[1][0][i] + part[1][1][i]) + (part[1][2][i] + part[1][3][i])) + bias;
-    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 4 * EPW) {
+    const int ee = threadIdx.x >> 2, i = threadIdx.x & 3, e = e0 + ee;
+    if (e < E && i < nt)
+      logits[(size_t)(t0 + i) * E + e] =
+          ((dots[ee][0][i] + dots[ee][1][i]) + (dots[ee][2][i] + dots[ee][3][i])) + (b ? b[e] : 0.0f);
   }
 }
 
