@@ -255,8 +255,8 @@ __device__ __forceinline__ void write_work_desc(WorkDesc* d, bool on, int e, int
 // ------------------------------------- small batches: top-k + dispatch, fused
 // One workgroup does, for P = T * k <= MAXP assignments, what router_topk_kernel and
 // dispatch_scatter_kernel do in two launches: top-k and weights per token (one wave per
-// token), histogram, exclusive scan, ordered scatter, work descriptors and token groups
-// -- all through LDS.
+// token), per-expert counts, exclusive scan, ordered lists, work descriptors and token
+// groups -- all through LDS.
 struct RouteIn {
   const float* logits;  // [T, E]
   const float* x;       // [T, H] rows the logits were computed from (close calls are recomputed)
@@ -308,6 +308,7 @@ struct RouteLds {
   float wts[MAXP];     // its routing weight
   int cnt[kMaxExperts], off[kMaxExperts], act_e[kMaxExperts];
   int na;
+  int cntc[MAXP / 64][kMaxExperts];  // per 64-assignment chunk: how many name the expert; then the count before the chunk
   unsigned long long ew[kMaxExperts * (sizeof(ExpertW) / 8)];  // the experts' weight pointers, staged early
   CloseCallLdsT<CCB> cc;
   int cc_tok[64], cc_n;
@@ -322,6 +323,9 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
   const int P = T * k;
   const float NEG = -__builtin_inff();
   const float tol = close_call_tolerance(r.H);
+  static_assert(MAXP <= NT && MAXP % 64 == 0, "assignment p belongs to thread p, chunk p / 64 to wave p / 64");
+  const int nchunk = (P + 63) >> 6;
+  for (int i = threadIdx.x; i < nchunk * kMaxExperts; i += NT) (&s.cntc[0][0])[i] = 0;
   if (threadIdx.x == 0) s.cc_n = 0;
   // the table of weight pointers is needed last (work descriptors); its load is started
   // first, so that its latency runs beside that of the logits
@@ -407,17 +411,34 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
     __syncthreads();
   }
   __syncthreads();
-  // histogram: wave wv counts experts wv, wv + NW, ... with ballots over the assignments
-  for (int e = wv; e < E; e += NW) {
-    int c = 0;
-    for (int p0 = 0; p0 < P; p0 += 64) {
-      const int p = p0 + lane;
-      c += __popcll(__ballot(p < P && s.ids[p] == e));
+  // Dispatch in O(P): thread p owns assignment p.  The lanes of a wave that name the same
+  // expert find one another in a loop over the distinct experts of the wave (a ballot per
+  // expert); the first of them records how many they are, the others their rank among
+  // them.  Per expert, a prefix over the chunks (waves) then gives every assignment its
+  // place in the expert's list: assignments stay in ascending order, as the reference's
+  // per-expert token loop visits them (expert_mlp_node.h:503-529).
+  const int my_p = threadIdx.x;
+  const bool live_p = my_p < P;
+  const int my_id = live_p ? s.ids[my_p] : -1;
+  unsigned long long same = 0ull, todo = __ballot(live_p);
+  while (todo != 0ull) {  // the same in every lane
+    const int id0 = __builtin_amdgcn_readlane(my_id, (int)__builtin_ctzll(todo));
+    const unsigned long long m = __ballot(my_id == id0);
+    if (my_id == id0) same = m;
+    todo &= ~m;
+  }
+  const int rank_in_chunk = __popcll(same & ((1ull << lane) - 1ull));
+  if (live_p && rank_in_chunk == 0) s.cntc[wv][my_id] = __popcll(same);
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += NT) {
+    int run = 0;
+    for (int c = 0; c < nchunk; ++c) {
+      const int v = s.cntc[c][e];
+      s.cntc[c][e] = run;
+      run += v;
     }
-    if (lane == 0) {
-      s.cnt[e] = c;
-      o.counts[e] = c;
-    }
+    s.cnt[e] = run;
+    o.counts[e] = run;
   }
   __syncthreads();
   // exclusive scan, active experts, token groups, M tiles: wave 0, four consecutive
@@ -468,23 +489,13 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
     }
   }
   __syncthreads();
-  // ordered scatter: rank of an assignment = matches before it (ballot prefix)
-  const unsigned inv_k = (65536u + (unsigned)k - 1u) / (unsigned)k;  // p / k == p * inv_k >> 16 for p <= 1024, k <= 16
-  for (int e = wv; e < E; e += NW) {
-    if (s.cnt[e] == 0) continue;
-    int basep = s.off[e];
-    for (int p0 = 0; p0 < P; p0 += 64) {
-      const int p = p0 + lane;
-      const bool hit = p < P && s.ids[p] == e;
-      const unsigned long long m = __ballot(hit);
-      if (hit) {
-        const int pos = basep + __popcll(m & ((1ull << lane) - 1ull));
-        o.list_tok[pos] = (int)(((unsigned)p * inv_k) >> 16);
-        o.list_w[pos] = s.wts[p];
-        o.pos_of_slot[p] = pos;
-      }
-      basep += __popcll(m);
-    }
+  // place of assignment p: the expert's offset + its assignments in earlier chunks + its rank in this one
+  if (live_p) {
+    const unsigned inv_k = (65536u + (unsigned)k - 1u) / (unsigned)k;  // p / k == p * inv_k >> 16 for p <= 1024, k <= 16
+    const int pos = s.off[my_id] + s.cntc[wv][my_id] + rank_in_chunk;
+    o.list_tok[pos] = (int)(((unsigned)my_p * inv_k) >> 16);
+    o.list_w[pos] = s.wts[my_p];
+    o.pos_of_slot[my_p] = pos;
   }
   for (int i = threadIdx.x; i < E; i += NT) {
     const bool on = i < s.na;
