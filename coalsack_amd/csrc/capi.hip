@@ -363,7 +363,7 @@ inline int stream_group_tokens(int64_t T) { return T <= 16 ? kStreamG : kStreamG
 
 int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, int64_t E,
                     const ExpertW* ew, Workspace& ws) {
-  dispatch_scatter_kernel<<<dim3((unsigned)E), 256, 0, g_stream>>>(
+  dispatch_scatter_kernel<<<dim3((unsigned)cdiv(std::max<int64_t>(P, 1), kDispatchThreads)), kDispatchThreads, 0, g_stream>>>(
       ids, pairs, (int)P, (int)k, (int)E, ws.counts, ew, ws.offsets, ws.desc,
       P <= kStreamMaxP ? ws.vlist : nullptr, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w,
       ws.pos, stream_group_tokens(P / std::max<int64_t>(k, 1)));

@@ -482,86 +482,86 @@ __global__ void pairs_to_ids_kernel(const float* __restrict__ pairs, int* __rest
 }
 
 // ----------------------------------------------------------------- dispatch
-// Workgroup e builds the whole per-expert histogram in LDS (every workgroup does: the
-// ids are L2-resident and LDS atomics are cheap, which saves a launch and any global
-// atomics), derives its offset, then writes the assignments naming e at offset + rank in
-// ascending order, so each expert's list is ascending in token index -- the order the
-// reference's per-expert token loop visits them (expert_mlp_node.h:503-529).  Workgroup 0
-// also publishes counts, offsets[0..E] and the compact list of experts with at least one
-// token (moe_weight_fetch_node.h:31-60).
-__global__ __launch_bounds__(256) void dispatch_scatter_kernel(
+// Workgroup c places the 1024 assignments [1024 c, 1024 c + 1024).  It counts, with LDS
+// atomics over all P expert ids (they are L2-resident; every workgroup does this, which
+// saves a launch and any global atomics), how many assignments name each expert in total
+// and how many of them lie before its own chunk; inside the chunk the lanes of a wave
+// that name the same expert find one another by ballots, and a prefix over the sixteen
+// waves completes the rank.  An assignment's place is offset(expert) + before + rank: each
+// expert's list is ascending in token index -- the order the reference's per-expert token
+// loop visits them (expert_mlp_node.h:503-529).  Ids below zero (assignments that do not
+// name the one expert of a node-level call) are skipped.  Workgroup 0 also publishes
+// counts, offsets[0..E], the work descriptors of the experts with at least one token
+// (moe_weight_fetch_node.h:31-60), the streaming kernel's token groups and the GEMM's M
+// tiles.
+constexpr int kDispatchThreads = 1024;
+__global__ __launch_bounds__(kDispatchThreads) void dispatch_scatter_kernel(
     const int* __restrict__ ids, const float* __restrict__ pairs, int P, int k, int E,
     int* __restrict__ counts, const ExpertW* __restrict__ ew, int* __restrict__ offsets,
     WorkDesc* __restrict__ desc, int* __restrict__ vlist, int* __restrict__ nv,
     int* __restrict__ mtiles, int* __restrict__ n_mtiles, int* __restrict__ list_tok,
     float* __restrict__ list_w, int* __restrict__ pos_of_slot, int group_tokens) {
-  const int e = blockIdx.x;
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  __shared__ int sh[8];
-  __shared__ int cnt[kMaxExperts], off_sh[kMaxExperts], act_e[kMaxExperts];
+  constexpr int NW = kDispatchThreads / 64;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const bool pub = blockIdx.x == 0;
+  const int chunk0 = blockIdx.x * kDispatchThreads;
+  __shared__ int cnt[kMaxExperts], before[kMaxExperts], off_sh[kMaxExperts], act_e[kMaxExperts];
+  __shared__ int wcnt[NW][kMaxExperts];
   __shared__ int na_sh;
-  cnt[threadIdx.x] = 0;  // kMaxExperts == blockDim
+  if (tid < kMaxExperts) cnt[tid] = 0, before[tid] = 0;
+  for (int i = tid; i < NW * kMaxExperts; i += kDispatchThreads) (&wcnt[0][0])[i] = 0;
   __syncthreads();
-  // each wave scans its own quarter of the assignments: the histogram, and how many name e
-  const int per_wave = ((P + 255) / 256) * 64;
-  const int p_lo = wv * per_wave, p_hi = min(P, p_lo + per_wave);
-  int hits = 0;
-  for (int p0 = p_lo; p0 < p_hi; p0 += 64 * 8) {  // eight loads in flight per lane
-    int id[8];
+  for (int p0 = 0; p0 < P; p0 += kDispatchThreads * 4) {  // four loads in flight per thread
+    int id[4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int p = p0 + 64 * j + lane;
-      id[j] = p < p_hi ? ids[p] : -1;
+    for (int j = 0; j < 4; ++j) {
+      const int p = p0 + kDispatchThreads * j + tid;
+      id[j] = p < P ? ids[p] : -1;
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      if (id[j] >= 0) atomicAdd(&cnt[id[j]], 1);
-      hits += __popcll(__ballot(id[j] == e));
+    for (int j = 0; j < 4; ++j) {
+      if (id[j] >= 0) {
+        atomicAdd(&cnt[id[j]], 1);
+        if (p0 + kDispatchThreads * j + tid < chunk0) atomicAdd(&before[id[j]], 1);
+      }
     }
   }
-  if (lane == 0) sh[4 + wv] = hits;
   __syncthreads();
-  const int mine = cnt[threadIdx.x];
-  int c = ((int)threadIdx.x < e) ? mine : 0;
-  c = (int)wave_sum((float)c);
-  if (lane == 0) sh[wv] = c;
-  if (e == 0 && (int)threadIdx.x < E) counts[threadIdx.x] = mine;
-  __syncthreads();
-  if (e == 0) {
-    // workgroup 0 publishes the scan, the active experts, the streaming kernel's token
-    // groups and the GEMM's M tiles: wave 0, four consecutive experts per lane,
-    // wave-wide prefix sums
-    if (wv == 0) {
-      int cc[4], tot = 0, nact = 0, ngrp = 0, nmt = 0;
+  // exclusive scan over the experts, active experts, token groups, M tiles: wave 0, four
+  // consecutive experts per lane, wave-wide prefix sums; every workgroup needs the offsets,
+  // workgroup 0 writes the results out
+  if (wv == 0) {
+    int cc[4], tot = 0, nact = 0, ngrp = 0, nmt = 0;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int ee = lane * 4 + j;
-        cc[j] = ee < E ? cnt[ee] : 0;
-        tot += cc[j];
-        nact += cc[j] > 0;
-        ngrp += (cc[j] + group_tokens - 1) / group_tokens;
-        nmt += (cc[j] + 63) / 64;
+    for (int j = 0; j < 4; ++j) {
+      const int ee = lane * 4 + j;
+      cc[j] = ee < E ? cnt[ee] : 0;
+      tot += cc[j];
+      nact += cc[j] > 0;
+      ngrp += group_count(cc[j], group_tokens);
+      nmt += (cc[j] + 63) / 64;
+    }
+    int s_tot = tot, s_act = nact, s_grp = ngrp, s_mt = nmt;  // inclusive scans over lanes
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t0 = __shfl_up(s_tot, o, 64), t1 = __shfl_up(s_act, o, 64);
+      const int t2 = __shfl_up(s_grp, o, 64), t3 = __shfl_up(s_mt, o, 64);
+      if (lane >= o) {
+        s_tot += t0;
+        s_act += t1;
+        s_grp += t2;
+        s_mt += t3;
       }
-      int s_tot = tot, s_act = nact, s_grp = ngrp, s_mt = nmt;  // inclusive scans over lanes
+    }
+    int run = s_tot - tot, slot = s_act - nact, gi = s_grp - ngrp, mi = s_mt - nmt;
 #pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        const int t0 = __shfl_up(s_tot, o, 64), t1 = __shfl_up(s_act, o, 64);
-        const int t2 = __shfl_up(s_grp, o, 64), t3 = __shfl_up(s_mt, o, 64);
-        if (lane >= o) {
-          s_tot += t0;
-          s_act += t1;
-          s_grp += t2;
-          s_mt += t3;
-        }
-      }
-      int run = s_tot - tot, slot = s_act - nact, gi = s_grp - ngrp, mi = s_mt - nmt;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int ee = lane * 4 + j;
-        if (ee < E) {
-          off_sh[ee] = run;
-          offsets[ee] = run;
-          if (cc[j] > 0) {
+    for (int j = 0; j < 4; ++j) {
+      const int ee = lane * 4 + j;
+      if (ee < E) {
+        off_sh[ee] = run;
+        if (pub) offsets[ee] = run;
+        if (cc[j] > 0) {
+          if (pub) {
             if (vlist) {
               for (int gb = 0; gb < cc[j]; gb += group_tokens) {
                 vlist[2 * gi] = slot;
@@ -574,48 +574,55 @@ __global__ __launch_bounds__(256) void dispatch_scatter_kernel(
               mtiles[2 * mi + 1] = m0;
               ++mi;
             }
-            act_e[slot++] = ee;
           }
-          run += cc[j];
+          act_e[slot++] = ee;
         }
+        run += cc[j];
       }
-      if (lane == 63) {
+    }
+    if (lane == 63) {
+      na_sh = s_act;
+      if (pub) {
         offsets[E] = s_tot;
-        na_sh = s_act;
         *nv = vlist ? s_grp : 0;
         *n_mtiles = s_mt;
       }
     }
-    __syncthreads();
-    if (threadIdx.x < E) {
-      const bool on = (int)threadIdx.x < na_sh;
-      const int e = on ? act_e[threadIdx.x] : 0;
-      write_work_desc(desc + threadIdx.x, on, e, cnt[e], off_sh[e], ew);
+  }
+  // this chunk: lanes of a wave that name the same expert, their rank among themselves
+  const int my_p = chunk0 + tid;
+  const int my_id = my_p < P ? ids[my_p] : -1;
+  unsigned long long same = 0ull, todo = __ballot(my_id >= 0);
+  while (todo != 0ull) {  // the same in every lane
+    const int id0 = __builtin_amdgcn_readlane(my_id, (int)__builtin_ctzll(todo));
+    const unsigned long long m = __ballot(my_id == id0);
+    if (my_id == id0) same = m;
+    todo &= ~m;
+  }
+  const int rank_in_wave = __popcll(same & ((1ull << lane) - 1ull));
+  if (my_id >= 0 && rank_in_wave == 0) wcnt[wv][my_id] = __popcll(same);
+  __syncthreads();
+  if (pub && tid < E) {
+    counts[tid] = cnt[tid];
+    const bool on = tid < na_sh;
+    const int e = on ? act_e[tid] : 0;
+    write_work_desc(desc + tid, on, e, cnt[e], off_sh[e], ew);
+  }
+  if (tid < E) {  // per expert: how many of the chunk's assignments sit in the waves before
+    int run = 0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const int v = wcnt[w][tid];
+      wcnt[w][tid] = run;
+      run += v;
     }
   }
-  // ... then writes them, in order, behind those of the waves before it
-  int base = sh[0] + sh[1] + sh[2] + sh[3];
-  for (int i = 0; i < wv; ++i) base += sh[4 + i];
-  for (int p0 = p_lo; p0 < p_hi; p0 += 64 * 8) {
-    int id[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int p = p0 + 64 * j + lane;
-      id[j] = p < p_hi ? ids[p] : -1;
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int p = p0 + 64 * j + lane;
-      const bool hit = id[j] == e;
-      const unsigned long long m = __ballot(hit);
-      if (hit) {
-        const int pos = base + __popcll(m & ((1ull << lane) - 1ull));
-        list_tok[pos] = p / k;
-        list_w[pos] = pairs[2 * (size_t)p + 1];
-        pos_of_slot[p] = pos;
-      }
-      base += __popcll(m);
-    }
+  __syncthreads();
+  if (my_id >= 0) {
+    const int pos = off_sh[my_id] + before[my_id] + wcnt[wv][my_id] + rank_in_wave;
+    list_tok[pos] = my_p / k;
+    list_w[pos] = pairs[2 * (size_t)my_p + 1];
+    pos_of_slot[my_p] = pos;
   }
 }
 
