@@ -1135,7 +1135,7 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
     mark(CSK_STAGE_PREP);
     mark(CSK_STAGE_ROUTER);
     // a workgroup takes one expert (latency) as long as all of them are resident at once, four beyond
-    if (cdiv(T, 4) * (L->E + 4) <= 5 * std::max(g_cus, 1))  // five of these workgroups fit a compute unit
+    if (cdiv(T, 4) * (L->E + 4) <= 4 * std::max(g_cus, 1) + 64)  // four of these workgroups fit a compute unit
       router_prep_logits_kernel<1><<<dim3((unsigned)(L->E + 4), (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
           hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, ws.xs, L->gate_w,
           L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);

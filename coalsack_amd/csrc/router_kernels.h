@@ -199,8 +199,19 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
     // four columns per thread, the row's loads all in flight at once and kept in registers
     // between the two passes (rows longer than 4096 take further rounds of the same)
     const float4* x4 = reinterpret_cast<const float4*>(hidden + (size_t)t * H);
+    const float4* nw4 = reinterpret_cast<const float4*>(norm_w);
     const int H4p = H >> 2;
     constexpr int kIter = 4;
+    const bool one_round = H4p <= 256 * kIter;  // the row and the norm weights are then read once, up front
+    float4 x0[kIter], w0[kIter];
+    if (one_round) {
+#pragma unroll
+      for (int j = 0; j < kIter; ++j) {
+        const int c = threadIdx.x + 256 * j;
+        x0[j] = c < H4p ? x4[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        w0[j] = (norm_w && c < H4p) ? nw4[c] : make_float4(1.f, 1.f, 1.f, 1.f);
+      }
+    }
     float den = 1.0f;
     if (norm_w) {
       float ss = 0.0f;
@@ -209,7 +220,7 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
 #pragma unroll
         for (int j = 0; j < kIter; ++j) {
           const int c = c0 + threadIdx.x + 256 * j;
-          xv[j] = c < H4p ? x4[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+          xv[j] = one_round ? x0[j] : (c < H4p ? x4[c] : make_float4(0.f, 0.f, 0.f, 0.f));
         }
 #pragma unroll
         for (int j = 0; j < kIter; ++j) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
@@ -220,13 +231,14 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
       ss = (part[0][0] + part[1][0]) + (part[2][0] + part[3][0]);
       den = sqrtf(ss / (float)H + eps);
     }
-    const float4* nw4 = reinterpret_cast<const float4*>(norm_w);
     for (int c0 = 0; c0 < H4p; c0 += 256 * kIter) {
       float4 xv[kIter], wv4[kIter];
 #pragma unroll
       for (int j = 0; j < kIter; ++j) {
         const int c = c0 + threadIdx.x + 256 * j;
-        if (c < H4p) {
+        if (one_round) {
+          xv[j] = x0[j], wv4[j] = w0[j];
+        } else if (c < H4p) {
           xv[j] = x4[c];
           if (norm_w) wv4[j] = nw4[c];
         }
@@ -281,6 +293,27 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
   auto row = [&](int i, int c) -> float4 {
     return reinterpret_cast<const float4*>(hidden + (size_t)(t0 + i) * H)[c];
   };
+  // the norm weights and the first expert's gate row are requested now, beside the token
+  // rows, not after the reductions that need only the rows
+  float4 wq[kMaxIter], gq[2][kMaxIter];
+  auto load_gate = [&](float4(&q)[kMaxIter], int ee) {
+    const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)min(e0 + ee, E - 1) * H);
+#pragma unroll
+    for (int j = 0; j < kMaxIter; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      q[j] = c < H4 ? g4[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
+  if (held) {
+    load_gate(gq[0], 0);
+    if (norm_w) {
+#pragma unroll
+      for (int j = 0; j < kMaxIter; ++j) {
+        const int c = threadIdx.x + 256 * j;
+        wq[j] = c < H4 ? w4[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
+  }
   // 1 / rms per token: the logits only have to be within the close-call tolerance of the
   // reference's (a token inside it is recomputed from the exactly normalised row the
   // prologue workgroups write), so the rows are scaled by a reciprocal here, one
@@ -320,7 +353,7 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
       for (int j = 0; j < kMaxIter; ++j) {
         const int c = threadIdx.x + 256 * j;
         if (c < H4) {
-          const float4 wv4 = w4[c];
+          const float4 wv4 = wq[j];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             if (i < nt) {
@@ -335,16 +368,6 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
     }
   }
   // the gate row of the next expert is requested before the current one is used
-  float4 gq[2][kMaxIter];
-  auto load_gate = [&](float4(&q)[kMaxIter], int ee) {
-    const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)min(e0 + ee, E - 1) * H);
-#pragma unroll
-    for (int j = 0; j < kMaxIter; ++j) {
-      const int c = threadIdx.x + 256 * j;
-      q[j] = c < H4 ? g4[c] : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-  };
-  if (held) load_gate(gq[0], 0);
 #pragma unroll
   for (int ee = 0; ee < EPW; ++ee) {
     const int e = min(e0 + ee, E - 1);  // a workgroup past the last expert repeats it; nothing is stored
