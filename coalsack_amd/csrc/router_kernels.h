@@ -675,23 +675,37 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
   const int t = blockIdx.y;
   const int d = (blockIdx.x * 256 + threadIdx.x) * 4;  // four adjacent columns per thread (H % 32 == 0)
   if (d >= H) return;
+  float4 res = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+  if (residual) res = *reinterpret_cast<const float4*>(residual + (size_t)t * H + d);  // requested first, used last
   float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-  for (int s = 0; s < k; ++s) {
-    const int pos = pos_of_slot[(size_t)t * k + s];
-    if (pos < 0) continue;  // empty expert tensor: skipped (expert_merge_node.h:111-113)
-    const float4 v = *reinterpret_cast<const float4*>(y + (size_t)pos * H + d);
-    if (pre_weighted) {
-      acc.x = acc.x + v.x, acc.y = acc.y + v.y, acc.z = acc.z + v.z, acc.w = acc.w + v.w;
-    } else {
-      const float w = pairs[2 * ((size_t)t * k + s) + 1];
-      const float4 wv = make_float4(w * v.x, w * v.y, w * v.z, w * v.w);
-      acc.x = acc.x + wv.x, acc.y = acc.y + wv.y, acc.z = acc.z + wv.z, acc.w = acc.w + wv.w;
+  // four slots at a time: their positions and weights are requested together, then their
+  // rows, so that a token's k rows cost two memory latencies, not 2 k; the sums stay in
+  // slot order
+  for (int s0 = 0; s0 < k; s0 += 4) {
+    int pos[4];
+    float w[4];
+    float4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int s = min(s0 + j, k - 1);
+      pos[j] = s0 + j < k ? pos_of_slot[(size_t)t * k + s] : -1;
+      w[j] = pre_weighted ? 1.0f : pairs[2 * ((size_t)t * k + s) + 1];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      v[j] = pos[j] >= 0 ? *reinterpret_cast<const float4*>(y + (size_t)pos[j] * H + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (pos[j] < 0) continue;  // empty expert tensor: skipped (expert_merge_node.h:111-113)
+      if (pre_weighted) {
+        acc.x = acc.x + v[j].x, acc.y = acc.y + v[j].y, acc.z = acc.z + v[j].z, acc.w = acc.w + v[j].w;
+      } else {
+        const float4 wv = make_float4(w[j] * v[j].x, w[j] * v[j].y, w[j] * v[j].z, w[j] * v[j].w);
+        acc.x = acc.x + wv.x, acc.y = acc.y + wv.y, acc.z = acc.z + wv.z, acc.w = acc.w + wv.w;
+      }
     }
   }
-  if (residual) {
-    const float4 r = *reinterpret_cast<const float4*>(residual + (size_t)t * H + d);
-    acc.x = r.x + acc.x, acc.y = r.y + acc.y, acc.z = r.z + acc.z, acc.w = r.w + acc.w;
-  }
+  if (residual) acc.x = res.x + acc.x, acc.y = res.y + acc.y, acc.z = res.z + acc.z, acc.w = res.w + acc.w;
   *reinterpret_cast<float4*>(out + (size_t)t * H + d) = acc;
 }
 
