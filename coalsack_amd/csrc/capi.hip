@@ -89,7 +89,7 @@ struct Workspace {
   int* counts = nullptr;    // [E]
   int* offsets = nullptr;   // [E+1]
   WorkDesc* desc = nullptr; // [E] work descriptors of the active experts
-  int* vlist = nullptr;     // [2 * P] token groups of the streaming kernel
+  StreamGroup* groups = nullptr;  // [P] token groups of the streaming kernel
   int* nv = nullptr;        // [1]
   int* list_tok = nullptr;  // [P]
   float* list_w = nullptr;  // [P]
@@ -100,7 +100,7 @@ struct Workspace {
   int* n_tiles = nullptr;
 
   void release() {
-    void* ps[] = {xn, xs, xg, logits, pairs, ids, counts, offsets, desc, vlist, nv,
+    void* ps[] = {xn, xs, xg, logits, pairs, ids, counts, offsets, desc, groups, nv,
                   list_tok, list_w, pos, act, y, tiles, n_tiles};
     for (void* p : ps)
       if (p) (void)hipFree(p);
@@ -133,7 +133,7 @@ struct Workspace {
     WS_ALLOC(counts, (size_t)nE);
     WS_ALLOC(offsets, (size_t)nE + 1);
     WS_ALLOC(desc, (size_t)nE);
-    WS_ALLOC(vlist, 2 * P);
+    WS_ALLOC(groups, P);
     WS_ALLOC(nv, 1);
     WS_ALLOC(list_tok, P);
     WS_ALLOC(list_w, P);
@@ -365,7 +365,7 @@ int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, in
                     const ExpertW* ew, Workspace& ws) {
   dispatch_scatter_kernel<<<dim3((unsigned)cdiv(std::max<int64_t>(P, 1), kDispatchThreads)), kDispatchThreads, 0, g_stream>>>(
       ids, pairs, (int)P, (int)k, (int)E, ws.counts, ew, ws.offsets, ws.desc,
-      P <= kStreamMaxP ? ws.vlist : nullptr, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w,
+      P <= kStreamMaxP ? ws.groups : nullptr, ws.nv, ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w,
       ws.pos, stream_group_tokens(P / std::max<int64_t>(k, 1)));
   return check_launch("dispatch_scatter_kernel");
 }
@@ -374,7 +374,7 @@ int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, in
 // layer is HBM-bound); grouped GEMM otherwise.
 template <int NMAT, int G>
 int launch_stream(ExpertStreamArgs a, int64_t P, Workspace& ws) {
-  a.vlist = ws.vlist;
+  a.groups = ws.groups;
   a.nv = ws.nv;
   // kStreamWgPerCu workgroups per compute unit in steady state; a batch so small that
   // every work unit can have a workgroup of its own (three fit a compute unit) gets that
@@ -1147,7 +1147,7 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
     mark(CSK_STAGE_DISPATCH);
     RouteIn rin{ws.logits, xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, L->ew_dev,
                 (int)T, (int)L->E, (int)L->k, (int)L->H, L->sigmoid, stream_group_tokens(T)};
-    RouteOut rout{ws.pairs, ws.ids, ws.pos, ws.counts, ws.offsets, ws.desc, ws.vlist, ws.nv,
+    RouteOut rout{ws.pairs, ws.ids, ws.pos, ws.counts, ws.offsets, ws.desc, ws.groups, ws.nv,
                   ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w};
     route_small_kernel<<<dim3(1), kRouteSmallThreads, 0, g_stream>>>(rin, rout);
     if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;

@@ -49,6 +49,25 @@ struct WorkDesc {
   ExpertW w;
 };
 
+// One entry per group of tokens of an expert that the streaming kernel contracts in one
+// pass over the expert's weights: everything a workgroup needs to start, in one record,
+// so that its first weight loads wait for two dependent reads (group count, record), not
+// for a chain through the group list and the expert's descriptor.
+struct StreamGroup {
+  ExpertW w;
+  int e;      // expert
+  int left;   // tokens of the expert from this group's first on (the group holds min(G, left))
+  int base;   // packed position of the group's first token
+  int pad;
+};
+
+__device__ __forceinline__ void write_stream_group(StreamGroup* g, const ExpertW* w, int e, int left, int base) {
+  g->w.q_gate = w->q_gate, g->w.s_gate = w->s_gate, g->w.q_up = w->q_up, g->w.s_up = w->s_up;
+  g->w.q_down = w->q_down, g->w.s_down = w->s_down;
+  g->w.b_gate = w->b_gate, g->w.b_up = w->b_up, g->w.b_down = w->b_down;
+  g->e = e, g->left = left, g->base = base, g->pad = 0;
+}
+
 // Pointers read out of device structures are generic to the compiler, which
 // would then use FLAT loads (tracked by both memory counters and therefore
 // always waited for in full).  These casts pin them to global memory.

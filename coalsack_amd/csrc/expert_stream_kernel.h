@@ -24,7 +24,7 @@ namespace csk {
 // unconditional.
 struct ExpertStreamArgs {
   const WorkDesc* desc;
-  const int* vlist;      // [2 * nv]: (expert slot, first token) of each group of G tokens
+  const StreamGroup* groups;  // [nv]: the groups of up to G tokens
   const int* nv;         // number of such groups
   const int* list_row;   // packed position -> row of A; null: row = packed position
   const uint4* A;        // [rows][nblk][8] x 16 B: 32 bf16 hi then 32 bf16 lo per block
@@ -124,16 +124,15 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
   int par = 0;
   for (int v = team; v < nvv; v += teams) {
     const int p_begin = tj, p_end = npair;
-    const WorkDesc* wd = a.desc + a.vlist[2 * v];
-    const int gbase = a.vlist[2 * v + 1];
-    const int gcount = min(G, wd->Te - gbase);
-    const int base = wd->base + gbase;
-    const CSK_GLOBAL u32x4* q0 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_gate : wd->w.q_down)) + n;
-    const CSK_GLOBAL u32x2* s0 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? wd->w.s_gate : wd->w.s_down)) + wv * 64 + lane;
-    const CSK_GLOBAL u32x4* q1 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? wd->w.q_up : wd->w.q_down)) + n;
-    const CSK_GLOBAL u32x2* s1 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? wd->w.s_up : wd->w.s_down)) + wv * 64 + lane;
-    const CSK_GLOBAL float* bp0 = as_global(MODE == 0 ? wd->w.b_gate : wd->w.b_down);
-    const CSK_GLOBAL float* bp1 = as_global(MODE == 0 ? wd->w.b_up : wd->w.b_down);
+    const StreamGroup* gr = a.groups + v;
+    const int gcount = min(G, gr->left);
+    const int base = gr->base;
+    const CSK_GLOBAL u32x4* q0 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? gr->w.q_gate : gr->w.q_down)) + n;
+    const CSK_GLOBAL u32x2* s0 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? gr->w.s_gate : gr->w.s_down)) + wv * 64 + lane;
+    const CSK_GLOBAL u32x4* q1 = as_global(reinterpret_cast<const u32x4*>(MODE == 0 ? gr->w.q_up : gr->w.q_down)) + n;
+    const CSK_GLOBAL u32x2* s1 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? gr->w.s_up : gr->w.s_down)) + wv * 64 + lane;
+    const CSK_GLOBAL float* bp0 = as_global(MODE == 0 ? gr->w.b_gate : gr->w.b_down);
+    const CSK_GLOBAL float* bp1 = as_global(MODE == 0 ? gr->w.b_up : gr->w.b_down);
 
     // activation rows of this token group -> LDS (every wave is past its last
     // read of the previous group: it has crossed that unit's barrier)

@@ -272,7 +272,7 @@ struct RouteOut {
   int* counts;        // [E]
   int* offsets;       // [E + 1]
   WorkDesc* desc;     // [E]
-  int* vlist;         // [2 * groups]
+  StreamGroup* groups;  // [token groups]
   int* nv;
   int* mtiles;        // [2 * M tiles]
   int* n_mtiles;
@@ -467,8 +467,7 @@ __device__ __forceinline__ void route_workgroup(const RouteIn& r, const RouteOut
         o.offsets[e] = run;
         if (c[j] > 0) {
           for (int gb = 0; gb < c[j]; gb += group_tokens) {
-            o.vlist[2 * gi] = slot;
-            o.vlist[2 * gi + 1] = gb;
+            write_stream_group(o.groups + gi, reinterpret_cast<const ExpertW*>(s.ew) + e, e, c[j] - gb, run + gb);
             ++gi;
           }
           for (int m0 = 0; m0 < c[j]; m0 += 64) {

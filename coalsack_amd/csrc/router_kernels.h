@@ -521,7 +521,7 @@ constexpr int kDispatchThreads = 1024;
 __global__ __launch_bounds__(kDispatchThreads) void dispatch_scatter_kernel(
     const int* __restrict__ ids, const float* __restrict__ pairs, int P, int k, int E,
     int* __restrict__ counts, const ExpertW* __restrict__ ew, int* __restrict__ offsets,
-    WorkDesc* __restrict__ desc, int* __restrict__ vlist, int* __restrict__ nv,
+    WorkDesc* __restrict__ desc, StreamGroup* __restrict__ groups, int* __restrict__ nv,
     int* __restrict__ mtiles, int* __restrict__ n_mtiles, int* __restrict__ list_tok,
     float* __restrict__ list_w, int* __restrict__ pos_of_slot, int group_tokens) {
   constexpr int NW = kDispatchThreads / 64;
@@ -585,10 +585,9 @@ __global__ __launch_bounds__(kDispatchThreads) void dispatch_scatter_kernel(
         if (pub) offsets[ee] = run;
         if (cc[j] > 0) {
           if (pub) {
-            if (vlist) {
+            if (groups) {
               for (int gb = 0; gb < cc[j]; gb += group_tokens) {
-                vlist[2 * gi] = slot;
-                vlist[2 * gi + 1] = gb;
+                write_stream_group(groups + gi, ew + ee, ee, cc[j] - gb, run + gb);
                 ++gi;
               }
             }
@@ -607,7 +606,7 @@ __global__ __launch_bounds__(kDispatchThreads) void dispatch_scatter_kernel(
       na_sh = s_act;
       if (pub) {
         offsets[E] = s_tot;
-        *nv = vlist ? s_grp : 0;
+        *nv = groups ? s_grp : 0;
         *n_mtiles = s_mt;
       }
     }
