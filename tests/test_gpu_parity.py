@@ -521,3 +521,12 @@ def test_long_batch_in_passes(lib, oracle):
     assert same.mean() > 0.99
     assert_layer_close(small[same], want[same])
     assert_layer_close(whole[same], want[same])
+
+
+@pytest.mark.parametrize("E,T,norm", [(128, 64, True), (128, 64, False), (200, 40, True), (130, 33, False)])
+def test_layer_many_experts_small_batch(lib, oracle, E, T, norm):
+    """Small batches over many experts: the prologue + logits kernel then gives a workgroup
+    four experts (the one-expert workgroups would not all be resident), with expert counts
+    that are not multiples of four and ragged token tiles."""
+    L = synth.LayerInputs(E, 4, 128, 96, seed=61, with_norm=True)
+    _check_layer(lib, oracle, L, T, norm=norm, residual=norm)
