@@ -530,3 +530,11 @@ def test_layer_many_experts_small_batch(lib, oracle, E, T, norm):
     that are not multiples of four and ragged token tiles."""
     L = synth.LayerInputs(E, 4, 128, 96, seed=61, with_norm=True)
     _check_layer(lib, oracle, L, T, norm=norm, residual=norm)
+
+
+@pytest.mark.parametrize("T", [3, 64, 65, 200])
+def test_layer_maximum_experts_and_top_k(lib, oracle, T):
+    """The limits of a layer: 256 experts, top-16 -- 64 tokens fill the single-workgroup
+    router (1024 assignments), 65 take the multi-workgroup one, 200 the grouped GEMM."""
+    L = synth.LayerInputs(256, 16, 64, 96, seed=71)
+    _check_layer(lib, oracle, L, T)
