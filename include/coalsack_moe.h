@@ -11,6 +11,13 @@
  * pointers come from csk_dev_alloc (or any hipMalloc).  All tensors are
  * row-major and contiguous, as dynamic_tensor is
  * (include/coalsack/tensor/dynamic_tensor.h:114-161).
+ *
+ * Threads: the library owns one GPU stream and one workspace, and serialises
+ * its entry points with a process-wide lock; callers may come from any thread
+ * (the reference drives each layer's nodes from that layer's scheduler thread,
+ * include/coalsack/nn/model_io_nodes.h:224) and need no locking of their
+ * own.  Device-pointer entry points are asynchronous on that stream; the
+ * host-buffer ones return when their results are in place.
  */
 #ifndef COALSACK_MOE_H
 #define COALSACK_MOE_H
