@@ -1241,13 +1241,26 @@ extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T
   REQUIRE_INIT();
   if (!L || !hidden || !out || T < 0) return fail(CSK_ERR_ARG, "csk_moe_forward_host: bad argument");
   if (T == 0) return CSK_OK;
-  float *dh = nullptr, *dout = nullptr;
+  // device copies of the caller's rows: kept between calls (a frame of a decoding engine
+  // comes back every few milliseconds) and grown on demand; the copies in, the kernels and
+  // the copies out are queued on the stream and awaited once
+  static float *dh = nullptr, *dout = nullptr;
+  static size_t cap = 0;
   const size_t n = (size_t)T * L->H;
-  HIP_TRY(hipMalloc((void**)&dh, n * sizeof(float)));
-  hipError_t e = hipMalloc((void**)&dout, n * sizeof(float));
+  if (n > cap) {
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    if (dh) (void)hipFree(dh);
+    if (dout) (void)hipFree(dout);
+    dh = dout = nullptr, cap = 0;
+    HIP_TRY(hipMalloc((void**)&dh, n * sizeof(float)));
+    HIP_TRY(hipMalloc((void**)&dout, n * sizeof(float)));
+    cap = n;
+  }
   int rc = CSK_OK;
-  if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("hipMalloc: ") + hipGetErrorString(e));
-  if (rc == CSK_OK) rc = csk_copy_h2d(dh, hidden, n * sizeof(float));
+  {
+    const hipError_t e = hipMemcpyAsync(dh, hidden, n * sizeof(float), hipMemcpyHostToDevice, g_stream);
+    if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("copy in: ") + hipGetErrorString(e));
+  }
   if (rc == CSK_OK && !pairs_out) rc = csk_moe_forward(L, dh, T, dout, flags);
   if (rc == CSK_OK && pairs_out) {
     // pass by pass, as csk_moe_forward does: the router output lives in the workspace of a pass
@@ -1262,10 +1275,12 @@ extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T
         rc = csk_copy_d2h(pairs_out + t0 * L->k * 2, g_ws.pairs, (size_t)tn * L->k * 2 * sizeof(float));
     }
   }
-  if (rc == CSK_OK) rc = csk_copy_d2h(out, dout, n * sizeof(float));
-  (void)hipStreamSynchronize(g_stream);
-  (void)hipFree(dh);
-  if (dout) (void)hipFree(dout);
+  if (rc == CSK_OK) {
+    const hipError_t e = hipMemcpyAsync(out, dout, n * sizeof(float), hipMemcpyDeviceToHost, g_stream);
+    if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("copy out: ") + hipGetErrorString(e));
+  }
+  const hipError_t es = hipStreamSynchronize(g_stream);
+  if (rc == CSK_OK && es != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("csk_moe_forward_host: ") + hipGetErrorString(es));
   return rc;
 }
 
