@@ -235,35 +235,39 @@ struct csk_layer {
 
 namespace {
 
-int validate_scales(const uint8_t* blocks, int64_t nblocks) {
-  for (int64_t b = 0; b < nblocks; ++b) {
-    const uint8_t s = blocks[b * 17];
-    if (s < 2 || s > 254)
-      return fail(CSK_ERR_SCALE, "MXFP4 scale byte " + std::to_string((int)s) + " at block " +
-                                     std::to_string(b) +
-                                     " is outside 2..254 (denormal / reserved scales unsupported)");
-  }
-  return CSK_OK;
-}
+// Upload `rows x K` reference blocks and repack into (q, s).  The staging buffer is kept
+// between calls (a checkpoint is hundreds of matrices of one size); the scale bytes are
+// checked by the pack kernel as it reads them, so the host touches the blocks only to hand
+// them to the copy.  On a scale outside 2..254 the planes of m hold partial data.
+uint8_t* g_stage = nullptr;
+size_t g_stage_cap = 0;
+unsigned long long* g_bad = nullptr;
 
-// Upload `rows x K` reference blocks and repack into (q, s).
 int pack_into(const uint8_t* host, csk_mxfp4& m) {
   const int64_t nblocks = m.rows * m.nblk;
-  int rc = validate_scales(host, nblocks);
-  if (rc != CSK_OK) return rc;
-  uint8_t* staging = nullptr;
-  HIP_TRY(hipMalloc((void**)&staging, (size_t)nblocks * 17));
-  hipError_t e = hipMemcpyAsync(staging, host, (size_t)nblocks * 17, hipMemcpyHostToDevice, g_stream);
-  if (e == hipSuccess) {
-    const long ent = m.entries();
-    pack_mxfp4_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(
-        staging, m.q, m.s, (int)m.rows, (int)m.nblk, ent);
-    e = hipGetLastError();
+  const size_t bytes = (size_t)nblocks * 17;
+  if (bytes > g_stage_cap) {
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    if (g_stage) (void)hipFree(g_stage);
+    g_stage = nullptr, g_stage_cap = 0;
+    HIP_TRY(hipMalloc((void**)&g_stage, bytes));
+    g_stage_cap = bytes;
   }
-  hipError_t e2 = hipStreamSynchronize(g_stream);
-  (void)hipFree(staging);
-  if (e != hipSuccess) return fail(CSK_ERR_HIP, std::string("pack: ") + hipGetErrorString(e));
-  if (e2 != hipSuccess) return fail(CSK_ERR_HIP, std::string("pack sync: ") + hipGetErrorString(e2));
+  if (!g_bad) HIP_TRY(hipMalloc((void**)&g_bad, sizeof(unsigned long long)));
+  HIP_TRY(hipMemsetAsync(g_bad, 0xFF, sizeof(unsigned long long), g_stream));
+  HIP_TRY(hipMemcpyAsync(g_stage, host, bytes, hipMemcpyHostToDevice, g_stream));
+  const long ent = m.entries();
+  pack_mxfp4_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(
+      g_stage, m.q, m.s, (int)m.rows, (int)m.nblk, ent, g_bad);
+  int rc = check_launch("pack_mxfp4_kernel");
+  if (rc != CSK_OK) return rc;
+  unsigned long long bad = 0;
+  HIP_TRY(hipMemcpyAsync(&bad, g_bad, sizeof bad, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  if (bad != ~0ull)
+    return fail(CSK_ERR_SCALE, "MXFP4 scale byte " + std::to_string((int)host[bad * 17]) + " at block " +
+                                   std::to_string(bad) +
+                                   " is outside 2..254 (denormal / reserved scales unsupported)");
   return CSK_OK;
 }
 
@@ -880,6 +884,7 @@ extern "C" int csk_layer_set_expert(csk_layer* L, int64_t e, const uint8_t* w_up
   if (w_up) {
     const uint8_t* src[3] = {w_up, w_gate, w_down};
     const int which[3] = {CSK_W_UP, CSK_W_GATE, CSK_W_DOWN};
+    L->expert_set[(size_t)e] = 0;  // a refused matrix (scale byte out of range) leaves the expert unset
     for (int i = 0; i < 3; ++i) {
       csk_mxfp4 m = L->view(e, which[i]);
       int rc = pack_into(src[i], m);

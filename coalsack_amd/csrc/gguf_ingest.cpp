@@ -13,6 +13,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
+#include <sys/mman.h>
 
 #include <string>
 #include <unordered_map>
@@ -62,6 +63,8 @@ struct Value {
 
 struct csk_gguf {
   FILE* fp = nullptr;
+  const uint8_t* map = nullptr;  // the file mapped read-only (tensor data is handed to the GPU copies from here); null: fread
+  size_t map_len = 0;
   uint32_t version = 0;
   uint64_t data_start = 0, file_size = 0;
   std::unordered_map<std::string, Value> meta;
@@ -150,6 +153,20 @@ bool read_at(csk_gguf* g, uint64_t off, void* dst, size_t n) {
   return rd(g->fp, dst, n);
 }
 
+// n bytes of the file at off without a copy: a pointer into the read-only mapping (made at
+// the first call), or, where the file cannot be mapped, into `fallback` filled by fread.
+const uint8_t* view_at(csk_gguf* g, uint64_t off, size_t n, std::vector<uint8_t>& fallback) {
+  if (off + n > g->file_size) return nullptr;
+  if (!g->map && g->map_len == 0) {
+    void* m = mmap(nullptr, (size_t)g->file_size, PROT_READ, MAP_PRIVATE, fileno(g->fp), 0);
+    g->map_len = (size_t)g->file_size;  // also marks the attempt
+    if (m != MAP_FAILED) g->map = static_cast<const uint8_t*>(m);
+  }
+  if (g->map) return g->map + off;
+  fallback.resize(n);
+  return read_at(g, off, fallback.data(), n) ? fallback.data() : nullptr;
+}
+
 }  // namespace
 
 extern "C" int csk_gguf_open(const char* path, csk_gguf** out) {
@@ -214,6 +231,7 @@ extern "C" int csk_gguf_open(const char* path, csk_gguf** out) {
 
 extern "C" void csk_gguf_close(csk_gguf* g) {
   if (!g) return;
+  if (g->map) munmap(const_cast<uint8_t*>(g->map), g->map_len);
   if (g->fp) fclose(g->fp);
   delete g;
 }
@@ -365,16 +383,15 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
       if (tw[i]->type == kGgmlQ4K || tw[i]->type == kGgmlQ6K)
         return bail(CSK_ERR_ARG, p + wn[i] + ": a K-quant expert slice must be a multiple of 256 values");
   const size_t bl[3] = {(size_t)F, (size_t)F, (size_t)H};
-  std::vector<uint8_t> w[3];
+  std::vector<uint8_t> w[3];  // used only where the file cannot be mapped
   std::vector<float> b[3];
-  for (int i = 0; i < 3; ++i) {
-    w[i].resize(sl[i]);
+  for (int i = 0; i < 3; ++i)
     if (tb[i]) b[i].resize(bl[i]);
-  }
   for (uint32_t e = 0; e < E; ++e) {
+    const uint8_t* wp[3];
     for (int i = 0; i < 3; ++i) {
-      if (!read_at(g, tw[i]->offset + (uint64_t)e * sl[i], w[i].data(), sl[i]))
-        return bail(CSK_ERR_ARG, "short read: " + p + wn[i]);
+      wp[i] = view_at(g, tw[i]->offset + (uint64_t)e * sl[i], sl[i], w[i]);
+      if (!wp[i]) return bail(CSK_ERR_ARG, "short read: " + p + wn[i]);
       if (tb[i] && !read_at(g, tb[i]->offset + (uint64_t)e * bl[i] * 4, b[i].data(), bl[i] * 4))
         return bail(CSK_ERR_ARG, "short read: " + p + bn[i]);
     }
@@ -383,10 +400,10 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
     if (f16) {
       const int which[3] = {CSK_W_UP, CSK_W_GATE, CSK_W_DOWN};
       for (int i = 0; i < 3 && rc == CSK_OK; ++i)
-        rc = csk_layer_set_expert_matrix(L, e, which[i], (int)tw[i]->type, w[i].data());
+        rc = csk_layer_set_expert_matrix(L, e, which[i], (int)tw[i]->type, wp[i]);
       if (rc == CSK_OK) rc = csk_layer_set_expert_f16(L, e, nullptr, nullptr, nullptr, bp[0], bp[1], bp[2]);
     } else {
-      rc = csk_layer_set_expert(L, e, w[0].data(), w[1].data(), w[2].data(), bp[0], bp[1], bp[2]);
+      rc = csk_layer_set_expert(L, e, wp[0], wp[1], wp[2], bp[0], bp[1], bp[2]);
     }
     if (rc != CSK_OK) return bail(rc, "");
   }

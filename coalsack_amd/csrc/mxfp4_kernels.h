@@ -48,8 +48,11 @@ __device__ __forceinline__ void entry_to_ref_block(uint4 q, uint8_t scale, uint8
 }
 
 // entries = ntile * nblk * 16
+// `bad` receives the lowest index of a block whose scale byte is outside 2..254 (the
+// conversion instruction is exact only inside that range); it must hold ~0 on entry.
 __global__ void pack_mxfp4_kernel(const uint8_t* __restrict__ src, uint4* __restrict__ q,
-                                  uint8_t* __restrict__ s, int rows, int nblk, long entries) {
+                                  uint8_t* __restrict__ s, int rows, int nblk, long entries,
+                                  unsigned long long* __restrict__ bad) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= entries) return;
   const int n = (int)(i & 15);
@@ -66,6 +69,7 @@ __global__ void pack_mxfp4_kernel(const uint8_t* __restrict__ src, uint4* __rest
   const uint8_t* blk = src + (row * nblk + kb) * 17;
   q[i] = ref_block_to_entry(blk);
   s[si] = blk[0];
+  if (bad && (blk[0] < 2 || blk[0] > 254)) atomicMin(bad, (unsigned long long)(row * nblk + kb));
 }
 
 __global__ void export_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t* __restrict__ s,
