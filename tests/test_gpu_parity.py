@@ -354,6 +354,10 @@ def test_layer_few_tokens_long_rows(lib, oracle):
     _check_layer(lib, oracle, L, 6, norm=True, residual=True)
     L = synth.LayerInputs(4, 2, 64, 3200, seed=24)
     _check_layer(lib, oracle, L, 5)
+    # rows longer than 4096: the prologue + logits kernel reads them in several rounds instead of holding them
+    L = synth.LayerInputs(6, 2, 4608, 64, seed=25, with_norm=True)
+    _check_layer(lib, oracle, L, 3, norm=True, residual=True)
+    _check_layer(lib, oracle, L, 7)
 
 
 def test_layer_many_tokens_per_expert(lib, oracle):
