@@ -7,14 +7,21 @@ on one MI355X through the C ABI.
 Prints ONE JSON line.  A step is one forward of the layer over one batch of T
 synthetic tokens with weights, input and output resident in HBM.  `value` is
 tokens/s of the whole layer; `roofline` describes the dominant kernel (gate/up
-projections), timed live with HIP events on the library's stream;
-`cpu_baseline` is the CPU checker (a restatement of the reference's
-single-threaded path) timed on this host on a bounded sample.
+projections), timed live by a start and a stop event attached to its dispatch on
+the library's stream (the kernel's own begin-to-end time, as a kernel trace
+reports it); `cpu_baseline` is the CPU checker (a restatement of the
+reference's single-threaded path) timed on this host on a bounded sample.
+
+The default line is the 120b-shaped layer (128 experts, 8 hot) at 16 tokens and
+carries, under `legs`, the same layer at 1 and at 4096 tokens and the 36-layer
+stack at 1, 8 and 64 tokens, each with its own `roofline` and `cpu_baseline`.
+Decode batches rotate over 8 layer instances x 8 token batches, so that no weight
+byte is touched again before more than the 256 MB last-level cache has streamed by.
 
 Workloads (BASELINE.json configs):
-  c2_20b_decode   32 experts, top-4, H = F = 2880, T in {1,2,4,8,16,32,64} (default, T=16)
+  c4_120b         128 experts, 8 hot experts (+2.0 router bias), T in {1,16,4096} (default, T=16)
+  c2_20b_decode   32 experts, top-4, H = F = 2880, T in {1,2,4,8,16,32,64}
   c3_20b_prefill  same layer, T = 2048
-  c4_120b         128 experts, 8 hot experts (+2.0 router bias), T in {1,16,4096}
   c5_stack        36 layers of the 120b shape with RMSNorm + residual, T in {1,8,64}
 Neighbouring paths (not the headline):
   gguf_ingest     one 20b-shaped block from a GGUF file into a resident layer
@@ -67,6 +74,12 @@ def gateup_bytes(H, F, T, k, U, f16=False):
     """Algorithmic bytes of the gate/up kernel: both matrices and biases of every
     distinct expert once, the fp32 activations in, the fp32 activations out."""
     return U * (2 * matrix_bytes(F, H, f16) + 2 * F * 4) + T * H * 4 + T * k * F * 4
+
+
+def down_bytes(H, F, T, k, U, f16=False):
+    """Algorithmic bytes of the down kernel: the matrix and bias of every distinct expert
+    once, the activations in, one fp32 row per assignment out."""
+    return U * (matrix_bytes(H, F, f16) + H * 4) + T * k * (F + H) * 4
 
 
 def layer_flops(E, k, H, F, T):
@@ -133,15 +146,18 @@ def time_forward(lib, fn, steps, warmup):
     return ms / steps
 
 
-def stage_profile(lib, fn, steps):
-    lib.stage_timing(True)
-    acc = {}
-    for _ in range(steps):
-        fn()
-        for kk, v in lib.stage_times().items():
-            acc[kk] = acc.get(kk, 0.0) + v
-    lib.stage_timing(False)
-    return {kk: v / steps for kk, v in acc.items()}
+def event_pair_overhead_ms(lib, reps=101):
+    """What two consecutive event records with nothing between them read: the part of a
+    `stage_ms` figure that is not the kernel."""
+    vals = []
+    for _ in range(reps):
+        e0, e1 = lib.event(), lib.event()
+        lib.record(e0)
+        lib.record(e1)
+        vals.append(lib.elapsed_ms(e0, e1))
+        lib.dll.csk_event_destroy(e0)
+        lib.dll.csk_event_destroy(e1)
+    return float(np.median(vals))
 
 
 def close_calls(L, hidden, k):
@@ -154,68 +170,148 @@ def close_calls(L, hidden, k):
     return int(np.count_nonzero(gaps.min(axis=1) <= 8 * 5.96e-8 * np.sqrt(hidden.shape[1])))
 
 
-def bench_layer(lib, synth, shape, T, steps, warmup, seed=1234):
-    """Times the forward over `nb` different token batches in rotation (decode sizes: the
-    set of selected experts, and with it the bytes streamed, varies from batch to batch)."""
-    L, layer = make_layer(lib, synth, shape, seed)
-    nb = 8 if T < 512 else 1
+def bench_layer(lib, synth, shape, T, steps, warmup, seed=1234, layers=None):
+    """Times exactly `steps` forwards.  Decode sizes rotate over nl layer instances x nb token
+    batches (layer index fastest): the experts selected, and with them the bytes streamed,
+    change from step to step, and a (layer, expert) pair comes back only after the other
+    layers' traffic -- far more than the last-level cache holds -- has passed.
+    `layers`: resident (LayerInputs, Layer) pairs to use instead of building new ones."""
+    decode = T < 512
+    nl, nb = (8, 8) if decode else (1, 1)
+    own = layers is None
+    if own:
+        layers = [make_layer(lib, synth, shape, seed, layer_index=i) for i in range(nl)]
+    layers = layers[:nl]
+    nl = len(layers)
+    L = layers[0][0]
+    f16 = bool(shape.get("f16"))
     hiddens = [synth.hidden_states(T, L.H, seed=T + 1000 * i) for i in range(nb)]
     d_ins = [lib.to_device(h) for h in hiddens]
     d_out = lib.dev_alloc(hiddens[0].nbytes)
+    ncombo = nl * nb
     turn = [0]
 
+    def combo(i):
+        return i % nl, (i // nl) % nb
+
     def fn():
-        layer.forward_device(d_ins[turn[0] % nb], T, d_out)
+        li, bi = combo(turn[0])
+        layers[li][1].forward_device(d_ins[bi], T, d_out)
         turn[0] += 1
-    steps = (steps + nb - 1) // nb * nb
-    ms = time_forward(lib, fn, steps, (warmup + nb - 1) // nb * nb)
-    stages = stage_profile(lib, fn, (max(5, min(steps, 50)) + nb - 1) // nb * nb)
-    Us, tmax = [], 0
-    for i in range(nb - 1, -1, -1):  # batch 0 last: its output is the one checked
-        layer.forward_device(d_ins[i], T, d_out)
+    ms = time_forward(lib, fn, steps, warmup)
+    timed_combos = [combo(i) for i in range(warmup, warmup + steps)]
+
+    # distinct experts of every combination (untimed)
+    U, tmax = {}, 0
+    for c in sorted(set(timed_combos) | {combo(i) for i in range(ncombo)}):
+        layers[c[0]][1].forward_device(d_ins[c[1]], T, d_out)
         if T <= 32768:
-            counts, _ = layer.last_dispatch(T)
-            Us.append(int(np.count_nonzero(counts)))
+            counts, _ = layers[c[0]][1].last_dispatch(T)
+            U[c] = int(np.count_nonzero(counts))
             tmax = max(tmax, int(counts.max()))
         else:  # taken in several passes: no single dispatch to read back; every expert is in use
-            Us.append(shape["E"])
-    U = float(np.mean(Us))
+            U[c] = shape["E"]
+
+    # per-stage and per-kernel times, every combination the same number of times
+    rounds = max(1, min(6, 200 // ncombo))
+    lib.stage_timing(True)
+    stage_acc, kern_acc, have_kern, gu_bytes, dn_bytes = {}, [0.0, 0.0], not f16, 0, 0
+    turn[0] = 0
+    for _ in range(rounds * ncombo):
+        c = combo(turn[0])
+        fn()
+        for kk, v in lib.stage_times().items():
+            stage_acc[kk] = stage_acc.get(kk, 0.0) + v
+        if have_kern:
+            g, d = lib.kernel_times()
+            kern_acc[0] += g
+            kern_acc[1] += d
+        gu_bytes += gateup_bytes(L.H, L.F, T, L.k, U[c], f16)
+        dn_bytes += down_bytes(L.H, L.F, T, L.k, U[c], f16)
+    lib.stage_timing(False)
+    n_prof = rounds * ncombo
+    stages = {kk: v / n_prof for kk, v in stage_acc.items()}
+    kernels = dict(gateup=kern_acc[0] / n_prof, down=kern_acc[1] / n_prof) if have_kern else None
+
+    # combination (0, 0) last: its output is the one checked against the CPU path
+    layers[0][1].forward_device(d_ins[0], T, d_out)
     hidden = hiddens[0]
     out = lib.to_host(d_out, (T, L.H))
-    f16 = bool(shape.get("f16"))
     L.f16_weights = None
     if f16:
         # the CPU leg needs the generated halves of the experts its token sample selects
         from coalsack_amd import capi
         ns = min(T, 2)
-        _, pairs = layer.forward(hidden[:ns], want_pairs=True)
-        L.f16_weights = {int(e): [layer.export_f16(int(e), w) for w in (capi.W_UP, capi.W_GATE, capi.W_DOWN)]
+        _, pairs = layers[0][1].forward(hidden[:ns], want_pairs=True)
+        L.f16_weights = {int(e): [layers[0][1].export_f16(int(e), w) for w in (capi.W_UP, capi.W_GATE, capi.W_DOWN)]
                          for e in sorted(set(pairs[..., 0].astype(int).ravel().tolist()))}
         L.f16_sample = ns
     for d in d_ins:
         lib.dev_free(d)
     lib.dev_free(d_out)
-    layer.close()
-    res = dict(T=T, ms_per_step=ms, tokens_per_s=T / (ms * 1e-3), distinct_experts=U,
-               stage_ms=stages, finite=bool(np.all(np.isfinite(out))),
-               max_tokens_per_expert=tmax, batches=nb, steps=steps,
-               close_call_tokens=sum(close_calls(L, h, L.k) for h in hiddens))
-    res["layer_bytes"] = layer_bytes(L.E, L.k, L.H, L.F, T, U, f16)
+    if own:
+        for _, layer in layers:
+            layer.close()
+    U_timed = float(np.mean([U[c] for c in timed_combos]))
+    res = dict(T=T, ms_per_step=ms, tokens_per_s=T / (ms * 1e-3), distinct_experts=U_timed,
+               stage_ms=stages, kernel_ms=kernels, finite=bool(np.all(np.isfinite(out))),
+               max_tokens_per_expert=tmax, batches=nb, layer_instances=nl, steps=steps,
+               close_call_tokens=sum(close_calls(layers[0][0], h, L.k) for h in hiddens))
+    res["layer_bytes"] = float(np.mean([layer_bytes(L.E, L.k, L.H, L.F, T, U[c], f16) for c in timed_combos]))
     res["layer_hbm_frac"] = res["layer_bytes"] / (ms * 1e-3) / (HBM_PEAK_GBS * 1e9)
     res["layer_flops"] = layer_flops(L.E, L.k, L.H, L.F, T)
     res["layer_fp4_frac"] = res["layer_flops"] / (ms * 1e-3) / (MFMA_FP4_PEAK_TFLOPS * 1e12)
-    gu = gateup_bytes(L.H, L.F, T, L.k, U, f16)
-    res["gateup_bytes"] = gu
-    res["gateup_gbs"] = gu / (stages["gateup"] * 1e-3) / 1e9
+    res["gateup_bytes"] = gu_bytes / n_prof
+    res["down_bytes"] = dn_bytes / n_prof
+    res["gateup_ms"] = kernels["gateup"] if kernels else stages["gateup"]
+    res["gateup_gbs"] = res["gateup_bytes"] / (res["gateup_ms"] * 1e-3) / 1e9
     return res, (L, hidden, out)
 
 
-def bench_stack(lib, synth, shape, T, steps, warmup, n_layers, seed=1234):
-    layers = []
-    for i in range(n_layers):
-        _, layer = make_layer(lib, synth, shape, seed, layer_index=i, norm=True)
-        layers.append(layer)
-    from coalsack_amd.capi import stack_forward
+def layer_roofline(res, shape, T, workload):
+    """`roofline` object of a layer measurement: its gate/up kernel."""
+    prefill = T >= 512
+    f16 = bool(shape.get("f16"))
+    fl = T * shape["k"] * 4 * shape["H"] * shape["F"]  # gate + up flops
+    clock = ("start/stop events on the kernel's dispatch (begin-to-end, as a kernel trace reports it)"
+             if res["kernel_ms"] else "events recorded around the launch")
+    if prefill:
+        roof = dict(bound="mfma",
+                    kernel=("expert_f16_gemm_kernel<0>" if f16 else "expert_gemm_mx_kernel<0>") + " (gate/up + SwiGLU)",
+                    achieved=fl / (res["gateup_ms"] * 1e-3) / 1e12,
+                    peak=MFMA_F16_PEAK_TFLOPS if f16 else MFMA_FP4_PEAK_TFLOPS, unit="TFLOP/s", traffic=None,
+                    algorithmic_flops=fl)
+    else:
+        roof = dict(bound="hbm",
+                    kernel=("expert_f16_kernel<0>" if f16 else "expert_stream_kernel<0,*>") + " (gate/up + SwiGLU)",
+                    achieved=res["gateup_gbs"], peak=HBM_PEAK_GBS, unit="GB/s", traffic=None,
+                    algorithmic_bytes=res["gateup_bytes"])
+    # HBM traffic of that kernel from a recorded counter run of this workload, where there is one
+    try:
+        rec = json.load(open(os.path.join(ROOT, "profiles", "traffic.json"))).get(f"{workload}:T={T}")
+    except (OSError, ValueError):
+        rec = None
+    if rec:
+        roof["traffic"] = rec["bytes"]
+        roof["traffic_source"] = rec["source"] + " (a recorded counter run, not measured in this run)"
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["kernel_ms"] = res["gateup_ms"]
+    roof["kernel_clock"] = clock
+    if res["kernel_ms"]:
+        roof["down_kernel_ms"] = res["kernel_ms"]["down"]
+        if prefill:
+            roof["down_achieved"] = fl / 2 / (res["kernel_ms"]["down"] * 1e-3) / 1e12
+        else:
+            roof["down_algorithmic_bytes"] = res["down_bytes"]
+            roof["down_achieved"] = res["down_bytes"] / (res["kernel_ms"]["down"] * 1e-3) / 1e9
+        roof["down_frac"] = roof["down_achieved"] / roof["peak"]
+    return roof
+
+
+def bench_stack(lib, synth, shape, T, steps, warmup, layers):
+    """36 resident layers, h <- h + MoE(RMSNorm(h)) each; `layers` = (LayerInputs, Layer) pairs."""
+    from coalsack_amd.capi import stack_forward, FWD_RMSNORM, FWD_RESIDUAL
+    handles = [layer for _, layer in layers]
     hidden = synth.hidden_states(T, shape["H"], seed=T)
     d_h = lib.to_device(hidden)
     d_h0 = lib.to_device(hidden)
@@ -223,26 +319,46 @@ def bench_stack(lib, synth, shape, T, steps, warmup, n_layers, seed=1234):
     def fn():
         # the stack updates the hidden states in place; start every step from the same N(0,1) input
         lib.copy_d2d(d_h, d_h0, hidden.nbytes)
-        stack_forward(lib, layers, d_h, T)
+        stack_forward(lib, handles, d_h, T)
     ms = time_forward(lib, fn, steps, warmup)
     out = lib.to_host(d_h, hidden.shape)
-    # untimed pass, layer by layer, to count the distinct experts each layer streams
-    from coalsack_amd.capi import FWD_RMSNORM, FWD_RESIDUAL
+    # untimed pass, layer by layer: distinct experts each layer streams, and the kernels' own times
     lib.copy_d2d(d_h, d_h0, hidden.nbytes)
-    total_bytes, distinct = 0, []
-    for layer in layers:
+    lib.stage_timing(True)
+    total_bytes, distinct, gu_bytes, gu_ms, dn_ms, side_ms = 0, [], 0, 0.0, 0.0, 0.0
+    first_out = None
+    for layer in handles:
         layer.forward_device(d_h, T, d_h, FWD_RMSNORM | FWD_RESIDUAL)
+        if first_out is None:
+            first_out = lib.to_host(d_h, hidden.shape)
+        st = lib.stage_times()
+        g, d = lib.kernel_times()
         counts, _ = layer.last_dispatch(T)
         U = int(np.count_nonzero(counts))
         distinct.append(U)
         total_bytes += layer_bytes(shape["E"], shape["k"], shape["H"], shape["F"], T, U) + shape["H"] * 4
+        gu_bytes += gateup_bytes(shape["H"], shape["F"], T, shape["k"], U)
+        gu_ms += g
+        dn_ms += d
+        side_ms += st["prep"] + st["router"] + st["dispatch"] + st["combine"]
+    lib.stage_timing(False)
     lib.dev_free(d_h)
     lib.dev_free(d_h0)
-    for layer in layers:
-        layer.close()
-    return dict(T=T, layers=n_layers, ms_per_step=ms, tokens_per_s=T / (ms * 1e-3),
+    return dict(T=T, layers=len(handles), ms_per_step=ms, tokens_per_s=T / (ms * 1e-3),
                 finite=bool(np.all(np.isfinite(out))), stack_bytes=total_bytes,
-                distinct_experts_per_layer=distinct)
+                distinct_experts_per_layer=distinct, gateup_bytes=gu_bytes, gateup_ms=gu_ms, down_ms=dn_ms,
+                side_stage_ms=side_ms, hidden=hidden, first_layer_out=first_out)
+
+
+def stack_roofline(res):
+    frac = res["stack_bytes"] / (res["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+    return dict(bound="hbm", kernel="whole stack (all kernels of 36 layers)",
+                achieved=frac * HBM_PEAK_GBS, peak=HBM_PEAK_GBS, unit="GB/s", traffic=None, frac=frac,
+                algorithmic_bytes=res["stack_bytes"],
+                gateup_kernels=dict(ms=res["gateup_ms"], algorithmic_bytes=res["gateup_bytes"],
+                                    frac=res["gateup_bytes"] / (res["gateup_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                    clock="start/stop events on each dispatch, summed over the 36 layers"),
+                down_kernels_ms=res["down_ms"], side_stages_ms_with_event_overhead=res["side_stage_ms"])
 
 
 def measured_copy_gbs(lib, nbytes=256 << 20, reps=10):
@@ -264,14 +380,17 @@ def measured_copy_gbs(lib, nbytes=256 << 20, reps=10):
     return 2 * nbytes * reps / (ms * 1e-3) / 1e9
 
 
-def cpu_baseline(L, hidden, gpu_out, budget_s=12.0):
+def cpu_baseline(L, hidden, gpu_out, budget_s=12.0, stack_layers=0):
     """Times the CPU checker (single thread, as the reference's layer runs) on
     the same layer and tokens; repeats the forward until about budget_s of CPU
-    work.  Host weights are replayed only for the experts the batch selects."""
+    work.  Host weights are replayed only for the experts the batch selects.
+    stack_layers > 0: the layer is the first of a stack of that many (RMSNorm in front,
+    residual add behind); the stack's rate is the layer's divided by the number of layers."""
     from oracle.binding import Oracle
     orc = Oracle()
     T = hidden.shape[0]
-    pairs = orc.router(hidden, L.gate_w, L.gate_b, L.k)
+    stack = stack_layers > 0
+    pairs = orc.router(orc.rmsnorm(hidden, L.norm_w, 1e-5) if stack else hidden, L.gate_w, L.gate_b, L.k)
     used = sorted(set(pairs[..., 0].astype(int).ravel().tolist()))
     per_gu, per_d = L.F * (L.H // 32) * 17, L.H * (L.F // 32) * 17
     wu = np.zeros(L.E * per_gu, np.uint8)
@@ -282,17 +401,20 @@ def cpu_baseline(L, hidden, gpu_out, budget_s=12.0):
         wg[e * per_gu:(e + 1) * per_gu] = L.blocks(e, 1)
         wd[e * per_d:(e + 1) * per_d] = L.blocks(e, 2)
     args = (hidden, L.E, L.k, L.H, L.F, L.gate_w, L.gate_b, wu, wg, wd, L.b_up, L.b_gate, L.b_down)
+    kw = dict(norm_w=L.norm_w, norm_eps=1e-5, residual=True) if stack else {}
+    _moe = orc.moe_layer
+    orc_moe_layer = lambda *a, **k2: _moe(*a, **kw, **k2)  # noqa: E731
     # bounded sample: at most Tm tokens of the batch, repeated
     t0 = time.perf_counter()
     Tm = min(T, 4)
-    ref, _ = orc.moe_layer(*args, max_tokens=Tm)
+    ref, _ = orc_moe_layer(*args, max_tokens=Tm)
     first = time.perf_counter() - t0
     per_tok = first / Tm
     Tm = int(max(1, min(T, budget_s / max(per_tok, 1e-6))))
     reps = int(max(1, min(50, budget_s / (per_tok * Tm))))
     t0 = time.perf_counter()
     for _ in range(reps):
-        ref, _ = orc.moe_layer(*args, max_tokens=Tm)
+        ref, _ = orc_moe_layer(*args, max_tokens=Tm)
     dt = time.perf_counter() - t0
     err = float(np.max(np.abs(gpu_out[:Tm] - ref[:Tm])) / max(1e-6, np.max(np.abs(ref[:Tm]))))
     # not reference behaviour (its layer runs on one thread): the same work farmed over the
@@ -308,7 +430,7 @@ def cpu_baseline(L, hidden, gpu_out, budget_s=12.0):
 
         def work(h):
             for _ in range(rounds):
-                orc.moe_layer(h, *args[1:], max_tokens=h.shape[0])
+                orc_moe_layer(h, *args[1:], max_tokens=h.shape[0])
         threads = [threading.Thread(target=work, args=(h,)) for h in slices]
         t0 = time.perf_counter()
         for th in threads:
@@ -316,12 +438,14 @@ def cpu_baseline(L, hidden, gpu_out, budget_s=12.0):
         for th in threads:
             th.join()
         dt_all = time.perf_counter() - t0
-        all_cores = dict(value=per * ncores * rounds / dt_all, unit="tokens/s", cores=ncores,
+        all_cores = dict(value=per * ncores * rounds / dt_all / max(1, stack_layers), unit="tokens/s", cores=ncores,
                          sample=f"{ncores} threads x {per} tokens x {rounds} rounds, {dt_all:.1f} s; "
                                 f"not reference behaviour")
-    return dict(value=Tm * reps / dt, unit="tokens/s", cores=1, kind="port", all_cores=all_cores,
+    return dict(value=Tm * reps / dt / max(1, stack_layers), unit="tokens/s", cores=1, kind="port", all_cores=all_cores,
                 sample=f"first {Tm} of {T} tokens x {reps} repeats, {dt:.1f} s on one host core "
-                       f"(CPU cost is linear in tokens x top_k)",
+                       f"(CPU cost is linear in tokens x top_k)"
+                       + (f"; first layer of the stack (RMSNorm + MoE + residual), rate divided by {stack_layers} "
+                          f"layers of identical shape" if stack else ""),
                 gpu_vs_cpu_max_rel_err=err)
 
 
@@ -353,15 +477,42 @@ def cpu_baseline_f16(L, hidden, gpu_out, budget_s=12.0):
                 gpu_vs_cpu_max_rel_err=err)
 
 
+def layer_leg(lib, synth, shape, workload, T, steps, warmup, layers, cpu, budget_s):
+    """One measured (workload, T) of a single layer as a JSON-able object."""
+    res, (L, hidden, out) = bench_layer(lib, synth, shape, T, steps, warmup, layers=layers)
+    leg = dict(workload=f"{workload} T={T}", tokens=T, value=res["tokens_per_s"], unit="tokens/s",
+               ms_per_step=res["ms_per_step"], steps=res["steps"], distinct_experts=res["distinct_experts"],
+               close_call_tokens=res["close_call_tokens"],
+               roofline=layer_roofline(res, shape, T, workload),
+               layer=dict(hbm_frac=res["layer_hbm_frac"], fp4_mfma_frac=res["layer_fp4_frac"],
+                          algorithmic_bytes=res["layer_bytes"], algorithmic_flops=res["layer_flops"],
+                          stage_ms={kk: round(v, 5) for kk, v in res["stage_ms"].items()},
+                          finite=res["finite"]),
+               cpu_baseline=cpu_baseline(L, hidden, out, budget_s) if cpu else None)
+    return leg, res, (L, hidden, out)
+
+
+def stack_leg(lib, synth, shape, T, steps, warmup, layers, cpu, budget_s):
+    res = bench_stack(lib, synth, shape, T, steps, warmup, layers)
+    return dict(workload=f"c5_stack: {len(layers)} x 120b-shaped MoE layer (RMSNorm + residual) T={T}", tokens=T,
+                value=res["tokens_per_s"], unit="tokens/s", ms_per_step=res["ms_per_step"], steps=steps,
+                distinct_experts_per_layer=res["distinct_experts_per_layer"], finite=res["finite"],
+                roofline=stack_roofline(res),
+                cpu_baseline=(cpu_baseline(layers[0][0], res["hidden"], res["first_layer_out"], budget_s,
+                                           stack_layers=len(layers)) if cpu else None))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2_20b_decode", choices=sorted(SHAPES))
+    ap.add_argument("--workload", default="c4_120b", choices=sorted(SHAPES))
     ap.add_argument("--tokens", type=int, default=0)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-sweep", action="store_true", help="only the headline batch size")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-sweep", action="store_true", help="only the headline batch size (no sweep)")
+    ap.add_argument("--no-legs", action="store_true",
+                    help="c4_120b: only the headline measurement, none of the other north-star legs")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run the 256 MiB copy kernel 10 times (known traffic, for profiler byte counters)")
     a = ap.parse_args()
@@ -388,24 +539,6 @@ def main():
         print(json.dumps(line))
         return
 
-    if a.workload == "c5_stack":
-        res = bench_stack(lib, synth, shape, T, a.steps, a.warmup, shape["layers"])
-        line = dict(metric="MoE stack tokens/s", value=res["tokens_per_s"], unit="tokens/s", n_gpus=1,
-                    steps=a.steps, warmup=a.warmup, ms_per_step=res["ms_per_step"],
-                    higher_is_better=True, scaling="weak", vs_baseline=None, dtype="mxfp4 x bf16(2-term) -> f32",
-                    data="synthetic",
-                    config=dict(workload=f"c5_stack: 36 x 120b-shaped MoE layer (RMSNorm + residual), T={T}",
-                                tokens=T, device=dev_name,
-                                distinct_experts_per_layer=res["distinct_experts_per_layer"]),
-                    roofline=dict(bound="hbm", kernel="whole stack (all kernels of 36 layers)",
-                                  achieved=res["stack_bytes"] / (res["ms_per_step"] * 1e-3) / 1e9,
-                                  peak=HBM_PEAK_GBS, unit="GB/s", traffic=None,
-                                  frac=res["stack_bytes"] / (res["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                                  algorithmic_bytes=res["stack_bytes"]),
-                    cpu_baseline=None, finite=res["finite"])
-        print(json.dumps(line))
-        return
-
     if a.calibrate:
         nbytes = 256 << 20
         src, dst = lib.dev_alloc(nbytes), lib.dev_alloc(nbytes)
@@ -414,70 +547,74 @@ def main():
         lib.synchronize()
         lib.dev_free(src)
         lib.dev_free(dst)
-    res, (L, hidden, out) = bench_layer(lib, synth, shape, T, a.steps, a.warmup)
+
+    is120 = a.workload in ("c4_120b", "c5_stack")
+    legs_wanted = a.workload == "c4_120b" and not a.no_legs and not a.tokens
+    # resident layers of the 120b shape: 36 for the stack legs, 8 for a decode rotation, 1 for prefill
+    n_res = 36 if (a.workload == "c5_stack" or legs_wanted) else (8 if T < 512 else 1)
+    layers120 = None
+    if is120:
+        layers120 = [make_layer(lib, synth, SHAPES["c5_stack"], 1234, layer_index=i, norm=True) for i in range(n_res)]
+
+    if a.workload == "c5_stack":
+        leg = stack_leg(lib, synth, shape, T, a.steps, a.warmup, layers120, not a.no_cpu, 12.0)
+        line = dict(metric="MoE stack tokens/s", value=leg["value"], unit="tokens/s", n_gpus=1,
+                    steps=a.steps, warmup=a.warmup, ms_per_step=leg["ms_per_step"],
+                    higher_is_better=True, scaling="weak", vs_baseline=None, dtype="mxfp4 x bf16(2-term) -> f32",
+                    data="synthetic",
+                    config=dict(workload=leg["workload"], tokens=T, device=dev_name,
+                                distinct_experts_per_layer=leg["distinct_experts_per_layer"]),
+                    roofline=leg["roofline"], cpu_baseline=leg["cpu_baseline"], finite=leg["finite"])
+        print(json.dumps(line))
+        return
+
+    head, res, (L, hidden, out) = layer_leg(lib, synth, shape, a.workload, T, a.steps, a.warmup, layers120,
+                                            not a.no_cpu, 12.0)
     prefill = T >= 512
     f16 = bool(shape.get("f16"))
-    if f16 and prefill:
-        st = res["stage_ms"]
-        fl = T * shape["k"] * 4 * shape["H"] * shape["F"]
-        roof = dict(bound="mfma", kernel="expert_f16_gemm_kernel<0> (gate/up + SwiGLU)", achieved=fl / (st["gateup"] * 1e-3) / 1e12,
-                    peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s", traffic=None)
-    elif f16:
-        roof = dict(bound="hbm", kernel="expert_f16_kernel<0> (gate/up + SwiGLU)",
-                    achieved=res["gateup_gbs"], peak=HBM_PEAK_GBS, unit="GB/s", traffic=None)
-    elif prefill:
-        st = res["stage_ms"]
-        fl = T * shape["k"] * 4 * shape["H"] * shape["F"]  # gate + up flops
-        roof = dict(bound="mfma", kernel="expert_gemm_mx_kernel<0> (gate/up + SwiGLU)", achieved=fl / (st["gateup"] * 1e-3) / 1e12,
-                    peak=MFMA_FP4_PEAK_TFLOPS, unit="TFLOP/s", traffic=None)
-    else:
-        roof = dict(bound="hbm", kernel="expert_stream_kernel<2,*> (gate/up + SwiGLU)",
-                    achieved=res["gateup_gbs"], peak=HBM_PEAK_GBS, unit="GB/s", traffic=None)
-    # measured HBM traffic of that kernel, where a counter run has been recorded for this workload
-    try:
-        rec = json.load(open(os.path.join(ROOT, "profiles", "traffic.json"))).get(f"{a.workload}:T={T}")
-    except (OSError, ValueError):
-        rec = None
-    if rec:
-        roof["traffic"] = rec["bytes"]
-        roof["traffic_source"] = rec["source"]
-    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof = head["roofline"]
     if roof["bound"] == "hbm":
         roof["measured_copy_gbs"] = round(measured_copy_gbs(lib), 1)
         roof["frac_of_measured_copy"] = roof["achieved"] / roof["measured_copy_gbs"]
-    roof["kernel_ms"] = res["stage_ms"]["gateup"]
-    roof["algorithmic_bytes"] = res["gateup_bytes"]
+    roof["event_pair_overhead_ms"] = round(event_pair_overhead_ms(lib), 5)
 
     sweep = []
-    if not a.no_sweep:
+    if not a.no_sweep and not legs_wanted:
         for Ts in shape["sweep"]:
             if Ts == T:
                 r = res
             else:
-                r, _ = bench_layer(lib, synth, shape, Ts, max(20, a.steps // 2), a.warmup)
+                r, _ = bench_layer(lib, synth, shape, Ts, max(20, a.steps // 2), a.warmup, layers=layers120)
             sweep.append(dict(T=Ts, tokens_per_s=round(r["tokens_per_s"], 1), ms_per_step=round(r["ms_per_step"], 5),
                               distinct_experts=r["distinct_experts"], close_call_tokens=r["close_call_tokens"],
                               layer_hbm_frac=round(r["layer_hbm_frac"], 4),
                               gateup_hbm_frac=round(r["gateup_gbs"] / HBM_PEAK_GBS, 4),
                               stage_ms={kk: round(v, 5) for kk, v in r["stage_ms"].items()}))
 
-    cpu = None if a.no_cpu else (cpu_baseline_f16(L, hidden, out) if f16 else cpu_baseline(L, hidden, out))
+    legs = []
+    if legs_wanted:
+        # the other configurations the target is stated on, in the same line
+        cpu = not a.no_cpu
+        legs.append(layer_leg(lib, synth, shape, "c4_120b", 1, a.steps, a.warmup, layers120, cpu, 8.0)[0])
+        legs.append(layer_leg(lib, synth, shape, "c4_120b", 4096, max(10, a.steps // 10), max(3, a.warmup // 5),
+                              layers120, cpu, 8.0)[0])
+        for Ts in SHAPES["c5_stack"]["sweep"]:
+            legs.append(stack_leg(lib, synth, SHAPES["c5_stack"], Ts, max(10, a.steps // 10), max(3, a.warmup // 5),
+                                  layers120, cpu, 8.0))
+
     line = dict(
-        metric="MoE layer tokens/s", value=res["tokens_per_s"], unit="tokens/s", n_gpus=1, steps=res["steps"],
-        warmup=a.warmup, ms_per_step=res["ms_per_step"], higher_is_better=True, scaling="weak",
+        metric="MoE layer tokens/s", value=head["value"], unit="tokens/s", n_gpus=1, steps=res["steps"],
+        warmup=a.warmup, ms_per_step=head["ms_per_step"], higher_is_better=True, scaling="weak",
         vs_baseline=None,
         dtype=("f16 x f16(2-term) -> f32" if f16 else
                "mxfp4 x fp6(3-term, block-scaled) -> f32" if prefill else "mxfp4 x bf16(2-term) -> f32"),
         data="synthetic",
         config=dict(workload=f"{a.workload}: E={shape['E']} top-{shape['k']} H={shape['H']} F={shape['F']} "
                              f"{'fp16' if f16 else 'MXFP4'}, T={T}" + (", 8 hot experts" if shape["hot"] else ""),
-                    tokens=T, distinct_experts=res["distinct_experts"], token_batches_in_rotation=res["batches"],
+                    tokens=T, distinct_experts=res["distinct_experts"],
+                    rotation=f"{res['layer_instances']} layer instances x {res['batches']} token batches",
                     close_call_tokens=res["close_call_tokens"], device=dev_name, compute_units=cus),
-        roofline=roof, cpu_baseline=cpu,
-        layer=dict(hbm_frac=res["layer_hbm_frac"], fp4_mfma_frac=res["layer_fp4_frac"],
-                   algorithmic_bytes=res["layer_bytes"], algorithmic_flops=res["layer_flops"],
-                   stage_ms=res["stage_ms"], finite=res["finite"]),
-        sweep=sweep)
+        roofline=roof, cpu_baseline=head["cpu_baseline"], layer=head["layer"], sweep=sweep, legs=legs)
     print(json.dumps(line))
 
 

@@ -36,6 +36,7 @@ SIGNATURES = {
     "csk_event_elapsed_ms": (C.c_int, [_P, _P, _F]),
     "csk_stage_timing": (C.c_int, [C.c_int]),
     "csk_stage_times": (C.c_int, [_F]),
+    "csk_kernel_times": (C.c_int, [_F]),
     "csk_mxfp4_upload": (C.c_int, [_P, _I64, _I64, C.POINTER(_P)]),
     "csk_mxfp4_free": (None, [_P]),
     "csk_mxfp4_dequant": (C.c_int, [_P, _P]),
@@ -198,6 +199,12 @@ class Library:
         ms = (C.c_float * len(self.STAGES))()
         self.check(self.dll.csk_stage_times(ms))
         return dict(zip(self.STAGES, list(ms)))
+
+    def kernel_times(self):
+        """(gate/up, down) kernel durations in ms of the last forward under stage timing."""
+        ms = (C.c_float * 2)()
+        self.check(self.dll.csk_kernel_times(ms))
+        return ms[0], ms[1]
 
     # -- MXFP4 matrices
     def mxfp4_upload(self, blocks, rows, K):

@@ -2,6 +2,7 @@
 // launches.  Declarations and reference citations are in
 // include/coalsack_moe.h.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <algorithm>
 #include <cstdio>
@@ -167,6 +168,21 @@ hipEvent_t g_stage_ev[CSK_N_STAGES + 1] = {};
 bool g_stage_valid = false;
 inline void mark(int i) {
   if (g_timing) (void)hipEventRecord(g_stage_ev[i], g_stream);
+}
+// With stage timing on, the two expert kernels of the MXFP4 path are launched with a start
+// and a stop event attached to the dispatch itself: their difference is the kernel's own
+// begin-to-end time (the clock a kernel trace reports), free of the cost of recording events
+// between launches.  [0] = gate/up, [1] = down.
+hipEvent_t g_kern_ev[2][2] = {};
+bool g_kern_valid = false;
+template <class Kern, class Args>
+inline void launch_expert_kernel(int which, Kern kernel, dim3 grid, dim3 block, size_t lds, const Args& a) {
+  if (g_timing) {
+    hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, g_stream, g_kern_ev[which][0], g_kern_ev[which][1], 0, a);
+    g_kern_valid = true;
+  } else {
+    kernel<<<grid, block, lds, g_stream>>>(a);
+  }
 }
 
 }  // namespace
@@ -386,7 +402,7 @@ int launch_stream(ExpertStreamArgs a, int64_t P, Workspace& ws) {
   const int64_t cus = std::max(g_cus, 1);
   const int64_t nwg = (G == kStreamG && P * npair <= 3 * cus) ? P * npair : kStreamWgPerCu * cus;  // (small P implies G == kStreamG)
   const size_t lds = (size_t)G * a.nblk * 128 + (size_t)2 * 4 * ((G + 3) / 4) * 8 * 16 * sizeof(float);
-  expert_stream_kernel<NMAT == 2 ? 0 : 1, G><<<dim3((unsigned)nwg), 256, lds, g_stream>>>(a);
+  launch_expert_kernel(NMAT == 2 ? 0 : 1, expert_stream_kernel<NMAT == 2 ? 0 : 1, G>, dim3((unsigned)nwg), dim3(256), lds, a);
   return check_launch("expert_stream_kernel");
 }
 
@@ -415,7 +431,8 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
     return fail(CSK_ERR_ARG, "batch too large for the grouped GEMM (activation rows or a weight plane exceed 4 GiB)");
   const int64_t max_mtiles = P / kGemmBM + std::min<int64_t>(E, P);
   const dim3 grid((unsigned)(cdiv(max_mtiles * ga.n_ntiles, kDies) * kDies));
-  expert_gemm_mx_kernel<NMAT == 2 ? 0 : 1><<<grid, 64 * kMxWaves, 3 * kMxStageChunks * 16, g_stream>>>(ga);
+  launch_expert_kernel(NMAT == 2 ? 0 : 1, expert_gemm_mx_kernel<NMAT == 2 ? 0 : 1>, grid, dim3(64 * kMxWaves),
+                       (size_t)3 * kMxStageChunks * 16, ga);
   return check_launch("expert_gemm_mx_kernel");
 }
 
@@ -624,10 +641,25 @@ extern "C" int csk_device_info(char* name, size_t cap, int* compute_units, size_
 
 extern "C" int csk_stage_timing(int enable) {
   REQUIRE_INIT();
-  if (enable && !g_stage_ev[0])
+  if (enable && !g_stage_ev[0]) {
     for (auto& e : g_stage_ev) HIP_TRY(hipEventCreate(&e));
+    for (auto& pair : g_kern_ev)
+      for (auto& e : pair) HIP_TRY(hipEventCreate(&e));
+  }
   g_timing = enable != 0;
   g_stage_valid = false;
+  g_kern_valid = false;
+  return CSK_OK;
+}
+extern "C" int csk_kernel_times(float* ms_out) {
+  REQUIRE_INIT();
+  if (!ms_out) return fail(CSK_ERR_ARG, "csk_kernel_times: null output");
+  if (!g_stage_valid || !g_kern_valid)
+    return fail(CSK_ERR_STATE, "no forward of an MXFP4 layer has run with stage timing enabled");
+  for (int i = 0; i < 2; ++i) {
+    HIP_TRY(hipEventSynchronize(g_kern_ev[i][1]));
+    HIP_TRY(hipEventElapsedTime(&ms_out[i], g_kern_ev[i][0], g_kern_ev[i][1]));
+  }
   return CSK_OK;
 }
 extern "C" int csk_stage_times(float* ms_out) {

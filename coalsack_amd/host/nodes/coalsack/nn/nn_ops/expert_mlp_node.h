@@ -4,17 +4,21 @@
 // below), for both kinds of weights process() distinguishes (:113-136): MXFP4
 // messages go to csk_expert_mlp_mxfp4, float16 tensors to csk_expert_mlp_f16.
 //
-// Weights are uploaded (repacked into the resident device layout) the first
-// time a storage pointer is seen and cached per node: moe_weight_provider
-// hands out the same storage from its own cache on every frame
-// (src/llm/moe_weight_provider.cpp:75-225), so a layer's experts become
-// resident after the first token.
+// Weights are uploaded (repacked into the resident device layout) and cached per
+// node, one entry per role (up, gate, down).  An entry keeps a copy of the host
+// tensor it was made from -- copies share the storage, so the storage cannot be
+// freed and its address handed to another tensor while the entry lives -- plus a
+// sampled stamp of its bytes.  A role whose tensor arrives with the same storage,
+// shape and stamp reuses the device copy; anything else (moe_weight_provider is an
+// LRU, src/llm/moe_weight_provider.cpp:102-132: an evicted slice comes back in new
+// storage) is uploaded again and the old device copy is freed, so a node never
+// holds more than three device matrices and three host references.
 #pragma once
 
+#include <cstring>
 #include <memory>
 #include <stdexcept>
 #include <string>
-#include <unordered_map>
 #include <vector>
 
 #include "coalsack/nn/nn_op_node.h"
@@ -35,8 +39,8 @@ class expert_mlp_node : public graph_node {
     set_output(output_);
   }
   ~expert_mlp_node() override {
-    for (auto& kv : resident_) csk_mxfp4_free(kv.second.handle);
-    for (auto& kv : resident16_) csk_f16_free(kv.second.handle);
+    for (auto& r : resident_) csk_mxfp4_free(r.handle);
+    for (auto& r : resident16_) csk_f16_free(r.handle);
   }
   expert_mlp_node(const expert_mlp_node&) = delete;
   expert_mlp_node& operator=(const expert_mlp_node&) = delete;
@@ -110,51 +114,84 @@ class expert_mlp_node : public graph_node {
     output_->send(out);
   }
 
+  // number of device copies made so far (tests: a reload must upload, a repeat must not)
+  size_t resident_uploads() const { return uploads_; }
+
  private:
-  struct resident {
-    csk_mxfp4* handle;
-    int64_t rows, cols;
-  };
+  enum role { ROLE_UP = 0, ROLE_GATE = 1, ROLE_DOWN = 2 };
 
   int act_code() const {
     return activation_type_ == activation_type::MODIFIED_SWIGLU ? CSK_ACT_MODIFIED_SWIGLU
                                                                 : CSK_ACT_STANDARD_SWIGLU;
   }
 
-  csk_mxfp4* resident_copy(const dynamic_mx_tensor& t) {
-    const uint8_t* key = t.data_ptr();
-    auto it = resident_.find(key);
-    if (it != resident_.end() && it->second.rows == t.dim(0) && it->second.cols == t.dim(1))
-      return it->second.handle;
-    if (it != resident_.end()) {
-      csk_mxfp4_free(it->second.handle);
-      resident_.erase(it);
+  // 64 eight-byte samples spread over the buffer, its length and its ends: enough to tell a
+  // rewritten or reused buffer from the one a device copy was made from, at no cost that matters
+  static uint64_t content_stamp(const uint8_t* p, size_t n) {
+    uint64_t h = 0x9E3779B97F4A7C15ull ^ n;
+    auto mix = [&h](uint64_t v) {
+      h ^= v + 0x9E3779B97F4A7C15ull + (h << 6) + (h >> 2);
+      h *= 0xBF58476D1CE4E5B9ull;
+    };
+    if (n < 8) {
+      for (size_t i = 0; i < n; ++i) mix(p[i]);
+      return h;
     }
+    const size_t step = (n - 8) / 63 ? (n - 8) / 63 : 1;
+    for (size_t off = 0; off + 8 <= n; off += step) {
+      uint64_t v;
+      std::memcpy(&v, p + off, 8);
+      mix(v);
+    }
+    uint64_t v;
+    std::memcpy(&v, p + n - 8, 8);
+    mix(v);
+    return h;
+  }
+
+  struct resident {
+    csk_mxfp4* handle = nullptr;
+    dynamic_mx_tensor held;  // shares the storage the copy was made from
+    uint64_t stamp = 0;
+  };
+
+  csk_mxfp4* resident_copy(role r, const dynamic_mx_tensor& t) {
+    resident& c = resident_[r];
+    const uint64_t stamp = content_stamp(t.data_ptr(), t.size_bytes());
+    if (c.handle && c.held.data_ptr() == t.data_ptr() && c.held.shape() == t.shape() && c.stamp == stamp)
+      return c.handle;
     csk_mxfp4* h = nullptr;
-    if (csk_mxfp4_upload(key, t.dim(0), t.dim(1), &h) != CSK_OK)
+    if (csk_mxfp4_upload(t.data_ptr(), t.dim(0), t.dim(1), &h) != CSK_OK)
       throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
-    resident_[key] = resident{h, t.dim(0), t.dim(1)};
+    if (c.handle) csk_mxfp4_free(c.handle);
+    c.handle = h;
+    c.held = t;
+    c.stamp = stamp;
+    ++uploads_;
     return h;
   }
 
   struct resident16 {
-    csk_f16* handle;
-    int64_t rows, cols;
+    csk_f16* handle = nullptr;
+    dynamic_tensor held;
+    uint64_t stamp = 0;
   };
 
-  csk_f16* resident_copy16(const dynamic_tensor& t) {
-    const uint16_t* key = t.data_ptr<uint16_t>();
-    auto it = resident16_.find(key);
-    if (it != resident16_.end() && it->second.rows == t.dim(0) && it->second.cols == t.dim(1))
-      return it->second.handle;
-    if (it != resident16_.end()) {
-      csk_f16_free(it->second.handle);
-      resident16_.erase(it);
-    }
+  csk_f16* resident_copy16(role r, const dynamic_tensor& t) {
+    resident16& c = resident16_[r];
+    const uint8_t* bytes = reinterpret_cast<const uint8_t*>(t.data_ptr<uint16_t>());
+    const uint64_t stamp = content_stamp(bytes, (size_t)t.dim(0) * (size_t)t.dim(1) * 2);
+    if (c.handle && c.held.data_ptr<uint16_t>() == t.data_ptr<uint16_t>() && c.held.shape() == t.shape() &&
+        c.stamp == stamp)
+      return c.handle;
     csk_f16* h = nullptr;
-    if (csk_f16_upload(key, t.dim(0), t.dim(1), &h) != CSK_OK)
+    if (csk_f16_upload(t.data_ptr<uint16_t>(), t.dim(0), t.dim(1), &h) != CSK_OK)
       throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
-    resident16_[key] = resident16{h, t.dim(0), t.dim(1)};
+    if (c.handle) csk_f16_free(c.handle);
+    c.handle = h;
+    c.held = t;
+    c.stamp = stamp;
+    ++uploads_;
     return h;
   }
 
@@ -225,8 +262,8 @@ class expert_mlp_node : public graph_node {
     dynamic_tensor output(dtype::float32, hidden.shape());
     int is_empty = 0;
     const int rc = csk_expert_mlp_f16(
-        expert_id_, hidden.data_ptr<float>(), tokens, hidden_dim, ffn, resident_copy16(w_up),
-        resident_copy16(w_gate), resident_copy16(w_down),
+        expert_id_, hidden.data_ptr<float>(), tokens, hidden_dim, ffn, resident_copy16(ROLE_UP, w_up),
+        resident_copy16(ROLE_GATE, w_gate), resident_copy16(ROLE_DOWN, w_down),
         has_bias ? inputs[4].data_ptr<float>() : nullptr, has_bias ? inputs[5].data_ptr<float>() : nullptr,
         has_bias ? inputs[6].data_ptr<float>() : nullptr, rp, top_k, act_code(),
         weight_before_ffn_ ? 1 : 0, output.data_ptr<float>(), &is_empty);
@@ -290,8 +327,8 @@ class expert_mlp_node : public graph_node {
     dynamic_tensor output(dtype::float32, hidden.shape());
     int is_empty = 0;
     const int rc = csk_expert_mlp_mxfp4(
-        expert_id_, hidden.data_ptr<float>(), tokens, hidden_dim, ffn, resident_copy(w_up),
-        resident_copy(w_gate), resident_copy(w_down),
+        expert_id_, hidden.data_ptr<float>(), tokens, hidden_dim, ffn, resident_copy(ROLE_UP, w_up),
+        resident_copy(ROLE_GATE, w_gate), resident_copy(ROLE_DOWN, w_down),
         has_bias ? b_up->get_tensor().data_ptr<float>() : nullptr,
         has_bias ? b_gate->get_tensor().data_ptr<float>() : nullptr,
         has_bias ? b_down->get_tensor().data_ptr<float>() : nullptr, rp, top_k, act_code(),
@@ -307,8 +344,9 @@ class expert_mlp_node : public graph_node {
   std::string output_name_, node_name_;
   activation_type activation_type_ = activation_type::MODIFIED_SWIGLU;
   bool weight_before_ffn_ = false;
-  std::unordered_map<const uint8_t*, resident> resident_;
-  std::unordered_map<const uint16_t*, resident16> resident16_;
+  resident resident_[3];
+  resident16 resident16_[3];
+  size_t uploads_ = 0;
 };
 
 }  // namespace coalsack

@@ -91,6 +91,11 @@ int csk_event_elapsed_ms(csk_event* a, csk_event* b, float* ms); /* waits for b 
 #define CSK_N_STAGES 6
 int csk_stage_timing(int enable);
 int csk_stage_times(float* ms_out);
+/* With stage timing enabled, the gate/up and the down kernel of an MXFP4 layer carry a
+ * start and a stop event on the dispatch itself: ms_out[0], ms_out[1] are their own
+ * begin-to-end durations in the last forward -- the figure a kernel trace reports, without
+ * the cost of the events recorded between launches that csk_stage_times includes. */
+int csk_kernel_times(float* ms_out2);
 
 /* ---- resident MXFP4 matrices ------------------------------------------- */
 

@@ -645,6 +645,65 @@ static void gpu_node_chain() {
   CHECK(worst <= 1e-3f);
 }
 
+// The provider behind the expert nodes is an LRU (src/llm/moe_weight_provider.cpp:102-132): a
+// slice that was evicted comes back in new storage, possibly at an address another matrix of
+// the same shape used before.  The node's device copies must follow: same storage and bytes
+// -> reused; new storage, rewritten bytes or tensors that changed roles -> uploaded again,
+// never a stale copy, never more than three device matrices.
+static void gpu_expert_weight_reload() {
+  std::printf("expert node: device copies follow reloaded / rewritten / swapped host weights\n");
+  std::mt19937 gen(99);
+  const int64_t H = 64, F = 64, S = 5, K = 1;  // H == F: all three matrices have the same shape
+  auto hidden = random_tensor({1, S, H}, gen, -1, 1);
+  dynamic_tensor router(dtype::float32, {1, S, K, 2});
+  for (int64_t t = 0; t < S; ++t) router.data_ptr<float>()[2 * t] = 0.0f, router.data_ptr<float>()[2 * t + 1] = 1.0f;
+  auto mk = [](const dynamic_tensor& t) { return std::make_shared<dynamic_tensor_message>(t); };
+  expert_mlp_node node(0);
+  node.set_input_names({"hidden", "w_up", "w_gate", "w_down", "router"});
+  node.set_output_name("out");
+  capture_node cap;
+  cap.set_input(node.get_output());
+  auto run_and_check = [&](const dynamic_mx_tensor& up, const dynamic_mx_tensor& gate, const dynamic_mx_tensor& down) {
+    node.process("default", result_message::ok({{"hidden", mk(hidden)},
+                                                {"w_up", std::make_shared<dynamic_mx_tensor_message>(up)},
+                                                {"w_gate", std::make_shared<dynamic_mx_tensor_message>(gate)},
+                                                {"w_down", std::make_shared<dynamic_mx_tensor_message>(down)},
+                                                {"router", mk(router)}}));
+    CHECK(!cap.got.empty() && cap.got.back()->is_ok());
+    if (cap.got.empty() || !cap.got.back()->is_ok()) return;
+    auto out = std::dynamic_pointer_cast<dynamic_tensor_message>(cap.got.back()->get_field("out"))->get_tensor();
+    std::vector<float> want(S * H);
+    int empty = 0;
+    orc_expert_mlp_mxfp4(0, hidden.data_ptr<float>(), S, H, F, up.data_ptr(), gate.data_ptr(), down.data_ptr(),
+                         nullptr, nullptr, nullptr, router.data_ptr<float>(), K, 0, 0, want.data(), &empty);
+    float worst = 0, scale = 0;
+    for (int64_t i = 0; i < S * H; ++i) {
+      worst = std::fmax(worst, std::fabs(out.data_ptr<float>()[i] - want[i]));
+      scale = std::fmax(scale, std::fabs(want[i]));
+    }
+    CHECK(worst <= 1e-3f * std::fmax(scale, 1e-6f));
+  };
+  {
+    auto up = random_mx(F, H, gen), gate = random_mx(F, H, gen), down = random_mx(H, F, gen);
+    run_and_check(up, gate, down);
+    CHECK(node.resident_uploads() == 3);
+    run_and_check(up, gate, down);  // same storage, same bytes: nothing is uploaded
+    CHECK(node.resident_uploads() == 3);
+    run_and_check(gate, up, down);  // the same two buffers in each other's role
+    CHECK(node.resident_uploads() == 5);
+    std::uniform_int_distribution<int> byte(0, 255);
+    for (size_t b = 0; b < up.num_blocks(); ++b)  // rewritten in place
+      for (int j = 1; j < 17; ++j) up.data_ptr()[17 * b + j] = (uint8_t)byte(gen);
+    run_and_check(gate, up, down);
+    CHECK(node.resident_uploads() == 6);
+  }  // the caller's references go away (an eviction); the node still holds the storage of its copies
+  for (int round = 0; round < 3; ++round) {  // reloads: fresh storage each time, wherever malloc puts it
+    auto up = random_mx(F, H, gen), gate = random_mx(F, H, gen), down = random_mx(H, F, gen);
+    run_and_check(up, gate, down);
+    CHECK(node.resident_uploads() == 9 + 3 * (size_t)round);
+  }
+}
+
 // Nodes of different layers may be driven from different threads (the reference runs each
 // layer's nodes on that layer's scheduler thread, layer_scheduler_node); the library
 // serialises the calls, so results must equal those of the same calls made one after another.
@@ -708,6 +767,7 @@ int main(int argc, char** argv) {
     gpu_dense_ffn_tests();
     gpu_matmul_tests();
     gpu_node_chain();
+    gpu_expert_weight_reload();
     gpu_norm_add_tests();
     gpu_concurrent_callers();
   } else {

@@ -89,7 +89,7 @@ def test_router_matches_oracle(lib, oracle, T, H, E, k, bias, sigmoid):
     L = _L()
     L.k, L.gate_w, L.gate_b = k, g, (b if b is not None else np.zeros(E, np.float32))
     real, near = classify_index_mismatches(oracle, h, L, got, want)
-    assert real == 0, (real, near)
+    assert (real, near) == (0, 0)
     # weights inherit the ~1e-6 relative difference between the two fp32 summation orders
     assert np.max(np.abs(got[same, :, 1] - want[same, :, 1])) <= 1e-5
     assert np.all(got[..., 1] > 0) and np.allclose(got[..., 1].sum(axis=1), 1.0, atol=1e-5) or sigmoid
@@ -268,7 +268,9 @@ def test_rmsnorm_and_add(lib, oracle):
 # ------------------------------------------------------------ whole layer
 
 def _check_layer(lib, oracle, L, T, bias=True, norm=False, residual=False, device_weights=False,
-                 oracle_tokens=-1, **opts):
+                 oracle_tokens=-1, subset=False, **opts):
+    """subset: the oracle replays only the experts the batch selects (real-shape layers whose
+    weights were generated on the device)."""
     hidden = synth.hidden_states(T, L.H, seed=T + 17)
     flags = (capi.FWD_RMSNORM if norm else 0) | (capi.FWD_RESIDUAL if residual else 0)
     with build_layer(lib, L, bias=bias, norm=norm, device_weights=device_weights, **opts) as layer:
@@ -281,11 +283,19 @@ def _check_layer(lib, oracle, L, T, bias=True, norm=False, residual=False, devic
         oopts["sigmoid"] = opts["sigmoid"]
     if "weight_before_ffn" in opts:
         oopts["weight_before_ffn"] = opts["weight_before_ffn"]
-    want, wpairs = oracle_layer(oracle, L, hidden, bias=bias, norm=norm, residual=residual,
-                                max_tokens=oracle_tokens, **oopts)
+    if subset:
+        assert bias and oracle_tokens < 0
+        want, wpairs = oracle_layer_subset(oracle, L, hidden, T, norm=norm, residual=residual, **oopts)
+    else:
+        want, wpairs = oracle_layer(oracle, L, hidden, bias=bias, norm=norm, residual=residual,
+                                    max_tokens=oracle_tokens, **oopts)
     xin = oracle.rmsnorm(hidden, L.norm_w, 1e-5) if norm else hidden
     real, near = classify_index_mismatches(oracle, xin, L, pairs, wpairs)
     assert real == 0, (real, near)
+    if not norm:
+        # the router sees the reference's own input: close calls are recomputed in the
+        # reference's summation order, so not even a near-tie may come out differently
+        assert near == 0, near
     same = np.all(pairs[..., 0] == wpairs[..., 0], axis=1)
     assert np.max(np.abs(pairs[same, :, 1] - wpairs[same, :, 1])) <= 1e-5
     # dispatch: per-expert token lists are {t : e in topk(t)} ascending, counts sum to T*k
@@ -373,6 +383,20 @@ def test_layer_120b_shape_skewed_16_tokens(lib, oracle):
     _check_layer(lib, oracle, L, 16, device_weights=True)
 
 
+@pytest.mark.parametrize("T", [32, 64])
+def test_layer_20b_shape_wide_token_groups(lib, oracle, T):
+    """BASELINE config 2 above 16 tokens: the six-token streaming kernels at K = 2880."""
+    L = synth.LayerInputs(32, 4, 2880, 2880, seed=52)
+    _check_layer(lib, oracle, L, T, device_weights=True, subset=True)
+
+
+@pytest.mark.parametrize("T", [1, 64])
+def test_layer_120b_shape_skewed_1_and_64_tokens(lib, oracle, T):
+    """BASELINE config 4 / 5 shape at the ends of the decode range, with the skewed bias."""
+    L = synth.LayerInputs(128, 4, 2880, 2880, seed=43, hot_experts=8)
+    _check_layer(lib, oracle, L, T, device_weights=True, subset=True)
+
+
 # ----------------------------------------------------- prefill (grouped GEMM)
 
 def _prefill_case(lib, oracle, L, T, ntok_oracle):
@@ -395,7 +419,7 @@ def _prefill_case(lib, oracle, L, T, ntok_oracle):
     assert np.allclose(pairs[..., 1].sum(axis=1), 1.0, atol=1e-5)
     want, wpairs = oracle_layer_subset(oracle, L, hidden, ntok_oracle)
     real, near = classify_index_mismatches(oracle, hidden[:ntok_oracle], L, pairs[:ntok_oracle], wpairs)
-    assert real == 0, (real, near)
+    assert (real, near) == (0, 0)
     same = np.all(pairs[:ntok_oracle, :, 0] == wpairs[..., 0], axis=1)
     assert_layer_close(got[:ntok_oracle][same], want[same])
     return counts
@@ -424,9 +448,9 @@ def test_prefill_ragged_small_shape(lib, oracle):
     with build_layer(lib, L) as layer:
         got, pairs = layer.forward(hidden, want_pairs=True)
     want, wpairs = oracle_layer(oracle, L, hidden)
-    same = np.all(pairs[..., 0] == wpairs[..., 0], axis=1)
-    assert same.mean() > 0.99
-    assert_layer_close(got[same], want[same])
+    real, near = classify_index_mismatches(oracle, hidden, L, pairs, wpairs)
+    assert (real, near) == (0, 0)
+    assert_layer_close(got, want)
 
 
 def test_concurrent_forwards_equal_sequential(lib):
@@ -483,13 +507,60 @@ def test_stack_config5(lib, oracle, E, k, H, F, T, n_layers):
                 want, wpairs = oracle_layer_subset(oracle, L, h, n, norm=True, residual=True)
             else:
                 want, wpairs = oracle_layer(oracle, L, h, norm=True, residual=True)
+            xin = oracle.rmsnorm(h[:n], L.norm_w, 1e-5)
+            real, near = classify_index_mismatches(oracle, xin, L, pairs[:n], wpairs[:n])
+            assert real == 0, (real, near)  # the router input carries the GPU's RMSNorm rounding: near-ties are tolerated
             same = np.all(pairs[:n, :, 0] == wpairs[:n, :, 0], axis=1)
-            assert same.mean() >= 0.9
             assert_layer_close(nxt[:n][same], want[:n][same])
             h = nxt
         assert np.array_equal(got_stack, h)
     finally:
         lib.dev_free(d_h)
+        for layer in layers:
+            layer.close()
+
+
+def test_stack_config5_36_resident_layers(lib, oracle):
+    """BASELINE config 5 as stated: 36 layers of the 120b shape resident at once (61 GB of
+    expert planes, generated on the device), decode batches of 1, 8 and 64 tokens.  The stack
+    call equals the layers called one at a time bit for bit; on sampled layers the output of
+    the layer matches the CPU path fed with that layer's actual input, on sampled tokens
+    (the host replays only the experts those tokens select)."""
+    from coalsack_amd.capi import stack_forward
+    flags = capi.FWD_RMSNORM | capi.FWD_RESIDUAL
+    E, k, H, F, n_layers = 128, 4, 2880, 2880, 36
+    Ls = [synth.LayerInputs(E, k, H, F, seed=91, layer=i, hot_experts=8, with_norm=True) for i in range(n_layers)]
+    layers = []
+    try:
+        for L in Ls:
+            layers.append(build_layer(lib, L, norm=True, device_weights=True))
+        for T, sampled in ((1, (0, 17, 35)), (8, (1, 20, 35)), (64, (2, 35))):
+            hidden = synth.hidden_states(T, H, seed=30 + T)
+            d_h = lib.to_device(hidden)
+            try:
+                stack_forward(lib, layers, d_h, T)
+                got_stack = lib.to_host(d_h, hidden.shape)
+            finally:
+                lib.dev_free(d_h)
+            h = hidden
+            n = min(T, 4)
+            for i, (L, layer) in enumerate(zip(Ls, layers)):
+                nxt, pairs = layer.forward(h, flags, want_pairs=True)
+                if i in sampled:
+                    want, wpairs = oracle_layer_subset(oracle, L, h, n, norm=True, residual=True)
+                    xin = oracle.rmsnorm(h[:n], L.norm_w, 1e-5)
+                    real, near = classify_index_mismatches(oracle, xin, L, pairs[:n], wpairs)
+                    assert real == 0, (T, i, real, near)
+                    same = np.all(pairs[:n, :, 0] == wpairs[..., 0], axis=1)
+                    assert same.any(), (T, i)
+                    # the residual stream grows through the stack: compare the layer's own
+                    # contribution (output minus residual input) to the bar as well
+                    assert_layer_close(nxt[:n][same], want[same])
+                    assert_layer_close((nxt[:n] - h[:n])[same], (want - h[:n])[same])
+                h = nxt
+            assert np.all(np.isfinite(got_stack))
+            assert np.array_equal(got_stack, h), T
+    finally:
         for layer in layers:
             layer.close()
 
@@ -521,8 +592,9 @@ def test_long_batch_in_passes(lib, oracle):
     # other kernels, another summation order: the same experts (no near-tie in this batch), weights to rounding
     assert np.array_equal(spairs[..., 0], pairs[..., 0]) and np.max(np.abs(spairs[..., 1] - pairs[..., 1])) < 1e-5
     want, wpairs = oracle_layer(oracle, L, hidden, norm=True, residual=True)
+    real, near = classify_index_mismatches(oracle, oracle.rmsnorm(hidden, L.norm_w, 1e-5), L, pairs, wpairs)
+    assert real == 0, (real, near)
     same = np.all(pairs[..., 0] == wpairs[..., 0], axis=1)
-    assert same.mean() > 0.99
     assert_layer_close(small[same], want[same])
     assert_layer_close(whole[same], want[same])
 
