@@ -69,6 +69,7 @@ SIGNATURES = {
     "csk_gguf_get_str": (C.c_int, [_P, C.c_char_p, C.c_char_p, C.c_size_t]),
     "csk_layer_from_gguf": (C.c_int, [_P, _I64, C.POINTER(_P)]),
     "csk_moe_forward": (C.c_int, [_P, _P, _I64, _P, C.c_int]),
+    "csk_moe_forward_noalloc": (C.c_int, [_P, _P, _I64, _P, C.c_int]),
     "csk_moe_forward_host": (C.c_int, [_P, _P, _I64, _P, _P, C.c_int]),
     "csk_moe_stack_forward": (C.c_int, [C.POINTER(_P), _I64, _P, _I64]),
     "csk_set_pass_tokens": (C.c_int, [_I64]),
@@ -519,6 +520,9 @@ class Layer:
 
     def forward_device(self, d_hidden, T, d_out, flags=0):
         self.lib.check(self.lib.dll.csk_moe_forward(self.h, d_hidden, T, d_out, flags))
+
+    def forward_device_noalloc(self, d_hidden, T, d_out, flags=0):
+        self.lib.check(self.lib.dll.csk_moe_forward_noalloc(self.h, d_hidden, T, d_out, flags))
 
     def forward(self, hidden, flags=0, want_pairs=False):
         hidden = _f32(hidden)

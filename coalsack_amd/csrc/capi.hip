@@ -99,6 +99,7 @@ struct Workspace {
   float* y = nullptr;       // [P,H]
   int* tiles = nullptr;     // prefill tile schedule
   int* n_tiles = nullptr;
+  bool fixed = false;       // carved out of the load-time device array: never grown, never freed
 
   void release() {
     void* ps[] = {xn, xs, xg, logits, pairs, ids, counts, offsets, desc, groups, nv,
@@ -109,6 +110,7 @@ struct Workspace {
   }
   int ensure(int64_t T_, int64_t E_, int64_t k_, int64_t H_, int64_t F_, bool need_xg) {
     if (T_ <= T && E_ <= E && k_ <= k && H_ <= H && F_ <= F && (!need_xg || xg)) return CSK_OK;
+    if (fixed) return fail(CSK_ERR_ARG, "shape exceeds the fixed workspace of the allocation-free forward");
     const int64_t nT = std::max(T, T_), nE = std::max(E, E_), nk = std::max(k, k_),
                   nH = std::max(H, H_), nF = std::max(F, F_);
     const bool had_xg = xg != nullptr;
@@ -149,6 +151,63 @@ struct Workspace {
   }
 };
 Workspace g_ws;
+Workspace* g_last_ws = &g_ws;  // the workspace the last forward ran in (csk_layer_last_dispatch reads it)
+
+// ---- fixed workspace of the allocation-free forward ------------------------
+// Callers that cannot allocate (code under graph capture, serving loops, harnesses that
+// forbid hipMalloc) get the decode-sized forward out of a workspace that exists from load
+// time on: one file-scope device array per GPU, carved into the buffers of a Workspace of
+// the maximum shape below.  The array's name is only a handle on the host; its device
+// address is asked for once per device (csk_init, that device current) and kept.
+constexpr int64_t kFixedMaxT = 64;      // tokens per call
+constexpr int64_t kFixedMaxP = 512;     // token-expert assignments per call (T * top_k)
+constexpr int64_t kFixedMaxDim = 3072;  // hidden_dim and expert_ffn_dim
+constexpr size_t fixed_align(size_t n) { return (n + 255) & ~(size_t)255; }
+constexpr size_t kFixedRowBytes = (size_t)kFixedMaxDim * 4;  // a row as f32, or as two bf16 terms
+constexpr size_t kFixedScratchBytes =
+    fixed_align(kFixedMaxT * kFixedRowBytes) * 2 +                                     // xn, xs
+    fixed_align(kFixedMaxP * kFixedRowBytes) * 3 +                                     // xg, act, y
+    fixed_align((size_t)kFixedMaxT * kMaxExperts * 4 * (1 + kRouterMaxSplits)) +       // logits
+    fixed_align(kFixedMaxP * 8) + fixed_align(kFixedMaxP * 4) * 4 +                    // pairs; ids, list_tok, list_w, pos
+    fixed_align(kMaxExperts * 4) + fixed_align((kMaxExperts + 1) * 4) +                // counts, offsets
+    fixed_align(kMaxExperts * sizeof(WorkDesc)) + fixed_align(kFixedMaxP * sizeof(StreamGroup)) +
+    fixed_align((size_t)4 * (kFixedMaxP / 16 + kMaxExperts + 1) * 4) + 2 * 256;        // tiles; nv, n_tiles
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kFixedScratchBytes];
+namespace {
+constexpr int kMaxDevices = 64;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each GPU that csk_init has seen
+Workspace g_ws_fixed;                             // carved out of g_scratch_ptr[g_device]
+
+void carve_fixed_workspace(Workspace& ws, unsigned char* base) {
+  size_t off = 0;
+  auto take = [&](size_t bytes) {
+    unsigned char* p = base + off;
+    off += fixed_align(bytes);
+    return p;
+  };
+  ws = Workspace();
+  ws.xn = reinterpret_cast<float*>(take(kFixedMaxT * kFixedRowBytes));
+  ws.xs = reinterpret_cast<uint16_t*>(take(kFixedMaxT * kFixedRowBytes));
+  ws.xg = reinterpret_cast<uint16_t*>(take(kFixedMaxP * kFixedRowBytes));
+  ws.act = reinterpret_cast<uint16_t*>(take(kFixedMaxP * kFixedRowBytes));
+  ws.y = reinterpret_cast<float*>(take(kFixedMaxP * kFixedRowBytes));
+  ws.logits = reinterpret_cast<float*>(take((size_t)kFixedMaxT * kMaxExperts * 4 * (1 + kRouterMaxSplits)));
+  ws.pairs = reinterpret_cast<float*>(take(kFixedMaxP * 8));
+  ws.ids = reinterpret_cast<int*>(take(kFixedMaxP * 4));
+  ws.list_tok = reinterpret_cast<int*>(take(kFixedMaxP * 4));
+  ws.list_w = reinterpret_cast<float*>(take(kFixedMaxP * 4));
+  ws.pos = reinterpret_cast<int*>(take(kFixedMaxP * 4));
+  ws.counts = reinterpret_cast<int*>(take(kMaxExperts * 4));
+  ws.offsets = reinterpret_cast<int*>(take((kMaxExperts + 1) * 4));
+  ws.desc = reinterpret_cast<WorkDesc*>(take(kMaxExperts * sizeof(WorkDesc)));
+  ws.groups = reinterpret_cast<StreamGroup*>(take(kFixedMaxP * sizeof(StreamGroup)));
+  ws.tiles = reinterpret_cast<int*>(take((size_t)4 * (kFixedMaxP / 16 + kMaxExperts + 1) * 4));
+  ws.nv = reinterpret_cast<int*>(take(4));
+  ws.n_tiles = reinterpret_cast<int*>(take(4));
+  ws.T = kFixedMaxT, ws.E = kMaxExperts, ws.k = kMaxTopK, ws.H = kFixedMaxDim, ws.F = kFixedMaxDim;
+  ws.fixed = true;
+}
 
 // extra buffers of the fp16 expert path
 struct F16Scratch {
@@ -616,6 +675,15 @@ extern "C" int csk_init(int device) {
     HIP_TRY(hipMalloc((void**)&g_zero, kZeroLen * sizeof(float)));
     HIP_TRY(hipMemset(g_zero, 0, kZeroLen * sizeof(float)));
   }
+  if (device >= kMaxDevices) return fail(CSK_ERR_HIP, "device index beyond the library's table");
+  if (!g_scratch_ptr[device]) {
+    // this GPU's copy of the load-time array (the device chosen above is current)
+    unsigned char* ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(CSK_ERR_HIP, "hipGetSymbolAddress returned a null address for the fixed workspace");
+    g_scratch_ptr[device] = ptr;
+  }
+  carve_fixed_workspace(g_ws_fixed, g_scratch_ptr[device]);
   g_device = device;
   g_cus = prop.multiProcessorCount;
   g_ready = true;
@@ -1159,11 +1227,11 @@ namespace {
 // kernels.
 int64_t g_pass_tokens = 32768;
 
-int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int flags) {
+int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int flags, Workspace& ws = g_ws) {
   int rc = CSK_OK;
-  Workspace& ws = g_ws;
   rc = ws.ensure(T, L->E, L->k, L->H, L->F, L->wbf);
   if (rc != CSK_OK) return rc;
+  g_last_ws = &ws;
   const int64_t P = T * L->k;
   const bool norm = (flags & CSK_FWD_RMSNORM) != 0;
   const float* xr = norm ? ws.xn : hidden;
@@ -1273,6 +1341,24 @@ extern "C" int csk_moe_forward(csk_layer* L, const float* hidden, int64_t T, flo
   return CSK_OK;
 }
 
+extern "C" int csk_moe_forward_noalloc(csk_layer* L, const float* hidden, int64_t T, float* out, int flags) {
+  REQUIRE_INIT();
+  if (!L || !hidden || !out || T < 0) return fail(CSK_ERR_ARG, "csk_moe_forward_noalloc: bad argument");
+  int rc = layer_ready(L, flags);
+  if (rc != CSK_OK) return rc;
+  if (L->f16) return fail(CSK_ERR_ARG, "csk_moe_forward_noalloc: MXFP4 layers only");
+  if (T > kFixedMaxT || T * L->k > kFixedMaxP || L->H > kFixedMaxDim || L->F > kFixedMaxDim)
+    return fail(CSK_ERR_ARG, "csk_moe_forward_noalloc: at most " + std::to_string(kFixedMaxT) + " tokens, " +
+                                 std::to_string(kFixedMaxP) + " token-expert assignments (T * top_k), hidden_dim and "
+                                 "expert_ffn_dim up to " + std::to_string(kFixedMaxDim) + "; got T = " +
+                                 std::to_string(T) + ", top_k = " + std::to_string(L->k) + ", H = " +
+                                 std::to_string(L->H) + ", F = " + std::to_string(L->F));
+  L->last_T = T;
+  if (T == 0) return CSK_OK;
+  // same kernels as csk_moe_forward, every buffer inside this GPU's load-time array
+  return forward_pass(L, hidden, T, out, flags, g_ws_fixed);
+}
+
 extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T, float* out,
                                     float* pairs_out, int flags) {
   REQUIRE_INIT();
@@ -1339,10 +1425,10 @@ extern "C" int csk_layer_last_dispatch(csk_layer* L, int32_t* counts_host, int32
     return fail(CSK_ERR_STATE, "the last forward took its batch in several passes: there is no single dispatch to report");
   if (L->last_T == 0) return fail(CSK_ERR_STATE, "no forward has run on this layer");
   if (counts_host) {
-    int rc = csk_copy_d2h(counts_host, g_ws.counts, (size_t)L->E * sizeof(int));
+    int rc = csk_copy_d2h(counts_host, g_last_ws->counts, (size_t)L->E * sizeof(int));
     if (rc != CSK_OK) return rc;
   }
-  if (tokens_host) return csk_copy_d2h(tokens_host, g_ws.list_tok, (size_t)L->last_T * L->k * sizeof(int));
+  if (tokens_host) return csk_copy_d2h(tokens_host, g_last_ws->list_tok, (size_t)L->last_T * L->k * sizeof(int));
   return CSK_OK;
 }
 

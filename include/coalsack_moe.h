@@ -219,6 +219,17 @@ int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out);
  * size -- tokens do not depend on one another -- so the workspace stays bounded. */
 int csk_moe_forward(csk_layer* L, const float* hidden_device, int64_t T, float* out_device,
                     int flags);
+/* csk_moe_forward for callers that cannot allocate device memory -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference.  Same arguments, same kernels and the same results bit for bit, but every
+ * intermediate buffer lives in a device array that is part of the library image (21 MB per
+ * GPU, held until the process ends), and the call makes no hipMalloc / hipFree.  Limits:
+ * MXFP4 layers, T <= 64 tokens, T * top_k <= 512, hidden_dim and expert_ffn_dim <= 3072;
+ * anything larger is refused with CSK_ERR_ARG.  All calls on a GPU share that array (it keeps
+ * the previous call's contents; nothing in it has to start at zero): calls that overlap on
+ * one GPU would race -- the library's lock and single stream order them. */
+int csk_moe_forward_noalloc(csk_layer* L, const float* hidden_device, int64_t T, float* out_device,
+                            int flags);
 /* Largest number of tokens one pass of csk_moe_forward takes (1..65536). */
 int csk_set_pass_tokens(int64_t tokens);
 /* Same through host buffers; also returns the router output [T,k,2] when
