@@ -97,7 +97,8 @@ class CskError(RuntimeError):
 
 
 def lib_path():
-    return os.path.join(_HERE, "libcoalsack_moe.so")
+    """The in-tree library, or the file COALSACK_MOE_LIB names (another build of it)."""
+    return os.environ.get("COALSACK_MOE_LIB") or os.path.join(_HERE, "libcoalsack_moe.so")
 
 
 def _ptr(a):

@@ -482,16 +482,23 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
   ga.act_type = a.act_type;
   ga.act_out = reinterpret_cast<u32x4*>(a.act_out);
   ga.y_out = a.y_out;
-  ga.n_ntiles = (int)cdiv(a.ntile, (NMAT == 2 ? 2 : 4) * kMxWaves);
-  // per-lane offsets into the activation rows and the weight planes are 32-bit
+  using Geom = MxGeom<kMxNG>;
+  constexpr int kMode = NMAT == 2 ? 0 : 1;
+  if (a.ntile % 2) return fail(CSK_ERR_ARG, "grouped GEMM: the number of output features must be a multiple of 32");
+  ga.n_ntiles = (int)cdiv(a.ntile, Geom::tiles_per_wg(kMode));
+  // per-lane offsets into the activation rows are 32-bit (the weight offsets are tile-relative)
   const int64_t a_rows = a.list_row ? T : P;
-  if (a_rows * mx3_row_blocks(a.nblk) * 96 >= ((int64_t)1 << 32) ||
-      (int64_t)a.ntile * a.nblk * 256 >= ((int64_t)1 << 32))
-    return fail(CSK_ERR_ARG, "batch too large for the grouped GEMM (activation rows or a weight plane exceed 4 GiB)");
+  if (a_rows * mx3_row_blocks(a.nblk) * 96 >= ((int64_t)1 << 32))
+    return fail(CSK_ERR_ARG, "batch too large for the grouped GEMM (activation rows exceed 4 GiB)");
+  static bool lds_attr_set[2] = {false, false};
+  if (!lds_attr_set[kMode]) {
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&expert_gemm_mx_kernel<kMode, kMxNG>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)Geom::kLdsBytes));
+    lds_attr_set[kMode] = true;
+  }
   const int64_t max_mtiles = P / kGemmBM + std::min<int64_t>(E, P);
   const dim3 grid((unsigned)(cdiv(max_mtiles * ga.n_ntiles, kDies) * kDies));
-  launch_expert_kernel(NMAT == 2 ? 0 : 1, expert_gemm_mx_kernel<NMAT == 2 ? 0 : 1>, grid, dim3(64 * kMxWaves),
-                       (size_t)3 * kMxStageChunks * 16, ga);
+  launch_expert_kernel(kMode, expert_gemm_mx_kernel<kMode, kMxNG>, grid, dim3(64 * kMxWaves), Geom::kLdsBytes, ga);
   return check_launch("expert_gemm_mx_kernel");
 }
 
@@ -1838,3 +1845,4 @@ extern "C" int csk_add(const float* a, const float* b, float* out, int64_t n) {
   HIP_TRY(hipStreamSynchronize(g_stream));
   return CSK_OK;
 }
+

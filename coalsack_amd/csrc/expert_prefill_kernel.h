@@ -15,15 +15,23 @@
 // tile (l%32)/16 of a pair of packed 16-row tiles, and its 16-byte packed entry
 // (32 nibbles in element order) is the operand.
 //
-// A workgroup of eight waves owns 64 tokens of one expert x 256 features (gate and
-// up rows together) or 512 down rows, and walks K in steps of 128 (4 blocks); the
-// kernel is bound by what the compute units can pull from L2, and the activation
-// tile is fetched once per workgroup, so the wide tile is what sets its speed.  The
-// activation tile (64 tokens x 4 blocks x 3 terms x 32 B) goes to LDS by
-// global_load_lds with a 16-byte XOR swizzle applied on the source side; weights
-// go straight to registers; both are requested two steps ahead (three LDS stages, one
-// barrier per step).
-// The gate/up epilogue applies bias + SwiGLU, stages the 64 x 128 tile in LDS as
+// A workgroup of four waves owns 64 tokens of one expert x (128 NG) weight rows -- gate and
+// up rows of the same 64 NG features together, or 128 NG down rows -- and walks K in steps
+// of 128 (4 blocks).  A wave owns NG groups of 32 weight rows (NG/2 gate groups and the NG/2
+// up groups of the same features) for all 64 tokens: NG x 2 accumulator tiles of 32 x 32.
+// The activations are the expensive operand (three terms of 32 bytes per 32 values against
+// 17 bytes of weights), so the tile is tall in weight rows: every activation fragment read
+// from LDS feeds NG matrix instructions, and NG = 4 is what still leaves two workgroups per
+// compute unit (128 accumulator + 80 weight registers per lane).  Measured with cycle
+// stamps per step: a wave spends 80-85 % of the K loop issuing matrix instructions at one
+// per ~40 cycles (the scaled form is a pair: scale load + product), 10-17 % waiting for the
+// next step's loads and 3-5 % at the barrier; a quarter of a workgroup's time lies outside
+// the loop (first loads, epilogue, the ragged last round of units).
+// The activation tile (64 tokens x 4 blocks x 3 terms x 32 B) goes to LDS by
+// global_load_lds with a 16-byte XOR swizzle applied on the source side; weights go
+// straight to registers; both are requested one step ahead (two LDS stages and register
+// sets, one barrier per step).
+// The gate/up epilogue applies bias + SwiGLU, stages each wave's 64 x 16 NG tile in LDS as
 // fp32 and re-quantises it to the three-term format the down GEMM reads.
 //
 // Restates include/coalsack/nn/nn_ops/expert_mlp_node.h:651-732 with the token
@@ -45,8 +53,8 @@ struct ExpertGemmMxArgs {
   const int* list_row;   // packed position -> row of A; null: row = packed position
   const uint4* A;        // [rows][mx3_row_blocks(nblk)][6] x 16 B (mx3.h); blocks past nblk are zeros
   int nblk;              // K / 32
-  int ntile;             // ceil(N / 16) weight row tiles
-  int n_ntiles;          // N tiles per M tile: ceil(ntile / 16) (MODE 0) or ceil(ntile / 32)
+  int ntile;             // N / 16 weight row tiles (even: N is a multiple of 32)
+  int n_ntiles;          // N tiles per M tile: ceil(ntile / (4 NG)) (MODE 0) or ceil(ntile / (8 NG))
   int N;
   int act_type;
   u32x4* act_out;        // MODE 0: [P][mx3_row_blocks(N / 32)][6] x 16 B
@@ -60,12 +68,48 @@ constexpr int kMxStageChunks = kGemmBM * 4 * kMx3ChunksPerBlock;  // 1536 x 16 B
 constexpr int kMxRowChunks = 4 * kMx3ChunksPerBlock;              // 24 chunks per token per step
 constexpr int kMxWaves = 4;                                       // waves per workgroup
 constexpr int kMxCopies = kMxStageChunks / 64 / kMxWaves;         // copy instructions per wave per step
-constexpr int kStepLoads = kMxCopies + 2 * 2 * 2;                 // load instructions per wave per step
+constexpr int kMxNG = 4;                                          // groups of 32 weight rows per wave
 
-template <int MODE>
-__global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_kernel(ExpertGemmMxArgs a) {
+// Geometry that follows from NG.
+template <int NG>
+struct MxGeom {
+  static_assert(NG >= 2 && NG % 2 == 0, "a wave pairs NG/2 gate groups with NG/2 up groups");
+  static constexpr int kStepLoads = kMxCopies + 4 * NG;  // load instructions per wave per step
+  // the wave's memory counter holds 63 loads: two steps of them in flight where they fit
+  // One step: the weight registers of a step are loaded while the step before it is
+  // contracted.  (Two steps ahead needs a third register set, which at NG = 4 no longer fits
+  // two workgroups per compute unit, and the second resident workgroup hides more latency
+  // than the deeper queue does.)
+  static constexpr int kAhead = 1;
+  static constexpr int kStages = kAhead + 1;
+  static constexpr int kEpiRow = 16 * NG + 1;  // floats per token in a wave's epilogue tile (+1: bank spread)
+  static constexpr size_t kLdsBytes =
+      (size_t)kStages * kMxStageChunks * 16 > (size_t)kMxWaves * kGemmBM * kEpiRow * 4
+          ? (size_t)kStages * kMxStageChunks * 16
+          : (size_t)kMxWaves * kGemmBM * kEpiRow * 4;
+  static constexpr int tiles_per_wg(int mode) { return mode == 0 ? 4 * NG : 8 * NG; }
+};
+
+__device__ __forceinline__ const char* uniform_ptr(const char* p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+}
+
+// Descriptor of a whole weight plane as a raw buffer (no stride, no range to speak of: the
+// offsets are tile arithmetic checked on the host).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t plane_rsrc(const void* p) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(uniform_ptr(reinterpret_cast<const char*>(p))), 0,
+                                           0x7fffffff, 0x00020000);
+}
+
+template <int MODE, int NG>
+__global__ __launch_bounds__(64 * kMxWaves, 2) void expert_gemm_mx_kernel(ExpertGemmMxArgs a) {
+  using G = MxGeom<NG>;
+  constexpr int kStepLoads = G::kStepLoads, kAhead = G::kAhead, kStages = G::kStages;
   extern __shared__ __align__(16) unsigned char smem[];
-  uint4* As = reinterpret_cast<uint4*>(smem);  // [3 stages][64 tokens][24 chunks]
+  uint4* As = reinterpret_cast<uint4*>(smem);  // [kStages][64 tokens][24 chunks]
   // Work unit = (M tile, N tile), numbered M-tile major.  Workgroups are handed to
   // the eight accelerator dies round-robin by linear id, and each die has its own L2:
   // die x takes the x-th contiguous eighth of the unit sequence, so that the
@@ -82,37 +126,43 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
   const int Te = wd->Te;
   const int base = wd->base + m0;
   const int mcount = min(kGemmBM, Te - m0);
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, and known to be
   const int n32 = lane & 31, kg = lane >> 5;
   const int n16 = n32 & 15, th = n32 >> 4;  // row within a packed tile, tile of the pair
   const int nblk = a.nblk;
   const int nsteps = (nblk + 3) >> 2;
   const int slots = scale_slots(nblk);
 
-  // this wave's two 32-row groups (each a pair of packed tiles).  Every address of the main
-  // loop is a wave-uniform base (advanced per step on the scalar unit) plus a 32-bit per-lane
-  // byte offset that never changes, so the loads cost no vector instructions.  Nothing is
-  // clamped: activation rows are padded with zero blocks to a whole number of steps, so the
-  // weight blocks read past K (the next tile's, or the slack behind the last plane) and the
-  // scale bytes read past K (slot padding, 127) are multiplied by exact zeros.
-  int tiles[2];  // this lane's packed tile in each group
-  const char* qbase[2];
-  const char* sbase[2];
-  uint32_t qoff[2], soff[2];
+  // Group g of this wave is the pair of packed tiles (t0(g), t0(g) + 1).  Every address of
+  // the main loop is a wave-uniform base (the group's plane and tile pair, advanced per step
+  // on the scalar unit) plus a 32-bit per-lane byte offset that never changes and is the
+  // same for every group, so the loads cost no vector instructions.  Nothing is clamped
+  // along K: activation rows are padded with zero blocks to a whole number of steps, so
+  // the weight blocks read past K (the next tile's, or the slack behind the last plane)
+  // and the scale bytes read past K (slot padding, 127) are multiplied by exact zeros.
+  // Groups past the last tile (ragged last N tile) re-read the last pair; their results
+  // are dropped.
+  auto group_tile = [&](int g) {
+    if (MODE == 0) return nt * (4 * NG) + wv * NG + 2 * (g % (NG / 2));
+    return nt * (8 * NG) + wv * (2 * NG) + 2 * g;
+  };
+  // One buffer descriptor per weight plane; a group's tile pair and the K step go into the
+  // scalar offset of the load, the lane's place within the pair into the vector offset.
+  const ExpertW& w = wd->w;
+  const auto q_rsrc0 = plane_rsrc(MODE == 0 ? w.q_gate : w.q_down);
+  const auto q_rsrc1 = plane_rsrc(MODE == 0 ? w.q_up : w.q_down);
+  const auto s_rsrc0 = plane_rsrc(MODE == 0 ? w.s_gate : w.s_down);
+  const auto s_rsrc1 = plane_rsrc(MODE == 0 ? w.s_up : w.s_down);
+  uint32_t goff_q[NG], goff_s[NG];  // byte offset of the group's tile pair in its planes
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    int t;
-    if (MODE == 0) t = nt * (2 * kMxWaves) + wv * 2 + th;
-    else t = nt * (4 * kMxWaves) + wv * 4 + 2 * s + th;
-    tiles[s] = t;
-    const int tc = min(t, a.ntile - 1);
-    const uint4* qb = MODE == 0 ? (s == 0 ? wd->w.q_gate : wd->w.q_up) : wd->w.q_down;
-    const uint8_t* sb = MODE == 0 ? (s == 0 ? wd->w.s_gate : wd->w.s_up) : wd->w.s_down;
-    qbase[s] = reinterpret_cast<const char*>(qb);
-    sbase[s] = reinterpret_cast<const char*>(sb);
-    qoff[s] = (uint32_t)((((size_t)tc * nblk + kg) * 16 + n16) * 16);  // entry (tile, block kg, row)
-    soff[s] = (uint32_t)scale_index(tc, kg, n16, slots);
+  for (int g = 0; g < NG; ++g) {
+    const int tc = min(group_tile(g), a.ntile - 2);
+    goff_q[g] = (uint32_t)__builtin_amdgcn_readfirstlane(tc * nblk * 256);
+    goff_s[g] = (uint32_t)__builtin_amdgcn_readfirstlane(tc * 256 * slots);
   }
+  const uint32_t qoff = (uint32_t)(((th * nblk + kg) * 16 + n16) * 16);  // entry (tile th, block kg, row)
+  const uint32_t soff = (uint32_t)scale_index(th, kg, n16, slots);
   const int rowblk = mx3_row_blocks(nblk);
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
@@ -130,18 +180,15 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
     aoff[c] = (uint32_t)(((size_t)row * rowblk * kMx3ChunksPerBlock + lc) * 16);
   }
   // LDS destination of copy c of this wave within a stage (wave-uniform)
-  const uint32_t lds_wave = lds0 + (uint32_t)__builtin_amdgcn_readfirstlane(kMxCopies * wv * 64 * 16);
+  const uint32_t lds_wave = lds0 + (uint32_t)(kMxCopies * wv * 64 * 16);
   struct BSet {
-    u32x4 q[2][2];     // [64-wide K chunk of the step][row group]
-    uint32_t s[2][2];  // byte 0 = the block's scale byte (the matrix instruction reads only that byte)
+    u32x4 q[2][NG];     // [64-wide K chunk of the step][row group]
+    uint32_t s[2][NG];  // byte 0 = the block's scale byte (the matrix instruction reads only that byte)
   };
   // The kStepLoads load instructions of step j, one at a time: n < kMxCopies copies a part
-  // of the activation tile into LDS, the next four fetch the weight entries, the last four
-  // the scale bytes.
-  // All loads are inline assembly in the scalar-base form.  Besides saving the address
-  // arithmetic this keeps them out of the compiler's wait tracking, which otherwise drains
-  // the whole queue once per loop iteration over a register it reuses; the explicit count at
-  // the step boundary is what guarantees their arrival.
+  // of the activation tile into LDS, the next 2 NG fetch the weight entries, the last 2 NG
+  // the scale bytes.  The LDS copies are inline assembly (nothing of theirs lives in a
+  // register; the explicit wait at the step boundary guarantees their arrival).
   auto issue_load = [&](int n, int stage, BSet& b, int j) {
     if (n < kMxCopies) {
       const char* abase = reinterpret_cast<const char*>(a.A) + (size_t)j * (4 * kMx3ChunksPerBlock * 16);
@@ -151,53 +198,44 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
                    : "v"(aoff[n]), "s"(abase), "s"(lds)
                    : "memory");
     } else {
-      const int m = (n - kMxCopies) & 3, kc = m >> 1, s = m & 1;
-      if (n < kMxCopies + 4) {
-        const char* base_q = qbase[s] + (size_t)j * 1024 + kc * 512;
-        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(b.q[kc][s]) : "v"(qoff[s]), "s"(base_q) : "memory");
+      // Weights: buffer loads the compiler can see.  Loads hidden in inline assembly would
+      // save its wait bookkeeping, but the register allocator moves values between register
+      // files around the matrix instructions, and a register it moves while an untracked load
+      // is still in flight takes stale data along (seen as rare wrong rows in ragged tiles).
+      const int m = (n - kMxCopies) % (2 * NG), kc = m / NG, g = m % NG;
+      const bool second = MODE == 0 && g >= NG / 2;  // up rows
+      if (n < kMxCopies + 2 * NG) {
+        const uint32_t so = goff_q[g] + (uint32_t)j * 1024u + (uint32_t)kc * 512u;
+        b.q[kc][g] = __builtin_amdgcn_raw_buffer_load_b128(second ? q_rsrc1 : q_rsrc0, qoff, so, 0);
       } else {
-        // a dword load at the byte's own (unaligned) address: the matrix instruction reads
-        // only byte 0 of its scale operand, so no widening instruction is needed
-        const char* base_s = sbase[s] + (size_t)((j & 3) * 64 + 32 * kc) * slots + (j >> 2);
-        asm volatile("global_load_dword %0, %1, %2" : "=v"(b.s[kc][s]) : "v"(soff[s]), "s"(base_s) : "memory");
+        // the block's scale byte (the matrix instruction reads only byte 0 of its scale operand)
+        const uint32_t so = goff_s[g] + (uint32_t)(((j & 3) * 64 + 32 * kc) * slots + (j >> 2));
+        b.s[kc][g] = __builtin_amdgcn_raw_buffer_load_b8(second ? s_rsrc1 : s_rsrc0, soff, so, 0);
       }
     }
   };
-  auto copy_a = [&](int stage, int j) {
-    BSet unused;
+  auto load_all = [&](int stage, BSet& b, int j) {
 #pragma unroll
-    for (int c = 0; c < kMxCopies; ++c) issue_load(c, stage, unused, j);
-  };
-  auto load_b = [&](BSet& b, int j) {
-#pragma unroll
-    for (int n = kMxCopies; n < kMxCopies + 8; ++n) issue_load(n, 0, b, j);
+    for (int n = 0; n < kStepLoads; ++n) issue_load(n, stage, b, j);
   };
 
-  floatx16 acc[2][2];  // [32-token sub-tile][row group]
+  floatx16 acc[2][NG];  // [32-token sub-tile][row group]
 #pragma unroll
   for (int ms = 0; ms < 2; ++ms)
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+    for (int g = 0; g < NG; ++g)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[ms][s][r] = 0.0f;
+      for (int r = 0; r < 16; ++r) acc[ms][g][r] = 0.0f;
 
   const int sw = (n32 >> 1) & 7;
-  // Fragment i = (kc, term, 32-token sub-tile) of a step feeds two matrix instructions
-  // (the two row groups).  Fragments are requested from LDS two ahead of their use, so
-  // the LDS latency is covered by the four matrix instructions in between.
-  // The loads of the step after next are issued one per fragment between the matrix
+  // Fragment i = (kc, term, 32-token sub-tile) of a step feeds NG matrix instructions (the
+  // wave's row groups).  Fragments are requested from LDS two ahead of their use.  The loads
+  // of the step being prefetched are issued a few per fragment between the matrix
   // instructions rather than in a burst at the step boundary: the texture address unit
-  // takes 16 cycles per 64-lane 128-bit load, and a burst of 14 per wave, 8 waves per
-  // compute unit, held every wave at the start of the step for longer than the step's
-  // matrix work.
-  auto compute = [&](const BSet& b, int stage, int j, BSet& bn, int stage_n, int jn) {
+  // takes 16 cycles per 64-lane 128-bit load, and a burst per wave would hold every wave at
+  // the start of the step.
+  auto compute = [&](const BSet& b, int stage, BSet& bn, int stage_n, int jn) {
     const u32x4* at = reinterpret_cast<const u32x4*>(As) + stage * kMxStageChunks;
-    i32x8 bw[2][2];
-#pragma unroll
-    for (int kc = 0; kc < 2; ++kc)
-#pragma unroll
-      for (int s = 0; s < 2; ++s)  // FP4 reads four registers
-        bw[kc][s] = (i32x8)__builtin_shufflevector(b.q[kc][s], b.q[kc][s], 0, 1, 2, 3, -1, -1, -1, -1);
     u32x4 flo[3], fhi[3];
     auto read_frag = [&](int i) {
       const int kc = i / 6, t = (i % 6) >> 1, ms = i & 1;
@@ -212,113 +250,118 @@ __global__ __launch_bounds__(64 * kMxWaves, 8 / kMxWaves) void expert_gemm_mx_ke
     for (int i = 0; i < 12; ++i) {
       const int kc = i / 6, ms = i & 1;
       if (i + 2 < 12) read_frag(i + 2);
-      issue_load(i, stage_n, bn, jn);
-      if (i + 12 < kStepLoads) issue_load(i + 12, stage_n, bn, jn);
+#pragma unroll
+      for (int n = i; n < kStepLoads; n += 12) issue_load(n, stage_n, bn, jn);
       __builtin_amdgcn_sched_barrier(0);
       // FP6 reads the first six registers; fhi[2] (register 6) is the term's scale byte
-      const i32x8 aw = (i32x8)__builtin_shufflevector(flo[i % 3], fhi[i % 3], 0, 1, 2, 3, 4, 5, 6, 7);
-      acc[ms][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aw, bw[kc][0], acc[ms][0], 2, 4, 0,
-                                                                   (int)fhi[i % 3][2], 0, (int)b.s[kc][0]);
-      acc[ms][1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aw, bw[kc][1], acc[ms][1], 2, 4, 0,
-                                                                   (int)fhi[i % 3][2], 0, (int)b.s[kc][1]);
+      i32x8 aw = (i32x8)__builtin_shufflevector(flo[i % 3], fhi[i % 3], 0, 1, 2, 3, 4, 5, 6, 7);
+      // the fragment stays in ordinary vector registers: left to itself the register allocator
+      // parks fragments in accumulation registers that it frees by moving parts of an
+      // accumulator tile out and back around the matrix instructions
+      asm volatile("" : "+v"(aw));
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        // FP4 reads four registers
+        const i32x8 bw = (i32x8)__builtin_shufflevector(b.q[kc][g], b.q[kc][g], 0, 1, 2, 3, -1, -1, -1, -1);
+        acc[ms][g] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(aw, bw, acc[ms][g], 2, 4, 0,
+                                                                     aw[6], 0, (int)b.s[kc][g]);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // Three LDS stages, loads two steps ahead.  A __syncthreads() would drain every
-  // outstanding load (its fence waits for vmcnt(0)), so the step boundary is an explicit
-  // count + bare barrier: a wave's loads of step j are older than the kStepLoads loads of
-  // step j+1, memory counters retire in order, so vmcnt(kStepLoads) means "my part of
-  // step j has landed", and the barrier extends that to the other waves' parts and
-  // tells that every wave is done reading the stage about to be overwritten.
-  constexpr int kWaitStep = (kStepLoads & 15) | (7 << 4) | (15 << 8) | ((kStepLoads >> 4) << 14);
-  // The first two steps are requested and awaited in full before the loop, so that the
-  // loop is entered with nothing in flight and its body is the steady state from the
-  // first iteration on (loads still pending at the loop entry would make the compiler's
-  // own wait insertion fall back to vmcnt(0) inside the loop).
-  BSet bs[3];
-  copy_a(0, 0);
-  load_b(bs[0], 0);
-  copy_a(1, min(1, nsteps - 1));
-  load_b(bs[1], min(1, nsteps - 1));
+  // kStages LDS stages and register sets, loads kAhead steps ahead.  The step boundary is
+  // an explicit wait + bare barrier: everything this wave requested for step j (during step
+  // j - kAhead) has landed once at most (kAhead - 1) steps' worth of its loads are still in
+  // flight (loads retire in order), and the barrier extends that to the other waves' parts
+  // of the activation tile and tells that every wave is done reading the stage about to
+  // be overwritten.
+  constexpr int kInFlight = (kAhead - 1) * kStepLoads;
+  constexpr int kWaitStep = (kInFlight & 15) | (7 << 4) | (15 << 8) | ((kInFlight >> 4) << 14);
+  BSet bs[kStages];
+#pragma unroll
+  for (int u = 0; u < kAhead; ++u) load_all(u, bs[u], min(u, nsteps - 1));
+  // the loop is entered with nothing in flight, so that its body is the steady state from the first iteration on
   __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0)
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int u = 0; u < kAhead; ++u)
 #pragma unroll
     for (int kc = 0; kc < 2; ++kc)
 #pragma unroll
-      for (int g = 0; g < 2; ++g)  // "use" the loaded registers so the compiler, too, knows they have arrived
-        asm volatile("" : "+v"(bs[i].q[kc][g]), "+v"(bs[i].s[kc][g]));
+      for (int g = 0; g < NG; ++g) asm volatile("" : "+v"(bs[u].q[kc][g]), "+v"(bs[u].s[kc][g]));
   __builtin_amdgcn_sched_barrier(0);
   auto step = [&](int u, int jj) {
     __builtin_amdgcn_s_waitcnt(kWaitStep);
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    compute(bs[u], u, jj, bs[(u + 2) % 3], (u + 2) % 3, min(jj + 2, nsteps - 1));
+    compute(bs[u], u, bs[(u + kAhead) % kStages], (u + kAhead) % kStages, min(jj + kAhead, nsteps - 1));
     __builtin_amdgcn_sched_barrier(0);
   };
-  // no control-flow joins between the steps of the steady state
-  for (int j = 0;; j += 3) {
+  static_assert(kStages == 2, "the K loop below alternates two stages");
+  for (int j = 0;; j += 2) {  // (exits in the middle rather than a conditional second step: no join inside the loop)
     step(0, j);
     if (j + 1 >= nsteps) break;
     step(1, j + 1);
     if (j + 2 >= nsteps) break;
-    step(2, j + 2);
-    if (j + 3 >= nsteps) break;
   }
-  // The re-reads requested past the last step are still in flight and the compiler does
-  // not know it (those loads are inline assembly): nothing may follow the loop before
-  // they have landed, or a register they are about to overwrite could be given a new role.
+  // the copies requested past the last step are still in flight: nothing may reuse their LDS before they land
   __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0)
   __builtin_amdgcn_sched_barrier(0);
 
   // epilogue: lane holds weight row n32 of each group; accumulator register r is token
   // (r % 4) + 8 * (r / 4) + 4 * kg of the 32-token sub-tile
   if (MODE == 0) {
-    // bias + activation into LDS as fp32 [token][block = wave][32 + 1], then one thread per
-    // (token, block) re-quantises 32 features to the three-term format
-    __syncthreads();  // the copies issued for the step after the last have landed; all waves are past their reads
-    float* stage = reinterpret_cast<float*>(smem);
-    const int row = tiles[0] * 16 + n16;  // feature
-    const bool rv = tiles[0] < a.ntile && row < a.N;
-    const float bg = rv ? wd->w.b_gate[row] : 0.0f;
-    const float bu = rv ? wd->w.b_up[row] : 0.0f;
+    // bias + activation into this wave's LDS tile as fp32 [token][16 NG features + 1], then
+    // one lane per token re-quantises 32 features at a time to the three-term format
+    __syncthreads();  // the copies issued for the steps after the last have landed; all waves are past their reads
+    float* tile = reinterpret_cast<float*>(smem) + (size_t)wv * kGemmBM * G::kEpiRow;
 #pragma unroll
-    for (int ms = 0; ms < 2; ++ms) {
+    for (int gi = 0; gi < NG / 2; ++gi) {
+      const int row = group_tile(gi) * 16 + n32;  // feature
+      const bool rv = row < a.N;
+      const float bg = rv ? wd->w.b_gate[row] : 0.0f;
+      const float bu = rv ? wd->w.b_up[row] : 0.0f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int tl = ms * 32 + (r & 3) + 8 * (r >> 2) + 4 * kg;
-        // features past N belong to the zero padding of the output rows
-        stage[(tl * kMxWaves + wv) * 33 + n32] =
-            rv ? moe_activation(acc[ms][0][r] + bg, acc[ms][1][r] + bu, a.act_type) : 0.0f;
+      for (int ms = 0; ms < 2; ++ms) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int tl = ms * 32 + (r & 3) + 8 * (r >> 2) + 4 * kg;
+          // features past N belong to the zero padding of the output rows
+          tile[tl * G::kEpiRow + 32 * gi + n32] =
+              rv ? moe_activation(acc[ms][gi][r] + bg, acc[ms][NG / 2 + gi][r] + bu, a.act_type) : 0.0f;
+        }
       }
     }
     __syncthreads();
-    const int tl = threadIdx.x / kMxWaves, blk = threadIdx.x % kMxWaves;
-    const int kb = nt * kMxWaves + blk;
+    const int tl = lane;
     const int out_rowblk = mx3_row_blocks(a.N >> 5);  // the down GEMM reads rows padded to whole steps
-    if (tl < mcount && kb < out_rowblk) {
-      float v[32];
+#pragma unroll 1
+    for (int bi = 0; bi < NG / 2; ++bi) {
+      const int kb = (nt * (4 * NG) + wv * NG) / 2 + bi;
+      if (tl < mcount && kb < out_rowblk) {
+        float v[32];
 #pragma unroll
-      for (int i = 0; i < 32; ++i) v[i] = stage[(tl * kMxWaves + blk) * 33 + i];
-      u32x4 out[kMx3ChunksPerBlock];
-      mx3_quantize_block(v, out);
-      u32x4* o = a.act_out + ((size_t)(base + tl) * out_rowblk + kb) * kMx3ChunksPerBlock;
+        for (int i = 0; i < 32; ++i) v[i] = tile[tl * G::kEpiRow + 32 * bi + i];
+        u32x4 out[kMx3ChunksPerBlock];
+        mx3_quantize_block(v, out);
+        u32x4* o = a.act_out + ((size_t)(base + tl) * out_rowblk + kb) * kMx3ChunksPerBlock;
 #pragma unroll
-      for (int c = 0; c < kMx3ChunksPerBlock; ++c) o[c] = out[c];
+        for (int c = 0; c < kMx3ChunksPerBlock; ++c) o[c] = out[c];
+      }
     }
   } else {
 #pragma unroll
-    for (int ms = 0; ms < 2; ++ms) {
+    for (int g = 0; g < NG; ++g) {
+      const int row = group_tile(g) * 16 + n32;
+      if (row >= a.N) continue;
+      const float bd = wd->w.b_down[row];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int tl = ms * 32 + (r & 3) + 8 * (r >> 2) + 4 * kg;
-        if (tl >= mcount) continue;
-        const size_t p = (size_t)(base + tl);
+      for (int ms = 0; ms < 2; ++ms) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          const int row = tiles[s] * 16 + n16;
-          if (tiles[s] < a.ntile && row < a.N) a.y_out[p * (size_t)a.N + row] = acc[ms][s][r] + wd->w.b_down[row];
+        for (int r = 0; r < 16; ++r) {
+          const int tl = ms * 32 + (r & 3) + 8 * (r >> 2) + 4 * kg;
+          if (tl >= mcount) continue;
+          a.y_out[(size_t)(base + tl) * (size_t)a.N + row] = acc[ms][g][r] + bd;
         }
       }
     }

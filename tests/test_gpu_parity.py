@@ -440,6 +440,22 @@ def test_prefill_120b_skewed_4096_tokens(lib, oracle):
     assert 0.4 < hot < 0.75, hot  # +2.0 logit offset on logits of std ~1.1
 
 
+@pytest.mark.parametrize("T,seed", [(512, 80), (1024, 79)])
+def test_prefill_repeatable_with_many_small_experts(lib, T, seed):
+    """128 experts with a skewed router at a few hundred tokens: most experts hold a handful
+    of tokens, so most M tiles are ragged and their padding rows repeat the last token --
+    the timing in which a load that the compiler does not track, or a register moved while
+    such a load is in flight, shows as a few wrong rows in some runs.  Every run must give
+    the same bits."""
+    L = synth.LayerInputs(128, 4, 2880, 2880, seed=seed, hot_experts=8)
+    hidden = synth.hidden_states(T, L.H, seed=T + 3)
+    with build_layer(lib, L, device_weights=True) as layer:
+        first = layer.forward(hidden)
+        assert np.all(np.isfinite(first))
+        for _ in range(11):
+            assert nbits_differ(layer.forward(hidden), first) == 0
+
+
 def test_prefill_ragged_small_shape(lib, oracle):
     """Token counts that are not multiples of the 64-token M tile, N not a multiple of
     the 128-feature N tile, K not a multiple of the 128-element K step."""
