@@ -59,6 +59,8 @@ SIGNATURES = {
     "csk_layer_dequant": (C.c_int, [_P, _I64, C.c_int, _P]),
     "csk_layer_export": (C.c_int, [_P, _I64, C.c_int, _P]),
     "csk_gguf_open": (C.c_int, [C.c_char_p, C.POINTER(_P)]),
+    "csk_gguf_open_shards": (C.c_int, [C.POINTER(C.c_char_p), _I64, C.POINTER(_P)]),
+    "csk_gguf_tensor_shard": (C.c_int, [_P, C.c_char_p, C.POINTER(C.c_int32)]),
     "csk_gguf_close": (None, [_P]),
     "csk_gguf_tensor_count": (C.c_int, [_P, C.POINTER(_I64)]),
     "csk_gguf_tensor_name": (C.c_int, [_P, _I64, C.c_char_p, C.c_size_t]),
@@ -378,12 +380,17 @@ class Library:
 
 
 class Gguf:
-    """An open GGUF file (csk_gguf_*): metadata and tensor table, no GPU needed."""
+    """An open GGUF checkpoint (csk_gguf_*): metadata and tensor table, no GPU needed.
+    `path` is one file, or the list of shard files of a split checkpoint."""
 
     def __init__(self, lib, path):
         self.lib = lib
         self.h = _P()
-        lib.check(lib.dll.csk_gguf_open(os.fsencode(path), C.byref(self.h)))
+        if isinstance(path, (list, tuple)):
+            arr = (C.c_char_p * len(path))(*[os.fsencode(p) for p in path])
+            lib.check(lib.dll.csk_gguf_open_shards(arr, len(path), C.byref(self.h)))
+        else:
+            lib.check(lib.dll.csk_gguf_open(os.fsencode(path), C.byref(self.h)))
 
     def close(self):
         if self.h:
@@ -412,6 +419,11 @@ class Gguf:
         self.lib.check(self.lib.dll.csk_gguf_tensor_info(self.h, name.encode(), C.byref(t), C.byref(nd),
                                                          dims, C.byref(off), C.byref(nb)))
         return dict(type=t.value, dims=list(dims)[:nd.value], offset=off.value, nbytes=nb.value)
+
+    def tensor_shard(self, name):
+        sh = C.c_int32()
+        self.lib.check(self.lib.dll.csk_gguf_tensor_shard(self.h, name.encode(), C.byref(sh)))
+        return sh.value
 
     def get_u32(self, key):
         v = C.c_uint32()

@@ -8,6 +8,7 @@
 //   src/llm/moe_weight_provider.cpp:75-225  expert slice = tensor offset + e * slice bytes,
 //                                           shape reversal (GGUF lists the fastest dim first)
 //   src/llm/llm_engine.cpp:135-225, 262-267, 714-753  architecture keys and tensor names
+//   src/gguf/gguf_multi_loader.cpp:25-76  split checkpoints: shards in order, duplicate names refused
 // Differences: every scalar array type is accepted (the reference rejects some), and
 // general.alignment is honoured when present (the reference assumes 32, the default).
 #include <stdint.h>
@@ -47,8 +48,9 @@ size_t scalar_size(uint32_t t) {
 struct TensorInfo {
   uint32_t type = 0;
   std::vector<uint64_t> dims;  // GGUF order: fastest-varying first
-  uint64_t offset = 0;         // absolute file offset
+  uint64_t offset = 0;         // absolute offset in its shard's file
   uint64_t nbytes = 0;
+  uint32_t shard = 0;          // which file of a split checkpoint
 };
 
 struct Value {
@@ -61,12 +63,20 @@ struct Value {
 
 }  // namespace
 
-struct csk_gguf {
+// One file of a checkpoint.
+struct GgufShard {
   FILE* fp = nullptr;
   const uint8_t* map = nullptr;  // the file mapped read-only (tensor data is handed to the GPU copies from here); null: fread
   size_t map_len = 0;
   uint32_t version = 0;
   uint64_t data_start = 0, file_size = 0;
+};
+
+// A checkpoint: one file, or the shards of a split one merged the way gguf_multi_loader
+// does (src/gguf/gguf_multi_loader.cpp:25-76): tensors keep the shard they came from, a
+// metadata key is answered by the first shard that has it.
+struct csk_gguf {
+  std::vector<GgufShard> shards;
   std::unordered_map<std::string, Value> meta;
   std::unordered_map<std::string, TensorInfo> tensors;
   std::vector<std::string> order;
@@ -147,92 +157,133 @@ const TensorInfo* find(const csk_gguf* g, const std::string& name) {
   return it == g->tensors.end() ? nullptr : &it->second;
 }
 
-bool read_at(csk_gguf* g, uint64_t off, void* dst, size_t n) {
-  if (off + n > g->file_size) return false;
-  if (fseeko(g->fp, (off_t)off, SEEK_SET) != 0) return false;
-  return rd(g->fp, dst, n);
+// [off, off + n) lies inside a file of `size` bytes (no sum that could wrap)
+bool in_file(uint64_t off, uint64_t n, uint64_t size) { return off <= size && n <= size - off; }
+
+bool read_at(GgufShard& sh, uint64_t off, void* dst, size_t n) {
+  if (!in_file(off, n, sh.file_size)) return false;
+  if (fseeko(sh.fp, (off_t)off, SEEK_SET) != 0) return false;
+  return rd(sh.fp, dst, n);
 }
 
 // n bytes of the file at off without a copy: a pointer into the read-only mapping (made at
 // the first call), or, where the file cannot be mapped, into `fallback` filled by fread.
-const uint8_t* view_at(csk_gguf* g, uint64_t off, size_t n, std::vector<uint8_t>& fallback) {
-  if (off + n > g->file_size) return nullptr;
-  if (!g->map && g->map_len == 0) {
-    void* m = mmap(nullptr, (size_t)g->file_size, PROT_READ, MAP_PRIVATE, fileno(g->fp), 0);
-    g->map_len = (size_t)g->file_size;  // also marks the attempt
-    if (m != MAP_FAILED) g->map = static_cast<const uint8_t*>(m);
+const uint8_t* view_at(GgufShard& sh, uint64_t off, size_t n, std::vector<uint8_t>& fallback) {
+  if (!in_file(off, n, sh.file_size)) return nullptr;
+  if (!sh.map && sh.map_len == 0) {
+    void* m = mmap(nullptr, (size_t)sh.file_size, PROT_READ, MAP_PRIVATE, fileno(sh.fp), 0);
+    sh.map_len = (size_t)sh.file_size;  // also marks the attempt
+    if (m != MAP_FAILED) sh.map = static_cast<const uint8_t*>(m);
   }
-  if (g->map) return g->map + off;
+  if (sh.map) return sh.map + off;
   fallback.resize(n);
-  return read_at(g, off, fallback.data(), n) ? fallback.data() : nullptr;
+  return read_at(sh, off, fallback.data(), n) ? fallback.data() : nullptr;
 }
+
+// the slice [rel, rel + n) of tensor t, checked against the tensor's own extent
+bool slice_in_tensor(const TensorInfo& t, uint64_t rel, uint64_t n) { return in_file(rel, n, t.nbytes); }
 
 }  // namespace
 
-extern "C" int csk_gguf_open(const char* path, csk_gguf** out) {
-  if (!path || !out) return fail(CSK_ERR_ARG, "csk_gguf_open: null argument");
-  *out = nullptr;
+namespace {
+// Parses one file into shard `idx` of g (header, key/value section, tensor table).
+int parse_shard(csk_gguf* g, uint32_t idx, const char* path) {
   FILE* fp = fopen(path, "rb");
   if (!fp) return fail(CSK_ERR_ARG, std::string("csk_gguf_open: cannot open ") + path);
-  csk_gguf* g = new csk_gguf;
-  g->fp = fp;
-  auto bad = [&](const std::string& why) {
-    fclose(fp);
-    delete g;
-    return fail(CSK_ERR_ARG, "csk_gguf_open: " + why);
-  };
+  g->shards.emplace_back();
+  GgufShard& sh = g->shards.back();
+  sh.fp = fp;
+  auto bad = [&](const std::string& why) { return fail(CSK_ERR_ARG, "csk_gguf_open: " + why); };
   fseeko(fp, 0, SEEK_END);
-  g->file_size = (uint64_t)ftello(fp);
+  sh.file_size = (uint64_t)ftello(fp);
   fseeko(fp, 0, SEEK_SET);
   uint32_t magic = 0;
   uint64_t n_tensors = 0, n_kv = 0;
   if (!rd(fp, &magic, 4) || magic != kMagic) return bad("not a GGUF file (bad magic)");
-  if (!rd(fp, &g->version, 4) || g->version < 2 || g->version > 3) return bad("unsupported GGUF version");
+  if (!rd(fp, &sh.version, 4) || sh.version < 2 || sh.version > 3) return bad("unsupported GGUF version");
   if (!rd(fp, &n_tensors, 8) || !rd(fp, &n_kv, 8)) return bad("truncated header");
-  if (n_tensors > g->file_size || n_kv > g->file_size) return bad("implausible header counts");
+  if (n_tensors > sh.file_size || n_kv > sh.file_size) return bad("implausible header counts");
+  std::unordered_map<std::string, Value> meta;
   for (uint64_t i = 0; i < n_kv; ++i) {
     std::string key;
     uint32_t type;
-    if (!rd_str(fp, key, g->file_size) || !rd(fp, &type, 4)) return bad("truncated metadata");
+    if (!rd_str(fp, key, sh.file_size) || !rd(fp, &type, 4)) return bad("truncated metadata");
     Value v;
-    const int r = read_value(fp, type, v, g->file_size);
+    const int r = read_value(fp, type, v, sh.file_size);
     if (r == 1) return bad("truncated metadata value of '" + key + "'");
     if (r == 2) return bad("unknown metadata type of '" + key + "'");
-    g->meta[key] = std::move(v);
+    meta[key] = std::move(v);
   }
+  std::vector<std::string> names;
   for (uint64_t i = 0; i < n_tensors; ++i) {
     std::string name;
     uint32_t nd;
     TensorInfo ti;
-    if (!rd_str(fp, name, g->file_size) || !rd(fp, &nd, 4) || nd > 4) return bad("truncated tensor table");
+    if (!rd_str(fp, name, sh.file_size) || !rd(fp, &nd, 4) || nd > 4) return bad("truncated tensor table");
     ti.dims.resize(nd);
     for (uint32_t d = 0; d < nd; ++d)
       if (!rd(fp, &ti.dims[d], 8)) return bad("truncated tensor table");
     if (!rd(fp, &ti.type, 4) || !rd(fp, &ti.offset, 8)) return bad("truncated tensor table");
     uint64_t ne = 1, be = 1, bb = 0;
-    for (uint64_t d : ti.dims) ne *= d;
-    if (type_geometry(ti.type, &be, &bb)) ti.nbytes = (ne + be - 1) / be * bb;
-    g->order.push_back(name);
+    for (uint64_t d : ti.dims)
+      if (__builtin_mul_overflow(ne, d, &ne)) return bad("tensor '" + name + "': element count overflows");
+    if (type_geometry(ti.type, &be, &bb)) {
+      const uint64_t blocks = ne / be + (ne % be != 0);
+      if (__builtin_mul_overflow(blocks, bb, &ti.nbytes)) return bad("tensor '" + name + "': size overflows");
+    }
+    ti.shard = idx;
+    if (g->tensors.count(name))  // gguf_multi_loader.cpp:64-67
+      return bad("Duplicate tensor name '" + name + "' in shard " + std::to_string(idx));
+    names.push_back(name);
     g->tensors[name] = std::move(ti);
   }
   uint64_t align = 32;
-  auto it = g->meta.find("general.alignment");
-  if (it != g->meta.end() && it->second.u >= 1 && it->second.u <= (1u << 20)) align = it->second.u;
+  auto it = meta.find("general.alignment");
+  if (it != meta.end() && it->second.u >= 1 && it->second.u <= (1u << 20)) align = it->second.u;
   const uint64_t pos = (uint64_t)ftello(fp);
-  g->data_start = (pos + align - 1) / align * align;
-  for (auto& kv : g->tensors) {
-    kv.second.offset += g->data_start;
-    if (kv.second.offset + kv.second.nbytes > g->file_size)
-      return bad("tensor '" + kv.first + "' reaches past the end of the file");
+  sh.data_start = (pos + align - 1) / align * align;
+  for (const std::string& name : names) {
+    TensorInfo& ti = g->tensors[name];
+    // relative offset -> absolute; both the sum and the tensor's end are checked without wrapping
+    if (sh.data_start > sh.file_size || ti.offset > sh.file_size - sh.data_start ||
+        !in_file(ti.offset + sh.data_start, ti.nbytes, sh.file_size))
+      return bad("tensor '" + name + "' reaches past the end of the file");
+    ti.offset += sh.data_start;
+    g->order.push_back(name);
+  }
+  for (auto& kv : meta)  // a key is answered by the first shard that has it (gguf_multi_loader.cpp:86-92)
+    if (!g->meta.count(kv.first)) g->meta[kv.first] = std::move(kv.second);
+  return CSK_OK;
+}
+}  // namespace
+
+extern "C" int csk_gguf_open_shards(const char* const* paths, int64_t n_paths, csk_gguf** out) {
+  if (!paths || !out || n_paths < 1) return fail(CSK_ERR_ARG, "csk_gguf_open: No GGUF files specified");
+  *out = nullptr;
+  csk_gguf* g = new csk_gguf;
+  g->shards.reserve((size_t)n_paths);
+  for (int64_t i = 0; i < n_paths; ++i) {
+    const int rc = paths[i] ? parse_shard(g, (uint32_t)i, paths[i]) : fail(CSK_ERR_ARG, "csk_gguf_open: null path");
+    if (rc != CSK_OK) {
+      csk_gguf_close(g);
+      return rc;
+    }
   }
   *out = g;
   return CSK_OK;
 }
 
+extern "C" int csk_gguf_open(const char* path, csk_gguf** out) {
+  if (!path || !out) return fail(CSK_ERR_ARG, "csk_gguf_open: null argument");
+  return csk_gguf_open_shards(&path, 1, out);
+}
+
 extern "C" void csk_gguf_close(csk_gguf* g) {
   if (!g) return;
-  if (g->map) munmap(const_cast<uint8_t*>(g->map), g->map_len);
-  if (g->fp) fclose(g->fp);
+  for (GgufShard& sh : g->shards) {
+    if (sh.map) munmap(const_cast<uint8_t*>(sh.map), sh.map_len);
+    if (sh.fp) fclose(sh.fp);
+  }
   delete g;
 }
 
@@ -261,6 +312,14 @@ extern "C" int csk_gguf_tensor_info(const csk_gguf* g, const char* name, uint32_
     for (size_t d = 0; d < 4; ++d) dims4[d] = d < t->dims.size() ? t->dims[d] : 1;
   if (file_offset) *file_offset = t->offset;
   if (nbytes) *nbytes = t->nbytes;
+  return CSK_OK;
+}
+
+extern "C" int csk_gguf_tensor_shard(const csk_gguf* g, const char* name, int32_t* shard) {
+  if (!g || !name || !shard) return fail(CSK_ERR_ARG, "csk_gguf_tensor_shard: null argument");
+  const TensorInfo* t = find(g, name);
+  if (!t) return fail(CSK_ERR_ARG, std::string("Tensor not found: ") + name);
+  *shard = (int32_t)t->shard;
   return CSK_OK;
 }
 
@@ -354,13 +413,13 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
   if (rc != CSK_OK) return bail(rc, "");
 
   std::vector<float> gw((size_t)E * H), gb;
-  if (!read_at(g, tg->offset, gw.data(), gw.size() * 4)) return bail(CSK_ERR_ARG, "short read: " + p + ".ffn_gate_inp.weight");
+  if (!slice_in_tensor(*tg, 0, gw.size() * 4) || !read_at(g->shards[tg->shard], tg->offset, gw.data(), gw.size() * 4)) return bail(CSK_ERR_ARG, "short read: " + p + ".ffn_gate_inp.weight");
   const TensorInfo* tgb = find(g, p + ".ffn_gate_inp.bias");
   if (tgb) {
     if (tgb->type != kGgmlF32 || tgb->dims.size() != 1 || tgb->dims[0] != E)
       return bail(CSK_ERR_ARG, p + ".ffn_gate_inp.bias: expected F32 [experts]");
     gb.resize(E);
-    if (!read_at(g, tgb->offset, gb.data(), (size_t)E * 4)) return bail(CSK_ERR_ARG, "short read: " + p + ".ffn_gate_inp.bias");
+    if (!read_at(g->shards[tgb->shard], tgb->offset, gb.data(), (size_t)E * 4)) return bail(CSK_ERR_ARG, "short read: " + p + ".ffn_gate_inp.bias");
   }
   rc = csk_layer_set_router(L, gw.data(), tgb ? gb.data() : nullptr);
   if (rc != CSK_OK) return bail(rc, "");
@@ -390,9 +449,13 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
   for (uint32_t e = 0; e < E; ++e) {
     const uint8_t* wp[3];
     for (int i = 0; i < 3; ++i) {
-      wp[i] = view_at(g, tw[i]->offset + (uint64_t)e * sl[i], sl[i], w[i]);
+      // the slice must lie inside the tensor as the table describes it, not merely inside the file
+      wp[i] = slice_in_tensor(*tw[i], (uint64_t)e * sl[i], sl[i])
+                  ? view_at(g->shards[tw[i]->shard], tw[i]->offset + (uint64_t)e * sl[i], sl[i], w[i])
+                  : nullptr;
       if (!wp[i]) return bail(CSK_ERR_ARG, "short read: " + p + wn[i]);
-      if (tb[i] && !read_at(g, tb[i]->offset + (uint64_t)e * bl[i] * 4, b[i].data(), bl[i] * 4))
+      if (tb[i] && (!slice_in_tensor(*tb[i], (uint64_t)e * bl[i] * 4, bl[i] * 4) ||
+                    !read_at(g->shards[tb[i]->shard], tb[i]->offset + (uint64_t)e * bl[i] * 4, b[i].data(), bl[i] * 4)))
         return bail(CSK_ERR_ARG, "short read: " + p + bn[i]);
     }
     const float* bp[3] = {tb[0] ? b[0].data() : nullptr, tb[1] ? b[1].data() : nullptr,
@@ -412,7 +475,7 @@ extern "C" int csk_layer_from_gguf(csk_gguf* g, int64_t block, csk_layer** out) 
     if (tn->type != kGgmlF32 || tn->dims.size() != 1 || tn->dims[0] != H)
       return bail(CSK_ERR_ARG, p + "." + norm_name + ": expected F32 [hidden]");
     std::vector<float> nw(H);
-    if (!read_at(g, tn->offset, nw.data(), (size_t)H * 4)) return bail(CSK_ERR_ARG, "short read: " + p + "." + norm_name);
+    if (!read_at(g->shards[tn->shard], tn->offset, nw.data(), (size_t)H * 4)) return bail(CSK_ERR_ARG, "short read: " + p + "." + norm_name);
     float eps = 1e-5f;  // graph_builder.h:154
     rc = csk_layer_set_norm(L, nw.data(), eps);
     if (rc != CSK_OK) return bail(rc, "");

@@ -185,9 +185,15 @@ int csk_layer_export_f16(const csk_layer* L, int64_t e, int which, uint16_t* hal
 /* ---------------------------------------------------------------- GGUF ingest
  * Reads a GGUF file's key/value section and tensor table (no tensor data) --
  * gguf_loader::load, src/gguf/gguf_loader.cpp:383-518.  Needs no GPU and no
- * csk_init.  One file; split (sharded) checkpoints are opened shard by shard. */
+ * csk_init. */
 typedef struct csk_gguf csk_gguf;
 int csk_gguf_open(const char* path, csk_gguf** out);
+/* A split checkpoint: the shards in order, merged as gguf_multi_loader::load does
+ * (src/gguf/gguf_multi_loader.cpp:25-76, used by src/llm/moe_weight_provider.cpp:75-100):
+ * a tensor belongs to the shard that lists it (a name in two shards is an error), a metadata
+ * key is answered by the first shard that has it.  csk_layer_from_gguf then reads every
+ * tensor from its own shard. */
+int csk_gguf_open_shards(const char* const* paths, int64_t n_paths, csk_gguf** out);
 void csk_gguf_close(csk_gguf* g);
 int csk_gguf_tensor_count(const csk_gguf* g, int64_t* n);
 int csk_gguf_tensor_name(const csk_gguf* g, int64_t index, char* buf, size_t cap);
@@ -195,6 +201,8 @@ int csk_gguf_tensor_name(const csk_gguf* g, int64_t index, char* buf, size_t cap
  * with 1), absolute file offset of the data, size in bytes (0: unknown type). */
 int csk_gguf_tensor_info(const csk_gguf* g, const char* name, uint32_t* ggml_type, int32_t* n_dims,
                          uint64_t* dims4, uint64_t* file_offset, uint64_t* nbytes);
+/* gguf_multi_loader::tensor_info::shard_idx: which file of a split checkpoint holds the tensor (0 for a single file) */
+int csk_gguf_tensor_shard(const csk_gguf* g, const char* name, int32_t* shard);
 /* gguf_loader::get_uint32 / get_string (any integer width is accepted) */
 int csk_gguf_get_u32(const csk_gguf* g, const char* key, uint32_t* value);
 int csk_gguf_get_str(const csk_gguf* g, const char* key, char* buf, size_t cap);

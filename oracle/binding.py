@@ -311,3 +311,67 @@ class RefCodec:
     def fp32_to_fp16(self, x):
         x = np.ascontiguousarray(x, np.float32).reshape(-1)
         return np.array([self.dll.ref_fp32_to_fp16(float(v)) for v in x], np.uint16)
+
+
+class RefGguf:
+    """The reference's own GGUF readers (gguf_loader / gguf_multi_loader), when oracle/_ref
+    was built.  `paths`: one file or the shards of a split checkpoint."""
+
+    def __init__(self, paths):
+        path = os.path.join(_HERE, "_ref", "libref_gguf.so")
+        if not os.path.exists(path):
+            raise FileNotFoundError(path)
+        self.dll = C.CDLL(path)
+        self.dll.ref_gguf_open.restype = C.c_void_p
+        self.dll.ref_gguf_open.argtypes = [C.POINTER(C.c_char_p), C.c_int64]
+        self.dll.ref_gguf_close.argtypes = [C.c_void_p]
+        self.dll.ref_gguf_tensor_count.restype = C.c_int64
+        self.dll.ref_gguf_tensor_count.argtypes = [C.c_void_p]
+        self.dll.ref_gguf_version.restype = C.c_uint32
+        self.dll.ref_gguf_version.argtypes = [C.c_void_p]
+        self.dll.ref_gguf_tensor_name.argtypes = [C.c_void_p, C.c_int64, C.c_char_p, C.c_size_t]
+        self.dll.ref_gguf_tensor_info.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(C.c_int32),
+                                                  C.POINTER(C.c_uint64), C.POINTER(C.c_uint64),
+                                                  C.POINTER(C.c_uint64), C.POINTER(C.c_int32)]
+        self.dll.ref_gguf_get_u32.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_uint32)]
+        self.dll.ref_gguf_get_str.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_size_t]
+        if isinstance(paths, (str, bytes, os.PathLike)):
+            paths = [paths]
+        arr = (C.c_char_p * len(paths))(*[os.fsencode(p) for p in paths])
+        self.h = self.dll.ref_gguf_open(arr, len(paths))
+
+    @property
+    def loaded(self):
+        return bool(self.h)
+
+    def close(self):
+        if self.h:
+            self.dll.ref_gguf_close(self.h)
+            self.h = None
+
+    def version(self):
+        return self.dll.ref_gguf_version(self.h)
+
+    def tensor_names(self):
+        buf = C.create_string_buffer(512)
+        out = []
+        for i in range(self.dll.ref_gguf_tensor_count(self.h)):
+            assert self.dll.ref_gguf_tensor_name(self.h, i, buf, 512) == 0
+            out.append(buf.value.decode())
+        return out
+
+    def tensor_info(self, name):
+        t, nd, off, nb, sh = C.c_uint32(), C.c_int32(), C.c_uint64(), C.c_uint64(), C.c_int32()
+        dims = (C.c_uint64 * 4)()
+        if self.dll.ref_gguf_tensor_info(self.h, name.encode(), C.byref(t), C.byref(nd), dims, C.byref(off),
+                                         C.byref(nb), C.byref(sh)) != 0:
+            return None
+        return dict(type=t.value, dims=list(dims)[:nd.value], offset=off.value, nbytes=nb.value, shard=sh.value)
+
+    def get_u32(self, key):
+        v = C.c_uint32()
+        return v.value if self.dll.ref_gguf_get_u32(self.h, key.encode(), C.byref(v)) == 0 else None
+
+    def get_str(self, key):
+        buf = C.create_string_buffer(1024)
+        return buf.value.decode() if self.dll.ref_gguf_get_str(self.h, key.encode(), buf, 1024) == 0 else None

@@ -238,3 +238,29 @@ def test_layer_from_gguf_kquant_experts(lib, oracle, tmp_path):
                                L.b_gate, L.b_down, norm_w=L.norm_w, norm_eps=1e-5)
     assert np.all(np.isfinite(want))
     assert_layer_close(got, want)
+
+
+@pytest.mark.gpu
+def test_layer_from_split_checkpoint_equals_single_file(lib, tmp_path):
+    """A block whose tensors are spread over two shard files (gguf_multi_loader,
+    moe_weight_provider.cpp:75-100): every tensor is read from its own shard, and the layer is
+    bit-identical to the one built from a single file."""
+    E, k, H, F = 6, 2, 96, 160
+    L = synth.LayerInputs(E, k, H, F, seed=31, with_norm=True)
+    tensors = gw.moe_block_tensors(L, 0)
+    one = str(tmp_path / "one.gguf")
+    gw.write_gguf(one, _meta(E=E, k=k), tensors)
+    first = [t for t in tensors if "ffn_up" in t[0] or "gate_inp" in t[0]]
+    second = [t for t in tensors if t not in first]
+    a, b = str(tmp_path / "s-00001-of-00002.gguf"), str(tmp_path / "s-00002-of-00002.gguf")
+    gw.write_gguf(a, _meta(E=E, k=k), [("pad.weight", gw.GGML_F32, [7], np.zeros(7, np.float32).tobytes())] + first)
+    gw.write_gguf(b, [("general.architecture", gw.STR, "gpt-oss")], second)
+    hidden = synth.hidden_states(9, H, seed=5)
+    flags = capi.FWD_RMSNORM | capi.FWD_RESIDUAL
+    with lib.gguf(one) as g1, lib.gguf([a, b]) as g2:
+        assert g2.tensor_shard("blk.0.ffn_down_exps.weight") == 1 and g2.tensor_shard("blk.0.ffn_up_exps.weight") == 0
+        with g1.layer(0) as l1, g2.layer(0) as l2:
+            for e in (0, E - 1):
+                for which in range(3):
+                    assert np.array_equal(l2.export(e, which), L.blocks(e, which))
+            assert nbits_differ(l2.forward(hidden, flags), l1.forward(hidden, flags)) == 0
