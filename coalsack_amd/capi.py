@@ -43,6 +43,7 @@ SIGNATURES = {
     "csk_mxfp4_export": (C.c_int, [_P, _P]),
     "csk_f16_upload": (C.c_int, [_P, _I64, _I64, C.POINTER(_P)]),
     "csk_f16_upload_ggml": (C.c_int, [C.c_int, _P, _I64, _I64, C.POINTER(_P)]),
+    "csk_f16_upload_f32": (C.c_int, [_P, _I64, _I64, C.POINTER(_P)]),
     "csk_f16_free": (None, [_P]),
     "csk_f16_export": (C.c_int, [_P, _P]),
     "csk_layer_create": (C.c_int, [_I64, _I64, _I64, _I64, C.POINTER(_P)]),
@@ -88,6 +89,8 @@ SIGNATURES = {
     "csk_expert_merge": (C.c_int, [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]),
     "csk_rmsnorm": (C.c_int, [_P, _P, _P, _I64, _I64, C.c_float]),
     "csk_add": (C.c_int, [_P, _P, _P, _I64]),
+    "csk_add_broadcast": (C.c_int, [_P, _P, C.c_int, _P, _P, C.c_int, C.c_int, _P]),
+    "csk_moe_router_f64": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P, _P]),
 }
 
 
@@ -240,6 +243,13 @@ class Library:
         self.check(self.dll.csk_f16_upload(_ptr(w), rows, K, C.byref(h)))
         return h
 
+    def f16_upload_f32(self, w):
+        """fp32 [rows, K] weights kept as two fp16 terms (csk_f16_upload_f32)."""
+        w = _f32(w)
+        h = _P()
+        self.check(self.dll.csk_f16_upload_f32(_ptr(w), w.shape[0], w.shape[1], C.byref(h)))
+        return h
+
     def f16_upload_ggml(self, ggml_type, data, rows, K):
         """data: uint8 stream of a [rows, K] matrix stored as ggml F16 (1), Q4_K (12) or Q6_K (14)."""
         data = _u8(data)
@@ -277,12 +287,13 @@ class Library:
         return None if empty.value else out
 
     def dense_ffn_f16(self, hidden, w_gate, w_up, w_down, b_gate=None, b_up=None, b_down=None):
-        """dense_ffn_node with float16 weights [F,H], [F,H], [H,F]; uploads them for the call."""
+        """dense_ffn_node with float16 (or float32) weights [F,H], [F,H], [H,F]; uploads them for the call."""
         hidden = _f32(hidden)
         b_gate, b_up, b_down = _f32(b_gate), _f32(b_up), _f32(b_down)
         T, H = hidden.shape
         F = w_gate.shape[0]
-        hs = [self.f16_upload(w) for w in (w_gate, w_up, w_down)]
+        up = self.f16_upload_f32 if w_gate.dtype == np.float32 else self.f16_upload
+        hs = [up(w) for w in (w_gate, w_up, w_down)]
         try:
             out = np.empty((T, H), np.float32)
             self.check(self.dll.csk_dense_ffn_f16(_ptr(hidden), T, H, F, hs[0], hs[1], hs[2], _ptr(b_gate),
@@ -293,10 +304,10 @@ class Library:
         return out
 
     def matmul_transpose_f16(self, a, w):
-        """a [M,K] f32 x w [N,K]^T (float16) -> [M,N]; uploads w for the call."""
+        """a [M,K] f32 x w [N,K]^T (float16 or float32) -> [M,N]; uploads w for the call."""
         a = _f32(a)
         M, K = a.shape
-        h = self.f16_upload(w)
+        h = self.f16_upload_f32(w) if w.dtype == np.float32 else self.f16_upload(w)
         try:
             out = np.empty((M, w.shape[0]), np.float32)
             self.check(self.dll.csk_matmul_transpose_f16(_ptr(a), M, K, h, _ptr(out)))
@@ -312,6 +323,36 @@ class Library:
         out = np.empty((T, k, 2), np.float32)
         self.check(self.dll.csk_moe_router(_ptr(hidden), T, H, _ptr(gate_w), E, _ptr(gate_b), k,
                                            int(sigmoid), _ptr(out)))
+        return out
+
+    def moe_router_f64(self, hidden, gate_w, gate_b, k, sigmoid=False, want_logits=False):
+        """moe_router_node on float64 inputs: float32 pairs [T,k,2] (and the float64 logits)."""
+        hidden = np.ascontiguousarray(hidden, np.float64)
+        gate_w = np.ascontiguousarray(gate_w, np.float64)
+        gate_b = _f32(gate_b)
+        T, H = hidden.shape
+        E = gate_w.shape[0]
+        out = np.empty((T, k, 2), np.float32)
+        logits = np.empty((T, E), np.float64) if want_logits else None
+        self.check(self.dll.csk_moe_router_f64(_ptr(hidden), T, H, _ptr(gate_w), E, _ptr(gate_b), k,
+                                               int(sigmoid), _ptr(out), _ptr(logits)))
+        return (out, logits) if want_logits else out
+
+    ADD_DTYPES = {np.dtype(np.float32): 0, np.dtype(np.float64): 1, np.dtype(np.int32): 2, np.dtype(np.int64): 3}
+
+    def add_broadcast(self, a, b):
+        """add_node with broadcasting; both arrays float32, float64, int32 or int64."""
+        a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+        if a.dtype != b.dtype:
+            raise ValueError("add: input dtype mismatch")
+        sa, sb = np.array(a.shape, np.int64), np.array(b.shape, np.int64)
+        try:
+            shape = np.broadcast_shapes(a.shape, b.shape)
+        except ValueError:
+            shape = (0,)
+        out = np.empty(shape, a.dtype)
+        self.check(self.dll.csk_add_broadcast(_ptr(a), _ptr(sa), a.ndim, _ptr(b), _ptr(sb), b.ndim,
+                                              self.ADD_DTYPES[a.dtype], _ptr(out)))
         return out
 
     def moe_router_logits(self, hidden, gate_w, gate_b):

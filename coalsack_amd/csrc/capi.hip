@@ -18,6 +18,7 @@
 #include "expert_f16_kernel.h"
 #include "mxfp4_kernels.h"
 #include "router_kernels.h"
+#include "node_extra_kernels.h"
 
 using namespace csk;
 
@@ -313,7 +314,7 @@ namespace {
 // Upload `rows x K` reference blocks and repack into (q, s).  The staging buffer is kept
 // between calls (a checkpoint is hundreds of matrices of one size); the scale bytes are
 // checked by the pack kernel as it reads them, so the host touches the blocks only to hand
-// them to the copy.  On a scale outside 2..254 the planes of m hold partial data.
+// them to the copy.  After a refused block the planes of m hold partial data.
 uint8_t* g_stage = nullptr;
 size_t g_stage_cap = 0;
 unsigned long long* g_bad = nullptr;
@@ -340,9 +341,8 @@ int pack_into(const uint8_t* host, csk_mxfp4& m) {
   HIP_TRY(hipMemcpyAsync(&bad, g_bad, sizeof bad, hipMemcpyDeviceToHost, g_stream));
   HIP_TRY(hipStreamSynchronize(g_stream));
   if (bad != ~0ull)
-    return fail(CSK_ERR_SCALE, "MXFP4 scale byte " + std::to_string((int)host[bad * 17]) + " at block " +
-                                   std::to_string(bad) +
-                                   " is outside 2..254 (denormal / reserved scales unsupported)");
+    return fail(CSK_ERR_SCALE, "MXFP4 scale byte 255 on the non-zero block " + std::to_string(bad) +
+                                   ": its values (codes x 2^127) overflow fp32");
   return CSK_OK;
 }
 
@@ -559,11 +559,12 @@ int F16Scratch::ensure(size_t rows_, size_t width_) {
   return CSK_OK;
 }
 
+// rows of K values read from source rows of Ksrc values (Ksrc = K, or K / 2: each row twice over)
 int launch_f16_split(const float* x, int64_t rows, int64_t K, const int* gather_tok,
-                     const float* gather_w, uint16_t* out, float* rscale) {
+                     const float* gather_w, uint16_t* out, float* rscale, int64_t Ksrc = 0) {
   if (rows == 0) return CSK_OK;
   f16_split_rows_kernel<<<dim3((unsigned)rows), 256, 0, g_stream>>>(
-      x, (long)K, gather_tok, gather_w, reinterpret_cast<u32x4*>(out), rscale);
+      x, (long)K, (long)(Ksrc ? Ksrc : K), gather_tok, gather_w, reinterpret_cast<u32x4*>(out), rscale);
   return check_launch("f16_split_rows_kernel");
 }
 
@@ -605,10 +606,13 @@ int launch_f16_projection(int64_t E, int64_t T, int64_t P, int64_t K, int64_t N,
 // Experts with fp16 weights over the dispatched tokens: ws.y[P,H] <- down(act(gate, up)).
 // x is [T,H] fp32.  Up to 64 tokens every expert's tokens form groups of 16 (one pass over
 // the weights per group, HBM-bound); beyond that groups of 64.
+// dup: the weights are fp32 matrices kept as two fp16 terms side by side ([F, 2 H] and
+// [H, 2 F]), so every activation row is contracted twice over.
 int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int act_type,
                     const float* x, bool weight_before_ffn, int64_t gather_rows, Workspace& ws,
-                    bool timed = false, bool identity_rows = false) {
+                    bool timed = false, bool identity_rows = false, bool dup = false) {
   const int64_t P = T * k;
+  const int64_t KH = dup ? 2 * H : H, KF = dup ? 2 * F : F;
   int rc = g_f16.ensure((size_t)P, (size_t)F);
   if (rc != CSK_OK) return rc;
   ExpertF16Args a{};
@@ -617,11 +621,11 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   a.act_type = act_type;
   if (weight_before_ffn) {
     // rows gathered per dispatch position and scaled by the routing weight first
-    rc = launch_f16_split(x, gather_rows, H, ws.list_tok, ws.list_w, ws.xg, g_f16.rs_x);
+    rc = launch_f16_split(x, gather_rows, KH, ws.list_tok, ws.list_w, ws.xg, g_f16.rs_x, H);
     a.list_row = nullptr;
     a.B = reinterpret_cast<const u32x4*>(ws.xg);
   } else {
-    rc = launch_f16_split(x, T, H, nullptr, nullptr, ws.xs, g_f16.rs_x);
+    rc = launch_f16_split(x, T, KH, nullptr, nullptr, ws.xs, g_f16.rs_x, H);
     a.list_row = identity_rows ? nullptr : ws.list_tok;  // identity: position p is token p
     a.B = reinterpret_cast<const u32x4*>(ws.xs);
   }
@@ -636,7 +640,7 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   const int64_t max_mtiles = P / 64 + std::min<int64_t>(E, P);
   auto gemm_grid = [&](int n_ntiles) { return dim3((unsigned)(cdiv(max_mtiles * n_ntiles, kF16Dies) * kF16Dies)); };
   a.rscale = g_f16.rs_x;
-  a.nkb = (int)f16_block_count(H);
+  a.nkb = (int)f16_block_count(KH);
   a.N = (int)F;
   a.ntile = (int)f16_tile_count(F);
   a.out = g_f16.actf;
@@ -651,8 +655,8 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   }
   if ((rc = check_launch("expert_f16_kernel<0>")) != CSK_OK) return rc;
   if (timed) mark(CSK_STAGE_DOWN);
-  if ((rc = launch_f16_split(g_f16.actf, P, F, nullptr, nullptr, ws.act, g_f16.rs_a)) != CSK_OK) return rc;
-  return launch_f16_projection(E, T, P, F, H, ws.act, g_f16.rs_a, ws.y, ws);
+  if ((rc = launch_f16_split(g_f16.actf, P, KF, nullptr, nullptr, ws.act, g_f16.rs_a, F)) != CSK_OK) return rc;
+  return launch_f16_projection(E, T, P, KF, H, ws.act, g_f16.rs_a, ws.y, ws);
 }
 
 int check_dims(int64_t E, int64_t k, int64_t H, int64_t F) {
@@ -1077,7 +1081,9 @@ extern "C" int csk_layer_export(const csk_layer* L, int64_t e, int which, uint8_
 
 struct csk_f16 {
   u32x4* w = nullptr;
-  int64_t rows = 0, K = 0;
+  int64_t rows = 0, K = 0;  // K: columns of the resident fp16 matrix
+  int64_t Ksrc = 0;         // columns of the matrix the caller gave: K, or K / 2 for fp32 weights kept as [hi | lo]
+  bool split() const { return K != Ksrc; }
 };
 
 namespace {
@@ -1132,6 +1138,93 @@ int f16_export_from(const u32x4* src, int64_t rows, int64_t K, uint16_t* halves)
 }
 }  // namespace
 
+namespace {
+// Device staging of the host-pointer entry points.  A node-level call needs a handful of
+// buffers whose sizes repeat from frame to frame (one call per expert node per frame), so
+// blocks are kept in a small pool instead of going back to hipFree -- which synchronises the
+// device -- and to hipMalloc on the next call.  The entry points hold the library's lock and
+// end with the stream idle, so a block returned at scope exit is free for the next call.
+struct StagingPool {
+  struct Block {
+    void* p;
+    size_t cap;
+  };
+  std::vector<Block> idle;
+  size_t idle_bytes = 0;
+  static constexpr size_t kMaxIdleBytes = (size_t)1 << 30;
+  static constexpr size_t kMaxIdleBlocks = 64;
+  static size_t size_class(size_t bytes) {  // powers of two from 4 KiB on
+    size_t c = 4096;
+    while (c < bytes) c <<= 1;
+    return c;
+  }
+  int take(size_t bytes, void** out, size_t* cap) {
+    const size_t want = size_class(bytes);
+    for (size_t i = 0; i < idle.size(); ++i) {
+      if (idle[i].cap == want) {
+        *out = idle[i].p, *cap = want;
+        idle_bytes -= want;
+        idle[i] = idle.back();
+        idle.pop_back();
+        return CSK_OK;
+      }
+    }
+    HIP_TRY(hipMalloc(out, want));
+    *cap = want;
+    return CSK_OK;
+  }
+  void give(void* p, size_t cap) {
+    if (idle.size() >= kMaxIdleBlocks || idle_bytes + cap > kMaxIdleBytes) {
+      (void)hipFree(p);
+      return;
+    }
+    idle.push_back(Block{p, cap});
+    idle_bytes += cap;
+  }
+};
+StagingPool g_staging;
+
+// Scoped device buffer for the host-pointer entry points.
+struct DevBuf {
+  void* p = nullptr;
+  size_t cap = 0;
+  ~DevBuf() {
+    if (p) g_staging.give(p, cap);
+  }
+  int alloc(size_t bytes) {
+    if (p) {
+      if (bytes <= cap) return CSK_OK;
+      g_staging.give(p, cap);
+      p = nullptr, cap = 0;
+    }
+    return g_staging.take(bytes ? bytes : 1, &p, &cap);
+  }
+  int upload(const void* host, size_t bytes) {
+    int rc = alloc(bytes);
+    if (rc != CSK_OK) return rc;
+    HIP_TRY(hipMemcpyAsync(p, host, bytes, hipMemcpyHostToDevice, g_stream));
+    return CSK_OK;
+  }
+  template <class T>
+  T* as() {
+    return reinterpret_cast<T*>(p);
+  }
+};
+
+// Tokens are independent in every node-level operation, so a long batch is taken in passes:
+// grids that have one row of workgroups per token stay inside the launch limits and the
+// 32-bit counts of token-expert assignments cannot overflow, whatever T is.
+constexpr int64_t kNodePassTokens = 16384;
+template <class F>
+int for_token_passes(int64_t T, F&& f) {
+  for (int64_t t0 = 0; t0 < T; t0 += kNodePassTokens) {
+    const int rc = f(t0, std::min(kNodePassTokens, T - t0));
+    if (rc != CSK_OK) return rc;
+  }
+  return CSK_OK;
+}
+}  // namespace
+
 extern "C" int csk_f16_upload(const uint16_t* halves, int64_t rows, int64_t K, csk_f16** out) {
   REQUIRE_INIT();
   if (!halves || !out || rows <= 0 || K <= 0)
@@ -1139,7 +1232,7 @@ extern "C" int csk_f16_upload(const uint16_t* halves, int64_t rows, int64_t K, c
   if (rows > (int64_t)kZeroLen || K > (int64_t)kZeroLen)
     return fail(CSK_ERR_ARG, "csk_f16_upload: dimensions above 65536 are not supported");
   csk_f16* m = new csk_f16;
-  m->rows = rows, m->K = K;
+  m->rows = rows, m->K = K, m->Ksrc = K;
   int rc = dev_alloc(&m->w, (size_t)f16_entries(rows, K));
   if (rc == CSK_OK) rc = f16_pack_into(halves, kGgmlF16Type, rows, K, m->w);
   if (rc != CSK_OK) {
@@ -1156,9 +1249,43 @@ extern "C" int csk_f16_upload_ggml(int ggml_type, const void* data, int64_t rows
   if (rows > (int64_t)kZeroLen || K > (int64_t)kZeroLen)
     return fail(CSK_ERR_ARG, "csk_f16_upload_ggml: dimensions above 65536 are not supported");
   csk_f16* m = new csk_f16;
-  m->rows = rows, m->K = K;
+  m->rows = rows, m->K = K, m->Ksrc = K;
   int rc = dev_alloc(&m->w, (size_t)f16_entries(rows, K));
   if (rc == CSK_OK) rc = f16_pack_into(data, ggml_type, rows, K, m->w);
+  if (rc != CSK_OK) {
+    csk_f16_free(m);
+    return rc;
+  }
+  *out = m;
+  return CSK_OK;
+}
+extern "C" int csk_f16_upload_f32(const float* w_host, int64_t rows, int64_t K, csk_f16** out) {
+  REQUIRE_INIT();
+  if (!w_host || !out || rows <= 0 || K <= 0)
+    return fail(CSK_ERR_ARG, "csk_f16_upload_f32: need a matrix with rows > 0 and K > 0");
+  if (rows > (int64_t)kZeroLen || 2 * K > (int64_t)kZeroLen)
+    return fail(CSK_ERR_ARG, "csk_f16_upload_f32: at most 65536 rows and 32768 columns");
+  csk_f16* m = new csk_f16;
+  m->rows = rows, m->K = 2 * K, m->Ksrc = K;
+  const long ent = f16_entries(rows, 2 * K);
+  DevBuf stage;
+  int rc = dev_alloc(&m->w, (size_t)ent);
+  if (rc == CSK_OK) rc = stage.upload(w_host, (size_t)rows * K * 4);
+  if (rc == CSK_OK && !g_bad && hipMalloc((void**)&g_bad, sizeof(unsigned long long)) != hipSuccess)
+    rc = fail(CSK_ERR_HIP, "hipMalloc failed");
+  unsigned long long bad = ~0ull;
+  if (rc == CSK_OK) {
+    hipError_t e = hipMemsetAsync(g_bad, 0xFF, sizeof(unsigned long long), g_stream);
+    f32_split_pack_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(stage.as<float>(), m->w, rows, K,
+                                                                              ent, g_bad);
+    if (e == hipSuccess) e = hipGetLastError();
+    if (e == hipSuccess) e = hipMemcpyAsync(&bad, g_bad, sizeof bad, hipMemcpyDeviceToHost, g_stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(g_stream);
+    if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("csk_f16_upload_f32: ") + hipGetErrorString(e));
+  }
+  if (rc == CSK_OK && bad != ~0ull)
+    rc = fail(CSK_ERR_ARG, "csk_f16_upload_f32: weight " + std::to_string(bad) +
+                               " is not finite or larger than 65504 in magnitude");
   if (rc != CSK_OK) {
     csk_f16_free(m);
     return rc;
@@ -1175,7 +1302,7 @@ extern "C" void csk_f16_free(csk_f16* m) {
 extern "C" int csk_f16_export(const csk_f16* m, uint16_t* halves_out) {
   REQUIRE_INIT();
   if (!m || !halves_out) return fail(CSK_ERR_ARG, "csk_f16_export: null argument");
-  return f16_export_from(m->w, m->rows, m->K, halves_out);
+  return f16_export_from(m->w, m->rows, m->K, halves_out);  // [rows, 2 K] = [hi | lo] for fp32 weights
 }
 
 extern "C" int csk_layer_set_expert_f16(csk_layer* L, int64_t e, const uint16_t* w_up,
@@ -1441,29 +1568,6 @@ extern "C" int csk_layer_last_dispatch(csk_layer* L, int32_t* counts_host, int32
 
 // ============================================================ node-level ops
 
-namespace {
-// Scoped device buffer for the host-pointer entry points.
-struct DevBuf {
-  void* p = nullptr;
-  ~DevBuf() {
-    if (p) (void)hipFree(p);
-  }
-  int alloc(size_t bytes) {
-    HIP_TRY(hipMalloc(&p, bytes ? bytes : 1));
-    return CSK_OK;
-  }
-  int upload(const void* host, size_t bytes) {
-    int rc = alloc(bytes);
-    if (rc != CSK_OK) return rc;
-    HIP_TRY(hipMemcpyAsync(p, host, bytes, hipMemcpyHostToDevice, g_stream));
-    return CSK_OK;
-  }
-  template <class T>
-  T* as() {
-    return reinterpret_cast<T*>(p);
-  }
-};
-}  // namespace
 
 namespace {
 int router_host(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
@@ -1494,19 +1598,24 @@ int router_host(const float* hidden, int64_t T, int64_t H, const float* gate_w, 
   if (T == 0) return CSK_OK;
   DevBuf dx, dg, db, dl, dp, di;
   int rc;
-  if ((rc = dx.upload(hidden, (size_t)T * H * 4)) != CSK_OK) return rc;
   if ((rc = dg.upload(gate_w, (size_t)E * H * 4)) != CSK_OK) return rc;
   if (gate_b && (rc = db.upload(gate_b, (size_t)E * 4)) != CSK_OK) return rc;
-  if ((rc = dl.alloc((size_t)T * E * 4 * (1 + kRouterMaxSplits))) != CSK_OK) return rc;
-  if ((rc = dp.alloc((size_t)T * k * 8)) != CSK_OK) return rc;
-  if ((rc = di.alloc((size_t)T * k * 4)) != CSK_OK) return rc;
-  rc = launch_router(dx.as<float>(), dg.as<float>(), gate_b ? db.as<float>() : nullptr, T, E, H, k,
-                     sigmoid, dl.as<float>(), dp.as<float>(), di.as<int>());
-  if (rc != CSK_OK) return rc;
-  if (out_pairs) HIP_TRY(hipMemcpyAsync(out_pairs, dp.p, (size_t)T * k * 8, hipMemcpyDeviceToHost, g_stream));
-  if (out_logits) HIP_TRY(hipMemcpyAsync(out_logits, dl.p, (size_t)T * E * 4, hipMemcpyDeviceToHost, g_stream));
-  HIP_TRY(hipStreamSynchronize(g_stream));
-  return CSK_OK;
+  return for_token_passes(T, [&](int64_t t0, int64_t tn) -> int {
+    int rc;
+    if ((rc = dx.upload(hidden + t0 * H, (size_t)tn * H * 4)) != CSK_OK) return rc;
+    if ((rc = dl.alloc((size_t)tn * E * 4 * (1 + kRouterMaxSplits))) != CSK_OK) return rc;
+    if ((rc = dp.alloc((size_t)tn * k * 8)) != CSK_OK) return rc;
+    if ((rc = di.alloc((size_t)tn * k * 4)) != CSK_OK) return rc;
+    rc = launch_router(dx.as<float>(), dg.as<float>(), gate_b ? db.as<float>() : nullptr, tn, E, H, k,
+                       sigmoid, dl.as<float>(), dp.as<float>(), di.as<int>());
+    if (rc != CSK_OK) return rc;
+    if (out_pairs)
+      HIP_TRY(hipMemcpyAsync(out_pairs + t0 * k * 2, dp.p, (size_t)tn * k * 8, hipMemcpyDeviceToHost, g_stream));
+    if (out_logits)
+      HIP_TRY(hipMemcpyAsync(out_logits + t0 * E, dl.p, (size_t)tn * E * 4, hipMemcpyDeviceToHost, g_stream));
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return CSK_OK;
+  });
 }
 }  // namespace
 
@@ -1542,12 +1651,8 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
   const int nb = (b_up != nullptr) + (b_gate != nullptr) + (b_down != nullptr);
   if (nb != 0 && nb != 3) return fail(CSK_ERR_ARG, "expert_mlp: biases must be all present or all absent");
   Workspace& ws = g_ws;
-  int rc = ws.ensure(T, 1, k, H, F, weight_before_ffn != 0);
-  if (rc != CSK_OK) return rc;
-  const int64_t P = T * k;
   DevBuf dx, dpairs, dbu, dbg, dbd, dew, dout;
-  if ((rc = dx.upload(hidden, (size_t)T * H * 4)) != CSK_OK) return rc;
-  if ((rc = dpairs.upload(pairs, (size_t)P * 8)) != CSK_OK) return rc;
+  int rc;
   if (nb == 3) {
     if ((rc = dbu.upload(b_up, (size_t)F * 4)) != CSK_OK) return rc;
     if ((rc = dbg.upload(b_gate, (size_t)F * 4)) != CSK_OK) return rc;
@@ -1560,41 +1665,49 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
   w.b_up = nb ? dbu.as<float>() : g_zero;
   w.b_down = nb ? dbd.as<float>() : g_zero;
   if ((rc = dew.upload(&w, sizeof w)) != CSK_OK) return rc;
-  if ((rc = dout.alloc((size_t)T * H * 4)) != CSK_OK) return rc;
-  select_expert_ids_kernel<<<dim3((unsigned)cdiv(P, 256)), 256, 0, g_stream>>>(
-      dpairs.as<float>(), ws.ids, (int)P, expert_id);
-  if ((rc = check_launch("select_expert_ids_kernel")) != CSK_OK) return rc;
-  HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
-  HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
-  if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
-  const uint16_t* xa;
-  const int* list_row;
-  if (weight_before_ffn) {
-    // The expert's token count is only known on the device, and at most T
-    // tokens can select it: gather T rows.  Positions past the count read the
-    // zeroed tail of the lists (token 0, weight 0) and are never consumed.
-    rc = stream_path(T, H, F)
-             ? launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xg, T, H, ws.list_tok, ws.list_w)
-             : launch_mx3(dx.as<float>(), ws.xg, T, H, ws.list_tok, ws.list_w);
+  // a pass in which no token selects the expert still writes its rows (zeros, :509-512)
+  return for_token_passes(T, [&](int64_t t0, int64_t tn) -> int {
+    int rc = ws.ensure(tn, 1, k, H, F, weight_before_ffn != 0);
     if (rc != CSK_OK) return rc;
-    xa = ws.xg;
-    list_row = nullptr;
-  } else {
-    rc = stream_path(T, H, F)
-             ? launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xs, T, H, nullptr, nullptr)
-             : launch_mx3(dx.as<float>(), ws.xs, T, H, nullptr, nullptr);
+    const int64_t P = tn * k;
+    if ((rc = dx.upload(hidden + t0 * H, (size_t)tn * H * 4)) != CSK_OK) return rc;
+    if ((rc = dpairs.upload(pairs + t0 * k * 2, (size_t)P * 8)) != CSK_OK) return rc;
+    if ((rc = dout.alloc((size_t)tn * H * 4)) != CSK_OK) return rc;
+    select_expert_ids_kernel<<<dim3((unsigned)cdiv(P, 256)), 256, 0, g_stream>>>(
+        dpairs.as<float>(), ws.ids, (int)P, expert_id);
+    if ((rc = check_launch("select_expert_ids_kernel")) != CSK_OK) return rc;
+    HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
+    HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
+    if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
+    const uint16_t* xa;
+    const int* list_row;
+    if (weight_before_ffn) {
+      // The expert's token count is only known on the device, and at most tn
+      // tokens can select it: gather tn rows.  Positions past the count read the
+      // zeroed tail of the lists (token 0, weight 0) and are never consumed.
+      rc = stream_path(tn, H, F)
+               ? launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xg, tn, H, ws.list_tok, ws.list_w)
+               : launch_mx3(dx.as<float>(), ws.xg, tn, H, ws.list_tok, ws.list_w);
+      if (rc != CSK_OK) return rc;
+      xa = ws.xg;
+      list_row = nullptr;
+    } else {
+      rc = stream_path(tn, H, F)
+               ? launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xs, tn, H, nullptr, nullptr)
+               : launch_mx3(dx.as<float>(), ws.xs, tn, H, nullptr, nullptr);
+      if (rc != CSK_OK) return rc;
+      xa = ws.xs;
+      list_row = ws.list_tok;
+    }
+    rc = run_experts(1, tn, k, H, F, activation, xa, list_row, ws);
     if (rc != CSK_OK) return rc;
-    xa = ws.xs;
-    list_row = ws.list_tok;
-  }
-  rc = run_experts(1, T, k, H, F, activation, xa, list_row, ws);
-  if (rc != CSK_OK) return rc;
-  expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)T), 256, 0, g_stream>>>(
-      ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
-  if ((rc = check_launch("expand_expert_rows_kernel")) != CSK_OK) return rc;
-  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
-  HIP_TRY(hipStreamSynchronize(g_stream));
-  return CSK_OK;
+    expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)tn), 256, 0, g_stream>>>(
+        ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
+    if ((rc = check_launch("expand_expert_rows_kernel")) != CSK_OK) return rc;
+    HIP_TRY(hipMemcpyAsync(out + t0 * H, dout.p, (size_t)tn * H * 4, hipMemcpyDeviceToHost, g_stream));
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return CSK_OK;
+  });
 }
 
 extern "C" int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T, int64_t H, int64_t F,
@@ -1610,6 +1723,8 @@ extern "C" int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T,
   for (int64_t p = 0; p < T * k && !any; ++p) any = (int)pairs[2 * p] == expert_id;
   *is_empty = !any;
   if (!any) return CSK_OK;
+  if (w_up->split() || w_gate->split() || w_down->split())
+    return fail(CSK_ERR_ARG, "expert_mlp: all weights must be FLOAT16");
   if (w_up->rows != F || w_up->K != H)
     return fail(CSK_ERR_ARG, "expert_mlp: w_up must be [" + std::to_string(F) + ", " + std::to_string(H) + "], got [" +
                                  std::to_string(w_up->rows) + ", " + std::to_string(w_up->K) + "]");
@@ -1624,12 +1739,8 @@ extern "C" int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T,
   if (nb != 0 && nb != 3) return fail(CSK_ERR_ARG, "expert_mlp: biases must be all present or all absent");
   Workspace& ws = g_ws;
   const int64_t Hp = cdiv(H, 32) * 32, Fp = cdiv(F, 32) * 32;  // activation rows are whole blocks
-  int rc = ws.ensure(T, 1, k, Hp, Fp, weight_before_ffn != 0);
-  if (rc != CSK_OK) return rc;
-  const int64_t P = T * k;
   DevBuf dx, dpairs, dbu, dbg, dbd, dew, dout;
-  if ((rc = dx.upload(hidden, (size_t)T * H * 4)) != CSK_OK) return rc;
-  if ((rc = dpairs.upload(pairs, (size_t)P * 8)) != CSK_OK) return rc;
+  int rc;
   if (nb == 3) {
     if ((rc = dbu.upload(b_up, (size_t)F * 4)) != CSK_OK) return rc;
     if ((rc = dbg.upload(b_gate, (size_t)F * 4)) != CSK_OK) return rc;
@@ -1643,23 +1754,30 @@ extern "C" int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T,
   w.b_up = nb ? dbu.as<float>() : g_zero;
   w.b_down = nb ? dbd.as<float>() : g_zero;
   if ((rc = dew.upload(&w, sizeof w)) != CSK_OK) return rc;
-  if ((rc = dout.alloc((size_t)T * H * 4)) != CSK_OK) return rc;
-  select_expert_ids_kernel<<<dim3((unsigned)cdiv(P, 256)), 256, 0, g_stream>>>(
-      dpairs.as<float>(), ws.ids, (int)P, expert_id);
-  if ((rc = check_launch("select_expert_ids_kernel")) != CSK_OK) return rc;
-  HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
-  HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
-  if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
-  // with weight_before_ffn at most T tokens can select the expert: T rows are gathered; the
-  // ones past its count read the zeroed tail of the lists and are never consumed
-  rc = run_experts_f16(1, T, k, H, F, activation, dx.as<float>(), weight_before_ffn != 0, T, ws);
-  if (rc != CSK_OK) return rc;
-  expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)T), 256, 0, g_stream>>>(
-      ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
-  if ((rc = check_launch("expand_expert_rows_kernel")) != CSK_OK) return rc;
-  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
-  HIP_TRY(hipStreamSynchronize(g_stream));
-  return CSK_OK;
+  return for_token_passes(T, [&](int64_t t0, int64_t tn) -> int {
+    int rc = ws.ensure(tn, 1, k, Hp, Fp, weight_before_ffn != 0);
+    if (rc != CSK_OK) return rc;
+    const int64_t P = tn * k;
+    if ((rc = dx.upload(hidden + t0 * H, (size_t)tn * H * 4)) != CSK_OK) return rc;
+    if ((rc = dpairs.upload(pairs + t0 * k * 2, (size_t)P * 8)) != CSK_OK) return rc;
+    if ((rc = dout.alloc((size_t)tn * H * 4)) != CSK_OK) return rc;
+    select_expert_ids_kernel<<<dim3((unsigned)cdiv(P, 256)), 256, 0, g_stream>>>(
+        dpairs.as<float>(), ws.ids, (int)P, expert_id);
+    if ((rc = check_launch("select_expert_ids_kernel")) != CSK_OK) return rc;
+    HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
+    HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
+    if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
+    // with weight_before_ffn at most tn tokens can select the expert: tn rows are gathered; the
+    // ones past its count read the zeroed tail of the lists and are never consumed
+    rc = run_experts_f16(1, tn, k, H, F, activation, dx.as<float>(), weight_before_ffn != 0, tn, ws);
+    if (rc != CSK_OK) return rc;
+    expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)tn), 256, 0, g_stream>>>(
+        ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
+    if ((rc = check_launch("expand_expert_rows_kernel")) != CSK_OK) return rc;
+    HIP_TRY(hipMemcpyAsync(out + t0 * H, dout.p, (size_t)tn * H * 4, hipMemcpyDeviceToHost, g_stream));
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return CSK_OK;
+  });
 }
 
 namespace {
@@ -1683,19 +1801,19 @@ extern "C" int csk_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int6
   REQUIRE_INIT();
   if (!hidden || !w_gate || !w_up || !w_down || !out || T < 0)
     return fail(CSK_ERR_ARG, "csk_dense_ffn_f16: null argument");
-  if (w_gate->rows != F || w_gate->K != H || w_up->rows != F || w_up->K != H)
+  if (w_gate->split() != w_up->split() || w_gate->split() != w_down->split())
+    return fail(CSK_ERR_ARG, "dense_ffn: weight tensors must all be FLOAT16 or all FLOAT32");
+  if (w_gate->rows != F || w_gate->Ksrc != H || w_up->rows != F || w_up->Ksrc != H)
     return fail(CSK_ERR_ARG, "dense_ffn: gate_w/up_w shape mismatch");
-  if (w_down->rows != H || w_down->K != F)
+  if (w_down->rows != H || w_down->Ksrc != F)
     return fail(CSK_ERR_ARG, "dense_ffn: down_w shape mismatch, expected [" + std::to_string(H) + ", " +
                                  std::to_string(F) + "], got [" + std::to_string(w_down->rows) + ", " +
-                                 std::to_string(w_down->K) + "]");
+                                 std::to_string(w_down->Ksrc) + "]");
   if (T == 0) return CSK_OK;
-  if (T > (int64_t)1 << 24) return fail(CSK_ERR_ARG, "dense_ffn: more than 2^24 tokens");
+  const bool dup = w_gate->split();  // fp32 weights as two fp16 terms: rows are contracted twice over
   Workspace& ws = g_ws;
-  int rc = ws.ensure(T, 1, 1, cdiv(H, 32) * 32, cdiv(F, 32) * 32, false);
-  if (rc != CSK_OK) return rc;
   DevBuf dx, dbg, dbu, dbd, dew;
-  if ((rc = dx.upload(hidden, (size_t)T * H * 4)) != CSK_OK) return rc;
+  int rc;
   // each bias is optional on its own (dense_ffn_node.h:196-197, 213)
   if (b_gate && (rc = dbg.upload(b_gate, (size_t)F * 4)) != CSK_OK) return rc;
   if (b_up && (rc = dbu.upload(b_up, (size_t)F * 4)) != CSK_OK) return rc;
@@ -1708,13 +1826,18 @@ extern "C" int csk_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int6
   w.b_up = b_up ? dbu.as<float>() : g_zero;
   w.b_down = b_down ? dbd.as<float>() : g_zero;
   if ((rc = dew.upload(&w, sizeof w)) != CSK_OK) return rc;
-  dense_desc_kernel<<<1, 256, 0, g_stream>>>(ws.desc, dew.as<ExpertW>(), (int)T, ws.tiles, ws.n_tiles);
-  if ((rc = check_launch("dense_desc_kernel")) != CSK_OK) return rc;
-  rc = run_experts_f16(1, T, 1, H, F, CSK_ACT_STANDARD_SWIGLU, dx.as<float>(), false, T, ws, false, true);
-  if (rc != CSK_OK) return rc;
-  HIP_TRY(hipMemcpyAsync(out, ws.y, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
-  HIP_TRY(hipStreamSynchronize(g_stream));
-  return CSK_OK;
+  return for_token_passes(T, [&](int64_t t0, int64_t tn) -> int {
+    int rc = ws.ensure(tn, 1, 1, cdiv(dup ? 2 * H : H, 32) * 32, cdiv(dup ? 2 * F : F, 32) * 32, false);
+    if (rc != CSK_OK) return rc;
+    if ((rc = dx.upload(hidden + t0 * H, (size_t)tn * H * 4)) != CSK_OK) return rc;
+    dense_desc_kernel<<<1, 256, 0, g_stream>>>(ws.desc, dew.as<ExpertW>(), (int)tn, ws.tiles, ws.n_tiles);
+    if ((rc = check_launch("dense_desc_kernel")) != CSK_OK) return rc;
+    rc = run_experts_f16(1, tn, 1, H, F, CSK_ACT_STANDARD_SWIGLU, dx.as<float>(), false, tn, ws, false, true, dup);
+    if (rc != CSK_OK) return rc;
+    HIP_TRY(hipMemcpyAsync(out + t0 * H, ws.y, (size_t)tn * H * 4, hipMemcpyDeviceToHost, g_stream));
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return CSK_OK;
+  });
 }
 
 extern "C" int csk_matmul_transpose_f16(const float* a_host, int64_t M, int64_t K, const csk_f16* w,
@@ -1722,29 +1845,31 @@ extern "C" int csk_matmul_transpose_f16(const float* a_host, int64_t M, int64_t 
   REQUIRE_INIT();
   if (!a_host || !w || !out || M < 0 || K <= 0)
     return fail(CSK_ERR_ARG, "csk_matmul_transpose_f16: null argument");
-  if (w->K != K) return fail(CSK_ERR_ARG, "matmul_transpose_mixed: incompatible dimensions");
+  if (w->Ksrc != K) return fail(CSK_ERR_ARG, "matmul_transpose_mixed: incompatible dimensions");
   if (M == 0) return CSK_OK;
-  if (M > (int64_t)1 << 24) return fail(CSK_ERR_ARG, "matmul_transpose_mixed: more than 2^24 rows");
-  const int64_t N = w->rows;
+  const int64_t N = w->rows, K2 = w->K;  // K2 = 2 K for an fp32 weight kept as two fp16 terms
   Workspace& ws = g_ws;
-  // rows of A take the place of the activations of a down projection: [M, K] -> [M, N]
-  int rc = ws.ensure(M, 1, 1, cdiv(N, 32) * 32, cdiv(K, 32) * 32, false);
-  if (rc == CSK_OK) rc = g_f16.ensure((size_t)M, 1);
-  if (rc != CSK_OK) return rc;
   DevBuf da, dew;
-  if ((rc = da.upload(a_host, (size_t)M * K * 4)) != CSK_OK) return rc;
+  int rc;
   ExpertW ew{};
   ew.q_down = reinterpret_cast<const uint4*>(w->w);
   ew.b_gate = ew.b_up = ew.b_down = g_zero;
   if ((rc = dew.upload(&ew, sizeof ew)) != CSK_OK) return rc;
-  dense_desc_kernel<<<1, 256, 0, g_stream>>>(ws.desc, dew.as<ExpertW>(), (int)M, ws.tiles, ws.n_tiles);
-  if ((rc = check_launch("dense_desc_kernel")) != CSK_OK) return rc;
-  if ((rc = launch_f16_split(da.as<float>(), M, K, nullptr, nullptr, ws.act, g_f16.rs_a)) != CSK_OK) return rc;
-  rc = launch_f16_projection(1, M, M, K, N, ws.act, g_f16.rs_a, ws.y, ws);
-  if (rc != CSK_OK) return rc;
-  HIP_TRY(hipMemcpyAsync(out, ws.y, (size_t)M * N * 4, hipMemcpyDeviceToHost, g_stream));
-  HIP_TRY(hipStreamSynchronize(g_stream));
-  return CSK_OK;
+  return for_token_passes(M, [&](int64_t m0, int64_t mn) -> int {
+    // rows of A take the place of the activations of a down projection: [mn, K] -> [mn, N]
+    int rc = ws.ensure(mn, 1, 1, cdiv(N, 32) * 32, cdiv(K2, 32) * 32, false);
+    if (rc == CSK_OK) rc = g_f16.ensure((size_t)mn, 1);
+    if (rc != CSK_OK) return rc;
+    if ((rc = da.upload(a_host + m0 * K, (size_t)mn * K * 4)) != CSK_OK) return rc;
+    dense_desc_kernel<<<1, 256, 0, g_stream>>>(ws.desc, dew.as<ExpertW>(), (int)mn, ws.tiles, ws.n_tiles);
+    if ((rc = check_launch("dense_desc_kernel")) != CSK_OK) return rc;
+    if ((rc = launch_f16_split(da.as<float>(), mn, K2, nullptr, nullptr, ws.act, g_f16.rs_a, K)) != CSK_OK) return rc;
+    rc = launch_f16_projection(1, mn, mn, K2, N, ws.act, g_f16.rs_a, ws.y, ws);
+    if (rc != CSK_OK) return rc;
+    HIP_TRY(hipMemcpyAsync(out + m0 * N, ws.y, (size_t)mn * N * 4, hipMemcpyDeviceToHost, g_stream));
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    return CSK_OK;
+  });
 }
 
 extern "C" int csk_expert_token_mxfp4(const float* x, const uint8_t* w_up, const uint8_t* w_gate,
@@ -1843,6 +1968,105 @@ extern "C" int csk_add(const float* a, const float* b, float* out, int64_t n) {
   if ((rc = check_launch("add_kernel")) != CSK_OK) return rc;
   HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)n * 4, hipMemcpyDeviceToHost, g_stream));
   HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+extern "C" int csk_add_broadcast(const void* a, const int64_t* shape_a, int nd_a, const void* b,
+                                 const int64_t* shape_b, int nd_b, int dtype, void* out) {
+  REQUIRE_INIT();
+  if (!a || !b || !out || nd_a < 0 || nd_b < 0 || (nd_a && !shape_a) || (nd_b && !shape_b))
+    return fail(CSK_ERR_ARG, "csk_add_broadcast: bad argument");
+  if (dtype < CSK_DT_FLOAT32 || dtype > CSK_DT_INT64) return fail(CSK_ERR_ARG, "add: unsupported dtype");
+  const int nd = std::max(nd_a, nd_b);
+  auto list = [](const int64_t* s, int n) {
+    std::string r;
+    for (int i = 0; i < n; ++i) r += (i ? "," : "") + std::to_string(s[i]);
+    return r;
+  };
+  if (nd > kMaxBroadcastDims)
+    return fail(CSK_ERR_ARG, "add: more than " + std::to_string(kMaxBroadcastDims) + " dimensions are not supported");
+  for (int i = 0; i < nd_a; ++i)
+    if (shape_a[i] < 0) return fail(CSK_ERR_ARG, "csk_add_broadcast: negative dimension");
+  for (int i = 0; i < nd_b; ++i)
+    if (shape_b[i] < 0) return fail(CSK_ERR_ARG, "csk_add_broadcast: negative dimension");
+  // dynamic_tensor::broadcast_shape (dynamic_tensor.h:218-238), trailing dimensions aligned
+  BroadcastDims d{};
+  d.nd = nd;
+  int64_t n = 1, na = 1, nb = 1;
+  for (int i = 0; i < nd; ++i) {
+    const int64_t da = i < nd_a ? shape_a[nd_a - 1 - i] : 1, db = i < nd_b ? shape_b[nd_b - 1 - i] : 1;
+    if (!(da == db || da == 1 || db == 1))
+      return fail(CSK_ERR_ARG, "Broadcast failed: Shape A=[" + list(shape_a, nd_a) + "], Shape B=[" +
+                                   list(shape_b, nd_b) + "]");
+    const int q = nd - 1 - i;
+    d.out[q] = (da == 0 || db == 0) ? 0 : std::max(da, db);
+    d.sa[q] = (i < nd_a && da != 1) ? na : 0;
+    d.sb[q] = (i < nd_b && db != 1) ? nb : 0;
+    if (__builtin_mul_overflow(n, d.out[q], &n) || __builtin_mul_overflow(na, da, &na) ||
+        __builtin_mul_overflow(nb, db, &nb))
+      return fail(CSK_ERR_ARG, "csk_add_broadcast: element count overflows");
+  }
+  if (n == 0) return CSK_OK;
+  const size_t esz = (dtype == CSK_DT_FLOAT32 || dtype == CSK_DT_INT32) ? 4 : 8;
+  DevBuf da_, db_, dout;
+  int rc;
+  if ((rc = da_.upload(a, (size_t)na * esz)) != CSK_OK) return rc;
+  if ((rc = db_.upload(b, (size_t)nb * esz)) != CSK_OK) return rc;
+  if ((rc = dout.alloc((size_t)n * esz)) != CSK_OK) return rc;
+  const dim3 grid((unsigned)std::min<int64_t>(cdiv(n, 256), 1 << 20));
+  switch (dtype) {
+    case CSK_DT_FLOAT32:
+      add_broadcast_kernel<float><<<grid, 256, 0, g_stream>>>(da_.as<float>(), db_.as<float>(), dout.as<float>(), n, d);
+      break;
+    case CSK_DT_FLOAT64:
+      add_broadcast_kernel<double><<<grid, 256, 0, g_stream>>>(da_.as<double>(), db_.as<double>(), dout.as<double>(), n, d);
+      break;
+    case CSK_DT_INT32:
+      add_broadcast_kernel<int32_t><<<grid, 256, 0, g_stream>>>(da_.as<int32_t>(), db_.as<int32_t>(), dout.as<int32_t>(), n, d);
+      break;
+    default:
+      add_broadcast_kernel<int64_t><<<grid, 256, 0, g_stream>>>(da_.as<int64_t>(), db_.as<int64_t>(), dout.as<int64_t>(), n, d);
+      break;
+  }
+  if ((rc = check_launch("add_broadcast_kernel")) != CSK_OK) return rc;
+  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)n * esz, hipMemcpyDeviceToHost, g_stream));
+  HIP_TRY(hipStreamSynchronize(g_stream));
+  return CSK_OK;
+}
+
+extern "C" int csk_moe_router_f64(const double* hidden, int64_t T, int64_t H, const double* gate_w, int64_t E,
+                                  const float* gate_b, int64_t k, int sigmoid, float* out_pairs,
+                                  double* out_logits) {
+  REQUIRE_INIT();
+  if (!hidden || !gate_w || !out_pairs || T < 0) return fail(CSK_ERR_ARG, "csk_moe_router_f64: null argument");
+  if (E <= 0 || E > (int64_t)kZeroLen || k <= 0 || k > E || H <= 0 || H > (1 << 30) / E)
+    return fail(CSK_ERR_ARG, "csk_moe_router_f64: need 1 <= top_k <= E <= 65536 and H * E <= 2^30");
+  if (T == 0) return CSK_OK;
+  DevBuf dx, dg, db, dl, dv, di, dw, dp;
+  int rc;
+  if ((rc = dg.upload(gate_w, (size_t)E * H * 8)) != CSK_OK) return rc;
+  if (gate_b && (rc = db.upload(gate_b, (size_t)E * 4)) != CSK_OK) return rc;
+  // passes small enough that tokens x experts and tokens x hidden fit 32-bit launch arithmetic
+  const int64_t pass = std::max<int64_t>(1, std::min<int64_t>(kNodePassTokens, ((int64_t)1 << 28) / std::max(E, H)));
+  for (int64_t t0 = 0; t0 < T; t0 += pass) {
+    const int64_t tn = std::min(pass, T - t0);
+    if ((rc = dx.upload(hidden + t0 * H, (size_t)tn * H * 8)) != CSK_OK) return rc;
+    if ((rc = dl.alloc((size_t)tn * E * 8)) != CSK_OK) return rc;
+    if ((rc = dv.alloc((size_t)tn * E * 8)) != CSK_OK) return rc;
+    if ((rc = di.alloc((size_t)tn * E * 4)) != CSK_OK) return rc;
+    if ((rc = dw.alloc((size_t)tn * k * 4)) != CSK_OK) return rc;
+    if ((rc = dp.alloc((size_t)tn * k * 8)) != CSK_OK) return rc;
+    router_f64_logits_kernel<<<dim3((unsigned)cdiv(E, 64), (unsigned)cdiv(tn, 4)), 256, 0, g_stream>>>(
+        dx.as<double>(), dg.as<double>(), gate_b ? db.as<float>() : nullptr, dl.as<double>(), (int)tn, (int)E, (int)H);
+    if ((rc = check_launch("router_f64_logits_kernel")) != CSK_OK) return rc;
+    router_f64_topk_kernel<<<dim3((unsigned)cdiv(tn, 64)), 64, 0, g_stream>>>(
+        dl.as<double>(), dv.as<double>(), di.as<int>(), dw.as<float>(), dp.as<float>(), (int)tn, (int)E, (int)k, sigmoid);
+    if ((rc = check_launch("router_f64_topk_kernel")) != CSK_OK) return rc;
+    HIP_TRY(hipMemcpyAsync(out_pairs + t0 * k * 2, dp.p, (size_t)tn * k * 8, hipMemcpyDeviceToHost, g_stream));
+    if (out_logits)
+      HIP_TRY(hipMemcpyAsync(out_logits + t0 * E, dl.p, (size_t)tn * E * 8, hipMemcpyDeviceToHost, g_stream));
+    HIP_TRY(hipStreamSynchronize(g_stream));
+  }
   return CSK_OK;
 }
 

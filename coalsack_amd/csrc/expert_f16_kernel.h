@@ -55,6 +55,38 @@ __global__ __launch_bounds__(256) void f16_pack_kernel(const uint16_t* __restric
   dst[idx] = u32x4{w[0], w[1], w[2], w[3]};
 }
 
+// Row-major fp32 [rows, K] -> tiles of the fp16 matrix [rows, 2 K] = [hi | lo], hi = fp16(w),
+// lo = fp16(w - hi): the two-term form of an fp32 weight (absolute error below 2^-25 for
+// |w| < 65504), contracted against activation rows that repeat themselves ([x | x], see
+// f16_split_rows_kernel), so that  x . w = x . hi + x . lo  comes out of the fp16 kernels
+// unchanged.  `bad` receives the lowest flat index of a weight whose magnitude is not finite
+// in fp16 (it must hold ~0 on entry).
+__global__ __launch_bounds__(256) void f32_split_pack_kernel(const float* __restrict__ src,
+                                                             u32x4* __restrict__ dst, long rows, long K,
+                                                             long entries,
+                                                             unsigned long long* __restrict__ bad) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= entries) return;
+  const long nkb = f16_block_count(2 * K);
+  const int lane = (int)(idx & 63);
+  const long kb = (idx >> 6) % nkb, tile = (idx >> 6) / nkb;
+  const long row = tile * 16 + (lane & 15), k0 = kb * 32 + 8 * (lane >> 4);
+  uint32_t w[4] = {0u, 0u, 0u, 0u};
+  if (row < rows) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const long k = k0 + j;
+      if (k >= 2 * K) continue;
+      const float v = src[row * K + (k < K ? k : k - K)];
+      if (!(fabsf(v) <= 65504.0f)) atomicMin(bad, (unsigned long long)(row * K + (k < K ? k : k - K)));
+      const _Float16 h = (_Float16)v;
+      const _Float16 r = k < K ? h : (_Float16)(v - (float)h);
+      w[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, r) << (16 * (j & 1));
+    }
+  }
+  dst[idx] = u32x4{w[0], w[1], w[2], w[3]};
+}
+
 // tiles -> row-major halves (the export used to check that packing changed no bit)
 __global__ __launch_bounds__(256) void f16_unpack_kernel(const u32x4* __restrict__ src,
                                                          uint16_t* __restrict__ dst, long rows,
@@ -194,7 +226,9 @@ __global__ __launch_bounds__(256) void synth_f16_kernel(u32x4* __restrict__ dst,
 // fp32 rows -> scaled two-term fp16 rows.  One workgroup per output row; the source row is
 // gather_tok[row] scaled by gather_w[row] when given (weight_before_ffn: the reference
 // multiplies the token by its routing weight in fp32 first, expert_mlp_node.h:766-772).
-__global__ __launch_bounds__(256) void f16_split_rows_kernel(const float* __restrict__ x, long K,
+// The logical row has K elements read from a source row of Ksrc: element k is source element
+// k mod Ksrc (K = Ksrc, or 2 Ksrc for the repeated rows that two-term fp32 weights need).
+__global__ __launch_bounds__(256) void f16_split_rows_kernel(const float* __restrict__ x, long K, long Ksrc,
                                                              const int* __restrict__ gather_tok,
                                                              const float* __restrict__ gather_w,
                                                              u32x4* __restrict__ out,
@@ -203,9 +237,9 @@ __global__ __launch_bounds__(256) void f16_split_rows_kernel(const float* __rest
   const long row = blockIdx.x;
   const long srow = gather_tok ? gather_tok[row] : row;
   const float gw = gather_w ? gather_w[row] : 1.0f;
-  const float* xr = x + srow * K;
+  const float* xr = x + srow * Ksrc;
   float m = 0.0f;
-  for (long i = threadIdx.x; i < K; i += 256) m = fmaxf(m, fabsf(xr[i] * gw));
+  for (long i = threadIdx.x; i < Ksrc; i += 256) m = fmaxf(m, fabsf(xr[i] * gw));
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
@@ -227,7 +261,7 @@ __global__ __launch_bounds__(256) void f16_split_rows_kernel(const float* __rest
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const long k = kb * 32 + c * 8 + j;
-      const float v = k < K ? (xr[k] * gw) * inv : 0.0f;
+      const float v = k < K ? (xr[k < Ksrc ? k : k - Ksrc] * gw) * inv : 0.0f;
       const _Float16 h = (_Float16)v;
       const _Float16 l = (_Float16)(v - (float)h);
       hi[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, h) << (16 * (j & 1));

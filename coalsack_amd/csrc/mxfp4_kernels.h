@@ -47,9 +47,19 @@ __device__ __forceinline__ void entry_to_ref_block(uint4 q, uint8_t scale, uint8
   for (int j = 0; j < 16; ++j) blk[1 + j] = (uint8_t)(code[j] | (code[j + 16] << 4));
 }
 
+// True when every code of the block is +0 or -0 (codes 0 and 8): the block is zero
+// whatever its scale byte says.
+__device__ __forceinline__ bool entry_is_zero(const uint4& e) {
+  return ((e.x | e.y | e.z | e.w) & 0x77777777u) == 0u;
+}
+
 // entries = ntile * nblk * 16
-// `bad` receives the lowest index of a block whose scale byte is outside 2..254 (the
-// conversion instruction is exact only inside that range); it must hold ~0 on entry.
+// Scale bytes: every byte the reference decodes to a finite value is kept as it is
+// (gguf_dequant.h:419-433: 0 and 1 are 2^-128 and 2^-127 on the doubled code table; ggml
+// writes 0 for an all-zero block).  Byte 255 is 2^127 in the reference and "not a number" to
+// the matrix instruction: on a block of zeros it is stored as 254 (the block is zero either
+// way), on any other block the reference's own values overflow fp32 and `bad` receives the
+// lowest such block index (it must hold ~0 on entry).
 __global__ void pack_mxfp4_kernel(const uint8_t* __restrict__ src, uint4* __restrict__ q,
                                   uint8_t* __restrict__ s, int rows, int nblk, long entries,
                                   unsigned long long* __restrict__ bad) {
@@ -67,9 +77,14 @@ __global__ void pack_mxfp4_kernel(const uint8_t* __restrict__ src, uint4* __rest
     return;
   }
   const uint8_t* blk = src + (row * nblk + kb) * 17;
-  q[i] = ref_block_to_entry(blk);
-  s[si] = blk[0];
-  if (bad && (blk[0] < 2 || blk[0] > 254)) atomicMin(bad, (unsigned long long)(row * nblk + kb));
+  const uint4 e = ref_block_to_entry(blk);
+  q[i] = e;
+  uint8_t sb = blk[0];
+  if (sb == 255) {
+    if (entry_is_zero(e)) sb = 254;
+    else if (bad) atomicMin(bad, (unsigned long long)(row * nblk + kb));
+  }
+  s[si] = sb;
 }
 
 __global__ void export_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t* __restrict__ s,
@@ -103,9 +118,23 @@ __global__ void dequant_mxfp4_kernel(const uint4* __restrict__ q, const uint8_t*
   const size_t si = scale_index(tile, kb, n, scale_slots(nblk));
   if (row >= rows) return;
   const uint4 e = q[i];
-  const float sc = e8m0_scale(s[si]);
   const uint32_t w[4] = {e.x, e.y, e.z, e.w};
   float* o = dst + (row * nblk + kb) * 32;
+  if (s[si] < 2) {
+    // scale bytes 0 and 1: the products are fp32 denormals, which the conversion instruction
+    // does not produce; the reference's own arithmetic instead (doubled code table times
+    // 2^-128 or 2^-127, gguf_dequant.h:413-455).  The expert kernels treat these blocks as
+    // what they are to any contraction: zero to within 1e-37.
+    const float half_scale = __uint_as_float(0x00200000u << s[si]);
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+      const uint32_t code = (w[j >> 3] >> (4 * (j & 7))) & 15u;
+      const int mag = (code & 7u) < 5u ? (int)(code & 7u) : ((code & 7u) == 5u ? 6 : ((code & 7u) == 6u ? 8 : 12));
+      o[j] = (float)((code & 8u) ? -mag : mag) * half_scale;
+    }
+    return;
+  }
+  const float sc = e8m0_scale(s[si]);
 #pragma unroll
   for (int d = 0; d < 4; ++d) {
     bf16x2 r0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[d], sc, 0);

@@ -52,6 +52,17 @@ class dynamic_tensor {
   template <class T>
   const T* data_ptr() const { return reinterpret_cast<const T*>(bytes_->data()); }
   bool empty() const { return numel() == 0; }
+  // :218-238
+  static std::vector<int64_t> broadcast_shape(const std::vector<int64_t>& a, const std::vector<int64_t>& b) {
+    const size_t nd = a.size() > b.size() ? a.size() : b.size();
+    std::vector<int64_t> r(nd);
+    for (size_t i = 0; i < nd; ++i) {
+      const int64_t da = i < a.size() ? a[a.size() - 1 - i] : 1, db = i < b.size() ? b[b.size() - 1 - i] : 1;
+      if (da != db && da != 1 && db != 1) throw std::invalid_argument("Incompatible shapes for broadcasting");
+      r[nd - 1 - i] = (da == 0 || db == 0) ? 0 : (da > db ? da : db);
+    }
+    return r;
+  }
 };
 
 }  // namespace coalsack

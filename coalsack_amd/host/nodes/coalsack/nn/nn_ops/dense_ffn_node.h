@@ -1,34 +1,35 @@
 // dense_ffn_node backed by the gfx950 library: same class name, input order, output
 // and error texts as include/coalsack/nn/nn_ops/dense_ffn_node.h of the reference (cited
-// by line below); float16 weights run in csk_dense_ffn_f16.  Weights are uploaded at the
-// first sight of their storage pointer and cached per node (the engine feeds the same
-// weight tensors every frame, src/llm/llm_engine.cpp:755-771).
+// by line below); float16 and float32 weights both run in csk_dense_ffn_f16 (float32 ones
+// as two fp16 terms).  The node keeps one device copy per weight role, replaced when the
+// tensor it is handed changes (the engine feeds the same weight tensors every frame,
+// src/llm/llm_engine.cpp:755-771).
 #pragma once
 
 #include <stdexcept>
 #include <string>
-#include <unordered_map>
 #include <vector>
 
 #include "coalsack/nn/nn_op_node.h"
+#include "coalsack/nn/nn_ops/resident_weight.h"
 #include "coalsack_moe.h"
 
 namespace coalsack {
 
 // output = down_proj(silu(gate_proj(x)) * up_proj(x)) for every token (:14-27).
-// Inputs: hidden [B, S, D] f32, gate_w / up_w [ffn, D], down_w [D, ffn] float16,
+// Inputs: hidden [B, S, D] f32, gate_w / up_w [ffn, D], down_w [D, ffn] all float16 or all float32,
 // optionally gate_b, up_b [ffn], down_b [D] f32.
 class dense_ffn_node : public variadic_op_node {
  public:
   dense_ffn_node() : variadic_op_node("dense_ffn", 4) {}  // :30
-  ~dense_ffn_node() override {
-    for (auto& kv : resident_) csk_f16_free(kv.second.handle);
-  }
+  ~dense_ffn_node() override = default;
   dense_ffn_node(const dense_ffn_node&) = delete;
   dense_ffn_node& operator=(const dense_ffn_node&) = delete;
   std::string get_proc_name() const override { return "dense_ffn"; }  // :32
   // not in the reference (its compute is reached through process only): for tests
   dynamic_tensor compute_test(const std::vector<dynamic_tensor>& inputs) { return compute(inputs); }
+  // number of device copies made so far (tests: a changed weight must upload, a repeat must not)
+  size_t resident_uploads() const { return uploads_; }
 
  protected:
   dynamic_tensor compute(const std::vector<dynamic_tensor>& inputs) override {  // :35-118
@@ -59,14 +60,10 @@ class dense_ffn_node : public variadic_op_node {
       throw std::runtime_error("dense_ffn: down_w shape mismatch, expected [" + std::to_string(hidden_dim) +
                                ", " + std::to_string(ffn_dim) + "], got [" + std::to_string(down_w.dim(0)) +
                                ", " + std::to_string(down_w.dim(1)) + "]");
-    // the reference also has a scalar branch for FLOAT32 weights (:101-114); the engine
-    // hands this node float16 ones unless the checkpoint stores them as F32
-    if (wt != dtype::float16)
-      throw std::runtime_error("dense_ffn: FLOAT32 weights are not supported on this build");
     dynamic_tensor output(dtype::float32, {hidden.dim(0), hidden.dim(1), hidden_dim});
     if (tokens == 0) return output;
-    const int rc = csk_dense_ffn_f16(hidden.data_ptr<float>(), tokens, hidden_dim, ffn_dim, resident_copy(gate_w),
-                                     resident_copy(up_w), resident_copy(down_w),
+    const int rc = csk_dense_ffn_f16(hidden.data_ptr<float>(), tokens, hidden_dim, ffn_dim, resident_copy(0, gate_w),
+                                     resident_copy(1, up_w), resident_copy(2, down_w),
                                      has_bias ? inputs[4].data_ptr<float>() : nullptr,
                                      has_bias ? inputs[5].data_ptr<float>() : nullptr,
                                      has_bias ? inputs[6].data_ptr<float>() : nullptr, output.data_ptr<float>());
@@ -75,26 +72,11 @@ class dense_ffn_node : public variadic_op_node {
   }
 
  private:
-  struct resident {
-    csk_f16* handle;
-    int64_t rows, cols;
-  };
-  csk_f16* resident_copy(const dynamic_tensor& t) {
-    const uint16_t* key = t.data_ptr<uint16_t>();
-    auto it = resident_.find(key);
-    if (it != resident_.end() && it->second.rows == t.dim(0) && it->second.cols == t.dim(1))
-      return it->second.handle;
-    if (it != resident_.end()) {
-      csk_f16_free(it->second.handle);
-      resident_.erase(it);
-    }
-    csk_f16* h = nullptr;
-    if (csk_f16_upload(key, t.dim(0), t.dim(1), &h) != CSK_OK)
-      throw std::runtime_error(std::string("dense_ffn: ") + csk_last_error());
-    resident_[key] = resident{h, t.dim(0), t.dim(1)};
-    return h;
+  csk_f16* resident_copy(int role, const dynamic_tensor& t) {
+    return resident_[role].get(t, t.dim(0), t.dim(1), 0, "dense_ffn", &uploads_);
   }
-  std::unordered_map<const uint16_t*, resident> resident_;
+  csk_resident::weight_slot resident_[3];  // gate, up, down
+  size_t uploads_ = 0;
 };
 
 }  // namespace coalsack

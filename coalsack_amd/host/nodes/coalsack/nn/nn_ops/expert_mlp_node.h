@@ -23,6 +23,7 @@
 
 #include "coalsack/nn/nn_op_node.h"
 #include "coalsack/tensor/dynamic_mx_tensor_message.h"
+#include "coalsack/nn/nn_ops/resident_weight.h"
 #include "coalsack_moe.h"
 
 namespace coalsack {
@@ -125,29 +126,7 @@ class expert_mlp_node : public graph_node {
                                                                 : CSK_ACT_STANDARD_SWIGLU;
   }
 
-  // 64 eight-byte samples spread over the buffer, its length and its ends: enough to tell a
-  // rewritten or reused buffer from the one a device copy was made from, at no cost that matters
-  static uint64_t content_stamp(const uint8_t* p, size_t n) {
-    uint64_t h = 0x9E3779B97F4A7C15ull ^ n;
-    auto mix = [&h](uint64_t v) {
-      h ^= v + 0x9E3779B97F4A7C15ull + (h << 6) + (h >> 2);
-      h *= 0xBF58476D1CE4E5B9ull;
-    };
-    if (n < 8) {
-      for (size_t i = 0; i < n; ++i) mix(p[i]);
-      return h;
-    }
-    const size_t step = (n - 8) / 63 ? (n - 8) / 63 : 1;
-    for (size_t off = 0; off + 8 <= n; off += step) {
-      uint64_t v;
-      std::memcpy(&v, p + off, 8);
-      mix(v);
-    }
-    uint64_t v;
-    std::memcpy(&v, p + n - 8, 8);
-    mix(v);
-    return h;
-  }
+  static uint64_t content_stamp(const uint8_t* p, size_t n) { return csk_resident::content_stamp(p, n); }
 
   struct resident {
     csk_mxfp4* handle = nullptr;

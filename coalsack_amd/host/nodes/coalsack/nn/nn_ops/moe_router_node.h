@@ -1,7 +1,8 @@
 // moe_router_node backed by the gfx950 library: same class name, setters, test
 // wrappers, input order, output format and error texts as
 // include/coalsack/nn/nn_ops/moe_router_node.h of the reference (cited by line
-// below); the body calls csk_moe_router instead of the scalar CPU loops.
+// below); the body calls csk_moe_router (float32) or csk_moe_router_f64 (float64) instead
+// of the scalar CPU loops.
 //
 // Place this directory in front of the reference's include path to swap the
 // node in; it needs only coalsack/nn/nn_op_node.h and the C ABI header.
@@ -16,8 +17,8 @@
 
 namespace coalsack {
 
-// Inputs: hidden_states [batch, seq_len, hidden_dim] f32, gate_weights
-// [num_experts, hidden_dim] f32, optional gate_bias [num_experts] f32.
+// Inputs: hidden_states [batch, seq_len, hidden_dim] and gate_weights
+// [num_experts, hidden_dim], both f32 or both f64; optional gate_bias [num_experts] f32.
 // Output: [batch, seq_len, top_k, 2] f32 = (expert index, routing weight),
 // slots in descending logit order (moe_router_node.h:13-21).
 class moe_router_node : public variadic_op_node {
@@ -67,15 +68,24 @@ class moe_router_node : public variadic_op_node {
       throw std::runtime_error("moe_router: gate_bias must have num_experts=" +
                                std::to_string(num_experts_) + " elements, got " +
                                std::to_string(inputs[2].dim(0)));
-    // the GPU path computes in f32; the reference's float64 branch (:116-119) is not offered
-    if (hidden.get_dtype() != dtype::float32 || gate.get_dtype() != dtype::float32)
-      throw std::runtime_error("moe_router: only float32 supported on the GPU path");
+    // :115-122: the element type of the hidden states picks float or double arithmetic.  The
+    // reference reads the gate weights as that type whatever they hold; here a gate of
+    // another type is refused instead of being reinterpreted.
+    const dtype dt = hidden.get_dtype();
+    if (dt != dtype::float32 && dt != dtype::float64)
+      throw std::runtime_error("moe_router: only float32 and float64 supported");
+    if (gate.get_dtype() != dt)
+      throw std::runtime_error("moe_router: gate_weights must have the element type of hidden_states");
 
     dynamic_tensor output(dtype::float32, {batch, seq_len, top_k_, 2});
-    const int rc = csk_moe_router(hidden.data_ptr<float>(), batch * seq_len, hidden_dim,
-                                  gate.data_ptr<float>(), num_experts_,
-                                  has_bias ? inputs[2].data_ptr<float>() : nullptr, top_k_,
-                                  use_sigmoid_gating_ ? 1 : 0, output.data_ptr<float>());
+    const float* bias = has_bias ? inputs[2].data_ptr<float>() : nullptr;
+    const int rc = dt == dtype::float32
+                       ? csk_moe_router(hidden.data_ptr<float>(), batch * seq_len, hidden_dim, gate.data_ptr<float>(),
+                                        num_experts_, bias, top_k_, use_sigmoid_gating_ ? 1 : 0,
+                                        output.data_ptr<float>())
+                       : csk_moe_router_f64(hidden.data_ptr<double>(), batch * seq_len, hidden_dim,
+                                            gate.data_ptr<double>(), num_experts_, bias, top_k_,
+                                            use_sigmoid_gating_ ? 1 : 0, output.data_ptr<float>(), nullptr);
     if (rc != CSK_OK) throw std::runtime_error(std::string("moe_router: ") + csk_last_error());
     return output;
   }

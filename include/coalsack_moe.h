@@ -34,7 +34,7 @@ extern "C" {
 #define CSK_ERR_HIP 2          /* a HIP runtime call failed                      */
 #define CSK_ERR_RANGE 3        /* expert index outside [0, E)                    */
 #define CSK_ERR_ALL_EMPTY 4    /* merge: every expert tensor is empty            */
-#define CSK_ERR_SCALE 5        /* MXFP4 scale byte outside the exact range 2..254 */
+#define CSK_ERR_SCALE 5        /* MXFP4 scale byte 255 on a non-zero block (overflows fp32) */
 #define CSK_ERR_STATE 6        /* layer not fully populated                      */
 
 /* expert_mlp_node::activation_type (include/coalsack/nn/nn_ops/expert_mlp_node.h:27-30) */
@@ -109,7 +109,10 @@ int csk_kernel_times(float* ms_out2);
 int csk_mxfp4_upload(const uint8_t* blocks17_host, int64_t rows, int64_t K, csk_mxfp4** out);
 void csk_mxfp4_free(csk_mxfp4* m);
 /* Dequantise the resident copy on the GPU into host_out[rows*K]; bit-identical
- * to dequantize_block_mxfp4 (gguf_dequant.h:437-455) for scale bytes 2..254. */
+ * to dequantize_block_mxfp4 (gguf_dequant.h:437-455) for every scale byte the upload
+ * accepts: 0..254, and 255 on blocks of zeros (kept as 254: such a block is zero either way,
+ * so csk_mxfp4_export returns it with scale byte 254).  Blocks with scale bytes 0 and 1
+ * hold fp32 denormals (|w| <= 12 * 2^-127); the expert kernels contract them as zeros. */
 int csk_mxfp4_dequant(const csk_mxfp4* m, float* host_out);
 /* Recover the 17-byte blocks from the resident copy (round-trip check). */
 int csk_mxfp4_export(const csk_mxfp4* m, uint8_t* blocks17_host);
@@ -132,7 +135,15 @@ void csk_f16_free(csk_f16* m);
  * include/coalsack/gguf/gguf_dequant.h:149-258, 458-487).  rows * K must be a multiple
  * of 256 for the K-quants. */
 int csk_f16_upload_ggml(int ggml_type, const void* data_host, int64_t rows, int64_t K, csk_f16** out);
-/* Recover the row-major halves from the resident copy (round-trip check). */
+/* The same from a row-major fp32 matrix -- the FLOAT32 weights dense_ffn_node and
+ * matmul_transpose_mixed_node also accept (dense_ffn_node.h:57-60, 101-114;
+ * matmul_transpose_mixed_node.h:29-31, 91-101).  Kept as two fp16 terms side by side,
+ * [rows, 2 K] = [fp16(w) | fp16(w - fp16(w))] (absolute error below 2^-25; |w| <= 65504), and
+ * contracted against each activation row twice over, so the fp16 kernels serve both kinds.
+ * Accepted by csk_dense_ffn_f16 and csk_matmul_transpose_f16. */
+int csk_f16_upload_f32(const float* w_host, int64_t rows, int64_t K, csk_f16** out);
+/* Recover the row-major halves from the resident copy (round-trip check); [rows, 2 K] for a
+ * matrix that came in as fp32. */
 int csk_f16_export(const csk_f16* m, uint16_t* halves_host);
 
 /* ---- one MoE layer, weights resident ------------------------------------ */
@@ -308,6 +319,26 @@ int csk_expert_merge(const float* router_pairs, int64_t T, int64_t k, int64_t E,
 /* rmsnorm_node::compute (rmsnorm_node.h:62-83) and add_node (add_node.h:8-55) */
 int csk_rmsnorm(const float* x, const float* weight, float* out, int64_t T, int64_t H, float eps);
 int csk_add(const float* a, const float* b, float* out, int64_t n);
+/* add_node over operands of different shapes and of the node's other element types
+ * (add_node.h:16-50 through elementwise_binary_op, elementwise_helpers.h:9-66): numpy-style
+ * broadcasting over trailing dimensions as dynamic_tensor::broadcast_shape defines it
+ * (dynamic_tensor.h:218-238).  dtype is one of CSK_DT_*; both operands and the result have
+ * it.  `out` holds the broadcast shape's element count.  Shapes that do not broadcast return
+ * CSK_ERR_ARG with the reference's text "Broadcast failed: Shape A=[..], Shape B=[..]".  At
+ * most 8 dimensions.  Integer sums wrap. */
+#define CSK_DT_FLOAT32 0
+#define CSK_DT_FLOAT64 1
+#define CSK_DT_INT32 2
+#define CSK_DT_INT64 3
+int csk_add_broadcast(const void* a, const int64_t* shape_a, int nd_a, const void* b,
+                      const int64_t* shape_b, int nd_b, int dtype, void* out);
+/* moe_router_node::compute_impl<double> (moe_router_node.h:115-118, 141-214): float64 hidden
+ * states [T,H] and gate weights [E,H], float32 bias [E] or NULL; logits are the reference's
+ * sequential float64 sums bit for bit, selection runs on them, weights and the [T,k,2]
+ * output are float32.  out_logits ([T,E] float64) may be NULL. */
+int csk_moe_router_f64(const double* hidden, int64_t T, int64_t H, const double* gate_w, int64_t E,
+                       const float* gate_b, int64_t k, int sigmoid, float* out_pairs,
+                       double* out_logits);
 
 #ifdef __cplusplus
 }

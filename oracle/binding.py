@@ -81,6 +81,16 @@ class Oracle:
         d.orc_dense_ffn_f16.argtypes = [_P, _I64, _I64, _I64] + [_P] * 7
         d.orc_matmul_transpose_f16.restype = None
         d.orc_matmul_transpose_f16.argtypes = [_P, _P, _P, _I64, _I64, _I64]
+        d.orc_matmul_transpose_f32.restype = None
+        d.orc_matmul_transpose_f32.argtypes = [_P, _P, _P, _I64, _I64, _I64]
+        d.orc_matmul_transpose_batched.restype = None
+        d.orc_matmul_transpose_batched.argtypes = [_P, _I64, _P, _I64, C.c_int, _I64, _P, _I64, _I64, _I64]
+        d.orc_dense_ffn_f32.restype = C.c_int
+        d.orc_dense_ffn_f32.argtypes = [_P, _I64, _I64, _I64] + [_P] * 7
+        d.orc_add_broadcast.restype = C.c_int
+        d.orc_add_broadcast.argtypes = [_P, _P, C.c_int, _P, _P, C.c_int, C.c_int, _P, _P]
+        d.orc_router_f64.restype = C.c_int
+        d.orc_router_f64.argtypes = [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P, _P]
         d.orc_expert_merge.restype = C.c_int
         d.orc_expert_merge.argtypes = [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]
         d.orc_rmsnorm.restype = None
@@ -216,6 +226,81 @@ class Oracle:
         out = np.empty((M, N), np.float32)
         self.dll.orc_matmul_transpose_f16(_p(a), _p(b), _p(out), M, K, N)
         return out
+
+    def matmul_transpose_f32(self, a, b):
+        """matmul_transpose_mixed_node with a float32 weight: a [M,K], b [N,K] -> [M,N]."""
+        a, b = _f32(a), _f32(b)
+        M, K = a.shape
+        N = b.shape[0]
+        out = np.empty((M, N), np.float32)
+        self.dll.orc_matmul_transpose_f32(_p(a), _p(b), _p(out), M, K, N)
+        return out
+
+    def matmul_transpose_batched(self, a, b):
+        """a [*, M, K] float32, b [*, N, K] float16 or float32; the node's batch rule
+        (output matrix i pairs matrix i % n_a of a with matrix i % n_b of b)."""
+        a = _f32(a)
+        b = _f16(b) if b.dtype == np.float16 else _f32(b)
+        M, K = a.shape[-2:]
+        N = b.shape[-2]
+        batch = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+        n_out = int(np.prod(batch, dtype=np.int64))
+        n_a, n_b = a.size // (M * K), b.size // (N * K)
+        out = np.empty(tuple(batch) + (M, N), np.float32)
+        self.dll.orc_matmul_transpose_batched(_p(a), n_a, _p(b), n_b, int(b.dtype == np.float16), n_out,
+                                              _p(out), M, K, N)
+        return out
+
+    def dense_ffn_f32(self, hidden, w_gate, w_up, w_down, b_gate=None, b_up=None, b_down=None):
+        """dense_ffn_node with FLOAT32 weights: hidden [T,H]; w_gate/w_up [F,H], w_down [H,F]."""
+        hidden = _f32(hidden)
+        w_gate, w_up, w_down = _f32(w_gate), _f32(w_up), _f32(w_down)
+        b_gate, b_up, b_down = _f32(b_gate), _f32(b_up), _f32(b_down)
+        T, H = hidden.shape
+        F = w_gate.shape[0]
+        out = np.empty((T, H), np.float32)
+        rc = self.dll.orc_dense_ffn_f32(_p(hidden), T, H, F, _p(w_gate), _p(w_up), _p(w_down), _p(b_gate),
+                                        _p(b_up), _p(b_down), _p(out))
+        if rc:
+            raise ValueError(f"orc_dense_ffn_f32 rc={rc}")
+        return out
+
+    _ADD_DTYPES = {np.dtype(np.float32): 0, np.dtype(np.float64): 1, np.dtype(np.int32): 2, np.dtype(np.int64): 3}
+
+    def add_broadcast(self, a, b):
+        """add_node over two arrays of one element type; None when the shapes do not broadcast."""
+        a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+        assert a.dtype == b.dtype
+        nd = max(a.ndim, b.ndim)
+        sa = np.array(a.shape, np.int64)
+        sb = np.array(b.shape, np.int64)
+        oshape = np.zeros(max(nd, 1), np.int64)
+        # size the output before the call: the shape is a function of the inputs' shapes alone
+        try:
+            shape = np.broadcast_shapes(a.shape, b.shape)
+        except ValueError:
+            shape = (0,)
+        out = np.empty(shape, a.dtype)
+        rc = self.dll.orc_add_broadcast(_p(a), _p(sa), a.ndim, _p(b), _p(sb), b.ndim,
+                                        self._ADD_DTYPES[a.dtype], _p(out), _p(oshape))
+        if rc:
+            return None
+        assert tuple(oshape[:nd]) == tuple(shape), (oshape, shape)
+        return out
+
+    def router_f64(self, hidden, gate_w, gate_b, k, sigmoid=False, want_logits=False):
+        hidden = np.ascontiguousarray(hidden, np.float64)
+        gate_w = np.ascontiguousarray(gate_w, np.float64)
+        gate_b = _f32(gate_b)
+        T, H = hidden.shape
+        E = gate_w.shape[0]
+        out = np.empty((T, k, 2), np.float32)
+        logits = np.empty((T, E), np.float64) if want_logits else None
+        rc = self.dll.orc_router_f64(_p(hidden), T, H, _p(gate_w), E, _p(gate_b), k, int(sigmoid),
+                                     _p(out), _p(logits))
+        if rc:
+            raise ValueError(f"orc_router_f64 rc={rc}")
+        return (out, logits) if want_logits else out
 
     def expert_merge(self, pairs, expert_outs, H, pre_weighted=False):
         pairs = _f32(pairs)

@@ -49,6 +49,24 @@
  *        - float64 matrix product over the fp16 weights widened exactly, shapes
  *          that exercise both column paths and every remainder, identity /
  *          one-hot weights.  PARITY UNPINNED at the last ulp, as above.
+ *   orc_matmul_transpose_f32 / orc_matmul_transpose_batched
+ *        - float64 matrix product, the same shapes as the fp16 function, equality
+ *          with the fp16 function on weights fp16 holds exactly; batched: each
+ *          output matrix against numpy's broadcast matmul where the modulus
+ *          indexing and broadcasting agree (one side without batch dims, or
+ *          equal batch shapes), and the modulus rule itself on a [2,1]x[1,3]
+ *          batch where they differ.  PARITY UNPINNED at the last ulp, as above.
+ *   orc_dense_ffn_f32
+ *        - independent float64 evaluation; equality with a numpy float32
+ *          sequential loop on small shapes (the rounding order is fully stated
+ *          by the scalar source).
+ *   orc_add_broadcast
+ *        - numpy's broadcasting add for all four element types, shapes with
+ *          leading, inner and both-sided 1s, zero-sized dims, refused shapes.
+ *   orc_router_f64
+ *        - the float32 known answers widened to float64, brute-force argsort of
+ *          float64 logits (numpy sequential sums are not used: logits compared
+ *          to math.fsum within 1e-12), tie order of all-equal logits.
  *   orc_expert_merge
  *        - definition sum_k w_k * y_{e_k}; one-hot weights reduce to a copy;
  *          linearity; error cases.
@@ -643,6 +661,80 @@ __attribute__((target("f16c,avx2,fma"))) void orc_matmul_transpose_f16(const flo
   }
 }
 
+/* matmul_transpose_mixed_node.h:116-196 (compute_matmul_avx2): the same with an fp32 B. */
+__attribute__((target("avx2,fma"))) void orc_matmul_transpose_f32(const float* a, const float* b, float* out,
+                                                                  int64_t M, int64_t K, int64_t N) {
+  for (int64_t i = 0; i < M; ++i) {
+    const float* ar = a + i * K;
+    for (int64_t j = 0; j < N; ++j) {
+      const float* br = b + j * K;
+      const int tiled = j < (N / 4) * 4;
+      int64_t k = 0;
+      __m256 sum = _mm256_setzero_ps();
+      if (tiled) {
+        __m256 sa = _mm256_setzero_ps(), sb = _mm256_setzero_ps();
+        for (; k + 16 <= K; k += 16) {
+          sa = _mm256_fmadd_ps(_mm256_loadu_ps(ar + k), _mm256_loadu_ps(br + k), sa);
+          sb = _mm256_fmadd_ps(_mm256_loadu_ps(ar + k + 8), _mm256_loadu_ps(br + k + 8), sb);
+        }
+        sum = _mm256_add_ps(sa, sb);
+      }
+      for (; k + 8 <= K; k += 8) sum = _mm256_fmadd_ps(_mm256_loadu_ps(ar + k), _mm256_loadu_ps(br + k), sum);
+      float r = hsum_avx2(sum);
+      for (; k < K; ++k) r = __builtin_fmaf(ar[k], br[k], r);
+      out[i * N + j] = r;
+    }
+  }
+}
+
+/* matmul_transpose_mixed_node.h:47-110: leading (batch) dimensions.  The output has the
+ * broadcast batch shape; matrix `batch` of it pairs matrix batch % n_a of A with matrix
+ * batch % n_b of B -- a modulus, not a stride walk, exactly as the node indexes them. */
+void orc_matmul_transpose_batched(const float* a, int64_t n_a, const void* b, int64_t n_b, int b_is_f16,
+                                  int64_t n_out, float* out, int64_t M, int64_t K, int64_t N) {
+  for (int64_t batch = 0; batch < n_out; ++batch) {
+    const float* am = a + (batch % n_a) * M * K;
+    float* om = out + batch * M * N;
+    if (b_is_f16)
+      orc_matmul_transpose_f16(am, (const uint16_t*)b + (batch % n_b) * N * K, om, M, K, N);
+    else
+      orc_matmul_transpose_f32(am, (const float*)b + (batch % n_b) * N * K, om, M, K, N);
+  }
+}
+
+/* dense_ffn_node.h:122-153 (compute_token_f32): FLOAT32 weights, plain scalar loops -- every
+ * product and every sum rounded on its own (the function carries no target attribute, so a
+ * -O2 build without -march contracts nothing).  Each bias optional. */
+int orc_dense_ffn_f32(const float* hidden, int64_t T, int64_t H, int64_t F, const float* w_gate,
+                      const float* w_up, const float* w_down, const float* b_gate, const float* b_up,
+                      const float* b_down, float* out) {
+  if (T < 0 || H <= 0 || F <= 0) return ORC_ERR_ARG;
+  float* act = (float*)malloc((size_t)F * sizeof(float));
+  if (!act) return ORC_ERR_ARG;
+  for (int64_t t = 0; t < T; ++t) {
+    const float* x = hidden + t * H;
+    for (int64_t o = 0; o < F; ++o) {
+      float gate_sum = 0.0f, up_sum = 0.0f;
+      for (int64_t i = 0; i < H; ++i) {
+        gate_sum += x[i] * w_gate[o * H + i];
+        up_sum += x[i] * w_up[o * H + i];
+      }
+      if (b_gate) gate_sum += b_gate[o];
+      if (b_up) up_sum += b_up[o];
+      const float silu = gate_sum / (1.0f + expf(-gate_sum));
+      act[o] = silu * up_sum;
+    }
+    for (int64_t o = 0; o < H; ++o) {
+      float sum = 0.0f;
+      for (int64_t i = 0; i < F; ++i) sum += act[i] * w_down[o * F + i];
+      if (b_down) sum += b_down[o];
+      out[t * H + o] = sum;
+    }
+  }
+  free(act);
+  return ORC_OK;
+}
+
 /* ------------------------------------------------------------------ merge */
 
 /* expert_merge_node.h:30-134.  expert_outs[e] is [T,H] or NULL for an empty
@@ -785,4 +877,157 @@ int orc_moe_layer(const orc_layer_t* L, const float* hidden, int64_t T, float* o
   free(tmp);
   free(normed);
   return rc;
+}
+
+
+/* ------------------------------------------------- elementwise add, broadcast */
+
+/* elementwise_helpers.h:9-66 + add_node.h:8-55: numpy-style broadcasting over trailing
+ * dimensions (dynamic_tensor.h:218-238), one element type for both operands and the result.
+ * dtype: 0 float32, 1 float64, 2 int32, 3 int64.  out_shape receives the broadcast shape
+ * (max(nd_a, nd_b) entries); returns ORC_ERR_ARG when the shapes do not broadcast. */
+int orc_add_broadcast(const void* a, const int64_t* sa, int nd_a, const void* b, const int64_t* sb, int nd_b,
+                      int dtype, void* out, int64_t* out_shape) {
+  const int nd = nd_a > nd_b ? nd_a : nd_b;
+  int64_t stra[16], strb[16];
+  if (nd > 16) return ORC_ERR_ARG;
+  int64_t n = 1;
+  for (int i = 0; i < nd; ++i) {
+    const int64_t da = i < nd_a ? sa[nd_a - 1 - i] : 1, db = i < nd_b ? sb[nd_b - 1 - i] : 1;
+    if (!(da == db || da == 1 || db == 1)) return ORC_ERR_ARG;
+    out_shape[nd - 1 - i] = (da == 0 || db == 0) ? 0 : (da > db ? da : db);
+  }
+  for (int i = 0; i < nd; ++i) n *= out_shape[i];
+  /* row-major strides of each operand, aligned to the trailing dimensions; 0 where it repeats */
+  int64_t run = 1;
+  for (int i = 0; i < nd; ++i) {
+    const int d = nd - 1 - i;
+    if (i < nd_a) {
+      stra[d] = sa[nd_a - 1 - i] == 1 ? 0 : run;
+      run *= sa[nd_a - 1 - i];
+    } else {
+      stra[d] = 0;
+    }
+  }
+  run = 1;
+  for (int i = 0; i < nd; ++i) {
+    const int d = nd - 1 - i;
+    if (i < nd_b) {
+      strb[d] = sb[nd_b - 1 - i] == 1 ? 0 : run;
+      run *= sb[nd_b - 1 - i];
+    } else {
+      strb[d] = 0;
+    }
+  }
+  for (int64_t i = 0; i < n; ++i) {
+    int64_t t = i, ia = 0, ib = 0;
+    for (int d = nd - 1; d >= 0; --d) {
+      const int64_t idx = t % out_shape[d];
+      t /= out_shape[d];
+      ia += idx * stra[d];
+      ib += idx * strb[d];
+    }
+    switch (dtype) {
+      case 0: ((float*)out)[i] = ((const float*)a)[ia] + ((const float*)b)[ib]; break;
+      case 1: ((double*)out)[i] = ((const double*)a)[ia] + ((const double*)b)[ib]; break;
+      case 2: ((int32_t*)out)[i] = (int32_t)((uint32_t)((const int32_t*)a)[ia] + (uint32_t)((const int32_t*)b)[ib]); break;
+      case 3: ((int64_t*)out)[i] = (int64_t)((uint64_t)((const int64_t*)a)[ia] + (uint64_t)((const int64_t*)b)[ib]); break;
+      default: return ORC_ERR_ARG;
+    }
+  }
+  return ORC_OK;
+}
+
+/* ------------------------------------------------------------ router, float64 */
+
+/* moe_router_node.h:115-118, compute_impl<double> (:141-214): hidden states and gate weights
+ * are float64, the bias float32 widened per expert, logits sequential double sums, selection
+ * on the double logits (the same partial_sort restated above), weights computed in float
+ * from the double differences, output float32 pairs. */
+typedef struct {
+  double v;
+  int64_t i;
+} scored64;
+static int before64(const scored64* a, const scored64* b) { return a->v > b->v; }
+static void sift64(scored64* h, int64_t hole, int64_t len, scored64 val) {
+  /* libstdc++ __adjust_heap followed by __push_heap, comparator before64 */
+  const int64_t top = hole;
+  int64_t child = hole;
+  while (child < (len - 1) / 2) {
+    child = 2 * (child + 1);
+    if (before64(&h[child], &h[child - 1])) --child;
+    h[hole] = h[child];
+    hole = child;
+  }
+  if ((len & 1) == 0 && child == (len - 2) / 2) {
+    child = 2 * (child + 1);
+    h[hole] = h[child - 1];
+    hole = child - 1;
+  }
+  int64_t parent = (hole - 1) / 2;
+  while (hole > top && before64(&h[parent], &val)) {
+    h[hole] = h[parent];
+    hole = parent;
+    parent = (hole - 1) / 2;
+  }
+  h[hole] = val;
+}
+static void partial_sort64(scored64* first, int64_t middle, int64_t last) {
+  /* std::partial_sort = __heap_select + __sort_heap (GCC 11 stl_algo.h / stl_heap.h) */
+  if (middle >= 2)
+    for (int64_t parent = (middle - 2) / 2;; --parent) {
+      sift64(first, parent, middle, first[parent]);
+      if (parent == 0) break;
+    }
+  for (int64_t i = middle; i < last; ++i)
+    if (before64(&first[i], &first[0])) {
+      const scored64 val = first[i];
+      first[i] = first[0];
+      sift64(first, 0, middle, val);
+    }
+  for (int64_t end = middle; end > 1; --end) {
+    const scored64 val = first[end - 1];
+    first[end - 1] = first[0];
+    sift64(first, 0, end - 1, val);
+  }
+}
+
+int orc_router_f64(const double* hidden, int64_t T, int64_t H, const double* gate_w, int64_t E,
+                   const float* gate_b, int64_t k, int sigmoid, float* out_pairs, double* out_logits) {
+  if (T < 0 || H <= 0 || E <= 0 || k <= 0 || k > E) return ORC_ERR_ARG;
+  scored64* sc = (scored64*)malloc((size_t)E * sizeof(scored64));
+  float* w = (float*)malloc((size_t)k * sizeof(float));
+  if (!sc || !w) return ORC_ERR_ARG;
+  for (int64_t t = 0; t < T; ++t) {
+    const double* x = hidden + t * H;
+    for (int64_t e = 0; e < E; ++e) {
+      double sum = 0;
+      for (int64_t d = 0; d < H; ++d) sum += x[d] * gate_w[e * H + d];
+      sc[e].v = sum + (gate_b ? (double)gate_b[e] : 0.0);
+      sc[e].i = e;
+      if (out_logits) out_logits[t * E + e] = sc[e].v;
+    }
+    partial_sort64(sc, k, E);
+    if (sigmoid) {
+      for (int64_t j = 0; j < k; ++j) w[j] = 1.0f / (1.0f + expf(-(float)sc[j].v));
+    } else {
+      double mx = sc[0].v;
+      for (int64_t j = 1; j < k; ++j)
+        if (sc[j].v > mx) mx = sc[j].v;
+      float sum = 0.0f;
+      for (int64_t j = 0; j < k; ++j) {
+        w[j] = expf((float)(sc[j].v - mx));
+        sum += w[j];
+      }
+      const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+      for (int64_t j = 0; j < k; ++j) w[j] *= inv;
+    }
+    for (int64_t j = 0; j < k; ++j) {
+      out_pairs[(t * k + j) * 2] = (float)sc[j].i;
+      out_pairs[(t * k + j) * 2 + 1] = w[j];
+    }
+  }
+  free(sc);
+  free(w);
+  return ORC_OK;
 }

@@ -38,6 +38,12 @@ int orc_dense_ffn_f16(const float*, int64_t, int64_t, int64_t, const uint16_t*, 
 void orc_matmul_transpose_f16(const float*, const uint16_t*, float*, int64_t, int64_t, int64_t);
 void orc_rmsnorm(const float*, const float*, float*, int64_t, int64_t, float);
 void orc_add(const float*, const float*, float*, int64_t);
+void orc_matmul_transpose_batched(const float*, int64_t, const void*, int64_t, int, int64_t, float*, int64_t, int64_t,
+                                  int64_t);
+int orc_dense_ffn_f32(const float*, int64_t, int64_t, int64_t, const float*, const float*, const float*, const float*,
+                      const float*, const float*, float*);
+int orc_add_broadcast(const void*, const int64_t*, int, const void*, const int64_t*, int, int, void*, int64_t*);
+int orc_router_f64(const double*, int64_t, int64_t, const double*, int64_t, const float*, int64_t, int, float*, double*);
 }
 
 static int g_failed = 0, g_checks = 0;
@@ -102,6 +108,10 @@ static void cpu_router_argument_errors() {
   CHECK(throws_with([&] { node.compute_test(h3, g_bad); }, "moe_router: gate_weights shape mismatch, expected [8, 4], got [7, 4]"));
   CHECK(throws_with([&] { node.compute_test(h3, g, b_bad); }, "moe_router: gate_bias must have num_experts=8 elements, got 5"));
   CHECK(throws_with([&] { node.compute_test(h3, g, b2); }, "moe_router: gate_bias must be 1D"));
+  CHECK(throws_with([&] { node.compute_test(dynamic_tensor(dtype::int32, {1, 2, 4}), g); },
+                    "moe_router: only float32 and float64 supported"));
+  CHECK(throws_with([&] { node.compute_test(dynamic_tensor(dtype::float64, {1, 2, 4}), g); },
+                    "moe_router: gate_weights must have the element type of hidden_states"));
   // through process(): the exception becomes an error result with a null field (nn_op_node.h:306-314)
   capture_node cap;
   cap.set_input(node.get_output());
@@ -255,8 +265,8 @@ static void cpu_dense_ffn_argument_errors() {
   CHECK(throws_with([&] { node.compute_test({hidden, gate, up, random_half_tensor({8, 15}, gen, -1, 1)}); },
                     "dense_ffn: down_w shape mismatch, expected [8, 16], got [8, 15]"));
   CHECK(throws_with([&] { node.compute_test({hidden, random_tensor({16, 8}, gen, -1, 1), random_tensor({16, 8}, gen, -1, 1),
-                                             random_tensor({8, 16}, gen, -1, 1)}); },
-                    "dense_ffn: FLOAT32 weights are not supported on this build"));
+                                             down}); },
+                    "dense_ffn: weight tensors must all be FLOAT16 or all FLOAT32"));
 }
 
 static void cpu_matmul_argument_errors() {
@@ -270,7 +280,8 @@ static void cpu_matmul_argument_errors() {
   CHECK(throws_with([&] { node.compute_test(a, dynamic_tensor(dtype::int32, {5, 8})); }, "matmul_transpose_mixed: input B must be fp32 or fp16"));
   CHECK(throws_with([&] { node.compute_test(dynamic_tensor(dtype::float32, {8}), w); }, "matmul_transpose_mixed: inputs must be at least 2D"));
   CHECK(throws_with([&] { node.compute_test(a, random_half_tensor({5, 7}, gen, -1, 1)); }, "matmul_transpose_mixed: incompatible dimensions"));
-  CHECK(throws_with([&] { node.compute_test(a, random_tensor({5, 8}, gen, -1, 1)); }, "only a 2D fp16 input B is supported"));
+  CHECK(throws_with([&] { node.compute_test(a, random_half_tensor({3, 5, 8}, gen, -1, 1)); },
+                    "Incompatible shapes for broadcasting"));  // batch [2] against [3]
 }
 
 static void cpu_merge_argument_errors() {
@@ -304,7 +315,9 @@ static void cpu_norm_add_argument_errors() {
   CHECK(throws_with([&] { norm.compute_test(x, w2); }, "rmsnorm: weight shape must be [hidden_dim]"));
   CHECK(throws_with([&] { norm.compute_test(dynamic_tensor(dtype::float64, {2, 8}), w); }, "rmsnorm: only float32"));
   CHECK(throws_with([&] { add.compute_test(x, dynamic_tensor(dtype::float64, {2, 3, 8})); }, "add: input dtype mismatch"));
-  CHECK(throws_with([&] { add.compute_test(x, w); }, "add: broadcasting is not supported"));
+  CHECK(throws_with([&] { add.compute_test(x, w_bad); }, "Broadcast failed: Shape A=[2,3,8], Shape B=[7]"));
+  CHECK(throws_with([&] { add.compute_test(dynamic_tensor(dtype::float16, {2}), dynamic_tensor(dtype::float16, {2})); },
+                    "add: unsupported dtype"));
   // through process(): missing input names and upstream errors (nn_op_node.h:172-219)
   capture_node cap;
   cap.set_input(norm.get_output());
@@ -562,6 +575,115 @@ static void gpu_dense_ffn_tests() {
   }
 }
 
+// The branches beside the engine's own use of these nodes: float32 weights, batched
+// weights, broadcasting / other element types in add, float64 in the router.
+static void gpu_variant_branches() {
+  std::printf("variants: fp32 / batched matmul, fp32 dense_ffn, broadcasting add, float64 router\n");
+  std::mt19937 gen(31);
+  auto rel_worst = [](const float* got, const float* want, int64_t n) {
+    float worst = 0, scale = 0;
+    for (int64_t i = 0; i < n; ++i) {
+      worst = std::fmax(worst, std::fabs(got[i] - want[i]));
+      scale = std::fmax(scale, std::fabs(want[i]));
+    }
+    return worst / std::fmax(scale, 1e-6f);
+  };
+  {  // matmul: every pairing of batch shapes the node accepts, fp16 and fp32 B
+    struct shapes { std::vector<int64_t> a, b; };
+    for (const shapes& sh : std::vector<shapes>{{{2, 40, 72}, {130, 72}}, {{3, 4, 16}, {3, 5, 16}}, {{4, 16}, {3, 5, 16}},
+                                                {{2, 3, 4, 16}, {3, 5, 16}}, {{2, 1, 2, 8}, {1, 3, 3, 8}}, {{7, 37}, {29, 37}},
+                                                {{2, 1, 4, 16}, {70, 5, 16}}}) {
+      for (bool half : {true, false}) {
+        auto a = random_tensor(sh.a, gen, -1, 1);
+        auto b = half ? random_half_tensor(sh.b, gen, -0.2f, 0.2f) : random_tensor(sh.b, gen, -0.2f, 0.2f);
+        matmul_transpose_mixed_node node;
+        auto out = node.compute_test(a, b);
+        const int64_t m = a.dim(-2), k = a.dim(-1), n = b.dim(-2);
+        const int64_t n_a = a.numel() / (m * k), n_b = b.numel() / (n * k), n_out = out.numel() / (m * n);
+        CHECK(out.dim(-2) == m && out.dim(-1) == n && n_out >= std::max(n_a, n_b));
+        std::vector<float> want(out.numel());
+        orc_matmul_transpose_batched(a.data_ptr<float>(), n_a, b.data_ptr<uint8_t>(), n_b, half, n_out, want.data(), m, k, n);
+        CHECK(rel_worst(out.data_ptr<float>(), want.data(), out.numel()) <= (half ? 1e-3f : 2e-5f));
+        const size_t uploads = node.resident_uploads();
+        CHECK(uploads == (size_t)std::min<int64_t>(n_b, n_out) || n_b > matmul_transpose_mixed_node::kMaxResidentMatrices);
+        if (n_b <= matmul_transpose_mixed_node::kMaxResidentMatrices) {
+          node.compute_test(a, b);  // the same weight again: no new device copies
+          CHECK(node.resident_uploads() == uploads);
+        }
+      }
+    }
+  }
+  {  // dense_ffn with FLOAT32 weights, and a weight rewritten in place between frames
+    const int64_t B = 2, S = 9, H = 72, F = 130;
+    auto hidden = random_tensor({B, S, H}, gen, -1, 1);
+    auto gate = random_tensor({F, H}, gen, -0.2f, 0.2f), up = random_tensor({F, H}, gen, -0.2f, 0.2f);
+    auto down = random_tensor({H, F}, gen, -0.2f, 0.2f);
+    auto bg = random_tensor({F}, gen, -0.1f, 0.1f), bu = random_tensor({F}, gen, -0.1f, 0.1f), bd = random_tensor({H}, gen, -0.1f, 0.1f);
+    dense_ffn_node node;
+    std::vector<float> want(B * S * H);
+    for (int round = 0; round < 3; ++round) {
+      auto out = node.compute_test({hidden, gate, up, down, bg, bu, bd});
+      CHECK(orc_dense_ffn_f32(hidden.data_ptr<float>(), B * S, H, F, gate.data_ptr<float>(), up.data_ptr<float>(),
+                              down.data_ptr<float>(), bg.data_ptr<float>(), bu.data_ptr<float>(), bd.data_ptr<float>(),
+                              want.data()) == 0);
+      CHECK(rel_worst(out.data_ptr<float>(), want.data(), out.numel()) <= 2e-5f);
+      CHECK(node.resident_uploads() == (round < 2 ? 3u : 4u));
+      if (round == 1) up = random_tensor({F, H}, gen, -0.2f, 0.2f);  // a reloaded weight: new storage, new bytes
+    }
+  }
+  {  // add: broadcasting and the other element types, bit-exact
+    add_node add;
+    auto x = random_tensor({2, 5, 96}, gen, -2, 2), row = random_tensor({96}, gen, -2, 2), col = random_tensor({5, 1}, gen, -2, 2);
+    for (const dynamic_tensor* other : {&row, &col}) {
+      auto out = add.compute_test(x, *other);
+      CHECK(out.shape() == x.shape());
+      std::vector<float> want(x.numel());
+      int64_t oshape[8];
+      CHECK(orc_add_broadcast(x.data_ptr<float>(), x.shape().data(), 3, other->data_ptr<float>(), other->shape().data(),
+                              (int)other->ndim(), 0, want.data(), oshape) == 0);
+      CHECK(std::memcmp(out.data_ptr<float>(), want.data(), want.size() * 4) == 0);
+    }
+    dynamic_tensor i64a(dtype::int64, {3, 1}), i64b(dtype::int64, {1, 4}), f64a(dtype::float64, {2, 3}), f64b(dtype::float64, {3});
+    dynamic_tensor i32a(dtype::int32, {4}), i32b(dtype::int32, {1});
+    for (int i = 0; i < 3; ++i) i64a.data_ptr<int64_t>()[i] = (int64_t)1 << (40 + i);
+    for (int i = 0; i < 4; ++i) i64b.data_ptr<int64_t>()[i] = i - 2, i32a.data_ptr<int32_t>()[i] = (int32_t)(500000000u * (uint32_t)i);
+    i32b.data_ptr<int32_t>()[0] = 2000000000;  // wraps for i >= 1, like the reference's int32 sum on this target
+    for (int i = 0; i < 6; ++i) f64a.data_ptr<double>()[i] = 1.0 + i * 1e-13;
+    for (int i = 0; i < 3; ++i) f64b.data_ptr<double>()[i] = 1e-3 * i;
+    auto o64 = add.compute_test(i64a, i64b);
+    CHECK((o64.shape() == std::vector<int64_t>{3, 4}) && o64.get_dtype() == dtype::int64);
+    for (int i = 0; i < 3; ++i)
+      for (int j = 0; j < 4; ++j) CHECK(o64.data_ptr<int64_t>()[i * 4 + j] == ((int64_t)1 << (40 + i)) + j - 2);
+    auto o32 = add.compute_test(i32a, i32b);
+    for (int i = 0; i < 4; ++i)
+      CHECK(o32.data_ptr<int32_t>()[i] == (int32_t)(500000000u * (uint32_t)i + 2000000000u));
+    auto od = add.compute_test(f64a, f64b);
+    CHECK(od.get_dtype() == dtype::float64);
+    for (int i = 0; i < 6; ++i) CHECK(od.data_ptr<double>()[i] == f64a.data_ptr<double>()[i] + f64b.data_ptr<double>()[i % 3]);
+    CHECK(add.compute_test(dynamic_tensor(dtype::float32, {2, 0, 3}), dynamic_tensor(dtype::float32, {1, 3})).numel() == 0);
+  }
+  {  // router on float64 inputs: experts exactly the CPU path's
+    const int64_t B = 2, S = 8, H = 128, E = 32, K = 4;
+    dynamic_tensor h(dtype::float64, {B, S, H}), g(dtype::float64, {E, H});
+    std::uniform_real_distribution<double> d(-1, 1);
+    for (int64_t i = 0; i < h.numel(); ++i) h.data_ptr<double>()[i] = d(gen);
+    for (int64_t i = 0; i < g.numel(); ++i) g.data_ptr<double>()[i] = 0.2 * d(gen);
+    auto b = random_tensor({E}, gen, -0.01f, 0.01f);
+    for (bool sigmoid : {false, true}) {
+      moe_router_node node;
+      node.set_config(E, K);
+      node.set_sigmoid_gating(sigmoid);
+      auto out = node.compute_test(h, g, b);
+      CHECK((out.shape() == std::vector<int64_t>{B, S, K, 2}) && out.get_dtype() == dtype::float32);
+      std::vector<float> want(B * S * K * 2);
+      CHECK(orc_router_f64(h.data_ptr<double>(), B * S, H, g.data_ptr<double>(), E, b.data_ptr<float>(), K, sigmoid,
+                           want.data(), nullptr) == 0);
+      for (int64_t p = 0; p < B * S * K; ++p)
+        CHECK(out.data_ptr<float>()[2 * p] == want[2 * p] && std::fabs(out.data_ptr<float>()[2 * p + 1] - want[2 * p + 1]) < 1e-6f);
+    }
+  }
+}
+
 // router -> E expert nodes -> merge, wired with edges and result messages the way
 // llm_engine builds the block (src/llm/llm_engine.cpp:721-753), against the CPU checker.
 static void gpu_node_chain() {
@@ -766,6 +888,7 @@ int main(int argc, char** argv) {
     gpu_expert_fp16_tests();
     gpu_dense_ffn_tests();
     gpu_matmul_tests();
+    gpu_variant_branches();
     gpu_node_chain();
     gpu_expert_weight_reload();
     gpu_norm_add_tests();

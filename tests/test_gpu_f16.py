@@ -243,3 +243,67 @@ def test_matmul_transpose_matches_oracle(lib, oracle, M, K, N):
     assert_layer_close(got, want)
     with pytest.raises(capi.CskError, match="incompatible dimensions"):
         lib.matmul_transpose_f16(a[:, :K - 1] if K > 1 else a, w)
+
+
+@pytest.mark.parametrize("T,H,F", [(1, 64, 96), (7, 37, 29), (65, 96, 160), (3, 1024, 2048)])
+@pytest.mark.parametrize("bias", ["none", "all"])
+def test_dense_ffn_float32_weights_match_oracle(lib, oracle, T, H, F, bias):
+    """dense_ffn_node's FLOAT32 weight branch (dense_ffn_node.h:102-113): the weights travel as two
+    fp16 terms, so they are exact to 2^-25 absolute; the result is held to the layer bar against
+    the oracle's scalar fp32 loops and to 2e-5 of the largest output against float64."""
+    rng = np.random.default_rng([T, H, F, 32])
+    hidden = rng.standard_normal((T, H)).astype(np.float32)
+    w_gate, w_up = [(rng.standard_normal((F, H)) * 0.1).astype(np.float32) for _ in range(2)]
+    w_down = (rng.standard_normal((H, F)) * 0.1).astype(np.float32)
+    bg, bu, bd = [rng.standard_normal(n).astype(np.float32) * 0.1 for n in (F, F, H)]
+    if bias == "none":
+        bg = bu = bd = None
+    got = lib.dense_ffn_f16(hidden, w_gate, w_up, w_down, bg, bu, bd)
+    want = oracle.dense_ffn_f32(hidden, w_gate, w_up, w_down, bg, bu, bd)
+    assert_layer_close(got, want)
+    x = hidden.astype(np.float64)
+    g = x @ w_gate.astype(np.float64).T + (0 if bg is None else bg)
+    u = x @ w_up.astype(np.float64).T + (0 if bu is None else bu)
+    ref = (g / (1 + np.exp(-g)) * u) @ w_down.astype(np.float64).T + (0 if bd is None else bd)
+    assert np.abs(got - ref).max() <= 2e-5 * np.abs(ref).max()
+
+
+def test_dense_ffn_weight_types_must_agree(lib):
+    hidden = np.zeros((2, 8), np.float32)
+    h16 = [lib.f16_upload(np.zeros(s, np.float16)) for s in ((4, 8), (4, 8))]
+    h32 = lib.f16_upload_f32(np.zeros((8, 4), np.float32))
+    out = np.empty((2, 8), np.float32)
+    try:
+        rc = lib.dll.csk_dense_ffn_f16(hidden.ctypes.data, 2, 8, 4, h16[0], h16[1], h32, None, None, None,
+                                       out.ctypes.data)
+        assert rc == capi.ERR_ARG
+        assert "weight tensors must all be FLOAT16 or all FLOAT32" in lib.dll.csk_last_error().decode()
+    finally:
+        for h in h16 + [h32]:
+            lib.f16_free(h)
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 64, 96), (7, 37, 29), (64, 2880, 512), (65, 96, 160), (2, 5120, 1024)])
+def test_matmul_transpose_float32_weight_matches_oracle(lib, oracle, M, K, N):
+    """matmul_transpose_mixed_node's fp32 B (matmul_transpose_mixed_node.h:83-92)."""
+    rng = np.random.default_rng([M, K, N, 32])
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * 0.1).astype(np.float32)
+    got = lib.matmul_transpose_f16(a, w)
+    want = oracle.matmul_transpose_f32(a, w)
+    assert got.shape == (M, N)
+    assert_layer_close(got, want)
+    ref = a.astype(np.float64) @ w.astype(np.float64).T
+    assert np.abs(got - ref).max() <= 2e-5 * np.abs(ref).max()
+    with pytest.raises(capi.CskError, match="incompatible dimensions"):
+        lib.matmul_transpose_f16(a[:, :K - 1] if K > 1 else a, w)
+
+
+def test_float32_weight_upload_refuses_what_two_halves_cannot_hold(lib):
+    w = np.ones((4, 8), np.float32)
+    w[2, 3] = 1e6
+    with pytest.raises(capi.CskError, match="weight 19 is not finite or larger than 65504"):
+        lib.f16_upload_f32(w)
+    w[2, 3] = np.nan
+    with pytest.raises(capi.CskError, match="weight 19"):
+        lib.f16_upload_f32(w)

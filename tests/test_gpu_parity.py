@@ -31,25 +31,73 @@ def test_dequant_bit_exact_and_roundtrip(lib, oracle):
 
 
 def test_dequant_every_scale_and_code(lib, oracle):
+    """Every scale byte the reference decodes to finite values, 0 and 1 (fp32 denormals)
+    included, with all 16 codes in both nibble positions: bit-exact against the fixture
+    written from the reference's own codec."""
     g = np.load(__file__.replace("test_gpu_parity.py", "golden/mxfp4_codec.npz"))
-    blocks = g["blocks"][64 + 2:64 + 255]  # scale bytes 2..254, all 16 codes in both nibbles
+    blocks = g["blocks"][64:64 + 255]  # scale bytes 0..254
+    assert blocks[0, 0] == 0 and blocks[254, 0] == 254
     n = blocks.shape[0]
     h = lib.mxfp4_upload(blocks.reshape(-1), n, 32)
     try:
         got = lib.mxfp4_dequant(h, n, 32)
-        want = g["values"].reshape(-1, 32)[64 + 2:64 + 255]
+        want = g["values"].reshape(-1, 32)[64:64 + 255]
         assert nbits_differ(got, want.view(np.float32)) == 0
+        assert np.array_equal(lib.mxfp4_export(h, n, 32), blocks.reshape(-1))
     finally:
         lib.mxfp4_free(h)
 
 
-def test_upload_rejects_inexact_scales(lib):
+def test_scale_byte_255_only_on_zero_blocks(lib):
+    """2^127 times a non-zero code overflows fp32 in the reference itself: refused.  On a
+    block of zeros (codes 0 and 8) any scale byte is accepted; 255 is kept as 254."""
     blk = np.zeros(17, np.uint8)
-    for s in (0, 1, 255):
-        blk[0] = s
-        with pytest.raises(capi.CskError) as ei:
-            lib.mxfp4_upload(blk, 1, 32)
-        assert ei.value.code == capi.ERR_SCALE
+    blk[0] = 255
+    blk[1:] = [0x00, 0x08, 0x80, 0x88] * 4
+    h = lib.mxfp4_upload(blk, 1, 32)
+    try:
+        assert np.all(lib.mxfp4_dequant(h, 1, 32) == 0)
+        back = lib.mxfp4_export(h, 1, 32)
+        assert back[0] == 254 and np.array_equal(back[1:], blk[1:])
+    finally:
+        lib.mxfp4_free(h)
+    blk[5] = 0x10
+    with pytest.raises(capi.CskError, match="overflow fp32") as ei:
+        lib.mxfp4_upload(blk, 1, 32)
+    assert ei.value.code == capi.ERR_SCALE
+
+
+@pytest.mark.parametrize("T", [5, 130])
+def test_layer_with_zero_and_denormal_scale_blocks(lib, oracle, T):
+    """A checkpoint as ggml writes it: all-zero blocks carry scale byte 0; a few non-zero
+    blocks with scale bytes 0 and 1 (values below 1e-37) are thrown in.  Both regimes must
+    accept the layer and match the CPU path."""
+    L = synth.LayerInputs(4, 2, 128, 96, seed=57)
+    rng = np.random.default_rng(5)
+    W = {}
+    for e in range(L.E):
+        for which in range(3):
+            b = L.blocks(e, which).reshape(-1, 17).copy()
+            zero = rng.random(b.shape[0]) < 0.2
+            b[zero, 1:] = 0
+            b[zero, 0] = 0
+            tiny = rng.random(b.shape[0]) < 0.05
+            b[tiny, 0] = rng.integers(0, 2, int(tiny.sum()))
+            W[(e, which)] = b.reshape(-1)
+    hidden = synth.hidden_states(T, L.H, seed=T)
+    layer = lib.layer(L.E, L.k, L.H, L.F)
+    try:
+        layer.set_router(L.gate_w, L.gate_b)
+        for e in range(L.E):
+            layer.set_expert(e, W[(e, 0)], W[(e, 1)], W[(e, 2)], L.b_up[e], L.b_gate[e], L.b_down[e])
+            assert nbits_differ(layer.dequant(e, 2), oracle.dequant(W[(e, 2)], L.H * L.F).reshape(L.H, L.F)) == 0
+        got = layer.forward(hidden)
+    finally:
+        layer.close()
+    cat = lambda w: np.concatenate([W[(e, w)] for e in range(L.E)])  # noqa: E731
+    want, _ = oracle.moe_layer(hidden, L.E, L.k, L.H, L.F, L.gate_w, L.gate_b, cat(0), cat(1), cat(2),
+                               L.b_up, L.b_gate, L.b_down)
+    assert_layer_close(got, want)
 
 
 def test_device_generator_matches_host_replay(lib):
