@@ -153,11 +153,15 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
     }
 
     // tiles of a unit: (R, R) for gate/up, (2R, 2R+1) for down
-    auto load_step = [&](WSet& ws, int unit, int s) {
+    // `idle`: a refill whose data nobody will use (past the workgroup's last unit).  It is
+    // still issued, so that the count of loads in flight is the same on every path, but
+    // every step aims at the same 1 KiB of the unit, which the caches hold: the tail of a
+    // workgroup must not cost HBM traffic.
+    auto load_step = [&](WSet& ws, int unit, int s, bool idle) {
       const int ta = MODE == 0 ? unit : 2 * unit;
       const int tb = MODE == 0 ? unit : min(2 * unit + 1, a.ntile - 1);
       const size_t ea = (size_t)ta * nblk * 16, eb = (size_t)tb * nblk * 16;
-      const int kb = min(4 * (wv + 4 * s) + g, nblk - 1);
+      const int kb = idle ? g : min(4 * (wv + 4 * s) + g, nblk - 1);
       ws.q[s][0] = q0[ea + kb * 16];
       ws.q[s][1] = q1[eb + kb * 16];
     };
@@ -175,6 +179,7 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
 
     // Contracts unit `unit` out of ws and, step by step, refills ws with unit `next`.
     auto compute_unit = [&](WSet& ws, int unit, int next) {
+      const bool idle = next == unit;
       const float bias0 = ws.b0, bias1 = ws.b1;
       const u32x2 scb0 = ws.sc[0], scb1 = ws.sc[1];
       floatx4 acc[2][2];  // [tile of the pair][hi, lo term]: independent accumulation chains
@@ -210,7 +215,7 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
           acc[1][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ahi[cur].b, b1, acc[1][0], 0, 0, 0);
           acc[1][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(alo[cur].b, b1, acc[1][1], 0, 0, 0);
         }
-        load_step(ws, next, s);  // this step's registers are free: start the next unit's loads
+        load_step(ws, next, s, idle);  // this step's registers are free: start the next unit's loads
       }
       load_unit_scalars(ws.sc[0], ws.sc[1], ws.b0, ws.b1, next);
       float* rbuf = red + (size_t)par * 4 * LG * NV * 16;
@@ -258,13 +263,13 @@ __global__ __launch_bounds__(256) void expert_stream_kernel(ExpertStreamArgs a) 
 
     // One register set, refilled step by step as it is consumed: the loads of unit
     // t+1 are issued during unit t and stay one unit ahead of their use.  Refills
-    // are unconditional (past the last unit they re-read it), so that the number of
-    // loads in flight is the same on every path and the waits in front of the
-    // matrix cores stay partial.
+    // are unconditional (past the last unit they re-read one cached KiB of it), so
+    // that the number of loads in flight is the same on every path and the waits in
+    // front of the matrix cores stay partial.
     const int t_last = p_begin + ((p_end - 1 - p_begin) / W) * W;  // last unit of this workgroup
     WSet ws;
 #pragma unroll
-    for (int s = 0; s < NS; ++s) load_step(ws, p_begin, s);
+    for (int s = 0; s < NS; ++s) load_step(ws, p_begin, s, false);
     load_unit_scalars(ws.sc[0], ws.sc[1], ws.b0, ws.b1, p_begin);
     __syncthreads();  // the LDS copies have landed (the compiler waits for them before the barrier)
     for (int t = p_begin; t < p_end; t += W) compute_unit(ws, t, min(t + W, t_last));
