@@ -76,7 +76,7 @@ inline long cdiv(long a, long b) { return (a + b - 1) / b; }
 // Above this many token-expert assignments the token-group list of the
 // weight-streaming kernel is not built.
 constexpr int64_t kStreamMaxP = 2048;
-constexpr size_t kWeightSlack = 4096;  // bytes of mapped memory kept behind weight planes
+constexpr size_t kWeightSlack = 32768;  // bytes of mapped memory kept behind weight planes (the streaming kernel walks 96 blocks per tile whatever K is)
 constexpr int kStreamWgPerCu = 2;  // resident workgroups of the streaming kernel per compute unit
 
 // ---- workspace shared by every layer (single stream, one call at a time) --
@@ -378,11 +378,9 @@ int export_to_host(const csk_mxfp4& m, uint8_t* host_out) {
   return CSK_OK;
 }
 
-int launch_prep(const float* src, const float* norm_w, float eps, float* xn, uint16_t* xs,
-                int64_t rows, int64_t H, const int* gather_tok, const float* gather_w) {
+int launch_prep(const float* src, const float* norm_w, float eps, float* xn, int64_t rows, int64_t H) {
   if (rows == 0) return CSK_OK;
-  prep_kernel<<<dim3((unsigned)rows), 256, 0, g_stream>>>(src, norm_w, eps, xn, xs, (int)H,
-                                                          gather_tok, gather_w);
+  prep_kernel<<<dim3((unsigned)rows), 256, 0, g_stream>>>(src, norm_w, eps, xn, (int)H);
   return check_launch("prep_kernel");
 }
 
@@ -396,7 +394,7 @@ int launch_mx3(const float* x, uint16_t* x3, int64_t rows, int64_t H, const int*
   return check_launch("mx3_rows_kernel");
 }
 
-// Small batches stream the weights once (HBM-bound, bf16 two-term activations); larger
+// Small batches stream the weights once (HBM-bound, activations quantised in the kernel); larger
 // ones run the grouped GEMM on the block-scaled matrix instruction (three-term FP6
 // activations).  One decision per forward: it fixes the activation format of both GEMMs.
 bool stream_path(int64_t T, int64_t H, int64_t F) { return T <= 64 && H / 32 <= 96 && F / 32 <= 96; }
@@ -456,17 +454,19 @@ int launch_stream(ExpertStreamArgs a, int64_t P, Workspace& ws) {
   a.groups = ws.groups;
   a.nv = ws.nv;
   // kStreamWgPerCu workgroups per compute unit in steady state; a batch so small that
-  // every work unit can have a workgroup of its own (three fit a compute unit) gets that
+  // every work unit can have a resident workgroup of its own gets that
   const int64_t npair = NMAT == 2 ? a.ntile : (a.ntile + 1) / 2;
   const int64_t cus = std::max(g_cus, 1);
-  const int64_t nwg = (G == kStreamG && P * npair <= 3 * cus) ? P * npair : kStreamWgPerCu * cus;  // (small P implies G == kStreamG)
-  const size_t lds = (size_t)G * a.nblk * 128 + (size_t)2 * 4 * ((G + 3) / 4) * 8 * 16 * sizeof(float);
+  const int64_t nwg = (G == kStreamG && P * npair <= kStreamWgPerCu * cus) ? P * npair : kStreamWgPerCu * cus;  // (small P implies G == kStreamG)
+  // activation rows as three FP6 terms (96 B per block, 96 blocks per row: zeros past K) + the reduction buffers
+  const size_t lds = (size_t)G * 96 * (kMx3ChunksPerBlock * 16) + (size_t)2 * 4 * ((G + 3) / 4) * 8 * 16 * sizeof(float);
   launch_expert_kernel(NMAT == 2 ? 0 : 1, expert_stream_kernel<NMAT == 2 ? 0 : 1, G>, dim3((unsigned)nwg), dim3(256), lds, a);
   return check_launch("expert_stream_kernel");
 }
 
 template <int NMAT>
-int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspace& ws, bool stream) {
+int launch_experts(ExpertStreamArgs a, const uint16_t* a_mx3, uint16_t* act_mx3, int64_t E, int64_t T, int64_t P,
+                   Workspace& ws, bool stream) {
   if (stream)
     return stream_group_tokens(T) == kStreamG ? launch_stream<NMAT, kStreamG>(a, P, ws)
                                               : launch_stream<NMAT, kStreamGWide>(a, P, ws);
@@ -475,12 +475,12 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
   ga.mtiles = ws.tiles;
   ga.n_mtiles = ws.n_tiles;
   ga.list_row = a.list_row;
-  ga.A = a.A;
+  ga.A = reinterpret_cast<const uint4*>(a_mx3);
   ga.nblk = a.nblk;
   ga.ntile = a.ntile;
   ga.N = a.N;
   ga.act_type = a.act_type;
-  ga.act_out = reinterpret_cast<u32x4*>(a.act_out);
+  ga.act_out = reinterpret_cast<u32x4*>(act_mx3);
   ga.y_out = a.y_out;
   using Geom = MxGeom<kMxNG>;
   constexpr int kMode = NMAT == 2 ? 0 : 1;
@@ -502,38 +502,49 @@ int launch_experts(ExpertStreamArgs a, int64_t E, int64_t T, int64_t P, Workspac
   return check_launch("expert_gemm_mx_kernel");
 }
 
+// Activation rows of the expert MLPs.  The streaming path reads them as fp32 (`x`, row of a
+// packed position through list_row, optionally scaled by gather_w) and quantises them
+// itself; the grouped GEMM reads rows already written as three FP6 terms (`x_mx3`, indexed
+// through mx3_list_row or directly by packed position).
+struct ExpertInput {
+  const float* x;
+  const int* list_row;
+  const float* gather_w;
+  const uint16_t* x_mx3;
+  const int* mx3_list_row;
+};
+
 // Experts' MLPs over the dispatched tokens: ws.y[P,H] <- down(act(gate, up)).
-// x_split rows are indexed through list_row (token ids) or directly by packed
-// position when list_row is null.
 int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
-                int act_type, const uint16_t* x_split, const int* list_row, Workspace& ws,
-                bool timed = false) {
+                int act_type, const ExpertInput& in, Workspace& ws, bool timed = false) {
   const int64_t P = T * k;
   const bool stream = stream_path(T, H, F);
   ExpertStreamArgs a{};
   a.desc = ws.desc;
   a.act_type = act_type;
   // gate/up + activation
-  a.list_row = list_row;
-  a.A = reinterpret_cast<const uint4*>(x_split);
+  a.list_row = stream ? in.list_row : in.mx3_list_row;
+  a.gather_w = in.gather_w;
+  a.X = in.x;
   a.nblk = (int)(H / 32);
   a.N = (int)F;
   a.ntile = (int)cdiv(F, 16);
-  a.act_out = ws.act;
+  a.act_out = reinterpret_cast<float*>(ws.act);  // [P][F] fp32 (streaming) or three-term rows (GEMM), same bytes
   a.y_out = nullptr;
   if (timed) mark(CSK_STAGE_GATEUP);
-  int rc = launch_experts<2>(a, E, T, P, ws, stream);
+  int rc = launch_experts<2>(a, in.x_mx3, ws.act, E, T, P, ws, stream);
   if (rc != CSK_OK) return rc;
   if (timed) mark(CSK_STAGE_DOWN);
   // down
   a.list_row = nullptr;
-  a.A = reinterpret_cast<const uint4*>(ws.act);
+  a.gather_w = nullptr;
+  a.X = reinterpret_cast<const float*>(ws.act);
   a.nblk = (int)(F / 32);
   a.N = (int)H;
   a.ntile = (int)cdiv(H, 16);
   a.act_out = nullptr;
   a.y_out = ws.y;
-  return launch_experts<1>(a, E, T, P, ws, stream);
+  return launch_experts<1>(a, ws.act, nullptr, E, T, P, ws, stream);
 }
 
 int launch_combine(const float* y, const float* pairs, const int* pos, const float* residual,
@@ -1376,11 +1387,11 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
     // a workgroup takes one expert (latency) as long as all of them are resident at once, four beyond
     if (cdiv(T, 4) * (L->E + 4) <= 4 * std::max(g_cus, 1) + 64)  // four of these workgroups fit a compute unit
       router_prep_logits_kernel<1><<<dim3((unsigned)(L->E + 4), (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
-          hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, ws.xs, L->gate_w,
+          hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, L->gate_w,
           L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
     else
       router_prep_logits_kernel<4><<<dim3((unsigned)(cdiv(L->E, 4) + 4), (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
-          hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, ws.xs, L->gate_w,
+          hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, L->gate_w,
           L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
     if ((rc = check_launch("router_prep_logits_kernel")) != CSK_OK) return rc;
     mark(CSK_STAGE_DISPATCH);
@@ -1397,9 +1408,8 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
   } else {
     mark(CSK_STAGE_PREP);
     const bool stream = !L->f16 && stream_path(T, L->H, L->F);
-    if (norm || stream) {
-      rc = launch_prep(hidden, norm ? L->norm_w : nullptr, L->eps, norm ? ws.xn : nullptr,
-                       stream ? ws.xs : nullptr, T, L->H, nullptr, nullptr);
+    if (norm) {
+      rc = launch_prep(hidden, L->norm_w, L->eps, ws.xn, T, L->H);
       if (rc != CSK_OK) return rc;
     }
     if (!L->f16 && !stream && !L->wbf) {
@@ -1424,17 +1434,16 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
     g_stage_valid = g_timing;
     return rc;
   }
-  const uint16_t* xa = ws.xs;
-  const int* list_row = ws.list_tok;
-  if (L->wbf) {
-    rc = stream_path(T, L->H, L->F)
-             ? launch_prep(xr, nullptr, 0.f, nullptr, ws.xg, P, L->H, ws.list_tok, ws.list_w)
-             : launch_mx3(xr, ws.xg, P, L->H, ws.list_tok, ws.list_w);
-    if (rc != CSK_OK) return rc;
-    xa = ws.xg;
-    list_row = nullptr;
+  // streaming path: the kernel gathers, scales and quantises the fp32 rows itself;
+  // grouped GEMM: rows written as three FP6 terms beforehand (per token, or gathered and
+  // pre-scaled per dispatch position when the routing weight goes in front of the FFN)
+  ExpertInput in{xr, ws.list_tok, L->wbf ? ws.list_w : nullptr, ws.xs, ws.list_tok};
+  if (L->wbf && !stream_path(T, L->H, L->F)) {
+    if ((rc = launch_mx3(xr, ws.xg, P, L->H, ws.list_tok, ws.list_w)) != CSK_OK) return rc;
+    in.x_mx3 = ws.xg;
+    in.mx3_list_row = nullptr;
   }
-  rc = run_experts(L->E, T, L->k, L->H, L->F, L->act, xa, list_row, ws, true);
+  rc = run_experts(L->E, T, L->k, L->H, L->F, L->act, in, ws, true);
   if (rc != CSK_OK) return rc;
   mark(CSK_STAGE_COMBINE);
   rc = launch_combine(ws.y, ws.pairs, ws.pos, (flags & CSK_FWD_RESIDUAL) ? hidden : nullptr, out, T,
@@ -1679,27 +1688,21 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
     HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
     HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
     if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
-    const uint16_t* xa;
-    const int* list_row;
-    if (weight_before_ffn) {
-      // The expert's token count is only known on the device, and at most tn
-      // tokens can select it: gather tn rows.  Positions past the count read the
-      // zeroed tail of the lists (token 0, weight 0) and are never consumed.
-      rc = stream_path(tn, H, F)
-               ? launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xg, tn, H, ws.list_tok, ws.list_w)
-               : launch_mx3(dx.as<float>(), ws.xg, tn, H, ws.list_tok, ws.list_w);
+    ExpertInput in{dx.as<float>(), ws.list_tok, weight_before_ffn ? ws.list_w : nullptr, ws.xs, ws.list_tok};
+    if (!stream_path(tn, H, F)) {
+      if (weight_before_ffn) {
+        // The expert's token count is only known on the device, and at most tn
+        // tokens can select it: gather tn rows.  Positions past the count read the
+        // zeroed tail of the lists (token 0, weight 0) and are never consumed.
+        rc = launch_mx3(dx.as<float>(), ws.xg, tn, H, ws.list_tok, ws.list_w);
+        in.x_mx3 = ws.xg;
+        in.mx3_list_row = nullptr;
+      } else {
+        rc = launch_mx3(dx.as<float>(), ws.xs, tn, H, nullptr, nullptr);
+      }
       if (rc != CSK_OK) return rc;
-      xa = ws.xg;
-      list_row = nullptr;
-    } else {
-      rc = stream_path(tn, H, F)
-               ? launch_prep(dx.as<float>(), nullptr, 0.f, nullptr, ws.xs, tn, H, nullptr, nullptr)
-               : launch_mx3(dx.as<float>(), ws.xs, tn, H, nullptr, nullptr);
-      if (rc != CSK_OK) return rc;
-      xa = ws.xs;
-      list_row = ws.list_tok;
     }
-    rc = run_experts(1, tn, k, H, F, activation, xa, list_row, ws);
+    rc = run_experts(1, tn, k, H, F, activation, in, ws);
     if (rc != CSK_OK) return rc;
     expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)tn), 256, 0, g_stream>>>(
         ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
@@ -1948,7 +1951,7 @@ extern "C" int csk_rmsnorm(const float* x, const float* weight, float* out, int6
   if ((rc = dx.upload(x, (size_t)T * H * 4)) != CSK_OK) return rc;
   if ((rc = dw.upload(weight, (size_t)H * 4)) != CSK_OK) return rc;
   if ((rc = dout.alloc((size_t)T * H * 4)) != CSK_OK) return rc;
-  rc = launch_prep(dx.as<float>(), dw.as<float>(), eps, dout.as<float>(), nullptr, T, H, nullptr, nullptr);
+  rc = launch_prep(dx.as<float>(), dw.as<float>(), eps, dout.as<float>(), T, H);
   if (rc != CSK_OK) return rc;
   HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
   HIP_TRY(hipStreamSynchronize(g_stream));

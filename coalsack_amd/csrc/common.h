@@ -18,7 +18,7 @@ constexpr int kBlk = 32;        // MXFP4 block length along K
 constexpr int kMaxTopK = 16;
 constexpr int kMaxExperts = 256;
 constexpr int kStreamG = 4;      // tokens per pass of the weight-streaming expert kernel: batches of up to four tokens
-constexpr int kStreamGWide = 6;  // ... and larger ones (six rows of activations are what two workgroups per compute unit can hold in LDS)
+constexpr int kStreamGWide = 6;  // ... and larger ones (rows of 9 KiB as three FP6 terms: six per workgroup leave room for two workgroups per compute unit)
 
 // Resident weights of one expert.  Each matrix [rows, K] is stored as
 //   q: [rows/16][K/32][16] x 16 bytes -- byte b of an entry holds elements
@@ -97,13 +97,6 @@ __device__ __forceinline__ uint32_t float_to_bf16_bits(float x) {
   uint32_t u = __float_as_uint(x);
   u += 0x7FFFu + ((u >> 16) & 1u);
   return u >> 16;
-}
-
-// x = hi + lo + O(2^-17 |x|): two bf16 terms carry 16 mantissa bits.
-__device__ __forceinline__ void split_bf16(float x, uint16_t& hi, uint16_t& lo) {
-  const uint32_t h = float_to_bf16_bits(x);
-  hi = (uint16_t)h;
-  lo = (uint16_t)float_to_bf16_bits(x - bf16_bits_to_float(h));
 }
 
 // Sum over the 64 lanes, the same value returned in every lane: four cross-lane steps

@@ -1,4 +1,4 @@
-// Prologue (optional RMSNorm + bf16 hi/lo split of the activations), router
+// Prologue (optional RMSNorm of the activations), router
 // (gate GEMV, wavefront top-k, softmax over the selected k), dispatch
 // (histogram -> prefix scan -> ordered scatter) and the weighted combine.
 #pragma once
@@ -9,47 +9,22 @@
 namespace csk {
 
 // ---------------------------------------------------------------- prologue
-// One workgroup per row.  Optionally applies RMSNorm
-// (include/coalsack/nn/nn_ops/rmsnorm_node.h:62-83: rms = sqrt(sum x^2 / H +
-// eps), out = (x / rms) * w) and writes the result as f32 (xn, may be null)
-// and as two bf16 terms in the layout the expert kernels read:
-//   xs[row][kb][0..31] = hi, xs[row][kb][32..63] = lo   (kb = 32-element block)
-// With gather != null the rows are gathered and pre-scaled per packed dispatch
-// position (weight_before_ffn, expert_mlp_node.h:515-522):
-//   row p <- src[gather_tok[p]] * gather_w[p].
+// One workgroup per row: RMSNorm (include/coalsack/nn/nn_ops/rmsnorm_node.h:62-83:
+// rms = sqrt(sum x^2 / H + eps), out = (x / rms) * w), written as f32.
 __global__ __launch_bounds__(256) void prep_kernel(const float* __restrict__ src,
                                                    const float* __restrict__ norm_w, float eps,
-                                                   float* __restrict__ xn,
-                                                   uint16_t* __restrict__ xs, int H,
-                                                   const int* __restrict__ gather_tok,
-                                                   const float* __restrict__ gather_w) {
+                                                   float* __restrict__ xn, int H) {
   const int row = blockIdx.x;
-  const int srow = gather_tok ? gather_tok[row] : row;
-  const float* x = src + (size_t)srow * H;
-  const float gw = gather_w ? gather_w[row] : 1.0f;
-  float inv_den = 0.0f;
-  if (norm_w) {
-    float ss = 0.0f;
-    for (int d = threadIdx.x; d < H; d += 256) ss += x[d] * x[d];
-    ss = wave_sum(ss);
-    __shared__ float part[4];
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
-    __syncthreads();
-    ss = (part[0] + part[1]) + (part[2] + part[3]);
-    inv_den = sqrtf(ss / (float)H + eps);
-  }
-  for (int d = threadIdx.x; d < H; d += 256) {
-    float v = x[d];
-    if (norm_w) v = (v / inv_den) * norm_w[d];
-    if (xn) xn[(size_t)row * H + d] = v;
-    if (!xs) continue;
-    if (gather_w) v = v * gw;
-    uint16_t hi, lo;
-    split_bf16(v, hi, lo);
-    uint16_t* o = xs + ((size_t)row * (H / 32) + (d >> 5)) * 64 + (d & 31);
-    o[0] = hi;
-    o[32] = lo;
-  }
+  const float* x = src + (size_t)row * H;
+  float ss = 0.0f;
+  for (int d = threadIdx.x; d < H; d += 256) ss += x[d] * x[d];
+  ss = wave_sum(ss);
+  __shared__ float part[4];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = (part[0] + part[1]) + (part[2] + part[3]);
+  const float den = sqrtf(ss / (float)H + eps);
+  for (int d = threadIdx.x; d < H; d += 256) xn[(size_t)row * H + d] = (x[d] / den) * norm_w[d];
 }
 
 // ------------------------------------------------------------ router logits
@@ -177,7 +152,7 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(const float* __
 // One launch for small T: workgroups x in [0, ceil(E / EPW)) compute the logits of EPW experts
 // for the four tokens of tile y (the four waves split H, so all loads of a row are in flight
 // at once; the token rows stay in registers across the experts); the next four workgroups
-// run the prologue of one token of tile y each (RMSNorm, f32 copy, bf16 hi/lo split).  With
+// run the prologue of one token of tile y each (RMSNorm, written as f32).  With
 // RMSNorm the expert workgroups recompute each token's normalisation themselves -- 2 H flops
 // per token -- instead of waiting for the prologue.  EPW = 1 spreads a handful of tokens
 // over as many workgroups as there are experts (latency); EPW = 4 is for batches whose
@@ -187,7 +162,7 @@ __global__ __launch_bounds__(256) void router_logits_mfma_kernel(const float* __
 template <int EPW>
 __global__ __launch_bounds__(256) void router_prep_logits_kernel(
     const float* __restrict__ hidden, const float* __restrict__ norm_w, float eps,
-    float* __restrict__ xn, uint16_t* __restrict__ xs, const float* __restrict__ g,
+    float* __restrict__ xn, const float* __restrict__ g,
     const float* __restrict__ b, float* __restrict__ logits, int T, int E, int H) {
   __shared__ float part[4][4];
   __shared__ float dots[EPW][4][4];
@@ -195,7 +170,7 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
   const int n_ewg = (E + EPW - 1) / EPW;  // workgroups that compute logits
   if ((int)blockIdx.x >= n_ewg) {  // ---- prologue of token t (one of four per token tile)
     const int t = (blockIdx.x - n_ewg) + 4 * blockIdx.y;
-    if (blockIdx.x - n_ewg >= 4 || t >= T) return;
+    if (blockIdx.x - n_ewg >= 4 || t >= T || !norm_w) return;  // without a norm the rows are used as they are
     // four columns per thread, the row's loads all in flight at once and kept in registers
     // between the two passes (rows longer than 4096 take further rounds of the same)
     const float4* x4 = reinterpret_cast<const float4*>(hidden + (size_t)t * H);
@@ -253,15 +228,6 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
             v.z = (v.z / den) * wv4[j].z, v.w = (v.w / den) * wv4[j].w;
             reinterpret_cast<float4*>(xn + (size_t)t * H)[c] = v;
           }
-          uint16_t hi[4], lo[4];
-          split_bf16(v.x, hi[0], lo[0]);
-          split_bf16(v.y, hi[1], lo[1]);
-          split_bf16(v.z, hi[2], lo[2]);
-          split_bf16(v.w, hi[3], lo[3]);
-          const int d = 4 * c;  // four columns of one 32-column block
-          uint16_t* o = xs + ((size_t)t * (H / 32) + (d >> 5)) * 64 + (d & 31);
-          *reinterpret_cast<uint2*>(o) = make_uint2(hi[0] | ((uint32_t)hi[1] << 16), hi[2] | ((uint32_t)hi[3] << 16));
-          *reinterpret_cast<uint2*>(o + 32) = make_uint2(lo[0] | ((uint32_t)lo[1] << 16), lo[2] | ((uint32_t)lo[3] << 16));
         }
       }
     }
