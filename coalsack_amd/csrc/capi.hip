@@ -433,9 +433,10 @@ int launch_router(const float* x, const float* gate_w, const float* gate_b, int6
 
 // Tokens of an expert contracted per pass over its weights by the streaming kernel.  An
 // expert with more tokens than that is streamed once per group, so larger batches take
-// groups of six (at 32 tokens and top-4 of 32 experts a quarter fewer passes); up to 16
-// tokens few experts see more than four and the four-token kernel, which is the faster of
-// the two per byte, wins (measured at T = 8, 16, 32).
+// groups of seven (what two workgroups per compute unit can hold in LDS; measured against
+// six: 20b T = 64 162 -> 151 us, 120b T = 64 245 -> 239 us); up to 16 tokens few experts see
+// more than four, the second pass of those that do is served by the memory-side cache, and
+// the four-token form is marginally the faster one (measured at T = 8, 16, 32).
 inline int stream_group_tokens(int64_t T) { return T <= 16 ? kStreamG : kStreamGWide; }
 
 int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, int64_t E,
@@ -460,6 +461,12 @@ int launch_stream(ExpertStreamArgs a, int64_t P, Workspace& ws) {
   const int64_t nwg = (G == kStreamG && P * npair <= kStreamWgPerCu * cus) ? P * npair : kStreamWgPerCu * cus;  // (small P implies G == kStreamG)
   // activation rows as three FP6 terms (96 B per block, 96 blocks per row: zeros past K) + the reduction buffers
   const size_t lds = (size_t)G * 96 * (kMx3ChunksPerBlock * 16) + (size_t)2 * 4 * ((G + 3) / 4) * 8 * 16 * sizeof(float);
+  static bool lds_attr_set = false;  // per instantiation: dynamic LDS beyond the default limit is asked for once
+  if (!lds_attr_set) {
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&expert_stream_kernel<NMAT == 2 ? 0 : 1, G>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    lds_attr_set = true;
+  }
   launch_expert_kernel(NMAT == 2 ? 0 : 1, expert_stream_kernel<NMAT == 2 ? 0 : 1, G>, dim3((unsigned)nwg), dim3(256), lds, a);
   return check_launch("expert_stream_kernel");
 }

@@ -18,7 +18,7 @@ constexpr int kBlk = 32;        // MXFP4 block length along K
 constexpr int kMaxTopK = 16;
 constexpr int kMaxExperts = 256;
 constexpr int kStreamG = 4;      // tokens per pass of the weight-streaming expert kernel: batches of up to four tokens
-constexpr int kStreamGWide = 6;  // ... and larger ones (rows of 9 KiB as three FP6 terms: six per workgroup leave room for two workgroups per compute unit)
+constexpr int kStreamGWide = 7;  // ... and larger ones (rows of 9 KiB as three FP6 terms: seven per workgroup leave room for two workgroups per compute unit)
 
 // Resident weights of one expert.  Each matrix [rows, K] is stored as
 //   q: [rows/16][K/32][16] x 16 bytes -- byte b of an entry holds elements

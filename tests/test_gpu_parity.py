@@ -433,7 +433,7 @@ def test_layer_120b_shape_skewed_16_tokens(lib, oracle):
 
 @pytest.mark.parametrize("T", [32, 64])
 def test_layer_20b_shape_wide_token_groups(lib, oracle, T):
-    """BASELINE config 2 above 16 tokens: the six-token streaming kernels at K = 2880."""
+    """BASELINE config 2 above 16 tokens: the wide-group streaming kernels at K = 2880."""
     L = synth.LayerInputs(32, 4, 2880, 2880, seed=52)
     _check_layer(lib, oracle, L, T, device_weights=True, subset=True)
 
