@@ -138,7 +138,9 @@ __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs 
     auto load_step = [&](WSet& ws, int unit, int s, bool idle) {
       const int ta = MODE == 0 ? unit : 2 * unit;
       const int tb = MODE == 0 ? unit : min(2 * unit + 1, a.ntile - 1);
-      const uint32_t step = idle ? 0u : (uint32_t)(wv + 4 * s) * 1024u;  // four blocks of 16 rows x 16 B
+      // four blocks of 16 rows x 16 B per step; a step that lies wholly past K (its activations
+      // are zeros) re-reads the cached start of the tile instead of fetching the next tile's blocks
+      const uint32_t step = (idle || 4 * (wv + 4 * s) >= nblk) ? 0u : (uint32_t)(wv + 4 * s) * 1024u;
       ws.q[s][0] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc0, qoff, (uint32_t)ta * (uint32_t)nblk * 256u + step, 0);
       ws.q[s][1] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc1, qoff, (uint32_t)tb * (uint32_t)nblk * 256u + step, 0);
     };
