@@ -560,7 +560,7 @@ def main():
         leg = stack_leg(lib, synth, shape, T, a.steps, a.warmup, layers120, not a.no_cpu, 12.0)
         line = dict(metric="MoE stack tokens/s", value=leg["value"], unit="tokens/s", n_gpus=1,
                     steps=a.steps, warmup=a.warmup, ms_per_step=leg["ms_per_step"],
-                    higher_is_better=True, scaling="weak", vs_baseline=None, dtype="mxfp4 x bf16(2-term) -> f32",
+                    higher_is_better=True, scaling="weak", vs_baseline=None, dtype="mxfp4 x fp6(3-term, block-scaled) -> f32",
                     data="synthetic",
                     config=dict(workload=leg["workload"], tokens=T, device=dev_name,
                                 distinct_experts_per_layer=leg["distinct_experts_per_layer"]),
@@ -607,7 +607,7 @@ def main():
         warmup=a.warmup, ms_per_step=head["ms_per_step"], higher_is_better=True, scaling="weak",
         vs_baseline=None,
         dtype=("f16 x f16(2-term) -> f32" if f16 else
-               "mxfp4 x fp6(3-term, block-scaled) -> f32" if prefill else "mxfp4 x bf16(2-term) -> f32"),
+               "mxfp4 x fp6(3-term, block-scaled) -> f32"),
         data="synthetic",
         config=dict(workload=f"{a.workload}: E={shape['E']} top-{shape['k']} H={shape['H']} F={shape['F']} "
                              f"{'fp16' if f16 else 'MXFP4'}, T={T}" + (", 8 hot experts" if shape["hot"] else ""),
