@@ -397,7 +397,15 @@ int launch_mx3(const float* x, uint16_t* x3, int64_t rows, int64_t H, const int*
 // Small batches stream the weights once (HBM-bound, activations quantised in the kernel); larger
 // ones run the grouped GEMM on the block-scaled matrix instruction (three-term FP6
 // activations).  One decision per forward: it fixes the activation format of both GEMMs.
-bool stream_path(int64_t T, int64_t H, int64_t F) { return T <= 64 && H / 32 <= 96 && F / 32 <= 96; }
+// What counts is tokens per expert: a 64-token M tile of the GEMM that holds a handful of
+// tokens costs as much as a full one, while the streaming kernel passes over an expert once
+// per seven of its tokens.  Measured crossover: about twelve assignments per expert (20b
+// shape: T = 96 a tie, T = 128 the GEMM 16 % faster; 120b shape: T = 128 streaming 17 %
+// faster, T = 256 8 %, T = 512 the GEMM 33 % faster).
+bool stream_path(int64_t T, int64_t H, int64_t F, int64_t E, int64_t k) {
+  if (H / 32 > 96 || F / 32 > 96) return false;
+  return T <= 64 || (T * k <= 10 * E && T * k <= kStreamMaxP);
+}
 
 int launch_router(const float* x, const float* gate_w, const float* gate_b, int64_t T, int64_t E,
                   int64_t H, int64_t k, int sigmoid, float* logits, float* pairs, int* ids) {
@@ -525,7 +533,7 @@ struct ExpertInput {
 int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
                 int act_type, const ExpertInput& in, Workspace& ws, bool timed = false) {
   const int64_t P = T * k;
-  const bool stream = stream_path(T, H, F);
+  const bool stream = stream_path(T, H, F, E, k);
   ExpertStreamArgs a{};
   a.desc = ws.desc;
   a.act_type = act_type;
@@ -1408,13 +1416,13 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
                   ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w};
     route_small_kernel<<<dim3(1), kRouteSmallThreads, 0, g_stream>>>(rin, rout);
     if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
-    if (!L->f16 && !stream_path(T, L->H, L->F) && !L->wbf) {
+    if (!L->f16 && !stream_path(T, L->H, L->F, L->E, L->k) && !L->wbf) {
       // few tokens but rows too long for the streaming kernel: the GEMM wants the FP6 form
       if ((rc = launch_mx3(xr, ws.xs, T, L->H, nullptr, nullptr)) != CSK_OK) return rc;
     }
   } else {
     mark(CSK_STAGE_PREP);
-    const bool stream = !L->f16 && stream_path(T, L->H, L->F);
+    const bool stream = !L->f16 && stream_path(T, L->H, L->F, L->E, L->k);
     if (norm) {
       rc = launch_prep(hidden, L->norm_w, L->eps, ws.xn, T, L->H);
       if (rc != CSK_OK) return rc;
@@ -1445,7 +1453,7 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
   // grouped GEMM: rows written as three FP6 terms beforehand (per token, or gathered and
   // pre-scaled per dispatch position when the routing weight goes in front of the FFN)
   ExpertInput in{xr, ws.list_tok, L->wbf ? ws.list_w : nullptr, ws.xs, ws.list_tok};
-  if (L->wbf && !stream_path(T, L->H, L->F)) {
+  if (L->wbf && !stream_path(T, L->H, L->F, L->E, L->k)) {
     if ((rc = launch_mx3(xr, ws.xg, P, L->H, ws.list_tok, ws.list_w)) != CSK_OK) return rc;
     in.x_mx3 = ws.xg;
     in.mx3_list_row = nullptr;
@@ -1696,7 +1704,7 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
     HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
     if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
     ExpertInput in{dx.as<float>(), ws.list_tok, weight_before_ffn ? ws.list_w : nullptr, ws.xs, ws.list_tok};
-    if (!stream_path(tn, H, F)) {
+    if (!stream_path(tn, H, F, 1, k)) {
       if (weight_before_ffn) {
         // The expert's token count is only known on the device, and at most tn
         // tokens can select it: gather tn rows.  Positions past the count read the

@@ -445,6 +445,20 @@ def test_layer_120b_shape_skewed_1_and_64_tokens(lib, oracle, T):
     _check_layer(lib, oracle, L, T, device_weights=True, subset=True)
 
 
+@pytest.mark.parametrize("T", [160, 320])
+def test_layer_120b_shape_many_experts_few_tokens_each(lib, oracle, T):
+    """More than 64 tokens, but at most ten assignments per expert on average: such a batch
+    still takes the streaming kernels (groups of seven tokens; the hot experts take many)."""
+    L = synth.LayerInputs(128, 4, 2880, 2880, seed=44, hot_experts=8)
+    _check_layer(lib, oracle, L, T, device_weights=True, subset=True)
+
+
+@pytest.mark.parametrize("opts", [dict(weight_before_ffn=True, sigmoid=True), dict(act=1)])
+def test_layer_many_small_experts_beyond_64_tokens(lib, oracle, opts):
+    L = synth.LayerInputs(64, 4, 128, 96, seed=45)
+    _check_layer(lib, oracle, L, 150, **opts)
+
+
 # ----------------------------------------------------- prefill (grouped GEMM)
 
 def _prefill_case(lib, oracle, L, T, ntok_oracle):
