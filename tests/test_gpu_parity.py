@@ -418,6 +418,16 @@ def test_layer_few_tokens_long_rows(lib, oracle):
     _check_layer(lib, oracle, L, 7)
 
 
+@pytest.mark.parametrize("H,F", [(3072, 3072), (32, 3072), (3072, 32), (32, 32), (3040, 2976)])
+@pytest.mark.parametrize("T", [3, 23])
+def test_layer_streaming_row_length_limits(lib, oracle, H, F, T):
+    """The streaming kernels at the ends of the row lengths they accept: 3072 (every block
+    of the activation rows in LDS holds data, none is a zero tail), one block of 32, and
+    lengths whose last 128-wide step is partly past the row."""
+    L = synth.LayerInputs(5, 2, H, F, seed=11 + H // 32 + F // 64, with_norm=True)
+    _check_layer(lib, oracle, L, T, norm=True, residual=True)
+
+
 def test_layer_many_tokens_per_expert(lib, oracle):
     """More than 64 tokens on one expert: several passes of the M tiles."""
     L = synth.LayerInputs(4, 2, 128, 96, seed=3)
