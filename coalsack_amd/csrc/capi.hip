@@ -1210,12 +1210,85 @@ struct StagingPool {
 };
 StagingPool g_staging;
 
+// Pinned host memory between the caller's pageable buffers and the device.  A copy between
+// pageable memory and the device is staged by the runtime anyway and returns only when it is
+// done, one round trip per call; a node-level call makes five or six small ones.  Through
+// this arena they become plain host copies plus asynchronous transfers that overlap one
+// another and the kernels, and the call waits once, at its end.  Space is handed out in
+// order and taken back all at once when the stream is idle (finish_fetches, or the last
+// DevBuf of a call going out of scope); a transfer that does not fit takes the direct path.
+struct PinnedArena {
+  static constexpr size_t kBytes = (size_t)32 << 20;
+  static constexpr size_t kMaxTransfer = (size_t)4 << 20;
+  char* base = nullptr;
+  size_t used = 0;
+  bool failed = false;
+  void* take(size_t bytes) {
+    if (bytes == 0 || bytes > kMaxTransfer || failed) return nullptr;
+    if (!base) {
+      if (hipHostMalloc(reinterpret_cast<void**>(&base), kBytes, hipHostMallocDefault) != hipSuccess) {
+        (void)hipGetLastError();
+        base = nullptr, failed = true;
+        return nullptr;
+      }
+    }
+    const size_t at = (used + 255) & ~(size_t)255;
+    if (at + bytes > kBytes) return nullptr;
+    used = at + bytes;
+    return base + at;
+  }
+  void reset() { used = 0; }
+};
+PinnedArena g_pinned;
+int g_live_devbufs = 0;
+
+// Results on their way to the caller's memory: copied out of the arena once the stream is idle.
+struct PendingFetch {
+  void* host;
+  const void* pinned;
+  size_t bytes;
+};
+std::vector<PendingFetch> g_fetches;
+
+int fetch(void* host, const void* dev, size_t bytes) {
+  if (bytes == 0) return CSK_OK;
+  if (void* stage = g_pinned.take(bytes)) {
+    HIP_TRY(hipMemcpyAsync(stage, dev, bytes, hipMemcpyDeviceToHost, g_stream));
+    g_fetches.push_back(PendingFetch{host, stage, bytes});
+    return CSK_OK;
+  }
+  HIP_TRY(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, g_stream));
+  return CSK_OK;
+}
+
+// Waits for the stream, then completes the fetches.  Every transfer staged in the arena has
+// been consumed by then, so its space is free again.
+int finish_fetches() {
+  const hipError_t e = hipStreamSynchronize(g_stream);
+  if (e == hipSuccess)
+    for (const PendingFetch& f : g_fetches) std::memcpy(f.host, f.pinned, f.bytes);
+  g_fetches.clear();
+  g_pinned.reset();
+  if (e != hipSuccess) return fail(CSK_ERR_HIP, std::string("stream synchronize: ") + hipGetErrorString(e));
+  return CSK_OK;
+}
+
+#define CSK_TRY(expr)                  \
+  do {                                 \
+    const int _rc = (expr);            \
+    if (_rc != CSK_OK) return _rc;     \
+  } while (0)
+
 // Scoped device buffer for the host-pointer entry points.
 struct DevBuf {
   void* p = nullptr;
   size_t cap = 0;
+  DevBuf() { ++g_live_devbufs; }
+  DevBuf(const DevBuf&) = delete;
+  DevBuf& operator=(const DevBuf&) = delete;
   ~DevBuf() {
     if (p) g_staging.give(p, cap);
+    if (--g_live_devbufs == 0 && g_fetches.empty()) g_pinned.reset();  // the call is over, the stream idle
   }
   int alloc(size_t bytes) {
     if (p) {
@@ -1228,12 +1301,101 @@ struct DevBuf {
   int upload(const void* host, size_t bytes) {
     int rc = alloc(bytes);
     if (rc != CSK_OK) return rc;
+    if (void* stage = g_pinned.take(bytes)) {
+      std::memcpy(stage, host, bytes);
+      host = stage;
+    }
     HIP_TRY(hipMemcpyAsync(p, host, bytes, hipMemcpyHostToDevice, g_stream));
     return CSK_OK;
   }
   template <class T>
   T* as() {
     return reinterpret_cast<T*>(p);
+  }
+};
+
+// Several host arrays in one transfer: the pieces are laid out back to back (256-byte
+// aligned) in one device block and, when they fit, copied into the pinned arena and sent
+// together; otherwise each piece goes up by itself.  A reserved piece is filled by the caller
+// once the block's device address is known (a table of pointers into the same block).
+struct PackedUpload {
+  struct Piece {
+    const void* host;  // null: reserved, filled through fill()
+    size_t bytes, off;
+    std::vector<char> own;  // a reserved piece's contents when there is no stage: alive as long as the object
+  };
+  DevBuf dev;
+  std::vector<Piece> pieces;
+  size_t total = 0;
+  char* stage = nullptr;
+  size_t add(const void* host, size_t bytes) {
+    const size_t off = (total + 255) & ~(size_t)255;
+    pieces.push_back(Piece{host, bytes, off, {}});
+    total = off + bytes;
+    return off;
+  }
+  size_t reserve(size_t bytes) { return add(nullptr, bytes); }
+  int begin() {  // after the last add: the device block exists from here on
+    CSK_TRY(dev.alloc(total));
+    stage = static_cast<char*>(g_pinned.take(total));
+    return CSK_OK;
+  }
+  void fill(size_t off, const void* src, size_t bytes) {
+    if (stage) {
+      std::memcpy(stage + off, src, bytes);
+      return;
+    }
+    for (Piece& pc : pieces)
+      if (pc.off == off) pc.own.assign(static_cast<const char*>(src), static_cast<const char*>(src) + bytes);
+  }
+  template <class T>
+  T* at(size_t off) {
+    return reinterpret_cast<T*>(static_cast<char*>(dev.p) + off);
+  }
+  int commit() {
+    if (stage) {
+      for (const Piece& pc : pieces)
+        if (pc.host) std::memcpy(stage + pc.off, pc.host, pc.bytes);
+      HIP_TRY(hipMemcpyAsync(dev.p, stage, total, hipMemcpyHostToDevice, g_stream));
+      return CSK_OK;
+    }
+    for (const Piece& pc : pieces) {
+      const void* src = pc.host ? pc.host : static_cast<const void*>(pc.own.data());
+      if (pc.bytes && src)
+        HIP_TRY(hipMemcpyAsync(static_cast<char*>(dev.p) + pc.off, src, pc.bytes, hipMemcpyHostToDevice, g_stream));
+    }
+    return CSK_OK;
+  }
+};
+
+// What one pass of a node-level expert call sends up: the biases, the table of weight and bias
+// pointers (completed here with the biases' device addresses), the router output and the
+// hidden states of the pass -- one transfer.
+struct ExpertCallInputs {
+  PackedUpload up;
+  const ExpertW* ew = nullptr;
+  const float* pairs = nullptr;
+  const float* x = nullptr;
+  int send(ExpertW w, bool biases, const float* b_up, const float* b_gate, const float* b_down, int64_t F,
+           int64_t H, const float* host_pairs, int64_t P, const float* hidden, int64_t n_hidden) {
+    size_t o_bu = 0, o_bg = 0, o_bd = 0;
+    if (biases) {
+      o_bu = up.add(b_up, (size_t)F * 4);
+      o_bg = up.add(b_gate, (size_t)F * 4);
+      o_bd = up.add(b_down, (size_t)H * 4);
+    }
+    const size_t o_ew = up.reserve(sizeof(ExpertW));
+    const size_t o_pairs = up.add(host_pairs, (size_t)P * 8);
+    const size_t o_x = up.add(hidden, (size_t)n_hidden * 4);
+    CSK_TRY(up.begin());
+    w.b_up = biases ? up.at<float>(o_bu) : g_zero;
+    w.b_gate = biases ? up.at<float>(o_bg) : g_zero;
+    w.b_down = biases ? up.at<float>(o_bd) : g_zero;
+    up.fill(o_ew, &w, sizeof w);
+    ew = up.at<ExpertW>(o_ew);
+    pairs = up.at<float>(o_pairs);
+    x = up.at<float>(o_x);
+    return up.commit();
   }
 };
 
@@ -1539,7 +1701,12 @@ extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T
   }
   int rc = CSK_OK;
   {
-    const hipError_t e = hipMemcpyAsync(dh, hidden, n * sizeof(float), hipMemcpyHostToDevice, g_stream);
+    const void* src = hidden;
+    if (void* stage = g_pinned.take(n * sizeof(float))) {
+      std::memcpy(stage, hidden, n * sizeof(float));
+      src = stage;
+    }
+    const hipError_t e = hipMemcpyAsync(dh, src, n * sizeof(float), hipMemcpyHostToDevice, g_stream);
     if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("copy in: ") + hipGetErrorString(e));
   }
   if (rc == CSK_OK && !pairs_out) rc = csk_moe_forward(L, dh, T, dout, flags);
@@ -1556,13 +1723,9 @@ extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T
         rc = csk_copy_d2h(pairs_out + t0 * L->k * 2, g_ws.pairs, (size_t)tn * L->k * 2 * sizeof(float));
     }
   }
-  if (rc == CSK_OK) {
-    const hipError_t e = hipMemcpyAsync(out, dout, n * sizeof(float), hipMemcpyDeviceToHost, g_stream);
-    if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("copy out: ") + hipGetErrorString(e));
-  }
-  const hipError_t es = hipStreamSynchronize(g_stream);
-  if (rc == CSK_OK && es != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("csk_moe_forward_host: ") + hipGetErrorString(es));
-  return rc;
+  if (rc == CSK_OK) rc = fetch(out, dout, n * sizeof(float));
+  const int rs = finish_fetches();  // also when an earlier step failed: the stream is left idle
+  return rc == CSK_OK ? rs : rc;
 }
 
 extern "C" int csk_moe_stack_forward(csk_layer* const* layers, int64_t n_layers, float* hidden,
@@ -1634,10 +1797,10 @@ int router_host(const float* hidden, int64_t T, int64_t H, const float* gate_w, 
                        sigmoid, dl.as<float>(), dp.as<float>(), di.as<int>());
     if (rc != CSK_OK) return rc;
     if (out_pairs)
-      HIP_TRY(hipMemcpyAsync(out_pairs + t0 * k * 2, dp.p, (size_t)tn * k * 8, hipMemcpyDeviceToHost, g_stream));
+      CSK_TRY(fetch(out_pairs + t0 * k * 2, dp.p, (size_t)tn * k * 8));
     if (out_logits)
-      HIP_TRY(hipMemcpyAsync(out_logits + t0 * E, dl.p, (size_t)tn * E * 4, hipMemcpyDeviceToHost, g_stream));
-    HIP_TRY(hipStreamSynchronize(g_stream));
+      CSK_TRY(fetch(out_logits + t0 * E, dl.p, (size_t)tn * E * 4));
+    CSK_TRY(finish_fetches());
     return CSK_OK;
   });
 }
@@ -1645,9 +1808,14 @@ int router_host(const float* hidden, int64_t T, int64_t H, const float* gate_w, 
 
 namespace {
 __global__ void select_expert_ids_kernel(const float* __restrict__ pairs, int* __restrict__ ids,
-                                         int P, int expert_id) {
+                                         int P, int expert_id, int* __restrict__ list_tok,
+                                         float* __restrict__ list_w) {
   const int p = blockIdx.x * blockDim.x + threadIdx.x;
-  if (p < P) ids[p] = ((int)pairs[2 * (size_t)p] == expert_id) ? 0 : -1;
+  if (p >= P) return;
+  ids[p] = ((int)pairs[2 * (size_t)p] == expert_id) ? 0 : -1;
+  // positions of the lists that the dispatch leaves unwritten read as token 0, weight 0
+  list_tok[p] = 0;
+  list_w[p] = 0.0f;
 }
 }  // namespace
 
@@ -1675,45 +1843,33 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
   const int nb = (b_up != nullptr) + (b_gate != nullptr) + (b_down != nullptr);
   if (nb != 0 && nb != 3) return fail(CSK_ERR_ARG, "expert_mlp: biases must be all present or all absent");
   Workspace& ws = g_ws;
-  DevBuf dx, dpairs, dbu, dbg, dbd, dew, dout;
-  int rc;
-  if (nb == 3) {
-    if ((rc = dbu.upload(b_up, (size_t)F * 4)) != CSK_OK) return rc;
-    if ((rc = dbg.upload(b_gate, (size_t)F * 4)) != CSK_OK) return rc;
-    if ((rc = dbd.upload(b_down, (size_t)H * 4)) != CSK_OK) return rc;
-  }
   ExpertW w{};
   w.q_gate = w_gate->q, w.s_gate = w_gate->s, w.q_up = w_up->q, w.s_up = w_up->s;
   w.q_down = w_down->q, w.s_down = w_down->s;
-  w.b_gate = nb ? dbg.as<float>() : g_zero;
-  w.b_up = nb ? dbu.as<float>() : g_zero;
-  w.b_down = nb ? dbd.as<float>() : g_zero;
-  if ((rc = dew.upload(&w, sizeof w)) != CSK_OK) return rc;
   // a pass in which no token selects the expert still writes its rows (zeros, :509-512)
   return for_token_passes(T, [&](int64_t t0, int64_t tn) -> int {
     int rc = ws.ensure(tn, 1, k, H, F, weight_before_ffn != 0);
     if (rc != CSK_OK) return rc;
     const int64_t P = tn * k;
-    if ((rc = dx.upload(hidden + t0 * H, (size_t)tn * H * 4)) != CSK_OK) return rc;
-    if ((rc = dpairs.upload(pairs + t0 * k * 2, (size_t)P * 8)) != CSK_OK) return rc;
+    ExpertCallInputs up;
+    CSK_TRY(up.send(w, nb == 3, b_up, b_gate, b_down, F, H, pairs + t0 * k * 2, P, hidden + t0 * H, tn * H));
+    DevBuf dout;
     if ((rc = dout.alloc((size_t)tn * H * 4)) != CSK_OK) return rc;
     select_expert_ids_kernel<<<dim3((unsigned)cdiv(P, 256)), 256, 0, g_stream>>>(
-        dpairs.as<float>(), ws.ids, (int)P, expert_id);
+        up.pairs, ws.ids, (int)P, expert_id, ws.list_tok, ws.list_w);
     if ((rc = check_launch("select_expert_ids_kernel")) != CSK_OK) return rc;
-    HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
-    HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
-    if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
-    ExpertInput in{dx.as<float>(), ws.list_tok, weight_before_ffn ? ws.list_w : nullptr, ws.xs, ws.list_tok};
+    if ((rc = launch_dispatch(ws.ids, up.pairs, P, k, 1, up.ew, ws)) != CSK_OK) return rc;
+    ExpertInput in{up.x, ws.list_tok, weight_before_ffn ? ws.list_w : nullptr, ws.xs, ws.list_tok};
     if (!stream_path(tn, H, F, 1, k)) {
       if (weight_before_ffn) {
         // The expert's token count is only known on the device, and at most tn
         // tokens can select it: gather tn rows.  Positions past the count read the
         // zeroed tail of the lists (token 0, weight 0) and are never consumed.
-        rc = launch_mx3(dx.as<float>(), ws.xg, tn, H, ws.list_tok, ws.list_w);
+        rc = launch_mx3(up.x, ws.xg, tn, H, ws.list_tok, ws.list_w);
         in.x_mx3 = ws.xg;
         in.mx3_list_row = nullptr;
       } else {
-        rc = launch_mx3(dx.as<float>(), ws.xs, tn, H, nullptr, nullptr);
+        rc = launch_mx3(up.x, ws.xs, tn, H, nullptr, nullptr);
       }
       if (rc != CSK_OK) return rc;
     }
@@ -1722,8 +1878,8 @@ extern "C" int csk_expert_mlp_mxfp4(int expert_id, const float* hidden, int64_t 
     expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)tn), 256, 0, g_stream>>>(
         ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
     if ((rc = check_launch("expand_expert_rows_kernel")) != CSK_OK) return rc;
-    HIP_TRY(hipMemcpyAsync(out + t0 * H, dout.p, (size_t)tn * H * 4, hipMemcpyDeviceToHost, g_stream));
-    HIP_TRY(hipStreamSynchronize(g_stream));
+    CSK_TRY(fetch(out + t0 * H, dout.p, (size_t)tn * H * 4));
+    CSK_TRY(finish_fetches());
     return CSK_OK;
   });
 }
@@ -1757,43 +1913,31 @@ extern "C" int csk_expert_mlp_f16(int expert_id, const float* hidden, int64_t T,
   if (nb != 0 && nb != 3) return fail(CSK_ERR_ARG, "expert_mlp: biases must be all present or all absent");
   Workspace& ws = g_ws;
   const int64_t Hp = cdiv(H, 32) * 32, Fp = cdiv(F, 32) * 32;  // activation rows are whole blocks
-  DevBuf dx, dpairs, dbu, dbg, dbd, dew, dout;
-  int rc;
-  if (nb == 3) {
-    if ((rc = dbu.upload(b_up, (size_t)F * 4)) != CSK_OK) return rc;
-    if ((rc = dbg.upload(b_gate, (size_t)F * 4)) != CSK_OK) return rc;
-    if ((rc = dbd.upload(b_down, (size_t)H * 4)) != CSK_OK) return rc;
-  }
   ExpertW w{};
   w.q_gate = reinterpret_cast<const uint4*>(w_gate->w);
   w.q_up = reinterpret_cast<const uint4*>(w_up->w);
   w.q_down = reinterpret_cast<const uint4*>(w_down->w);
-  w.b_gate = nb ? dbg.as<float>() : g_zero;
-  w.b_up = nb ? dbu.as<float>() : g_zero;
-  w.b_down = nb ? dbd.as<float>() : g_zero;
-  if ((rc = dew.upload(&w, sizeof w)) != CSK_OK) return rc;
   return for_token_passes(T, [&](int64_t t0, int64_t tn) -> int {
     int rc = ws.ensure(tn, 1, k, Hp, Fp, weight_before_ffn != 0);
     if (rc != CSK_OK) return rc;
     const int64_t P = tn * k;
-    if ((rc = dx.upload(hidden + t0 * H, (size_t)tn * H * 4)) != CSK_OK) return rc;
-    if ((rc = dpairs.upload(pairs + t0 * k * 2, (size_t)P * 8)) != CSK_OK) return rc;
+    ExpertCallInputs up;
+    CSK_TRY(up.send(w, nb == 3, b_up, b_gate, b_down, F, H, pairs + t0 * k * 2, P, hidden + t0 * H, tn * H));
+    DevBuf dout;
     if ((rc = dout.alloc((size_t)tn * H * 4)) != CSK_OK) return rc;
     select_expert_ids_kernel<<<dim3((unsigned)cdiv(P, 256)), 256, 0, g_stream>>>(
-        dpairs.as<float>(), ws.ids, (int)P, expert_id);
+        up.pairs, ws.ids, (int)P, expert_id, ws.list_tok, ws.list_w);
     if ((rc = check_launch("select_expert_ids_kernel")) != CSK_OK) return rc;
-    HIP_TRY(hipMemsetAsync(ws.list_tok, 0, (size_t)P * sizeof(int), g_stream));
-    HIP_TRY(hipMemsetAsync(ws.list_w, 0, (size_t)P * sizeof(float), g_stream));
-    if ((rc = launch_dispatch(ws.ids, dpairs.as<float>(), P, k, 1, dew.as<ExpertW>(), ws)) != CSK_OK) return rc;
+    if ((rc = launch_dispatch(ws.ids, up.pairs, P, k, 1, up.ew, ws)) != CSK_OK) return rc;
     // with weight_before_ffn at most tn tokens can select the expert: tn rows are gathered; the
     // ones past its count read the zeroed tail of the lists and are never consumed
-    rc = run_experts_f16(1, tn, k, H, F, activation, dx.as<float>(), weight_before_ffn != 0, tn, ws);
+    rc = run_experts_f16(1, tn, k, H, F, activation, up.x, weight_before_ffn != 0, tn, ws);
     if (rc != CSK_OK) return rc;
     expand_expert_rows_kernel<<<dim3((unsigned)cdiv(H, 256), (unsigned)tn), 256, 0, g_stream>>>(
         ws.y, ws.ids, ws.pos, dout.as<float>(), (int)k, (int)H, 0);
     if ((rc = check_launch("expand_expert_rows_kernel")) != CSK_OK) return rc;
-    HIP_TRY(hipMemcpyAsync(out + t0 * H, dout.p, (size_t)tn * H * 4, hipMemcpyDeviceToHost, g_stream));
-    HIP_TRY(hipStreamSynchronize(g_stream));
+    CSK_TRY(fetch(out + t0 * H, dout.p, (size_t)tn * H * 4));
+    CSK_TRY(finish_fetches());
     return CSK_OK;
   });
 }
@@ -1852,8 +1996,8 @@ extern "C" int csk_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int6
     if ((rc = check_launch("dense_desc_kernel")) != CSK_OK) return rc;
     rc = run_experts_f16(1, tn, 1, H, F, CSK_ACT_STANDARD_SWIGLU, dx.as<float>(), false, tn, ws, false, true, dup);
     if (rc != CSK_OK) return rc;
-    HIP_TRY(hipMemcpyAsync(out + t0 * H, ws.y, (size_t)tn * H * 4, hipMemcpyDeviceToHost, g_stream));
-    HIP_TRY(hipStreamSynchronize(g_stream));
+    CSK_TRY(fetch(out + t0 * H, ws.y, (size_t)tn * H * 4));
+    CSK_TRY(finish_fetches());
     return CSK_OK;
   });
 }
@@ -1884,8 +2028,8 @@ extern "C" int csk_matmul_transpose_f16(const float* a_host, int64_t M, int64_t 
     if ((rc = launch_f16_split(da.as<float>(), mn, K2, nullptr, nullptr, ws.act, g_f16.rs_a, K)) != CSK_OK) return rc;
     rc = launch_f16_projection(1, mn, mn, K2, N, ws.act, g_f16.rs_a, ws.y, ws);
     if (rc != CSK_OK) return rc;
-    HIP_TRY(hipMemcpyAsync(out + m0 * N, ws.y, (size_t)mn * N * 4, hipMemcpyDeviceToHost, g_stream));
-    HIP_TRY(hipStreamSynchronize(g_stream));
+    CSK_TRY(fetch(out + m0 * N, ws.y, (size_t)mn * N * 4));
+    CSK_TRY(finish_fetches());
     return CSK_OK;
   });
 }
@@ -1943,8 +2087,8 @@ extern "C" int csk_expert_merge(const float* pairs, int64_t T, int64_t k, int64_
   rc = launch_combine(dy.as<float>(), dpairs.as<float>(), dpos.as<int>(), nullptr, dout.as<float>(),
                       T, k, H, pre_weighted);
   if (rc != CSK_OK) return rc;
-  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
-  HIP_TRY(hipStreamSynchronize(g_stream));
+  CSK_TRY(fetch(out, dout.p, (size_t)T * H * 4));
+  CSK_TRY(finish_fetches());
   return CSK_OK;
 }
 
@@ -1968,8 +2112,8 @@ extern "C" int csk_rmsnorm(const float* x, const float* weight, float* out, int6
   if ((rc = dout.alloc((size_t)T * H * 4)) != CSK_OK) return rc;
   rc = launch_prep(dx.as<float>(), dw.as<float>(), eps, dout.as<float>(), T, H);
   if (rc != CSK_OK) return rc;
-  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)T * H * 4, hipMemcpyDeviceToHost, g_stream));
-  HIP_TRY(hipStreamSynchronize(g_stream));
+  CSK_TRY(fetch(out, dout.p, (size_t)T * H * 4));
+  CSK_TRY(finish_fetches());
   return CSK_OK;
 }
 
@@ -1984,8 +2128,8 @@ extern "C" int csk_add(const float* a, const float* b, float* out, int64_t n) {
   if ((rc = dout.alloc((size_t)n * 4)) != CSK_OK) return rc;
   add_kernel<<<dim3((unsigned)cdiv(n, 256)), 256, 0, g_stream>>>(da.as<float>(), db.as<float>(), dout.as<float>(), n);
   if ((rc = check_launch("add_kernel")) != CSK_OK) return rc;
-  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)n * 4, hipMemcpyDeviceToHost, g_stream));
-  HIP_TRY(hipStreamSynchronize(g_stream));
+  CSK_TRY(fetch(out, dout.p, (size_t)n * 4));
+  CSK_TRY(finish_fetches());
   return CSK_OK;
 }
 
@@ -2047,8 +2191,8 @@ extern "C" int csk_add_broadcast(const void* a, const int64_t* shape_a, int nd_a
       break;
   }
   if ((rc = check_launch("add_broadcast_kernel")) != CSK_OK) return rc;
-  HIP_TRY(hipMemcpyAsync(out, dout.p, (size_t)n * esz, hipMemcpyDeviceToHost, g_stream));
-  HIP_TRY(hipStreamSynchronize(g_stream));
+  CSK_TRY(fetch(out, dout.p, (size_t)n * esz));
+  CSK_TRY(finish_fetches());
   return CSK_OK;
 }
 
@@ -2080,10 +2224,10 @@ extern "C" int csk_moe_router_f64(const double* hidden, int64_t T, int64_t H, co
     router_f64_topk_kernel<<<dim3((unsigned)cdiv(tn, 64)), 64, 0, g_stream>>>(
         dl.as<double>(), dv.as<double>(), di.as<int>(), dw.as<float>(), dp.as<float>(), (int)tn, (int)E, (int)k, sigmoid);
     if ((rc = check_launch("router_f64_topk_kernel")) != CSK_OK) return rc;
-    HIP_TRY(hipMemcpyAsync(out_pairs + t0 * k * 2, dp.p, (size_t)tn * k * 8, hipMemcpyDeviceToHost, g_stream));
+    CSK_TRY(fetch(out_pairs + t0 * k * 2, dp.p, (size_t)tn * k * 8));
     if (out_logits)
-      HIP_TRY(hipMemcpyAsync(out_logits + t0 * E, dl.p, (size_t)tn * E * 8, hipMemcpyDeviceToHost, g_stream));
-    HIP_TRY(hipStreamSynchronize(g_stream));
+      CSK_TRY(fetch(out_logits + t0 * E, dl.p, (size_t)tn * E * 8));
+    CSK_TRY(finish_fetches());
   }
   return CSK_OK;
 }

@@ -78,12 +78,14 @@ def test_reference_known_answer_two_by_two(lib):
 
 
 @pytest.mark.parametrize("T,H,F", [(5, 64, 96), (7, 37, 29), (3, 2880, 2880), (150, 96, 160),
-                                   (70, 45, 50)])
+                                   (70, 45, 50), (18000, 64, 32)])
 @pytest.mark.parametrize("bias", [False, True])
 @pytest.mark.parametrize("act,wbf", [(0, False), (1, False), (0, True)])
 def test_expert_node_matches_oracle(lib, oracle, T, H, F, bias, act, wbf):
     if H == 2880 and (bias or act or wbf):
         pytest.skip("large shape: one variant is enough")
+    if T == 18000 and (act or not bias):
+        pytest.skip("long batch (two passes, inputs past the pinned staging area): two variants are enough")
     rng = np.random.default_rng([T, H, F, act])
     hidden = rng.standard_normal((T, H)).astype(np.float32)
     w = random_f16_expert(rng, H, F, 0.1)
