@@ -1576,8 +1576,14 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
                 (int)T, (int)L->E, (int)L->k, (int)L->H, L->sigmoid, stream_group_tokens(T)};
     RouteOut rout{ws.pairs, ws.ids, ws.pos, ws.counts, ws.offsets, ws.desc, ws.groups, ws.nv,
                   ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w};
-    route_small_kernel<<<dim3(1), kRouteSmallThreads, 0, g_stream>>>(rin, rout);
-    if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
+    if (T <= kRouteTinyTokens && P <= kRouteTinyMaxP && !L->f16 && stream_path(T, L->H, L->F, L->E, L->k)) {
+      // a handful of tokens on the streaming kernels: each active expert is one token group
+      route_tiny_kernel<<<dim3(1), 256, 0, g_stream>>>(rin, rout);
+      if ((rc = check_launch("route_tiny_kernel")) != CSK_OK) return rc;
+    } else {
+      route_small_kernel<<<dim3(1), kRouteSmallThreads, 0, g_stream>>>(rin, rout);
+      if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;
+    }
     if (!L->f16 && !stream_path(T, L->H, L->F, L->E, L->k) && !L->wbf) {
       // few tokens but rows too long for the streaming kernel: the GEMM wants the FP6 form
       if ((rc = launch_mx3(xr, ws.xs, T, L->H, nullptr, nullptr)) != CSK_OK) return rc;

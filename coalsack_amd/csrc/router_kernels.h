@@ -624,6 +624,119 @@ __global__ __launch_bounds__(kRouteSmallThreads) void route_small_kernel(RouteIn
   route_workgroup<kRouteSmallThreads, kCcBatch, kRouteSmallMaxP>(in, out, lds);
 }
 
+// ------------------------- up to four tokens: top-k + dispatch, one wave per token
+// Four tokens name at most 4 k <= 64 assignments.  Wave t selects the experts of token t
+// (select_topk, close calls recomputed by the four waves together, as router_topk_kernel
+// does); then lane p of wave 0 places assignment p by counting, across the wave, the
+// assignments that come before it: those of experts with a lower index, and those of its own
+// expert from earlier tokens -- an expert's list stays ascending in token index, the order of
+// the reference's per-expert token loop (expert_mlp_node.h:503-529).  No histogram and no
+// scan, two barriers.  No expert has more than four tokens, so each active expert is one
+// token group of the weight-streaming kernels.  Writes what those kernels, the combine and
+// csk_layer_last_dispatch read: pairs, ids, positions, the lists, counts, the token groups
+// and their number; the grouped GEMM's descriptors and tiles are not written.
+constexpr int kRouteTinyTokens = 4;
+constexpr int kRouteTinyMaxP = 64;
+__global__ __launch_bounds__(256) void route_tiny_kernel(RouteIn r, RouteOut o) {
+  __shared__ CloseCallLds cc;
+  __shared__ float cc_thr[4];
+  __shared__ int cc_flag[4];
+  __shared__ int s_ids[kRouteTinyMaxP];
+  __shared__ float s_w[kRouteTinyMaxP];
+  constexpr int kEwWords = kMaxExperts * (int)(sizeof(ExpertW) / 8), kEwPerThread = (kEwWords + 255) / 256;
+  __shared__ unsigned long long s_ew[kEwWords];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int T = r.T, E = r.E, k = r.k, P = T * k;
+  const int t = wv;
+  const bool live = t < T;  // waves past the last token stay for the barriers
+  const float NEG = -__builtin_inff();
+  // the table of weight pointers is needed last (token groups); its load runs beside that of the logits
+  unsigned long long ew_reg[kEwPerThread];
+#pragma unroll
+  for (int i = 0; i < kEwPerThread; ++i) {
+    const int w = threadIdx.x + i * 256;
+    ew_reg[i] = w < E * (int)(sizeof(ExpertW) / 8) ? reinterpret_cast<const unsigned long long*>(r.ew)[w] : 0ull;
+  }
+  float v[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e = lane + 64 * j;
+    v[j] = (live && e < E) ? r.logits[(size_t)t * E + e] : NEG;
+  }
+  float my_val, vmax, runner_up;  // lane s keeps slot s
+  int my_idx;
+  bool close_call;
+  const float tol = close_call_tolerance(r.H);
+  select_topk(v, lane, E, k, my_val, my_idx, vmax, close_call, tol, runner_up);
+  close_call = close_call && live;
+  if (lane == 0) {
+    cc_flag[wv] = close_call;
+    cc_thr[wv] = runner_up - 2.0f * tol * fmaxf(1.0f, fabsf(runner_up));
+  }
+#pragma unroll
+  for (int i = 0; i < kEwPerThread; ++i) {
+    const int w = threadIdx.x + i * 256;
+    if (w < kEwWords) s_ew[w] = ew_reg[i];
+  }
+  if (__syncthreads_or(close_call)) {
+    for (int w = 0; w < 4; ++w) {
+      if (!cc_flag[w]) continue;
+      logits_reference_order_wg<256>(r.x + (size_t)w * r.H, r.g, r.b, r.logits + (size_t)w * E, E, r.H,
+                                     cc_thr[w], cc);
+      if (wv == w) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int e = lane + 64 * j;
+          v[j] = e < E ? cc.fixed[e] : NEG;
+        }
+        select_topk(v, lane, E, k, my_val, my_idx, vmax, close_call, 0.0f, runner_up);
+      }
+      __syncthreads();
+    }
+  }
+  if (live) {
+    const float w = routing_weight(my_val, vmax, lane, k, r.sigmoid);
+    if (lane < k) {
+      reinterpret_cast<float2*>(o.pairs)[(size_t)t * k + lane] = make_float2((float)my_idx, w);
+      o.ids[t * k + lane] = my_idx;
+      s_ids[t * k + lane] = my_idx;
+      s_w[t * k + lane] = w;
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) {
+    int c = 0;
+    for (int q = 0; q < P; ++q) c += s_ids[q] == e;
+    o.counts[e] = c;
+  }
+  if (wv != 0) return;
+  const bool lp = lane < P;
+  const int my = lp ? s_ids[lane] : 0x7fffffff;
+  int lower = 0, same_before = 0, same = 0;
+  for (int q = 0; q < P; ++q) {  // q is the same in every lane
+    const int idq = __builtin_amdgcn_readlane(my, q);
+    lower += idq < my;
+    same += idq == my;
+    same_before += (idq == my) && q < lane;
+  }
+  const bool first = lp && same_before == 0;  // the expert's first assignment stands for its token group
+  const unsigned long long firsts = __ballot(first);
+  int groups_before = 0;
+  for (unsigned long long m = firsts; m != 0ull; m &= m - 1ull) {
+    const int idq = __builtin_amdgcn_readlane(my, (int)__builtin_ctzll(m));
+    groups_before += idq < my;
+  }
+  if (lp) {
+    const int pos = lower + same_before;
+    const unsigned inv_k = (65536u + (unsigned)k - 1u) / (unsigned)k;  // p / k == p * inv_k >> 16 for p < 64, k <= 16
+    o.list_tok[pos] = (int)(((unsigned)lane * inv_k) >> 16);
+    o.list_w[pos] = s_w[lane];
+    o.pos_of_slot[lane] = pos;
+    if (first) write_stream_group(o.groups + groups_before, reinterpret_cast<const ExpertW*>(s_ew) + my, my, same, pos);
+  }
+  if (lane == 0) *o.nv = __popcll(firsts);
+}
+
 // ------------------------------------------------------------------ combine
 // out[t] = sum over slots in router order of w * y[pos(t, slot)]
 // (include/coalsack/nn/nn_ops/expert_merge_node.h:97-128), multiply and add
