@@ -537,6 +537,8 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   ExpertStreamArgs a{};
   a.desc = ws.desc;
   a.act_type = act_type;
+  // a single token of a routed layer names k different experts: k token groups, known here
+  a.nv_known = (stream && T == 1 && E > 1) ? (int)k : 0;
   // gate/up + activation
   a.list_row = stream ? in.list_row : in.mx3_list_row;
   a.gather_w = in.gather_w;

@@ -26,6 +26,7 @@ struct ExpertStreamArgs {
   const WorkDesc* desc;
   const StreamGroup* groups;  // [nv]: the groups of up to G tokens
   const int* nv;         // number of such groups
+  int nv_known;          // > 0: the number of groups is known at launch (one token: its k experts), *nv is not read
   const int* list_row;   // packed position -> row of X; null: row = packed position
   const float* gather_w; // packed position -> factor applied to its row (weight_before_ffn); null: 1
   const float* X;        // [rows][32 nblk] fp32 activation rows
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs 
   // Teams of W workgroups share one token group and interleave its units
   // (workgroup j takes units j, j + W, ...), so that at any moment a team reads one
   // contiguous window of the expert's planes.
-  const int nvv = *a.nv;
+  const int nvv = a.nv_known > 0 ? a.nv_known : *a.nv;  // one dependent read fewer in front of the first weights
   const int W = max(1, (int)gridDim.x / max(nvv, 1));
   const int teams = gridDim.x / W;
   const int team = blockIdx.x / W, tj = blockIdx.x % W;
