@@ -1290,7 +1290,10 @@ struct DevBuf {
   DevBuf& operator=(const DevBuf&) = delete;
   ~DevBuf() {
     if (p) g_staging.give(p, cap);
-    if (--g_live_devbufs == 0 && g_fetches.empty()) g_pinned.reset();  // the call is over, the stream idle
+    if (--g_live_devbufs == 0) {  // the call is over: the stream is idle, or the call failed and its fetches are void
+      g_fetches.clear();
+      g_pinned.reset();
+    }
   }
   int alloc(size_t bytes) {
     if (p) {
