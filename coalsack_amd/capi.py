@@ -78,6 +78,7 @@ SIGNATURES = {
     "csk_set_pass_tokens": (C.c_int, [_I64]),
     "csk_layer_last_dispatch": (C.c_int, [_P, _P, _P]),
     "csk_moe_router": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P]),
+    "csk_moe_router_resident": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P]),
     "csk_moe_router_logits": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _P]),
     "csk_expert_mlp_mxfp4": (C.c_int, [C.c_int, _P, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P,
                                        _I64, C.c_int, C.c_int, _P, C.POINTER(C.c_int)]),
@@ -323,6 +324,16 @@ class Library:
         out = np.empty((T, k, 2), np.float32)
         self.check(self.dll.csk_moe_router(_ptr(hidden), T, H, _ptr(gate_w), E, _ptr(gate_b), k,
                                            int(sigmoid), _ptr(out)))
+        return out
+
+    def moe_router_resident(self, hidden, gate_w_dev, E, gate_b_dev, k, sigmoid=False):
+        """csk_moe_router with the gate [E,H] (and bias, or None) already in device memory."""
+        hidden = _f32(hidden)
+        T, H = hidden.shape
+        out = np.empty((T, k, 2), np.float32)
+        self.check(self.dll.csk_moe_router_resident(_ptr(hidden), T, H, C.c_void_p(gate_w_dev), E,
+                                                    C.c_void_p(gate_b_dev) if gate_b_dev else None, k,
+                                                    int(sigmoid), _ptr(out)))
         return out
 
     def moe_router_f64(self, hidden, gate_w, gate_b, k, sigmoid=False, want_logits=False):

@@ -1769,7 +1769,8 @@ extern "C" int csk_layer_last_dispatch(csk_layer* L, int32_t* counts_host, int32
 
 namespace {
 int router_host(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
-                const float* gate_b, int64_t k, int sigmoid, float* out_pairs, float* out_logits);
+                const float* gate_b, int64_t k, int sigmoid, float* out_pairs, float* out_logits,
+                bool gate_on_device = false);
 }
 
 extern "C" int csk_moe_router(const float* hidden, int64_t T, int64_t H, const float* gate_w,
@@ -1778,6 +1779,14 @@ extern "C" int csk_moe_router(const float* hidden, int64_t T, int64_t H, const f
   REQUIRE_INIT();
   if (!out_pairs) return fail(CSK_ERR_ARG, "csk_moe_router: null argument");
   return router_host(hidden, T, H, gate_w, E, gate_b, k, sigmoid, out_pairs, nullptr);
+}
+
+extern "C" int csk_moe_router_resident(const float* hidden, int64_t T, int64_t H, const float* gate_w_dev,
+                                       int64_t E, const float* gate_b_dev, int64_t k, int sigmoid,
+                                       float* out_pairs) {
+  REQUIRE_INIT();
+  if (!out_pairs) return fail(CSK_ERR_ARG, "csk_moe_router: null argument");
+  return router_host(hidden, T, H, gate_w_dev, E, gate_b_dev, k, sigmoid, out_pairs, nullptr, /*gate_on_device=*/true);
 }
 
 extern "C" int csk_moe_router_logits(const float* hidden, int64_t T, int64_t H, const float* gate_w,
@@ -1789,23 +1798,27 @@ extern "C" int csk_moe_router_logits(const float* hidden, int64_t T, int64_t H, 
 
 namespace {
 int router_host(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
-                const float* gate_b, int64_t k, int sigmoid, float* out_pairs, float* out_logits) {
+                const float* gate_b, int64_t k, int sigmoid, float* out_pairs, float* out_logits,
+                bool gate_on_device) {
   if (!hidden || !gate_w || T < 0) return fail(CSK_ERR_ARG, "csk_moe_router: null argument");
   if (E <= 0 || E > kMaxExperts || k <= 0 || k > kMaxTopK || k > E || H <= 0 || H % 4)
     return fail(CSK_ERR_ARG, "csk_moe_router: need 1 <= top_k <= min(16, E), E <= 256, H a multiple of 4");
   if (T == 0) return CSK_OK;
   DevBuf dx, dg, db, dl, dp, di;
   int rc;
-  if ((rc = dg.upload(gate_w, (size_t)E * H * 4)) != CSK_OK) return rc;
-  if (gate_b && (rc = db.upload(gate_b, (size_t)E * 4)) != CSK_OK) return rc;
+  const float *gw = gate_w, *gb = gate_b;  // device addresses of the gate
+  if (!gate_on_device) {
+    if ((rc = dg.upload(gate_w, (size_t)E * H * 4)) != CSK_OK) return rc;
+    if (gate_b && (rc = db.upload(gate_b, (size_t)E * 4)) != CSK_OK) return rc;
+    gw = dg.as<float>(), gb = gate_b ? db.as<float>() : nullptr;
+  }
   return for_token_passes(T, [&](int64_t t0, int64_t tn) -> int {
     int rc;
     if ((rc = dx.upload(hidden + t0 * H, (size_t)tn * H * 4)) != CSK_OK) return rc;
     if ((rc = dl.alloc((size_t)tn * E * 4 * (1 + kRouterMaxSplits))) != CSK_OK) return rc;
     if ((rc = dp.alloc((size_t)tn * k * 8)) != CSK_OK) return rc;
     if ((rc = di.alloc((size_t)tn * k * 4)) != CSK_OK) return rc;
-    rc = launch_router(dx.as<float>(), dg.as<float>(), gate_b ? db.as<float>() : nullptr, tn, E, H, k,
-                       sigmoid, dl.as<float>(), dp.as<float>(), di.as<int>());
+    rc = launch_router(dx.as<float>(), gw, gb, tn, E, H, k, sigmoid, dl.as<float>(), dp.as<float>(), di.as<int>());
     if (rc != CSK_OK) return rc;
     if (out_pairs)
       CSK_TRY(fetch(out_pairs + t0 * k * 2, dp.p, (size_t)tn * k * 8));

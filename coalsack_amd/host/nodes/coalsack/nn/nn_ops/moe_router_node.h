@@ -1,8 +1,9 @@
 // moe_router_node backed by the gfx950 library: same class name, setters, test
 // wrappers, input order, output format and error texts as
 // include/coalsack/nn/nn_ops/moe_router_node.h of the reference (cited by line
-// below); the body calls csk_moe_router (float32) or csk_moe_router_f64 (float64) instead
-// of the scalar CPU loops.
+// below); the body calls csk_moe_router_resident (float32; the gate and its bias, the same
+// tensors every frame, are kept in device memory) or csk_moe_router_f64 (float64) instead of
+// the scalar CPU loops.
 //
 // Place this directory in front of the reference's include path to swap the
 // node in; it needs only coalsack/nn/nn_op_node.h and the C ABI header.
@@ -14,6 +15,7 @@
 
 #include "coalsack/nn/nn_op_node.h"
 #include "coalsack_moe.h"
+#include "resident_weight.h"
 
 namespace coalsack {
 
@@ -78,22 +80,33 @@ class moe_router_node : public variadic_op_node {
       throw std::runtime_error("moe_router: gate_weights must have the element type of hidden_states");
 
     dynamic_tensor output(dtype::float32, {batch, seq_len, top_k_, 2});
-    const float* bias = has_bias ? inputs[2].data_ptr<float>() : nullptr;
-    const int rc = dt == dtype::float32
-                       ? csk_moe_router(hidden.data_ptr<float>(), batch * seq_len, hidden_dim, gate.data_ptr<float>(),
-                                        num_experts_, bias, top_k_, use_sigmoid_gating_ ? 1 : 0,
-                                        output.data_ptr<float>())
-                       : csk_moe_router_f64(hidden.data_ptr<double>(), batch * seq_len, hidden_dim,
-                                            gate.data_ptr<double>(), num_experts_, bias, top_k_,
-                                            use_sigmoid_gating_ ? 1 : 0, output.data_ptr<float>(), nullptr);
+    int rc;
+    if (dt == dtype::float32) {
+      const float* gate_dev = static_cast<const float*>(gate_slot_.get(gate, "moe_router", &resident_uploads_));
+      const float* bias_dev =
+          has_bias ? static_cast<const float*>(bias_slot_.get(inputs[2], "moe_router", &resident_uploads_)) : nullptr;
+      rc = csk_moe_router_resident(hidden.data_ptr<float>(), batch * seq_len, hidden_dim, gate_dev, num_experts_,
+                                   bias_dev, top_k_, use_sigmoid_gating_ ? 1 : 0, output.data_ptr<float>());
+    } else {
+      const float* bias = has_bias ? inputs[2].data_ptr<float>() : nullptr;
+      rc = csk_moe_router_f64(hidden.data_ptr<double>(), batch * seq_len, hidden_dim, gate.data_ptr<double>(),
+                              num_experts_, bias, top_k_, use_sigmoid_gating_ ? 1 : 0, output.data_ptr<float>(),
+                              nullptr);
+    }
     if (rc != CSK_OK) throw std::runtime_error(std::string("moe_router: ") + csk_last_error());
     return output;
   }
+
+ public:
+  // device copies of the gate / bias made so far (a test hook: the same tensors must not go up twice)
+  size_t resident_uploads() const { return resident_uploads_; }
 
  private:
   int64_t num_experts_ = 0;
   int64_t top_k_ = 0;
   bool use_sigmoid_gating_ = false;
+  csk_resident::array_slot gate_slot_, bias_slot_;
+  size_t resident_uploads_ = 0;
 };
 
 }  // namespace coalsack

@@ -87,5 +87,45 @@ class weight_slot {
   uint64_t stamp_ = 0;
 };
 
+// A whole tensor kept as it is in device memory (the router's gate and bias): the same
+// rule -- the slot holds the tensor it copied and a stamp of its contents; another address,
+// shape, element type or stamp replaces the copy.
+class array_slot {
+ public:
+  array_slot() = default;
+  array_slot(const array_slot&) = delete;
+  array_slot& operator=(const array_slot&) = delete;
+  ~array_slot() {
+    if (dev_) csk_dev_free(dev_);
+  }
+
+  // device address of t's bytes; `who` prefixes the error text
+  const void* get(const dynamic_tensor& t, const char* who, size_t* uploads = nullptr) {
+    const uint8_t* base = t.data_ptr<uint8_t>();
+    const size_t bytes = t.bytes();
+    const uint64_t stamp = content_stamp(base, bytes);
+    if (dev_ && held_.data_ptr<uint8_t>() == base && held_.get_dtype() == t.get_dtype() &&
+        held_.shape() == t.shape() && stamp_ == stamp)
+      return dev_;
+    void* d = csk_dev_alloc(bytes ? bytes : 1);
+    if (!d) throw std::runtime_error(std::string(who) + ": " + csk_last_error());
+    if (csk_copy_h2d(d, base, bytes) != CSK_OK) {
+      csk_dev_free(d);
+      throw std::runtime_error(std::string(who) + ": " + csk_last_error());
+    }
+    if (dev_) csk_dev_free(dev_);
+    dev_ = d;
+    held_ = t;
+    stamp_ = stamp;
+    if (uploads) ++*uploads;
+    return d;
+  }
+
+ private:
+  void* dev_ = nullptr;
+  dynamic_tensor held_;
+  uint64_t stamp_ = 0;
+};
+
 }  // namespace csk_resident
 }  // namespace coalsack

@@ -271,6 +271,14 @@ int csk_layer_last_dispatch(csk_layer* L, int32_t* counts_host, int32_t* tokens_
  * weight). */
 int csk_moe_router(const float* hidden, int64_t T, int64_t H, const float* gate_w, int64_t E,
                    const float* gate_b, int64_t k, int sigmoid_gating, float* out_pairs);
+/* The same router for a caller that keeps the gate in device memory between frames
+ * (moe_router_node is handed the same gate tensors every frame): gate_w_dev [E,H] and
+ * gate_b_dev [E] or NULL are device pointers (csk_dev_alloc + csk_copy_h2d); hidden and
+ * out_pairs stay host pointers.  Replaces the same lines of the reference as
+ * csk_moe_router. */
+int csk_moe_router_resident(const float* hidden, int64_t T, int64_t H, const float* gate_w_dev,
+                            int64_t E, const float* gate_b_dev_or_null, int64_t k,
+                            int sigmoid_gating, float* out_pairs);
 /* The logits of that router as this library first computes them (fp32, tree-ordered
  * sums; [T,E]), before any recomputation in the reference's summation order -- a
  * diagnostic: the tests bound their distance from the reference's sequential sums,

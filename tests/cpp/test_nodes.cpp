@@ -826,6 +826,41 @@ static void gpu_expert_weight_reload() {
   }
 }
 
+// The router node is handed the same gate tensors every frame and keeps them in device
+// memory: same storage and bytes -> no upload; rewritten in place or reloaded elsewhere ->
+// a new copy, and the result is that of the new gate.
+static void gpu_router_gate_reload() {
+  std::printf("router node: device copy of the gate follows rewritten / reloaded host tensors\n");
+  std::mt19937 gen(7);
+  const int64_t S = 6, H = 64, E = 16, K = 2;
+  moe_router_node node;
+  node.set_config(E, K);
+  auto h = random_tensor({1, S, H}, gen, -1, 1);
+  auto check = [&](const dynamic_tensor& g, const dynamic_tensor& b) {
+    auto out = node.compute_test(h, g, b);
+    std::vector<float> want(S * K * 2);
+    orc_router(h.data_ptr<float>(), S, H, g.data_ptr<float>(), E, b.data_ptr<float>(), K, 0, want.data());
+    for (int64_t i = 0; i < S * K; ++i) {
+      CHECK(out.data_ptr<float>()[2 * i] == want[2 * i]);
+      CHECK(std::fabs(out.data_ptr<float>()[2 * i + 1] - want[2 * i + 1]) <= 1e-5f);
+    }
+  };
+  auto g = random_tensor({E, H}, gen, -0.5f, 0.5f), b = random_tensor({E}, gen, -0.1f, 0.1f);
+  check(g, b);
+  CHECK(node.resident_uploads() == 2);
+  check(g, b);  // same storage, same bytes
+  CHECK(node.resident_uploads() == 2);
+  for (int64_t i = 0; i < E * H; ++i) g.data_ptr<float>()[i] = -g.data_ptr<float>()[i];  // rewritten in place
+  check(g, b);
+  CHECK(node.resident_uploads() == 3);
+  b.data_ptr<float>()[E - 1] += 5.0f;  // the last expert now wins every token
+  check(g, b);
+  CHECK(node.resident_uploads() == 4);
+  auto g2 = random_tensor({E, H}, gen, -0.5f, 0.5f);  // a reload: other storage
+  check(g2, b);
+  CHECK(node.resident_uploads() == 5);
+}
+
 // Nodes of different layers may be driven from different threads (the reference runs each
 // layer's nodes on that layer's scheduler thread, layer_scheduler_node); the library
 // serialises the calls, so results must equal those of the same calls made one after another.
@@ -891,6 +926,7 @@ int main(int argc, char** argv) {
     gpu_variant_branches();
     gpu_node_chain();
     gpu_expert_weight_reload();
+    gpu_router_gate_reload();
     gpu_norm_add_tests();
     gpu_concurrent_callers();
   } else {

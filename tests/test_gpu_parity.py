@@ -143,6 +143,25 @@ def test_router_matches_oracle(lib, oracle, T, H, E, k, bias, sigmoid):
     assert np.all(got[..., 1] > 0) and np.allclose(got[..., 1].sum(axis=1), 1.0, atol=1e-5) or sigmoid
 
 
+@pytest.mark.parametrize("T,bias", [(1, True), (16, False), (300, True)])
+def test_router_with_resident_gate_equals_host_gate(lib, T, bias):
+    """csk_moe_router_resident (gate kept in device memory by the caller) is csk_moe_router."""
+    rng = np.random.default_rng(T)
+    E, H, k = 32, 2880, 4
+    h = rng.normal(0, 1, (T, H)).astype(np.float32)
+    g = rng.normal(0, 0.02, (E, H)).astype(np.float32)
+    b = rng.normal(0, 0.01, E).astype(np.float32) if bias else None
+    dg = lib.to_device(g)
+    db = lib.to_device(b) if bias else None
+    try:
+        got = lib.moe_router_resident(h, dg, E, db, k)
+    finally:
+        lib.dev_free(dg)
+        if db:
+            lib.dev_free(db)
+    assert np.array_equal(got, lib.moe_router(h, g, b, k))
+
+
 @pytest.mark.parametrize("T,E,H,sg", [(2048, 32, 2880, 0.02), (1024, 128, 2880, 0.02), (16, 32, 2880, 0.02),
                                       (2048, 32, 512, 0.05), (300, 200, 256, 0.05)])
 def test_router_logits_distance_from_sequential_sums(lib, oracle, T, E, H, sg):
