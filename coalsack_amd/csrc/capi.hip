@@ -1554,6 +1554,11 @@ namespace {
 // kernels.
 int64_t g_pass_tokens = 32768;
 
+// Largest batch routed by the single-workgroup kernel.  Its sixteen waves take the tokens four
+// at a time one after the other; beyond 32 tokens, selection spread over T / 4 workgroups
+// followed by the dispatch kernel is faster although it is a launch more (120b shape, routing
+// stage: 17.6 -> 15.7 us at T = 48, 20.8 -> 15.9 at T = 64; no gain at 32, a loss at 24).
+constexpr int64_t kRouteSmallTokens = 32;
 int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int flags, Workspace& ws = g_ws) {
   int rc = CSK_OK;
   rc = ws.ensure(T, L->E, L->k, L->H, L->F, L->wbf);
@@ -1585,6 +1590,14 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
       // a handful of tokens on the streaming kernels: each active expert is one token group
       route_tiny_kernel<<<dim3(1), 256, 0, g_stream>>>(rin, rout);
       if ((rc = check_launch("route_tiny_kernel")) != CSK_OK) return rc;
+    } else if (T > kRouteSmallTokens) {
+      // more tokens than the single workgroup has waves: selection spread over T / 4
+      // workgroups, then the dispatch kernel -- a launch more, each much shorter
+      router_topk_kernel<<<dim3((unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
+          ws.logits, ws.pairs, ws.ids, (int)T, (int)L->E, (int)L->k, L->sigmoid, xr, L->gate_w,
+          L->has_gate_b ? L->gate_b : nullptr, (int)L->H, ws.logits + T * L->E, 0);
+      if ((rc = check_launch("router_topk_kernel")) != CSK_OK) return rc;
+      if ((rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, L->ew_dev, ws)) != CSK_OK) return rc;
     } else {
       route_small_kernel<<<dim3(1), kRouteSmallThreads, 0, g_stream>>>(rin, rout);
       if ((rc = check_launch("route_small_kernel")) != CSK_OK) return rc;

@@ -718,10 +718,11 @@ def test_layer_many_experts_small_batch(lib, oracle, E, T, norm):
     _check_layer(lib, oracle, L, T, norm=norm, residual=norm)
 
 
-@pytest.mark.parametrize("T", [3, 4, 5, 64, 65, 200])
+@pytest.mark.parametrize("T", [3, 4, 5, 32, 33, 64, 65, 200])
 def test_layer_maximum_experts_and_top_k(lib, oracle, T):
     """The limits of a layer: 256 experts, top-16 -- four tokens fill the one-wave-per-token
-    router (64 assignments), 64 the single-workgroup one (1024 assignments), 65 take the
-    multi-workgroup one, 200 the grouped GEMM."""
+    router (64 assignments), 32 are the most the single-workgroup one takes (512 assignments),
+    33 to 64 go through the multi-workgroup selection and the dispatch kernel behind the fused
+    norm + logits kernel, 65 through the separate kernels, 200 take the grouped GEMM."""
     L = synth.LayerInputs(256, 16, 64, 96, seed=71)
     _check_layer(lib, oracle, L, T)
