@@ -503,6 +503,13 @@ def _prefill_case(lib, oracle, L, T, ntok_oracle):
         # tokens permutes the outputs bit for bit
         perm = np.random.default_rng(1).permutation(T)
         got_p = layer.forward(hidden[perm])
+        # ... nor on the kernels its batch takes: every token of the batch, sixteen at a time
+        # through the weight-streaming kernels (themselves checked against the CPU path on
+        # their own), selects the same experts and gives the same result to a fifth of the bar
+        for t0 in range(0, T, 16):
+            small, spairs = layer.forward(hidden[t0:t0 + 16], want_pairs=True)
+            assert np.array_equal(spairs[..., 0], pairs[t0:t0 + 16, :, 0]), t0
+            assert_layer_close(got[t0:t0 + 16], small, tol=2e-4)
     assert nbits_differ(got, again) == 0
     assert nbits_differ(got_p, got[perm]) == 0
     ids = pairs[..., 0].astype(int)
