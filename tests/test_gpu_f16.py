@@ -195,6 +195,36 @@ def test_f16_layer_20b_shape_device_weights(lib, oracle):
         assert_layer_close(got, want)
 
 
+def test_f16_layer_20b_shape_many_tokens(lib, oracle):
+    """The same layer at 1024 tokens (grouped GEMM, about 128 tokens per expert): the first
+    tokens against the CPU path, and every token against the same layer run sixteen tokens at
+    a time through the decode kernels -- same experts, same result to a fifth of the bar."""
+    L = synth.LayerInputs(32, 4, 2880, 2880, seed=31)
+    T = 1024
+    hidden = synth.hidden_states(T, L.H, seed=5)
+    with lib.layer(L.E, L.k, L.H, L.F, f16=True) as layer:
+        layer.set_router(L.gate_w, L.gate_b)
+        layer.fill_synthetic(31, 0)
+        for e in range(L.E):
+            layer.set_expert_f16(e, None, None, None, L.b_up[e], L.b_gate[e], L.b_down[e])
+        got, pairs = layer.forward(hidden, want_pairs=True)
+        for t0 in range(0, T, 16):
+            small, spairs = layer.forward(hidden[t0:t0 + 16], want_pairs=True)
+            assert np.array_equal(spairs[..., 0], pairs[t0:t0 + 16, :, 0]), t0
+            assert_layer_close(got[t0:t0 + 16], small, tol=2e-4)
+        nt = 2
+        want_pairs = oracle.router(hidden[:nt], L.gate_w, L.gate_b, L.k)
+        assert np.array_equal(pairs[:nt, :, 0], want_pairs[..., 0])
+        want = np.zeros_like(got[:nt])
+        for t in range(nt):
+            for j in range(L.k):
+                e = int(want_pairs[t, j, 0])
+                w = [layer.export_f16(e, which) for which in (capi.W_UP, capi.W_GATE, capi.W_DOWN)]
+                y = oracle.expert_token_f16(hidden[t], *w, L.b_up[e], L.b_gate[e], L.b_down[e])
+                want[t] += want_pairs[t, j, 1] * y
+        assert_layer_close(got[:nt], want)
+
+
 def test_layer_kinds_do_not_mix(lib):
     with lib.layer(2, 1, 32, 32, f16=True) as layer:
         with pytest.raises(capi.CskError, match="fp16 experts"):
