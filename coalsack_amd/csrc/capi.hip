@@ -497,7 +497,7 @@ int launch_experts(ExpertStreamArgs a, const uint16_t* a_mx3, uint16_t* act_mx3,
   ga.act_type = a.act_type;
   ga.act_out = reinterpret_cast<u32x4*>(act_mx3);
   ga.y_out = a.y_out;
-  using Geom = MxGeom<kMxNG>;
+  using Geom = MxGeom<kMxNG, 2>;
   constexpr int kMode = NMAT == 2 ? 0 : 1;
   if (a.ntile % 2) return fail(CSK_ERR_ARG, "grouped GEMM: the number of output features must be a multiple of 32");
   ga.n_ntiles = (int)cdiv(a.ntile, Geom::tiles_per_wg(kMode));

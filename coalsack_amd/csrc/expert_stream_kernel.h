@@ -38,15 +38,22 @@ struct ExpertStreamArgs {
   float* y_out;          // down: [P][N] fp32
 };
 
+// exp and the reciprocal are the hardware's own approximations (v_exp_f32 on x log2 e,
+// v_rcp_f32: one ulp each, a relative error near 1e-6 after the argument's rounding at
+// |x| <= 12), not libm's expf and an IEEE division: the epilogue of the grouped GEMM
+// evaluates 64 of these per lane and was spending more vector instructions on them than
+// on anything else.  Both regimes use this one function, so they agree with each other.
+__device__ __forceinline__ float fast_sigmoid_mul(float x, float slope) {  // x * sigmoid(slope x)
+  const float e = __builtin_amdgcn_exp2f(x * (-slope * 1.4426950408889634f));
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
 __device__ __forceinline__ float moe_activation(float gate_v, float up_v, int act_type) {
   if (act_type == 0) {  // expert_mlp_node.h:699-703
     const float x = fminf(gate_v, 7.0f);
     const float y = fminf(fmaxf(up_v, -7.0f), 7.0f);
-    const float glu = x / (1.0f + expf(1.702f * (-x)));
-    return glu * (y + 1.0f);
+    return fast_sigmoid_mul(x, 1.702f) * (y + 1.0f);
   }
-  const float silu = gate_v / (1.0f + expf(-gate_v));  // :705-706
-  return silu * up_v;
+  return fast_sigmoid_mul(gate_v, 1.0f) * up_v;  // :705-706
 }
 
 // ---------------------------------------------------------------------------
