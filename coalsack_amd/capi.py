@@ -24,6 +24,8 @@ SIGNATURES = {
     "csk_init": (C.c_int, [C.c_int]),
     "csk_last_error": (C.c_char_p, []),
     "csk_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_size_t)]),
+    "csk_device_memory": (C.c_int, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "csk_alloc_count": (C.c_int, [C.POINTER(C.c_uint64)]),
     "csk_dev_alloc": (_P, [C.c_size_t]),
     "csk_dev_free": (None, [_P]),
     "csk_copy_h2d": (C.c_int, [_P, _P, C.c_size_t]),
@@ -89,6 +91,7 @@ SIGNATURES = {
     "csk_expert_token_mxfp4": (C.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, C.c_int]),
     "csk_expert_merge": (C.c_int, [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]),
     "csk_rmsnorm": (C.c_int, [_P, _P, _P, _I64, _I64, C.c_float]),
+    "csk_rmsnorm_f64": (C.c_int, [_P, _P, _P, _I64, _I64, C.c_float]),
     "csk_add": (C.c_int, [_P, _P, _P, _I64]),
     "csk_add_broadcast": (C.c_int, [_P, _P, C.c_int, _P, _P, C.c_int, C.c_int, _P]),
     "csk_moe_router_f64": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P, _P]),
@@ -153,6 +156,18 @@ class Library:
         mem = C.c_size_t()
         self.check(self.dll.csk_device_info(name, 256, C.byref(cus), C.byref(mem)))
         return name.value.decode(), cus.value, mem.value
+
+    def device_memory(self):
+        """(free, total) bytes of device memory as the runtime reports them now."""
+        free, total = C.c_size_t(), C.c_size_t()
+        self.check(self.dll.csk_device_memory(C.byref(free), C.byref(total)))
+        return free.value, total.value
+
+    def alloc_count(self):
+        """Device allocations the library has made in this process so far."""
+        n = C.c_uint64()
+        self.check(self.dll.csk_alloc_count(C.byref(n)))
+        return n.value
 
     # -- device memory
     def dev_alloc(self, nbytes):
@@ -415,6 +430,14 @@ class Library:
         T, H = x.shape
         out = np.empty((T, H), np.float32)
         self.check(self.dll.csk_rmsnorm(_ptr(x), _ptr(w), _ptr(out), T, H, eps))
+        return out
+
+    def rmsnorm_f64(self, x, w, eps):
+        x = np.ascontiguousarray(x, np.float64)
+        w = np.ascontiguousarray(w, np.float64)
+        T, H = x.shape
+        out = np.empty((T, H), np.float64)
+        self.check(self.dll.csk_rmsnorm_f64(_ptr(x), _ptr(w), _ptr(out), T, H, eps))
         return out
 
     def add(self, a, b):

@@ -5,6 +5,7 @@
 #include <hip/hip_ext.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -63,11 +64,19 @@ int check_launch(const char* what) {
   return CSK_OK;
 }
 
+// Every device allocation of the library goes through here and is counted, so that a test
+// can hold the allocation-free entry point to its name (csk_alloc_count).
+std::atomic<uint64_t> g_alloc_count{0};
+inline hipError_t counted_malloc(void** p, size_t bytes) {
+  g_alloc_count.fetch_add(1, std::memory_order_relaxed);
+  return hipMalloc(p, bytes);
+}
+
 template <class T>
 int dev_alloc(T** p, size_t count) {
   *p = nullptr;
   if (count == 0) return CSK_OK;
-  HIP_TRY(hipMalloc(reinterpret_cast<void**>(p), count * sizeof(T)));
+  HIP_TRY(counted_malloc(reinterpret_cast<void**>(p), count * sizeof(T)));
   return CSK_OK;
 }
 
@@ -101,13 +110,16 @@ struct Workspace {
   int* tiles = nullptr;     // prefill tile schedule
   int* n_tiles = nullptr;
   bool fixed = false;       // carved out of the load-time device array: never grown, never freed
+  uint64_t runs = 0;        // forwards that have used this workspace
 
   void release() {
     void* ps[] = {xn, xs, xg, logits, pairs, ids, counts, offsets, desc, groups, nv,
                   list_tok, list_w, pos, act, y, tiles, n_tiles};
     for (void* p : ps)
       if (p) (void)hipFree(p);
+    const uint64_t r = runs;
     *this = Workspace();
+    runs = r + 1;  // (what a layer remembered of the old buffers no longer matches)
   }
   int ensure(int64_t T_, int64_t E_, int64_t k_, int64_t H_, int64_t F_, bool need_xg) {
     if (T_ <= T && E_ <= E && k_ <= k && H_ <= H && F_ <= F && (!need_xg || xg)) return CSK_OK;
@@ -152,7 +164,6 @@ struct Workspace {
   }
 };
 Workspace g_ws;
-Workspace* g_last_ws = &g_ws;  // the workspace the last forward ran in (csk_layer_last_dispatch reads it)
 
 // ---- fixed workspace of the allocation-free forward ------------------------
 // Callers that cannot allocate (code under graph capture, serving loops, harnesses that
@@ -286,6 +297,8 @@ struct csk_layer {
   float eps = 1e-5f;
   bool has_norm = false;
   int64_t last_T = 0;
+  const void* last_ws = nullptr;  // workspace of this layer's last forward, and that workspace's forward count then
+  uint64_t last_run = 0;
   // geometry of one expert's planes
   int64_t nblkH = 0, nblkF = 0, ntF = 0, ntH = 0;
   long ent_gu() const { return (long)(ntF * nblkH * 16); }  // gate or up: [F,H]
@@ -326,10 +339,10 @@ int pack_into(const uint8_t* host, csk_mxfp4& m) {
     HIP_TRY(hipStreamSynchronize(g_stream));
     if (g_stage) (void)hipFree(g_stage);
     g_stage = nullptr, g_stage_cap = 0;
-    HIP_TRY(hipMalloc((void**)&g_stage, bytes));
+    HIP_TRY(counted_malloc((void**)&g_stage, bytes));
     g_stage_cap = bytes;
   }
-  if (!g_bad) HIP_TRY(hipMalloc((void**)&g_bad, sizeof(unsigned long long)));
+  if (!g_bad) HIP_TRY(counted_malloc((void**)&g_bad, sizeof(unsigned long long)));
   HIP_TRY(hipMemsetAsync(g_bad, 0xFF, sizeof(unsigned long long), g_stream));
   HIP_TRY(hipMemcpyAsync(g_stage, host, bytes, hipMemcpyHostToDevice, g_stream));
   const long ent = m.entries();
@@ -349,7 +362,7 @@ int pack_into(const uint8_t* host, csk_mxfp4& m) {
 int dequant_to_host(const csk_mxfp4& m, float* host_out) {
   float* d = nullptr;
   const size_t n = (size_t)m.rows * m.K;
-  HIP_TRY(hipMalloc((void**)&d, n * sizeof(float)));
+  HIP_TRY(counted_malloc((void**)&d, n * sizeof(float)));
   const long ent = m.entries();
   dequant_mxfp4_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(
       m.q, m.s, d, (int)m.rows, (int)m.nblk, ent);
@@ -365,7 +378,7 @@ int dequant_to_host(const csk_mxfp4& m, float* host_out) {
 int export_to_host(const csk_mxfp4& m, uint8_t* host_out) {
   uint8_t* d = nullptr;
   const size_t n = (size_t)m.rows * m.nblk * 17;
-  HIP_TRY(hipMalloc((void**)&d, n));
+  HIP_TRY(counted_malloc((void**)&d, n));
   const long ent = m.entries();
   export_mxfp4_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(
       m.q, m.s, d, (int)m.rows, (int)m.nblk, ent);
@@ -711,7 +724,7 @@ extern "C" int csk_init(int device) {
     return fail(CSK_ERR_HIP, std::string("device is ") + prop.gcnArchName + ", this library is built for gfx950 only");
   if (!g_stream) HIP_TRY(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
   if (!g_zero) {
-    HIP_TRY(hipMalloc((void**)&g_zero, kZeroLen * sizeof(float)));
+    HIP_TRY(counted_malloc((void**)&g_zero, kZeroLen * sizeof(float)));
     HIP_TRY(hipMemset(g_zero, 0, kZeroLen * sizeof(float)));
   }
   if (device >= kMaxDevices) return fail(CSK_ERR_HIP, "device index beyond the library's table");
@@ -743,6 +756,21 @@ extern "C" int csk_device_info(char* name, size_t cap, int* compute_units, size_
   }
   if (compute_units) *compute_units = prop.multiProcessorCount;
   if (hbm_bytes) *hbm_bytes = prop.totalGlobalMem;
+  return CSK_OK;
+}
+
+extern "C" int csk_device_memory(size_t* free_bytes, size_t* total_bytes) {
+  REQUIRE_INIT();
+  size_t f = 0, t = 0;
+  HIP_TRY(hipMemGetInfo(&f, &t));
+  if (free_bytes) *free_bytes = f;
+  if (total_bytes) *total_bytes = t;
+  return CSK_OK;
+}
+
+extern "C" int csk_alloc_count(uint64_t* count) {
+  if (!count) return fail(CSK_ERR_ARG, "csk_alloc_count: null output");
+  *count = g_alloc_count.load(std::memory_order_relaxed);
   return CSK_OK;
 }
 
@@ -785,7 +813,7 @@ extern "C" void* csk_dev_alloc(size_t bytes) {
   }
   if (!t_device_bound && hipSetDevice(g_device) == hipSuccess) t_device_bound = true;
   void* p = nullptr;
-  hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+  hipError_t e = counted_malloc(&p, bytes ? bytes : 1);
   if (e != hipSuccess) {
     g_err = std::string("hipMalloc: ") + hipGetErrorString(e);
     return nullptr;
@@ -1130,7 +1158,7 @@ int f16_pack_into(const void* data, int type, int64_t rows, int64_t K, u32x4* ds
   if (!bytes)
     return fail(CSK_ERR_ARG, "fp16 experts take ggml types F16 (1), Q4_K (12) and Q6_K (14), K-quants with rows * K a multiple of 256");
   uint8_t* stage = nullptr;
-  HIP_TRY(hipMalloc((void**)&stage, bytes));
+  HIP_TRY(counted_malloc((void**)&stage, bytes));
   hipError_t e = hipMemcpyAsync(stage, data, bytes, hipMemcpyHostToDevice, g_stream);
   int rc = CSK_OK;
   if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("hipMemcpy: ") + hipGetErrorString(e));
@@ -1152,7 +1180,7 @@ int f16_pack_into(const void* data, int type, int64_t rows, int64_t K, u32x4* ds
 int f16_export_from(const u32x4* src, int64_t rows, int64_t K, uint16_t* halves) {
   uint16_t* stage = nullptr;
   const size_t n = (size_t)rows * K;
-  HIP_TRY(hipMalloc((void**)&stage, n * sizeof(uint16_t)));
+  HIP_TRY(counted_malloc((void**)&stage, n * sizeof(uint16_t)));
   const long ent = f16_entries(rows, K);
   f16_unpack_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(src, stage, rows, K, ent);
   int rc = check_launch("f16_unpack_kernel");
@@ -1197,7 +1225,7 @@ struct StagingPool {
         return CSK_OK;
       }
     }
-    HIP_TRY(hipMalloc(out, want));
+    HIP_TRY(counted_malloc(out, want));
     *cap = want;
     return CSK_OK;
   }
@@ -1464,7 +1492,7 @@ extern "C" int csk_f16_upload_f32(const float* w_host, int64_t rows, int64_t K, 
   DevBuf stage;
   int rc = dev_alloc(&m->w, (size_t)ent);
   if (rc == CSK_OK) rc = stage.upload(w_host, (size_t)rows * K * 4);
-  if (rc == CSK_OK && !g_bad && hipMalloc((void**)&g_bad, sizeof(unsigned long long)) != hipSuccess)
+  if (rc == CSK_OK && !g_bad && counted_malloc((void**)&g_bad, sizeof(unsigned long long)) != hipSuccess)
     rc = fail(CSK_ERR_HIP, "hipMalloc failed");
   unsigned long long bad = ~0ull;
   if (rc == CSK_OK) {
@@ -1563,7 +1591,8 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
   int rc = CSK_OK;
   rc = ws.ensure(T, L->E, L->k, L->H, L->F, L->wbf);
   if (rc != CSK_OK) return rc;
-  g_last_ws = &ws;
+  L->last_ws = &ws;
+  L->last_run = ++ws.runs;
   const int64_t P = T * L->k;
   const bool norm = (flags & CSK_FWD_RMSNORM) != 0;
   const float* xr = norm ? ws.xn : hidden;
@@ -1708,21 +1737,19 @@ extern "C" int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T
   REQUIRE_INIT();
   if (!L || !hidden || !out || T < 0) return fail(CSK_ERR_ARG, "csk_moe_forward_host: bad argument");
   if (T == 0) return CSK_OK;
-  // device copies of the caller's rows: kept between calls (a frame of a decoding engine
-  // comes back every few milliseconds) and grown on demand; the copies in, the kernels and
-  // the copies out are queued on the stream and awaited once
-  static float *dh = nullptr, *dout = nullptr;
-  static size_t cap = 0;
+  // device copies of the caller's rows, from the pool of staging blocks (a frame of a decoding
+  // engine comes back every few milliseconds and finds its blocks idle again: no allocation
+  // in steady state, nothing held that the pool's bounds do not cover); the copies in, the
+  // kernels and the copies out are queued on the stream and awaited once
   const size_t n = (size_t)T * L->H;
-  if (n > cap) {
-    HIP_TRY(hipStreamSynchronize(g_stream));
-    if (dh) (void)hipFree(dh);
-    if (dout) (void)hipFree(dout);
-    dh = dout = nullptr, cap = 0;
-    HIP_TRY(hipMalloc((void**)&dh, n * sizeof(float)));
-    HIP_TRY(hipMalloc((void**)&dout, n * sizeof(float)));
-    cap = n;
+  DevBuf dbh, dbo;
+  {
+    int rc0 = dbh.alloc(n * sizeof(float));
+    if (rc0 == CSK_OK) rc0 = dbo.alloc(n * sizeof(float));
+    if (rc0 != CSK_OK) return rc0;
   }
+  float* const dh = dbh.as<float>();
+  float* const dout = dbo.as<float>();
   int rc = CSK_OK;
   {
     const void* src = hidden;
@@ -1768,12 +1795,16 @@ extern "C" int csk_layer_last_dispatch(csk_layer* L, int32_t* counts_host, int32
   if (!L) return fail(CSK_ERR_ARG, "null layer");
   if (L->last_T < 0)
     return fail(CSK_ERR_STATE, "the last forward took its batch in several passes: there is no single dispatch to report");
-  if (L->last_T == 0) return fail(CSK_ERR_STATE, "no forward has run on this layer");
+  if (L->last_T == 0 || !L->last_ws) return fail(CSK_ERR_STATE, "no forward has run on this layer");
+  // the lists live in the workspace the forward ran in, which the next forward -- of any layer -- overwrites
+  const Workspace* ws = static_cast<const Workspace*>(L->last_ws);
+  if (ws->runs != L->last_run)
+    return fail(CSK_ERR_STATE, "another forward has run since this layer's last one: its dispatch lists are gone");
   if (counts_host) {
-    int rc = csk_copy_d2h(counts_host, g_last_ws->counts, (size_t)L->E * sizeof(int));
+    int rc = csk_copy_d2h(counts_host, ws->counts, (size_t)L->E * sizeof(int));
     if (rc != CSK_OK) return rc;
   }
-  if (tokens_host) return csk_copy_d2h(tokens_host, g_last_ws->list_tok, (size_t)L->last_T * L->k * sizeof(int));
+  if (tokens_host) return csk_copy_d2h(tokens_host, ws->list_tok, (size_t)L->last_T * L->k * sizeof(int));
   return CSK_OK;
 }
 
@@ -2150,6 +2181,24 @@ extern "C" int csk_rmsnorm(const float* x, const float* weight, float* out, int6
   rc = launch_prep(dx.as<float>(), dw.as<float>(), eps, dout.as<float>(), T, H);
   if (rc != CSK_OK) return rc;
   CSK_TRY(fetch(out, dout.p, (size_t)T * H * 4));
+  CSK_TRY(finish_fetches());
+  return CSK_OK;
+}
+
+extern "C" int csk_rmsnorm_f64(const double* x, const double* weight, double* out, int64_t T, int64_t H,
+                               float eps) {
+  REQUIRE_INIT();
+  if (!x || !weight || !out || T < 0 || H <= 0) return fail(CSK_ERR_ARG, "csk_rmsnorm_f64: bad argument");
+  if (T == 0) return CSK_OK;
+  DevBuf dx, dw, dout;
+  int rc;
+  if ((rc = dx.upload(x, (size_t)T * H * 8)) != CSK_OK) return rc;
+  if ((rc = dw.upload(weight, (size_t)H * 8)) != CSK_OK) return rc;
+  if ((rc = dout.alloc((size_t)T * H * 8)) != CSK_OK) return rc;
+  rmsnorm_f64_kernel<<<dim3((unsigned)cdiv(T, 8)), 512, 0, g_stream>>>(dx.as<double>(), dw.as<double>(),
+                                                                       dout.as<double>(), (long)T, (long)H, eps);
+  if ((rc = check_launch("rmsnorm_f64_kernel")) != CSK_OK) return rc;
+  CSK_TRY(fetch(out, dout.p, (size_t)T * H * 8));
   CSK_TRY(finish_fetches());
   return CSK_OK;
 }

@@ -182,4 +182,45 @@ __global__ __launch_bounds__(256) void add_broadcast_kernel(const V* __restrict_
   }
 }
 
+// ------------------------------------------------------------ rmsnorm, float64
+// out[i][j] = (x[i][j] / sqrt(sum_j x[i][j]^2 / H + eps)) * w[j]   (rmsnorm_node.h:62-83 with
+// T = double).  The sum of squares is the reference's: one product and one addition per
+// element, each rounded, in index order -- so one lane walks the row alone (eight rows per
+// workgroup, one per wave, the row staged through LDS in chunks so that the global reads are
+// coalesced); division, square root, x / rms and the product with w are IEEE operations and
+// are spread over the wave.  Bit-exact against the CPU path.
+constexpr int kRms64Chunk = 512;
+
+__global__ __launch_bounds__(512) void rmsnorm_f64_kernel(const double* __restrict__ x,
+                                                          const double* __restrict__ w,
+                                                          double* __restrict__ out, long T, long H,
+                                                          float eps) {
+#pragma clang fp contract(off)
+  __shared__ double stage[8][kRms64Chunk];
+  __shared__ double rms_sh[8];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const long row = (long)blockIdx.x * 8 + wv;
+  if (row >= T) return;  // (whole waves leave: what follows synchronises within a wave only)
+  const double* xr = x + row * H;
+  double ss = 0.0;
+  for (long c0 = 0; c0 < H; c0 += kRms64Chunk) {
+    const int n = (int)min((long)kRms64Chunk, H - c0);
+    for (int j = lane; j < n; j += 64) stage[wv][j] = xr[c0 + j];
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's LDS writes have landed
+    if (lane == 0) {
+      for (int j = 0; j < n; ++j) {
+        const double v = stage[wv][j];
+        ss += v * v;
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane == 0) rms_sh[wv] = sqrt(ss / (double)H + (double)eps);
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_s_waitcnt(0xc07f);
+  const double rms = rms_sh[wv];
+  for (long j = lane; j < H; j += 64) out[row * H + j] = (xr[j] / rms) * w[j];
+}
+
 }  // namespace csk

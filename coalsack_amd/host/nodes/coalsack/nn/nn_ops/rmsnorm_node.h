@@ -1,6 +1,6 @@
 // rmsnorm_node backed by the gfx950 library: same class name, setter, test wrapper
 // and error texts as include/coalsack/nn/nn_ops/rmsnorm_node.h of the reference
-// (cited by line below); the normalisation runs in csk_rmsnorm.
+// (cited by line below); the normalisation runs in csk_rmsnorm / csk_rmsnorm_f64.
 #pragma once
 
 #include <stdexcept>
@@ -31,13 +31,20 @@ class rmsnorm_node : public binary_op_node {
     const int64_t hidden_dim = shape.back();
     if (weight.ndim() != 1 || weight.dim(0) != hidden_dim)
       throw std::runtime_error("rmsnorm: weight shape must be [hidden_dim]");
-    // the reference also has a float64 branch; this build computes in float32 only
-    if (input.get_dtype() != dtype::float32 || weight.get_dtype() != dtype::float32)
-      throw std::runtime_error("rmsnorm: only float32 supported on this build");
-    dynamic_tensor output(dtype::float32, shape);
+    // float32 or float64, as the reference (:47-53).  The reference reads the weight as the
+    // input's element type whatever it holds (:65); a weight of another type is refused here
+    // instead of having its bytes reinterpreted.
+    const dtype dt = input.get_dtype();
+    if (dt != dtype::float32 && dt != dtype::float64)
+      throw std::runtime_error("rmsnorm: only float32 and float64 supported");
+    if (weight.get_dtype() != dt) throw std::runtime_error("rmsnorm: weight must have the input's element type");
+    dynamic_tensor output(dt, shape);
     if (outer_size == 0 || hidden_dim == 0) return output;
-    const int rc = csk_rmsnorm(input.data_ptr<float>(), weight.data_ptr<float>(), output.data_ptr<float>(),
-                               outer_size, hidden_dim, epsilon_);
+    const int rc = dt == dtype::float32
+                       ? csk_rmsnorm(input.data_ptr<float>(), weight.data_ptr<float>(), output.data_ptr<float>(),
+                                     outer_size, hidden_dim, epsilon_)
+                       : csk_rmsnorm_f64(input.data_ptr<double>(), weight.data_ptr<double>(),
+                                         output.data_ptr<double>(), outer_size, hidden_dim, epsilon_);
     if (rc != CSK_OK) throw std::runtime_error(std::string("rmsnorm: ") + csk_last_error());
     return output;
   }

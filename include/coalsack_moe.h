@@ -61,6 +61,11 @@ int csk_init(int device);
 const char* csk_last_error(void);
 /* name (NUL-terminated, cap bytes), compute-unit count, total device memory */
 int csk_device_info(char* name, size_t cap, int* compute_units, size_t* hbm_bytes);
+/* free and total device memory as the runtime reports them now (either may be NULL) */
+int csk_device_memory(size_t* free_bytes, size_t* total_bytes);
+/* number of device allocations the library has made in this process so far (every one of
+ * them goes through one counted call): unchanged across a call that allocates nothing */
+int csk_alloc_count(uint64_t* count);
 
 /* Device memory and timing for hosts with no HIP binding of their own. */
 void* csk_dev_alloc(size_t bytes);
@@ -326,6 +331,10 @@ int csk_expert_merge(const float* router_pairs, int64_t T, int64_t k, int64_t E,
                      const float* const* expert_outs, int pre_weighted, float* out);
 /* rmsnorm_node::compute (rmsnorm_node.h:62-83) and add_node (add_node.h:8-55) */
 int csk_rmsnorm(const float* x, const float* weight, float* out, int64_t T, int64_t H, float eps);
+/* the node's float64 branch (rmsnorm_node.h:49-50, compute_impl<double>): input, weight and
+ * output are doubles; sums, division, square root and products in double, in the
+ * reference's order -- the result equals the CPU's bit for bit */
+int csk_rmsnorm_f64(const double* x, const double* weight, double* out, int64_t T, int64_t H, float eps);
 int csk_add(const float* a, const float* b, float* out, int64_t n);
 /* add_node over operands of different shapes and of the node's other element types
  * (add_node.h:16-50 through elementwise_binary_op, elementwise_helpers.h:9-66): numpy-style

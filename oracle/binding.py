@@ -95,6 +95,8 @@ class Oracle:
         d.orc_expert_merge.argtypes = [_P, _I64, _I64, _I64, _I64, C.POINTER(_P), C.c_int, _P]
         d.orc_rmsnorm.restype = None
         d.orc_rmsnorm.argtypes = [_P, _P, _P, _I64, _I64, C.c_float]
+        d.orc_rmsnorm_f64.restype = None
+        d.orc_rmsnorm_f64.argtypes = [_P, _P, _P, _I64, _I64, C.c_float]
         d.orc_add.restype = None
         d.orc_add.argtypes = [_P, _P, _P, _I64]
         d.orc_moe_layer.restype = C.c_int
@@ -317,6 +319,14 @@ class Oracle:
         T, H = x.shape
         out = np.empty((T, H), np.float32)
         self.dll.orc_rmsnorm(_p(x), _p(w), _p(out), T, H, eps)
+        return out
+
+    def rmsnorm_f64(self, x, w, eps):
+        x = np.ascontiguousarray(x, np.float64)
+        w = np.ascontiguousarray(w, np.float64)
+        T, H = x.shape
+        out = np.empty((T, H), np.float64)
+        self.dll.orc_rmsnorm_f64(_p(x), _p(w), _p(out), T, H, eps)
         return out
 
     def add(self, a, b):

@@ -72,6 +72,14 @@
  *          linearity; error cases.
  *   orc_rmsnorm / orc_add
  *        - known answers test/test_rmsnorm.cpp:74-142 and closed form.
+ *   orc_rmsnorm_f64
+ *        - the same known answers in double (exact where they are exact: rows
+ *          of +-c give +-w c / sqrt(c^2 + eps) with one rounding per operation,
+ *          checked against Python's correctly rounded float arithmetic on
+ *          values chosen so that every intermediate is exact or a single
+ *          rounding), math.fsum for the sum of squares within 2 ulp on random
+ *          rows, scale covariance (x -> 2^k x, eps = 0, bit for bit), and
+ *          agreement with the float32 function to float32 precision.
  *
  * Build: gcc -O2 -shared -fPIC (the reference's Release flags are plain -O2,
  * CMakeLists.txt:19-21).  No -march: scalar code must not be contracted into
@@ -775,6 +783,21 @@ void orc_rmsnorm(const float* x, const float* w, float* out, int64_t T, int64_t 
       ss += v * v;
     }
     const float rms = sqrtf(ss / (float)H + eps);
+    for (int64_t j = 0; j < H; ++j) out[i * H + j] = (x[i * H + j] / rms) * w[j];
+  }
+}
+
+/* rmsnorm_node.h:47-53, :62-83 with T = double: the sums, the division by hidden_dim, the
+ * epsilon (a float member widened, :72) and the square root are all double; x / rms, then
+ * times w, each rounded (plain -O2 x86-64 has no fused multiply-add to contract them). */
+void orc_rmsnorm_f64(const double* x, const double* w, double* out, int64_t T, int64_t H, float eps) {
+  for (int64_t i = 0; i < T; ++i) {
+    double ss = 0.0;
+    for (int64_t j = 0; j < H; ++j) {
+      const double v = x[i * H + j];
+      ss += v * v;
+    }
+    const double rms = sqrt(ss / (double)H + (double)eps);
     for (int64_t j = 0; j < H; ++j) out[i * H + j] = (x[i * H + j] / rms) * w[j];
   }
 }

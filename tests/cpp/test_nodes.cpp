@@ -37,6 +37,7 @@ int orc_dense_ffn_f16(const float*, int64_t, int64_t, int64_t, const uint16_t*, 
                       const float*, const float*, const float*, float*);
 void orc_matmul_transpose_f16(const float*, const uint16_t*, float*, int64_t, int64_t, int64_t);
 void orc_rmsnorm(const float*, const float*, float*, int64_t, int64_t, float);
+void orc_rmsnorm_f64(const double*, const double*, double*, int64_t, int64_t, float);
 void orc_add(const float*, const float*, float*, int64_t);
 void orc_matmul_transpose_batched(const float*, int64_t, const void*, int64_t, int, int64_t, float*, int64_t, int64_t,
                                   int64_t);
@@ -313,7 +314,10 @@ static void cpu_norm_add_argument_errors() {
                     "rmsnorm: input must have at least 1 dimension"));
   CHECK(throws_with([&] { norm.compute_test(x, w_bad); }, "rmsnorm: weight shape must be [hidden_dim]"));
   CHECK(throws_with([&] { norm.compute_test(x, w2); }, "rmsnorm: weight shape must be [hidden_dim]"));
-  CHECK(throws_with([&] { norm.compute_test(dynamic_tensor(dtype::float64, {2, 8}), w); }, "rmsnorm: only float32"));
+  CHECK(throws_with([&] { norm.compute_test(dynamic_tensor(dtype::float16, {2, 8}), w); },
+                    "rmsnorm: only float32 and float64 supported"));  // rmsnorm_node.h:52
+  CHECK(throws_with([&] { norm.compute_test(dynamic_tensor(dtype::float64, {2, 8}), w); },
+                    "rmsnorm: weight must have the input's element type"));
   CHECK(throws_with([&] { add.compute_test(x, dynamic_tensor(dtype::float64, {2, 3, 8})); }, "add: input dtype mismatch"));
   CHECK(throws_with([&] { add.compute_test(x, w_bad); }, "Broadcast failed: Shape A=[2,3,8], Shape B=[7]"));
   CHECK(throws_with([&] { add.compute_test(dynamic_tensor(dtype::float16, {2}), dynamic_tensor(dtype::float16, {2})); },
@@ -354,6 +358,24 @@ static void gpu_norm_add_tests() {
   float worst = 0;
   for (size_t i = 0; i < want.size(); ++i) worst = std::fmax(worst, std::fabs(y.data_ptr<float>()[i] - want[i]));
   CHECK(worst <= 2e-6f);
+  {  // the float64 branch (rmsnorm_node.h:49-50): equal to the CPU's double arithmetic bit for bit
+    dynamic_tensor xd(dtype::float64, {B, S, H}), wd(dtype::float64, {H});
+    std::uniform_real_distribution<double> dx(-2.0, 2.0), dw(0.5, 1.5);
+    for (int64_t i = 0; i < B * S * H; ++i) xd.data_ptr<double>()[i] = dx(gen);
+    for (int64_t i = 0; i < H; ++i) wd.data_ptr<double>()[i] = dw(gen);
+    auto yd = norm.compute_test(xd, wd);
+    CHECK(yd.get_dtype() == dtype::float64 && yd.shape() == xd.shape());
+    std::vector<double> wantd((size_t)(B * S * H));
+    orc_rmsnorm_f64(xd.data_ptr<double>(), wd.data_ptr<double>(), wantd.data(), B * S, H, 1e-6f);
+    CHECK(std::memcmp(yd.data_ptr<double>(), wantd.data(), wantd.size() * sizeof(double)) == 0);
+    // test_rmsnorm.cpp:118-142 in double: 5 / sqrt(25) * 2 = 2
+    dynamic_tensor x1(dtype::float64, {1, 1}), w1d(dtype::float64, {1});
+    x1.data_ptr<double>()[0] = 5.0, w1d.data_ptr<double>()[0] = 2.0;
+    norm.set_epsilon(0.0f);
+    CHECK(norm.compute_test(x1, w1d).data_ptr<double>()[0] == 2.0);
+    norm.set_epsilon(1e-6f);
+    CHECK(norm.compute_test(dynamic_tensor(dtype::float64, {0, 8}), dynamic_tensor(dtype::float64, {8})).numel() == 0);
+  }
   auto z = add.compute_test(x, y);
   orc_add(x.data_ptr<float>(), y.data_ptr<float>(), want.data(), B * S * H);
   CHECK(std::memcmp(z.data_ptr<float>(), want.data(), want.size() * sizeof(float)) == 0);

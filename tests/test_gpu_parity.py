@@ -335,6 +335,22 @@ def test_rmsnorm_and_add(lib, oracle):
     assert np.array_equal(lib.add(x, x), oracle.add(x, x))
 
 
+def test_rmsnorm_f64_equals_cpu_bit_for_bit(lib, oracle):
+    """rmsnorm_node's float64 branch (rmsnorm_node.h:49-50): every operation is a double one
+    in the reference's order, so the result is the CPU's."""
+    assert lib.rmsnorm_f64(np.array([[5.0]]), np.array([2.0]), 0.0)[0, 0] == 2.0  # test_rmsnorm.cpp:118-142
+    rng = np.random.default_rng(11)
+    for T, H in ((1, 1), (3, 7), (9, 512), (5, 513), (17, 2880), (2, 5000)):
+        x = rng.normal(0, 2, (T, H))
+        w = rng.normal(1, 0.1, H)
+        for eps in (0.0, 1e-5):
+            assert np.array_equal(lib.rmsnorm_f64(x, w, eps), oracle.rmsnorm_f64(x, w, eps)), (T, H, eps)
+    x = np.zeros((2, 64))
+    assert np.array_equal(lib.rmsnorm_f64(x, np.ones(64), 1e-5), x)
+    got = lib.rmsnorm_f64(x, np.ones(64), 0.0)  # 0 / 0, as the reference computes it
+    assert np.all(np.isnan(got))
+
+
 # ------------------------------------------------------------ whole layer
 
 def _check_layer(lib, oracle, L, T, bias=True, norm=False, residual=False, device_weights=False,

@@ -185,6 +185,45 @@ def test_rmsnorm_known_answers(oracle):
     assert np.array_equal(oracle.add(x, x), x + x)
 
 
+def test_rmsnorm_f64_pinned(oracle):
+    """rmsnorm_node.h:49-50 / :62-83 with T = double.  Known answers in double; rows on which
+    every operation is exact or a single correctly rounded one (so Python's own IEEE double
+    arithmetic states the answer without restating the loop); the sum of squares against
+    math.fsum; exact scale covariance; agreement with the float32 function."""
+    import math
+    # test_rmsnorm.cpp:118-142 and :74-115 in double
+    assert oracle.rmsnorm_f64(np.array([[5.0]]), np.array([2.0]), 0.0)[0, 0] == 2.0
+    x = np.array([[1.0, 2.0, 3.0, 4.0]])
+    w = np.array([2.0, 0.5, 1.5, 1.0])
+    rms = math.sqrt(30.0 / 4.0)  # 30 and 7.5 are exact; one rounding in the root
+    assert np.array_equal(oracle.rmsnorm_f64(x, w, 0.0), np.array([[(v / rms) * g for v, g in zip(x[0], w)]]))
+    # rows of +-c: sum of squares H c^2 exact for small integers, mean = c^2 exact, eps widened from float
+    for c, H in ((3.0, 8), (0.5, 64), (7.0, 2880)):
+        eps = float(np.float32(1e-5))
+        row = np.array([[c if j % 2 == 0 else -c for j in range(H)]])
+        wv = np.linspace(0.5, 1.5, H)
+        r = math.sqrt(c * c + eps)
+        want = np.array([[(v / r) * g for v, g in zip(row[0], wv)]])
+        assert np.array_equal(oracle.rmsnorm_f64(row, wv, 1e-5), want)
+    # a dropped term, a wrong divisor or a float accumulator would show here
+    rng = np.random.default_rng(3)
+    x = rng.normal(0, 1, (4, 2880))
+    w = rng.normal(1, 0.02, 2880)
+    got = oracle.rmsnorm_f64(x, w, 1e-5)
+    for i in range(4):
+        ss = math.fsum(float(v) * float(v) for v in x[i])  # (rounded products, exactly summed)
+        r = math.sqrt(ss / 2880 + float(np.float32(1e-5)))
+        want = x[i] / r * w
+        assert np.max(np.abs(got[i] - want) / np.abs(want)) < 1e-13  # sequential vs compensated sum: a few ulp
+    # eps = 0: scaling the row by a power of two changes nothing (every operation scales exactly)
+    a = oracle.rmsnorm_f64(x, w, 0.0)
+    assert np.array_equal(oracle.rmsnorm_f64(x * 1024.0, w, 0.0), a)
+    assert np.array_equal(oracle.rmsnorm_f64(x, w * 0.25, 0.0), a * 0.25)
+    # against the float32 function on float32 data
+    xf, wf = x.astype(np.float32), w.astype(np.float32)
+    assert np.allclose(oracle.rmsnorm_f64(xf, wf, 1e-5), oracle.rmsnorm(xf, wf, 1e-5), rtol=2e-6, atol=1e-6)
+
+
 def test_layer_composition_equals_node_chain(oracle):
     """orc_moe_layer (token-by-token evaluation) is bit-identical to the node
     chain the reference wires: router -> E expert nodes -> merge."""
