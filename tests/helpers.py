@@ -75,6 +75,51 @@ def nbits_differ(a, b):
     return int(np.count_nonzero(a != b))
 
 
+# |w_gpu - w_cpu| for a routing weight.  The two sets of logits differ by summation order:
+# test_router_logits_distance_from_sequential_sums holds each logit within 3 units of
+# 2^-24 sqrt(H) max(1, |logit|) of the reference's sequential sum -- 9.6e-6 max(1, |logit|)
+# at H = 2880.  A softmax (or sigmoid) weight moves by at most w (1 - w) <= 1/4 per unit of
+# logit difference between two experts, i.e. by up to 1/4 x 2 x 9.6e-6 = 4.8e-6 for logits
+# of magnitude <= 1 and proportionally more for larger ones (observed: 5.5e-6 at 257
+# tokens).  1e-5 is that bound for the logit magnitudes of these configurations; 1e-6
+# would need every logit in the reference's sequential order, which the library computes
+# only where a selection depends on it (close calls).
+ROUTING_WEIGHT_TOL = 1e-5
+
+
+def oracle_layer_tokens(oracle, L, hidden, idx, threads=16):
+    """Oracle output and router pairs for the tokens hidden[idx] (any index set), replaying on
+    the host only the experts those tokens select; the tokens are farmed over threads (the
+    checker releases the interpreter lock inside a call and tokens are independent)."""
+    import threading
+    idx = np.asarray(idx, dtype=np.int64)
+    sub = np.ascontiguousarray(hidden[idx])
+    pairs = oracle.router(sub, L.gate_w, L.gate_b, L.k)
+    used = sorted(set(pairs[..., 0].astype(int).ravel().tolist()))
+    per_gu, per_d = L.F * (L.H // 32) * 17, L.H * (L.F // 32) * 17
+    wu = np.zeros(L.E * per_gu, np.uint8)
+    wg = np.zeros(L.E * per_gu, np.uint8)
+    wd = np.zeros(L.E * per_d, np.uint8)
+    for e in used:
+        wu[e * per_gu:(e + 1) * per_gu] = L.blocks(e, 0)
+        wg[e * per_gu:(e + 1) * per_gu] = L.blocks(e, 1)
+        wd[e * per_d:(e + 1) * per_d] = L.blocks(e, 2)
+    out = np.zeros((idx.size, L.H), np.float32)
+    opairs = np.zeros((idx.size, L.k, 2), np.float32)
+    chunks = [c for c in np.array_split(np.arange(idx.size), max(1, min(threads, idx.size))) if c.size]
+
+    def work(c):
+        o, p = oracle.moe_layer(np.ascontiguousarray(sub[c]), L.E, L.k, L.H, L.F, L.gate_w, L.gate_b, wu, wg, wd,
+                                L.b_up, L.b_gate, L.b_down)
+        out[c], opairs[c] = o, p
+    ts = [threading.Thread(target=work, args=(c,)) for c in chunks]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    return out, opairs
+
+
 def oracle_layer_subset(oracle, L, hidden, ntok, norm=False, residual=False, **opts):
     """Oracle output for the first ntok tokens, replaying on the host only the
     experts those tokens select (the others stay zero and are never read)."""
