@@ -95,6 +95,13 @@ SIGNATURES = {
     "csk_add": (C.c_int, [_P, _P, _P, _I64]),
     "csk_add_broadcast": (C.c_int, [_P, _P, C.c_int, _P, _P, C.c_int, C.c_int, _P]),
     "csk_moe_router_f64": (C.c_int, [_P, _I64, _I64, _P, _I64, _P, _I64, C.c_int, _P, _P]),
+    "csk_layer_create_view": (C.c_int, [_I64, _I64, _I64, _I64, C.POINTER(_P)]),
+    "csk_layer_attach_expert": (C.c_int, [_P, _I64, _P, _P, _P, _P, _P, _P]),
+    "csk_layer_detach_expert": (C.c_int, [_P, _I64]),
+    "csk_moe_frame_begin": (C.c_int, [_P, _P, _I64, _P, C.c_int, C.POINTER(C.c_int)]),
+    "csk_moe_frame_expert_rows": (C.c_int, [_P, _I64, _P]),
+    "csk_moe_frame_void": (C.c_int, [_P]),
+    "csk_moe_frame_merged": (C.c_int, [_P, _P, C.POINTER(C.c_int)]),
 }
 
 

@@ -299,6 +299,22 @@ struct csk_layer {
   int64_t last_T = 0;
   const void* last_ws = nullptr;  // workspace of this layer's last forward, and that workspace's forward count then
   uint64_t last_run = 0;
+  // A view layer owns no expert matrices: expert e's planes are those of three csk_mxfp4
+  // handles attached by the caller.  It has a workspace of its own, so that what a frame
+  // leaves there (router output, per-assignment rows) stays until the next frame of this
+  // layer whatever other layers do meanwhile.
+  bool is_view = false;
+  std::vector<char> attached;
+  void* own_ws = nullptr;  // Workspace*
+  struct Frame {
+    bool live = false, experts_ran = false, rows_fetched = false, voided = false;
+    int64_t T = 0;
+    int flags = 0;
+    float *d_hidden = nullptr, *d_out = nullptr;
+    size_t cap = 0;  // floats in d_hidden / d_out
+    std::vector<float> pairs, y;
+    std::vector<int> pos;
+  } frame;
   // geometry of one expert's planes
   int64_t nblkH = 0, nblkF = 0, ntF = 0, ntH = 0;
   long ent_gu() const { return (long)(ntF * nblkH * 16); }  // gate or up: [F,H]
@@ -927,7 +943,7 @@ extern "C" int csk_mxfp4_export(const csk_mxfp4* m, uint8_t* host_out) {
 
 // ============================================================ layer
 
-static int layer_create(int64_t E, int64_t k, int64_t H, int64_t F, bool f16, csk_layer** out) {
+static int layer_create(int64_t E, int64_t k, int64_t H, int64_t F, bool f16, csk_layer** out, bool view = false) {
   REQUIRE_INIT();
   if (!out) return fail(CSK_ERR_ARG, "csk_layer_create: null out");
   int rc = check_dims(E, k, H, F);
@@ -935,6 +951,11 @@ static int layer_create(int64_t E, int64_t k, int64_t H, int64_t F, bool f16, cs
   csk_layer* L = new csk_layer;
   L->E = E, L->k = k, L->H = H, L->F = F;
   L->f16 = f16;
+  L->is_view = view;
+  if (view) {
+    L->attached.assign((size_t)E, 0);
+    L->own_ws = new Workspace;
+  }
   L->nblkH = H / 32, L->nblkF = F / 32, L->ntF = cdiv(F, 16), L->ntH = cdiv(H, 16);
   L->expert_set.assign((size_t)E, 0);
   L->expert_bias.assign((size_t)E, 0);
@@ -944,7 +965,9 @@ static int layer_create(int64_t E, int64_t k, int64_t H, int64_t F, bool f16, cs
   if (rc == CSK_OK) rc = dev_alloc(&L->gate_b, (size_t)E);
   // kWeightSlack: the grouped GEMM reads up to three blocks (and the scale loads three
   // bytes) past the end of a plane; behind the last plane that must still be mapped memory
-  if (f16) {
+  if (view) {
+    // no planes of its own
+  } else if (f16) {
     if (rc == CSK_OK) rc = dev_alloc(&L->h_all, (size_t)E * L->ent16_expert());
   } else {
     if (rc == CSK_OK) rc = dev_alloc(&L->q_all, (size_t)E * L->ent_expert() + kWeightSlack / sizeof(uint4));
@@ -960,7 +983,9 @@ static int layer_create(int64_t E, int64_t k, int64_t H, int64_t F, bool f16, cs
   }
   for (int64_t e = 0; e < E; ++e) {
     ExpertW& w = L->ew_host[(size_t)e];
-    if (f16) {
+    if (view) {
+      w = ExpertW{};
+    } else if (f16) {
       w.q_gate = reinterpret_cast<const uint4*>(L->view16(e, CSK_W_GATE));
       w.q_up = reinterpret_cast<const uint4*>(L->view16(e, CSK_W_UP));
       w.q_down = reinterpret_cast<const uint4*>(L->view16(e, CSK_W_DOWN));
@@ -991,9 +1016,14 @@ extern "C" void csk_layer_destroy(csk_layer* L) {
   if (!L) return;
   API_LOCK();
   if (g_stream) (void)hipStreamSynchronize(g_stream);
-  void* ps[] = {L->gate_w, L->gate_b, L->q_all, L->s_all, L->h_all, L->bias_all, L->ew_dev, L->norm_w};
+  void* ps[] = {L->gate_w, L->gate_b, L->q_all, L->s_all, L->h_all, L->bias_all, L->ew_dev, L->norm_w,
+                L->frame.d_hidden, L->frame.d_out};
   for (void* p : ps)
     if (p) (void)hipFree(p);
+  if (L->own_ws) {
+    static_cast<Workspace*>(L->own_ws)->release();
+    delete static_cast<Workspace*>(L->own_ws);
+  }
   delete L;
 }
 
@@ -1587,16 +1617,23 @@ int64_t g_pass_tokens = 32768;
 // followed by the dispatch kernel is faster although it is a launch more (120b shape, routing
 // stage: 17.6 -> 15.7 us at T = 48, 20.8 -> 15.9 at T = 64; no gain at 32, a loss at 24).
 constexpr int64_t kRouteSmallTokens = 32;
-int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int flags, Workspace& ws = g_ws) {
+// phase 0: the whole forward; 1: up to and including the dispatch (router output and lists
+// are in ws); 2: the rest (experts and combine) of a pass whose phase 1 ran in the same ws.
+int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int flags, Workspace& ws = g_ws,
+                 int phase = 0) {
   int rc = CSK_OK;
-  rc = ws.ensure(T, L->E, L->k, L->H, L->F, L->wbf);
-  if (rc != CSK_OK) return rc;
-  L->last_ws = &ws;
-  L->last_run = ++ws.runs;
+  if (phase != 2) {
+    rc = ws.ensure(T, L->E, L->k, L->H, L->F, L->wbf);
+    if (rc != CSK_OK) return rc;
+    L->last_ws = &ws;
+    L->last_run = ++ws.runs;
+  }
   const int64_t P = T * L->k;
   const bool norm = (flags & CSK_FWD_RMSNORM) != 0;
   const float* xr = norm ? ws.xn : hidden;
-  if (P <= 1024 && T <= 64) {
+  if (phase == 2) {
+    // routed already
+  } else if (P <= 1024 && T <= 64) {
     // small batch: prologue + logits in one launch, top-k + dispatch in another
     mark(CSK_STAGE_PREP);
     mark(CSK_STAGE_ROUTER);
@@ -1654,6 +1691,7 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
     rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, L->ew_dev, ws);
     if (rc != CSK_OK) return rc;
   }
+  if (phase == 1) return CSK_OK;
   if (L->f16) {
     rc = run_experts_f16(L->E, T, L->k, L->H, L->F, L->act, xr, L->wbf != 0, P, ws, true);
     if (rc != CSK_OK) return rc;
@@ -1787,6 +1825,152 @@ extern "C" int csk_moe_stack_forward(csk_layer* const* layers, int64_t n_layers,
     int rc = csk_moe_forward(layers[i], hidden, T, hidden, CSK_FWD_RMSNORM | CSK_FWD_RESIDUAL);
     if (rc != CSK_OK) return rc;
   }
+  return CSK_OK;
+}
+
+// ---------------------------------------------------------------- view layers and frames
+// What the drop-in node classes share per MoE block: the expert nodes own the resident
+// matrices, a view layer points at them, and a frame runs router, dispatch, every selected
+// expert and the merge as the fused forward does -- begun by the router node, read back by
+// the expert nodes (their rows) and the merge node (the merged rows).
+
+extern "C" int csk_layer_create_view(int64_t E, int64_t k, int64_t H, int64_t F, csk_layer** out) {
+  return layer_create(E, k, H, F, false, out, true);
+}
+
+extern "C" int csk_layer_attach_expert(csk_layer* L, int64_t e, const csk_mxfp4* up, const csk_mxfp4* gate,
+                                       const csk_mxfp4* down, const float* b_up, const float* b_gate,
+                                       const float* b_down) {
+  REQUIRE_INIT();
+  if (!L || !L->is_view) return fail(CSK_ERR_ARG, "csk_layer_attach_expert: not a view layer");
+  if (e < 0 || e >= L->E || !up || !gate || !down) return fail(CSK_ERR_ARG, "csk_layer_attach_expert: bad argument");
+  if (up->rows != L->F || up->K != L->H || gate->rows != L->F || gate->K != L->H || down->rows != L->H ||
+      down->K != L->F)
+    return fail(CSK_ERR_ARG, "csk_layer_attach_expert: matrix shapes do not match the layer");
+  HIP_TRY(hipStreamSynchronize(g_stream));  // nothing in flight reads the entry that is about to change
+  L->frame.live = false;
+  ExpertW& w = L->ew_host[(size_t)e];
+  w.q_gate = gate->q, w.s_gate = gate->s, w.q_up = up->q, w.s_up = up->s, w.q_down = down->q, w.s_down = down->s;
+  int rc = upload_biases(L, e, b_up, b_gate, b_down);  // also publishes the entry
+  if (rc != CSK_OK) return rc;
+  L->attached[(size_t)e] = 1;
+  L->expert_set[(size_t)e] = 1;
+  return CSK_OK;
+}
+
+extern "C" int csk_layer_detach_expert(csk_layer* L, int64_t e) {
+  REQUIRE_INIT();
+  if (!L || !L->is_view || e < 0 || e >= L->E) return fail(CSK_ERR_ARG, "csk_layer_detach_expert: bad argument");
+  HIP_TRY(hipStreamSynchronize(g_stream));  // a frame in flight may still be reading the matrices
+  L->frame.live = false;
+  L->attached[(size_t)e] = 0;
+  L->expert_set[(size_t)e] = 0;
+  L->ew_host[(size_t)e] = ExpertW{};
+  HIP_TRY(hipMemcpy(L->ew_dev + e, &L->ew_host[(size_t)e], sizeof(ExpertW), hipMemcpyHostToDevice));
+  return CSK_OK;
+}
+
+extern "C" int csk_moe_frame_begin(csk_layer* L, const float* hidden, int64_t T, float* pairs_out, int flags,
+                                   int* experts_running) {
+  REQUIRE_INIT();
+  if (!L || !L->is_view || !hidden || !pairs_out || !experts_running || T <= 0)
+    return fail(CSK_ERR_ARG, "csk_moe_frame_begin: bad argument");
+  if (!L->has_gate) return fail(CSK_ERR_STATE, "router weights not set");
+  if ((flags & CSK_FWD_RMSNORM) && !L->has_norm) return fail(CSK_ERR_STATE, "RMSNorm weight not set");
+  if (T > g_pass_tokens) return fail(CSK_ERR_ARG, "csk_moe_frame_begin: a frame is one pass (at most " + std::to_string(g_pass_tokens) + " tokens)");
+  csk_layer::Frame& f = L->frame;
+  *experts_running = 0;
+  f.live = false;
+  const size_t n = (size_t)T * L->H;
+  if (n > f.cap) {
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    if (f.d_hidden) (void)hipFree(f.d_hidden);
+    if (f.d_out) (void)hipFree(f.d_out);
+    f.d_hidden = f.d_out = nullptr, f.cap = 0;
+    HIP_TRY(counted_malloc((void**)&f.d_hidden, n * sizeof(float)));
+    HIP_TRY(counted_malloc((void**)&f.d_out, n * sizeof(float)));
+    f.cap = n;
+  }
+  Workspace& ws = *static_cast<Workspace*>(L->own_ws);
+  {
+    const void* src = hidden;
+    if (void* stage = g_pinned.take(n * sizeof(float))) {
+      std::memcpy(stage, hidden, n * sizeof(float));
+      src = stage;
+    }
+    HIP_TRY(hipMemcpyAsync(f.d_hidden, src, n * sizeof(float), hipMemcpyHostToDevice, g_stream));
+  }
+  int rc = forward_pass(L, f.d_hidden, T, f.d_out, flags, ws, 1);
+  const size_t np = (size_t)T * L->k;
+  f.pairs.resize(np * 2);
+  if (rc == CSK_OK) rc = fetch(f.pairs.data(), ws.pairs, np * 2 * sizeof(float));
+  const int rs = finish_fetches();
+  if (rc == CSK_OK) rc = rs;
+  if (rc != CSK_OK) return rc;
+  std::memcpy(pairs_out, f.pairs.data(), np * 2 * sizeof(float));
+  L->last_T = T;
+  f.T = T, f.flags = flags;
+  f.live = true, f.experts_ran = false, f.rows_fetched = false, f.voided = false;
+  // every expert the frame selects has to be attached: the expert kernels follow the
+  // descriptors of the selected experts, and only of those
+  for (size_t p = 0; p < np; ++p) {
+    const int e = (int)f.pairs[2 * p];
+    if (e < 0 || e >= L->E || !L->attached[(size_t)e]) return CSK_OK;
+  }
+  rc = forward_pass(L, f.d_hidden, T, f.d_out, flags, ws, 2);
+  if (rc != CSK_OK) {
+    f.live = false;
+    return rc;
+  }
+  f.experts_ran = true;
+  *experts_running = 1;
+  return CSK_OK;
+}
+
+extern "C" int csk_moe_frame_expert_rows(csk_layer* L, int64_t e, float* out) {
+  REQUIRE_INIT();
+  if (!L || !L->is_view || !out || e < 0 || e >= L->E) return fail(CSK_ERR_ARG, "csk_moe_frame_expert_rows: bad argument");
+  csk_layer::Frame& f = L->frame;
+  if (!f.live || !f.experts_ran) return fail(CSK_ERR_STATE, "csk_moe_frame_expert_rows: no frame with running experts");
+  const size_t np = (size_t)f.T * L->k, H = (size_t)L->H;
+  if (!f.rows_fetched) {
+    Workspace& ws = *static_cast<Workspace*>(L->own_ws);
+    f.y.resize(np * H);
+    f.pos.resize(np);
+    HIP_TRY(hipMemcpyAsync(f.y.data(), ws.y, np * H * sizeof(float), hipMemcpyDeviceToHost, g_stream));
+    HIP_TRY(hipMemcpyAsync(f.pos.data(), ws.pos, np * sizeof(int), hipMemcpyDeviceToHost, g_stream));
+    HIP_TRY(hipStreamSynchronize(g_stream));
+    f.rows_fetched = true;
+  }
+  // row t = the expert's output for token t if t selected it (first matching slot, as
+  // expert_mlp_node.h:503-529), else the zeros the caller's tensor already holds
+  for (int64_t t = 0; t < f.T; ++t)
+    for (int64_t s2 = 0; s2 < L->k; ++s2) {
+      const size_t p = (size_t)t * L->k + s2;
+      if ((int64_t)(int)f.pairs[2 * p] == e) {
+        std::memcpy(out + (size_t)t * H, f.y.data() + (size_t)f.pos[p] * H, H * sizeof(float));
+        break;
+      }
+    }
+  return CSK_OK;
+}
+
+extern "C" int csk_moe_frame_void(csk_layer* L) {
+  API_LOCK();
+  if (!L || !L->is_view) return fail(CSK_ERR_ARG, "csk_moe_frame_void: not a view layer");
+  L->frame.voided = true;
+  return CSK_OK;
+}
+
+extern "C" int csk_moe_frame_merged(csk_layer* L, float* out, int* available) {
+  REQUIRE_INIT();
+  if (!L || !L->is_view || !out || !available) return fail(CSK_ERR_ARG, "csk_moe_frame_merged: bad argument");
+  csk_layer::Frame& f = L->frame;
+  *available = 0;
+  if (!f.live || !f.experts_ran || f.voided) return CSK_OK;
+  CSK_TRY(fetch(out, f.d_out, (size_t)f.T * L->H * sizeof(float)));
+  CSK_TRY(finish_fetches());
+  *available = 1;
   return CSK_OK;
 }
 

@@ -1,7 +1,9 @@
 // expert_merge_node backed by the gfx950 library: same class name, setters,
 // test wrapper, input order and error texts as
 // include/coalsack/nn/nn_ops/expert_merge_node.h of the reference (cited by
-// line below); the weighted sum runs in csk_expert_merge.
+// line below); the weighted sum runs in csk_expert_merge -- or, when the inputs are exactly
+// what the expert nodes of a frame emitted (moe_block_context.h), is the frame's own merged
+// rows, which are on the device already.
 #pragma once
 
 #include <stdexcept>
@@ -9,6 +11,7 @@
 #include <vector>
 
 #include "coalsack/nn/nn_op_node.h"
+#include "coalsack/nn/nn_ops/moe_block_context.h"
 #include "coalsack_moe.h"
 
 namespace coalsack {
@@ -52,6 +55,7 @@ class expert_merge_node : public variadic_op_node {
     if (router.get_dtype() != dtype::float32) throw std::runtime_error("expert_merge: only float32 supported");
 
     dynamic_tensor output(dtype::float32, {batch, seq_len, hidden_dim});
+    if (from_frame(router, inputs, output)) return output;
     const int rc = csk_expert_merge(router.data_ptr<float>(), batch * seq_len, top_k_, num_experts_,
                                     hidden_dim, outs.data(), weight_before_ffn_ ? 1 : 0,
                                     output.data_ptr<float>());
@@ -59,10 +63,48 @@ class expert_merge_node : public variadic_op_node {
     return output;
   }
 
+ public:
+  // merges answered by a frame's own merged rows (a test hook)
+  size_t merges_from_frames() const { return merges_from_frames_; }
+
  private:
+  // The frame's merged rows stand for this merge if the router tensor is the frame's and
+  // every expert output is the very tensor the expert node of that frame emitted from it
+  // (a live input), or belongs to an expert no token of the frame selected (an empty one).
+  bool from_frame(const dynamic_tensor& router, const std::vector<dynamic_tensor>& inputs, dynamic_tensor& output) {
+    auto ctx = csk_resident::moe_block_context::find(router.data_ptr<float>());
+    if (!ctx) return false;
+    std::lock_guard<std::mutex> g(ctx->m);
+    const auto& f = ctx->frame;
+    if (!f.valid || !f.experts_running || ctx->E != num_experts_ || ctx->k != top_k_ ||
+        ctx->weight_before_ffn != (weight_before_ffn_ ? 1 : 0))
+      return false;
+    if ((size_t)router.numel() != f.pairs.size() ||
+        std::memcmp(router.data_ptr<float>(), f.pairs.data(), f.pairs.size() * sizeof(float)) != 0)
+      return false;
+    if (output.dim(0) * output.dim(1) != f.T || output.dim(2) != ctx->H) return false;
+    std::vector<char> selected((size_t)num_experts_, 0);
+    for (size_t p = 0; p < f.pairs.size() / 2; ++p) {
+      const int e = static_cast<int>(f.pairs[2 * p]);
+      if (e < 0 || e >= num_experts_) return false;
+      selected[(size_t)e] = 1;
+    }
+    for (int64_t e = 0; e < num_experts_; ++e) {
+      const dynamic_tensor& t = inputs[(size_t)e + 1];
+      const bool live = t.ndim() == 3 && t.dim(0) > 0;
+      if (live != (selected[(size_t)e] != 0)) return false;
+      if (live && t.data_ptr<float>() != f.emitted[(size_t)e]) return false;
+    }
+    int available = 0;
+    if (csk_moe_frame_merged(ctx->layer, output.data_ptr<float>(), &available) != CSK_OK || !available) return false;
+    ++merges_from_frames_;
+    return true;
+  }
+
   int64_t num_experts_ = 0;
   int64_t top_k_ = 0;
   bool weight_before_ffn_ = false;
+  size_t merges_from_frames_ = 0;
 };
 
 }  // namespace coalsack

@@ -8,11 +8,19 @@
 // node, one entry per role (up, gate, down).  An entry keeps a copy of the host
 // tensor it was made from -- copies share the storage, so the storage cannot be
 // freed and its address handed to another tensor while the entry lives -- plus a
-// sampled stamp of its bytes.  A role whose tensor arrives with the same storage,
-// shape and stamp reuses the device copy; anything else (moe_weight_provider is an
+// stamp of its bytes (resident_weight.h: a hash of all of them by default).  A role whose
+// tensor arrives with the same storage, shape and stamp reuses the device copy; anything else (moe_weight_provider is an
 // LRU, src/llm/moe_weight_provider.cpp:102-132: an evicted slice comes back in new
 // storage) is uploaded again and the old device copy is freed, so a node never
 // holds more than three device matrices and three host references.
+//
+// With MXFP4 weights the node also takes part in its block's frames (moe_block_context.h):
+// it attaches its three resident matrices and its biases to the context the router tensor
+// leads to, and when a frame's experts are already running on the device and every tensor
+// it is handed is the one it attached, it copies its rows out of the frame instead of
+// computing them again.  A tensor that changed is uploaded and computed here, as before,
+// the frame's merged rows are declared void, and the new copy is attached for the next
+// frame.
 #pragma once
 
 #include <cstring>
@@ -23,6 +31,7 @@
 
 #include "coalsack/nn/nn_op_node.h"
 #include "coalsack/tensor/dynamic_mx_tensor_message.h"
+#include "coalsack/nn/nn_ops/moe_block_context.h"
 #include "coalsack/nn/nn_ops/resident_weight.h"
 #include "coalsack_moe.h"
 
@@ -40,6 +49,7 @@ class expert_mlp_node : public graph_node {
     set_output(output_);
   }
   ~expert_mlp_node() override {
+    detach();
     for (auto& r : resident_) csk_mxfp4_free(r.handle);
     for (auto& r : resident16_) csk_f16_free(r.handle);
   }
@@ -117,6 +127,9 @@ class expert_mlp_node : public graph_node {
 
   // number of device copies made so far (tests: a reload must upload, a repeat must not)
   size_t resident_uploads() const { return uploads_; }
+  // outputs taken from a frame the router node had started / computed by this node itself
+  size_t rows_from_frames() const { return rows_from_frames_; }
+  size_t rows_computed() const { return rows_computed_; }
 
  private:
   enum role { ROLE_UP = 0, ROLE_GATE = 1, ROLE_DOWN = 2 };
@@ -142,12 +155,71 @@ class expert_mlp_node : public graph_node {
     csk_mxfp4* h = nullptr;
     if (csk_mxfp4_upload(t.data_ptr(), t.dim(0), t.dim(1), &h) != CSK_OK)
       throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
-    if (c.handle) csk_mxfp4_free(c.handle);
+    if (c.handle) {
+      detach();  // the view layer must not point at a matrix that is about to be freed
+      csk_mxfp4_free(c.handle);
+    }
     c.handle = h;
     c.held = t;
     c.stamp = stamp;
     ++uploads_;
     return h;
+  }
+
+  // -- the block's frames (moe_block_context.h)
+  struct bias_held {
+    dynamic_tensor t;
+    uint64_t stamp = 0;
+  };
+  void detach() {
+    if (auto ctx = attached_to_.lock()) {
+      std::lock_guard<std::mutex> g(ctx->m);
+      if (ctx->layer) (void)csk_layer_detach_expert(ctx->layer, expert_id_);
+      ctx->frame.experts_running = false;  // (a frame in flight was built on the old matrices)
+    }
+    attached_to_.reset();
+  }
+  // biases as attached: same storage and stamp?
+  bool biases_unchanged(bool has_bias, const dynamic_tensor* b[3]) const {
+    if (has_bias != attached_bias_) return false;
+    if (!has_bias) return true;
+    for (int i = 0; i < 3; ++i)
+      if (b[i]->data_ptr<uint8_t>() != bias_[i].t.data_ptr<uint8_t>() ||
+          csk_resident::content_stamp(b[i]->data_ptr<uint8_t>(), b[i]->bytes()) != bias_[i].stamp)
+        return false;
+    return true;
+  }
+  // Points the context's view layer at this node's matrices (creating the layer when this is
+  // the first expert of the block to arrive) so that the next frame can run here.
+  void attach(const std::shared_ptr<csk_resident::moe_block_context>& ctx, int64_t hidden_dim, int64_t ffn,
+              csk_mxfp4* up, csk_mxfp4* gate, csk_mxfp4* down, bool has_bias, const dynamic_tensor* b[3]) {
+    std::lock_guard<std::mutex> g(ctx->m);
+    if (expert_id_ < 0 || expert_id_ >= ctx->E) return;
+    if (!ctx->layer) {
+      if (csk_layer_create_view(ctx->E, ctx->k, hidden_dim, ffn, &ctx->layer) != CSK_OK) {
+        ctx->layer = nullptr;
+        return;
+      }
+      ctx->H = hidden_dim, ctx->F = ffn;
+      ctx->activation = act_code(), ctx->weight_before_ffn = weight_before_ffn_ ? 1 : 0;
+      ctx->sigmoid = -1;  // the router node passes the options on with its own
+    }
+    if (ctx->H != hidden_dim || ctx->F != ffn) return;
+    // every expert node of a block has the same options; if not, the block has no frames
+    if (ctx->activation != act_code() || ctx->weight_before_ffn != (weight_before_ffn_ ? 1 : 0)) {
+      ctx->activation = ctx->weight_before_ffn = -2;
+      return;
+    }
+    if (csk_layer_attach_expert(ctx->layer, expert_id_, up, gate, down, has_bias ? b[0]->data_ptr<float>() : nullptr,
+                                has_bias ? b[1]->data_ptr<float>() : nullptr,
+                                has_bias ? b[2]->data_ptr<float>() : nullptr) != CSK_OK)
+      return;
+    attached_to_ = ctx;
+    attached_bias_ = has_bias;
+    for (int i = 0; has_bias && i < 3; ++i) {
+      bias_[i].t = *b[i];
+      bias_[i].stamp = csk_resident::content_stamp(b[i]->data_ptr<uint8_t>(), b[i]->bytes());
+    }
   }
 
   struct resident16 {
@@ -303,16 +375,52 @@ class expert_mlp_node : public graph_node {
       throw std::runtime_error("expert_mlp: expert_ffn_dim must be a multiple of 32 for MXFP4, got " +
                                std::to_string(ffn));
 
+    // resident copies of the three matrices (an unchanged tensor costs its stamp)
+    const size_t uploads_before = uploads_;
+    csk_mxfp4* d_up = resident_copy(ROLE_UP, w_up);
+    csk_mxfp4* d_gate = resident_copy(ROLE_GATE, w_gate);
+    csk_mxfp4* d_down = resident_copy(ROLE_DOWN, w_down);
+    const dynamic_tensor* biases[3] = {has_bias ? &b_up->get_tensor() : nullptr,
+                                       has_bias ? &b_gate->get_tensor() : nullptr,
+                                       has_bias ? &b_down->get_tensor() : nullptr};
+
+    // the block's frame, if the router tensor leads to one and it is this (hidden, router) pair
+    auto ctx = csk_resident::moe_block_context::find(rp);
+    bool in_frame = false, frame_running = false;
+    if (ctx) {
+      std::lock_guard<std::mutex> g(ctx->m);
+      in_frame = ctx->frame_matches(hidden, router);
+      frame_running = in_frame && ctx->frame.experts_running;
+    }
+    const bool mine = ctx && attached_to_.lock() == ctx && uploads_ == uploads_before &&
+                      biases_unchanged(has_bias, biases);
     dynamic_tensor output(dtype::float32, hidden.shape());
+    if (frame_running && mine) {
+      // the frame computed this expert from the very matrices and biases handed in now
+      std::lock_guard<std::mutex> g(ctx->m);
+      if (ctx->frame.experts_running && csk_moe_frame_expert_rows(ctx->layer, expert_id_, output.data_ptr<float>()) == CSK_OK) {
+        ctx->frame.emitted[(size_t)expert_id_] = output.data_ptr<float>();
+        ++rows_from_frames_;
+        return output;
+      }
+    }
+    if (frame_running) {
+      // the frame ran on matrices that are not the ones handed in: its merged rows are void
+      std::lock_guard<std::mutex> g(ctx->m);
+      (void)csk_moe_frame_void(ctx->layer);
+    }
     int is_empty = 0;
     const int rc = csk_expert_mlp_mxfp4(
-        expert_id_, hidden.data_ptr<float>(), tokens, hidden_dim, ffn, resident_copy(ROLE_UP, w_up),
-        resident_copy(ROLE_GATE, w_gate), resident_copy(ROLE_DOWN, w_down),
-        has_bias ? b_up->get_tensor().data_ptr<float>() : nullptr,
-        has_bias ? b_gate->get_tensor().data_ptr<float>() : nullptr,
-        has_bias ? b_down->get_tensor().data_ptr<float>() : nullptr, rp, top_k, act_code(),
+        expert_id_, hidden.data_ptr<float>(), tokens, hidden_dim, ffn, d_up, d_gate, d_down,
+        has_bias ? biases[0]->data_ptr<float>() : nullptr, has_bias ? biases[1]->data_ptr<float>() : nullptr,
+        has_bias ? biases[2]->data_ptr<float>() : nullptr, rp, top_k, act_code(),
         weight_before_ffn_ ? 1 : 0, output.data_ptr<float>(), &is_empty);
     if (rc != CSK_OK) throw std::runtime_error(std::string("expert_mlp: ") + csk_last_error());
+    ++rows_computed_;
+    if (in_frame && !mine) {
+      if (attached_to_.lock() != ctx) detach();
+      attach(ctx, hidden_dim, ffn, d_up, d_gate, d_down, has_bias, biases);
+    }
     if (is_empty) return dynamic_tensor(dtype::float32, {0});
     return output;
   }
@@ -326,6 +434,10 @@ class expert_mlp_node : public graph_node {
   resident resident_[3];
   resident16 resident16_[3];
   size_t uploads_ = 0;
+  std::weak_ptr<csk_resident::moe_block_context> attached_to_;
+  bool attached_bias_ = false;
+  bias_held bias_[3];
+  size_t rows_from_frames_ = 0, rows_computed_ = 0;
 };
 
 }  // namespace coalsack

@@ -4,12 +4,14 @@
 // A node keeps one slot per weight role (and per matrix of a batched weight).  A slot
 // remembers the tensor its copy was made from -- the tensor object shares the storage, so
 // that storage cannot be freed and handed out again for other bytes while the slot holds
-// it -- and a stamp of its contents; a tensor with another address, shape, element type or
-// stamp replaces the copy, the old device memory is released.  A node therefore holds a
-// bounded number of device copies whatever the weight provider evicts and reloads.
+// it -- and a stamp of its contents (a hash of every byte unless the host opts for a
+// sampled one, below); a tensor with another address, shape, element type or stamp
+// replaces the copy, the old device memory is released.  A node therefore holds a bounded
+// number of device copies whatever the weight provider evicts and reloads.
 #pragma once
 
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
 #include <stdexcept>
 #include <string>
@@ -20,9 +22,31 @@
 namespace coalsack {
 namespace csk_resident {
 
-// 64 eight-byte samples spread over the buffer, its length and its ends: enough to tell a
-// rewritten or reused buffer from the one a device copy was made from, at no cost that matters
-inline uint64_t content_stamp(const uint8_t* p, size_t n) {
+// How a slot decides that the bytes behind an unchanged address are still the bytes its
+// device copy was made from.
+//   full    (default) every byte is hashed, every frame: exact.  The reference reads its host
+//           weights anew on every frame, so a caller may rewrite a tensor in place between
+//           two frames -- a patched weight, a provider that recycles a slot for another
+//           expert's slice -- and must get the new values.  Costs one pass over the weights
+//           at memory speed (about 0.3 ms per 4.4 MB matrix on one core).
+//   sampled 64 eight-byte samples spread over the buffer, its length and its ends: for hosts
+//           whose weight tensors are never rewritten in place -- the reference's own
+//           moe_weight_provider is one: every load is a fresh tensor, and the slot keeps the
+//           old storage alive, so a new slice cannot appear at an old address.  A rewrite
+//           that misses all the samples goes unnoticed.  Chosen per process with
+//           set_content_check(content_check::sampled) or COALSACK_RESIDENT_CHECK=sampled.
+enum class content_check { full, sampled };
+
+inline content_check& content_check_policy() {
+  static content_check policy = [] {
+    const char* e = std::getenv("COALSACK_RESIDENT_CHECK");
+    return e && std::string(e) == "sampled" ? content_check::sampled : content_check::full;
+  }();
+  return policy;
+}
+inline void set_content_check(content_check c) { content_check_policy() = c; }
+
+inline uint64_t sampled_stamp(const uint8_t* p, size_t n) {
   uint64_t h = 0x9E3779B97F4A7C15ull ^ n;
   auto mix = [&h](uint64_t v) {
     h ^= v + 0x9E3779B97F4A7C15ull + (h << 6) + (h >> 2);
@@ -42,6 +66,32 @@ inline uint64_t content_stamp(const uint8_t* p, size_t n) {
   std::memcpy(&v, p + n - 8, 8);
   mix(v);
   return h;
+}
+
+// Every byte: four independent multiply-xor lanes over 32-byte strides (the lanes keep four
+// multiplications in flight, which is what lets one core run this at memory speed), folded
+// together with the length and the tail.
+inline uint64_t full_hash(const uint8_t* p, size_t n) {
+  uint64_t a = 0x9E3779B97F4A7C15ull ^ n, b = 0xBF58476D1CE4E5B9ull, c = 0x94D049BB133111EBull, d = 0xD6E8FEB86659FD93ull;
+  size_t i = 0;
+  for (; i + 32 <= n; i += 32) {
+    uint64_t v[4];
+    std::memcpy(v, p + i, 32);
+    a = (a ^ v[0]) * 0x9FB21C651E98DF25ull;
+    b = (b ^ v[1]) * 0xC2B2AE3D27D4EB4Full;
+    c = (c ^ v[2]) * 0x165667B19E3779F9ull;
+    d = (d ^ v[3]) * 0x27D4EB2F165667C5ull;
+    a ^= a >> 29, b ^= b >> 31, c ^= c >> 30, d ^= d >> 28;
+  }
+  uint64_t t = 0;
+  for (int sh = 0; i < n; ++i, sh = (sh + 8) & 63) t ^= (uint64_t)p[i] << sh, t *= 0x9E3779B97F4A7C15ull;
+  uint64_t h = a ^ (b << 1 | b >> 63) ^ (c << 2 | c >> 62) ^ (d << 3 | d >> 61) ^ t;
+  h ^= h >> 33, h *= 0xFF51AFD7ED558CCDull, h ^= h >> 33;
+  return h;
+}
+
+inline uint64_t content_stamp(const uint8_t* p, size_t n) {
+  return content_check_policy() == content_check::full ? full_hash(p, n) : sampled_stamp(p, n);
 }
 
 // One [rows, cols] float16 or float32 matrix, `index` matrices into the tensor's data.

@@ -264,6 +264,37 @@ int csk_moe_forward_host(csk_layer* L, const float* hidden, int64_t T, float* ou
  * updated in place. */
 int csk_moe_stack_forward(csk_layer* const* layers, int64_t n_layers, float* hidden_device,
                           int64_t T);
+/* ---- one MoE block behind the reference's node classes (src/llm/llm_engine.cpp:721-753,
+ * include/coalsack/llm/graph_builder.h:289-372: router node -> weight fetch -> one expert
+ * node per expert -> merge node).  The expert nodes own the resident matrices; a view layer
+ * points at them, and a frame runs the block as csk_moe_forward_host does while every node
+ * still emits what the reference's node emits. */
+/* A layer without expert matrices of its own (router, biases and norm as any layer). */
+int csk_layer_create_view(int64_t E, int64_t k, int64_t H, int64_t F, csk_layer** out);
+/* Expert e of a view := these three resident matrices (owned by the caller: detach before
+ * freeing one) and these biases (host pointers, copied; all three or none). */
+int csk_layer_attach_expert(csk_layer* L, int64_t e, const csk_mxfp4* up, const csk_mxfp4* gate,
+                            const csk_mxfp4* down, const float* b_up, const float* b_gate,
+                            const float* b_down);
+int csk_layer_detach_expert(csk_layer* L, int64_t e);
+/* moe_router_node's part (moe_router_node.h:51-124): uploads hidden [T,H] (host), runs router
+ * and dispatch, returns the router output [T,k,2] in pairs_out; if every expert the frame
+ * selects is attached, the experts and the merge are then started on the device and
+ * *experts_running is 1 (else 0: the expert nodes compute on their own, as without a view). */
+int csk_moe_frame_begin(csk_layer* L, const float* hidden, int64_t T, float* pairs_out, int flags,
+                        int* experts_running);
+/* expert_mlp_node's part (expert_mlp_node.h:503-529): into out [T,H] (host, zero-filled by the
+ * caller) the rows of the tokens that selected expert e -- what the node emits.  The first
+ * call of a frame waits for the experts and fetches all rows at once. */
+int csk_moe_frame_expert_rows(csk_layer* L, int64_t e, float* out);
+/* An expert node found that its weights are no longer the attached ones and computed its
+ * output itself: the frame's merged rows must not be used. */
+int csk_moe_frame_void(csk_layer* L);
+/* expert_merge_node's part (expert_merge_node.h:30-134): the merged rows [T,H] of the frame
+ * if its experts ran and nothing voided it (*available = 1), bit-identical to
+ * csk_moe_forward_host; else *available = 0 and out is untouched. */
+int csk_moe_frame_merged(csk_layer* L, float* out, int* available);
+
 /* Intermediate results of the last csk_moe_forward on L, for tests:
  * per-expert token counts [E] and the packed token list (token ids grouped by
  * expert, ascending within an expert) [T*k]. */

@@ -840,12 +840,201 @@ static void gpu_expert_weight_reload() {
       for (int j = 1; j < 17; ++j) up.data_ptr()[17 * b + j] = (uint8_t)byte(gen);
     run_and_check(gate, up, down);
     CHECK(node.resident_uploads() == 6);
+    // one byte flipped in place, at an offset the sampled stamp does not look at: the default
+    // (every byte hashed) sees it and uploads again ...
+    const size_t n = down.size_bytes(), step = (n - 8) / 63;
+    const size_t off = step + 9;  // between the second and the third sample
+    CHECK(step > 24 && off + 1 < 2 * step);
+    down.data_ptr()[off] ^= 0x10;
+    run_and_check(gate, up, down);
+    CHECK(node.resident_uploads() == 7);
+    // ... the sampled stamp, which a host may choose when its weights are never rewritten in
+    // place, does not: that is its stated contract (the result is that of the old bytes)
+    csk_resident::set_content_check(csk_resident::content_check::sampled);
+    run_and_check(gate, up, down);  // the policy changed, so the stamps differ: three uploads
+    CHECK(node.resident_uploads() == 10);
+    down.data_ptr()[off] ^= 0x10;
+    const size_t before = node.resident_uploads();
+    node.process("default", result_message::ok({{"hidden", mk(hidden)},
+                                                {"w_up", std::make_shared<dynamic_mx_tensor_message>(gate)},
+                                                {"w_gate", std::make_shared<dynamic_mx_tensor_message>(up)},
+                                                {"w_down", std::make_shared<dynamic_mx_tensor_message>(down)},
+                                                {"router", mk(router)}}));
+    CHECK(node.resident_uploads() == before);
+    down.data_ptr()[0] ^= 0x01;  // a sampled byte: noticed in either mode
+    run_and_check(gate, up, down);
+    CHECK(node.resident_uploads() == before + 1);
+    csk_resident::set_content_check(csk_resident::content_check::full);
+    run_and_check(gate, up, down);
+    CHECK(node.resident_uploads() == before + 4);
   }  // the caller's references go away (an eviction); the node still holds the storage of its copies
+  const size_t base_uploads = node.resident_uploads();
   for (int round = 0; round < 3; ++round) {  // reloads: fresh storage each time, wherever malloc puts it
     auto up = random_mx(F, H, gen), gate = random_mx(F, H, gen), down = random_mx(H, F, gen);
     run_and_check(up, gate, down);
-    CHECK(node.resident_uploads() == 9 + 3 * (size_t)round);
+    CHECK(node.resident_uploads() == base_uploads + 3 * (size_t)(round + 1));
   }
+}
+
+// One MoE block wired as the engine wires it (llm_engine.cpp:721-753): router node, one
+// expert node per expert, merge node.  From the second frame on the block runs as one fused
+// forward behind the nodes; the nodes' outputs stay what the reference's nodes emit, the
+// merged result equals csk_moe_forward_host bit for bit, and anything that cannot be proved
+// -- a weight rewritten in place, an expert not yet attached, an expert output that did not
+// come from the frame -- takes the per-node path and is right all the same.
+static void gpu_block_frames() {
+  std::printf("block: router + experts + merge share frames; reloads and mixed paths\n");
+  std::mt19937 gen(4242);
+  const int64_t E = 8, K = 2, H = 96, F = 160;
+  auto gate = random_tensor({E, H}, gen, -0.3f, 0.3f), gate_b = random_tensor({E}, gen, -0.05f, 0.05f);
+  std::vector<dynamic_mx_tensor> wu, wg, wd;
+  std::vector<dynamic_tensor> bu, bg, bd;
+  for (int64_t e = 0; e < E; ++e) {
+    wu.push_back(random_mx(F, H, gen)), wg.push_back(random_mx(F, H, gen)), wd.push_back(random_mx(H, F, gen));
+    bu.push_back(random_tensor({F}, gen, -0.01f, 0.01f)), bg.push_back(random_tensor({F}, gen, -0.01f, 0.01f));
+    bd.push_back(random_tensor({H}, gen, -0.01f, 0.01f));
+  }
+  auto mk = [](const dynamic_tensor& t) { return std::make_shared<dynamic_tensor_message>(t); };
+  auto mx = [](const dynamic_mx_tensor& t) { return std::make_shared<dynamic_mx_tensor_message>(t); };
+  moe_router_node router;
+  router.set_config(E, K);
+  router.set_input_names({"hidden", "gate_w", "gate_b"});
+  router.set_output_name("router_out");
+  capture_node rcap;
+  rcap.set_input(router.get_output());
+  std::vector<std::unique_ptr<expert_mlp_node>> experts;
+  std::vector<std::unique_ptr<capture_node>> ecaps;
+  for (int64_t e = 0; e < E; ++e) {
+    experts.emplace_back(new expert_mlp_node((int)e));
+    experts.back()->set_input_names({"hidden", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "router"});
+    experts.back()->set_output_name("out");
+    ecaps.emplace_back(new capture_node);
+    ecaps.back()->set_input(experts.back()->get_output());
+  }
+  expert_merge_node merge;
+  merge.set_config(E, K);
+
+  struct frame_result {
+    dynamic_tensor merged, router_out;
+    std::vector<dynamic_tensor> outs;
+    int active = 0;
+  };
+  // `foreign`: hand the merge node a copy of one live expert output instead of the tensor the node emitted
+  auto run_frame = [&](const dynamic_tensor& hidden, bool foreign = false) {
+    frame_result r;
+    auto hm = mk(hidden);
+    router.process("default", result_message::ok({{"hidden", hm}, {"gate_w", mk(gate)}, {"gate_b", mk(gate_b)}}));
+    auto rm = std::dynamic_pointer_cast<dynamic_tensor_message>(rcap.got.back()->get_field("router_out"));
+    r.router_out = rm->get_tensor();
+    std::vector<dynamic_tensor> merge_in{r.router_out};
+    for (int64_t e = 0; e < E; ++e) {
+      experts[e]->process("default", result_message::ok({{"hidden", hm}, {"w_up", mx(wu[e])}, {"w_gate", mx(wg[e])},
+                                                         {"w_down", mx(wd[e])}, {"b_up", mk(bu[e])},
+                                                         {"b_gate", mk(bg[e])}, {"b_down", mk(bd[e])}, {"router", rm}}));
+      CHECK(ecaps[e]->got.back()->is_ok());
+      auto t = std::dynamic_pointer_cast<dynamic_tensor_message>(ecaps[e]->got.back()->get_field("out"))->get_tensor();
+      r.active += t.numel() != 0;
+      if (foreign && t.numel() != 0) {
+        dynamic_tensor copy(dtype::float32, t.shape());
+        std::memcpy(copy.data_ptr<float>(), t.data_ptr<float>(), t.bytes());
+        t = copy;
+        foreign = false;
+      }
+      merge_in.push_back(t);
+      r.outs.push_back(t);
+    }
+    r.merged = merge.compute_test(merge_in);
+    return r;
+  };
+  // the same block as an ordinary resident layer: what csk_moe_forward_host gives
+  auto fused = [&](const dynamic_tensor& hidden) {
+    csk_layer* L = nullptr;
+    CHECK(csk_layer_create(E, K, H, F, &L) == CSK_OK);
+    CHECK(csk_layer_set_router(L, gate.data_ptr<float>(), gate_b.data_ptr<float>()) == CSK_OK);
+    for (int64_t e = 0; e < E; ++e)
+      CHECK(csk_layer_set_expert(L, e, wu[e].data_ptr(), wg[e].data_ptr(), wd[e].data_ptr(), bu[e].data_ptr<float>(),
+                                 bg[e].data_ptr<float>(), bd[e].data_ptr<float>()) == CSK_OK);
+    dynamic_tensor out(dtype::float32, hidden.shape());
+    CHECK(csk_moe_forward_host(L, hidden.data_ptr<float>(), hidden.dim(0) * hidden.dim(1), out.data_ptr<float>(),
+                               nullptr, 0) == CSK_OK);
+    csk_layer_destroy(L);
+    return out;
+  };
+  auto same_bits = [](const dynamic_tensor& a, const dynamic_tensor& b) {
+    return a.shape() == b.shape() && std::memcmp(a.data_ptr<float>(), b.data_ptr<float>(), a.bytes()) == 0;
+  };
+  auto close = [](const dynamic_tensor& a, const dynamic_tensor& b) {
+    if (a.shape() != b.shape()) return false;
+    float worst = 0, scale = 0;
+    for (int64_t i = 0; i < a.numel(); ++i) {
+      worst = std::fmax(worst, std::fabs(a.data_ptr<float>()[i] - b.data_ptr<float>()[i]));
+      scale = std::fmax(scale, std::fabs(b.data_ptr<float>()[i]));
+    }
+    return worst <= 1e-5f * std::fmax(scale, 1e-6f);
+  };
+  auto rows_from_frames = [&] {
+    size_t n = 0;
+    for (auto& x : experts) n += x->rows_from_frames();
+    return n;
+  };
+
+  // all 8 experts of a 24-token batch are selected: frame 1 is computed node by node and attaches them
+  auto hidden = random_tensor({1, 24, H}, gen, -1, 1);
+  auto f1 = run_frame(hidden);
+  CHECK(f1.active == E);
+  CHECK(router.frames_begun() == 0 && rows_from_frames() == 0 && merge.merges_from_frames() == 0);
+  auto want = fused(hidden);
+  CHECK(close(f1.merged, want));
+  // frame 2: one fused forward behind the nodes
+  auto f2 = run_frame(hidden);
+  CHECK(router.frames_begun() == 1 && router.frames_with_experts() == 1);
+  CHECK(rows_from_frames() == (size_t)E && merge.merges_from_frames() == 1);
+  CHECK(same_bits(f2.merged, want));
+  CHECK(same_bits(f2.router_out, f1.router_out) || close(f2.router_out, f1.router_out));
+  for (int64_t e = 0; e < E; ++e) CHECK(close(f2.outs[e], f1.outs[e]));  // each node still emits its own dense rows
+  // other tokens, fewer of them: some experts may stay unselected ({0}-shaped outputs, as ever)
+  auto hidden3 = random_tensor({1, 3, H}, gen, -1, 1);
+  auto f3 = run_frame(hidden3);
+  CHECK(f3.active <= 6 && merge.merges_from_frames() == 2);
+  CHECK(same_bits(f3.merged, fused(hidden3)));
+  for (int64_t e = 0; e < E; ++e) CHECK((f3.outs[e].numel() == 0) == (f3.outs[e].ndim() == 1));
+  // an expert output that did not come from the frame: the merge node computes on what it was given
+  auto f4 = run_frame(hidden, true);
+  CHECK(merge.merges_from_frames() == 2 && close(f4.merged, want));
+  // a weight rewritten in place between two frames: that node uploads and computes itself, the
+  // frame's merged rows are void, everything follows the new bytes; the next frame is fused again
+  std::uniform_int_distribution<int> byte(0, 255);
+  for (size_t b = 0; b < wu[3].num_blocks(); ++b)
+    for (int j = 1; j < 17; ++j) wu[3].data_ptr()[17 * b + j] = (uint8_t)byte(gen);
+  const size_t before_rows = rows_from_frames(), before_up = experts[3]->resident_uploads();
+  auto f5 = run_frame(hidden);
+  auto want5 = fused(hidden);
+  CHECK(experts[3]->resident_uploads() == before_up + 1 && merge.merges_from_frames() == 2);
+  CHECK(rows_from_frames() < before_rows + (size_t)E);
+  CHECK(close(f5.merged, want5) && !close(f5.merged, want));
+  auto f6 = run_frame(hidden);
+  CHECK(merge.merges_from_frames() == 3 && same_bits(f6.merged, want5));
+  // a bias replaced by another tensor: same story
+  bd[5] = random_tensor({H}, gen, -0.02f, 0.02f);
+  auto f7 = run_frame(hidden);
+  auto want7 = fused(hidden);
+  CHECK(merge.merges_from_frames() == 3 && close(f7.merged, want7));
+  auto f8 = run_frame(hidden);
+  CHECK(merge.merges_from_frames() == 4 && same_bits(f8.merged, want7));
+  // the router's gate rewritten in place: the view layer's copy follows it
+  for (int64_t i = 0; i < gate.numel(); ++i) gate.data_ptr<float>()[i] = -gate.data_ptr<float>()[i];
+  auto f9 = run_frame(hidden);
+  CHECK(merge.merges_from_frames() == 5 && same_bits(f9.merged, fused(hidden)));
+  // an expert node goes away while attached: the block falls back to the per-node path for its experts
+  experts[2].reset(new expert_mlp_node(2));
+  experts[2]->set_input_names({"hidden", "w_up", "w_gate", "w_down", "b_up", "b_gate", "b_down", "router"});
+  experts[2]->set_output_name("out");
+  ecaps[2]->got.clear();
+  ecaps[2]->set_input(experts[2]->get_output());
+  auto f10 = run_frame(hidden);
+  CHECK(merge.merges_from_frames() == 5 && close(f10.merged, fused(hidden)));
+  auto f11 = run_frame(hidden);
+  CHECK(merge.merges_from_frames() == 6 && same_bits(f11.merged, fused(hidden)));
 }
 
 // The router node is handed the same gate tensors every frame and keeps them in device
@@ -948,6 +1137,7 @@ int main(int argc, char** argv) {
     gpu_variant_branches();
     gpu_node_chain();
     gpu_expert_weight_reload();
+    gpu_block_frames();
     gpu_router_gate_reload();
     gpu_norm_add_tests();
     gpu_concurrent_callers();

@@ -141,8 +141,9 @@ CHECKED = {"get_dtype", "shape", "ndim", "dim", "numel", "bytes", "data_ptr", "e
            "get_field", "get_fields", "is_ok", "is_error", "get_error_message", "get_frame_number",
            "set_frame_number", "get_timestamp", "set_timestamp", "send", "get_tensor", "get_mx_tensor"}
 LIBRARY = {"size", "push_back", "emplace_back", "begin", "end", "empty", "data", "what", "resize", "find", "count",
-           "c_str", "back", "reserve", "assign", "clear"}
-OWN = {"get", "split"}
+           "c_str", "back", "reserve", "assign", "clear", "lock", "reset", "expired", "erase"}
+# the nodes' own helpers: resident_weight.h's slots, moe_block_context.h's frame bookkeeping
+OWN = {"get", "split", "frame_matches", "publish", "unpublish", "usable"}
 
 
 def test_nodes_call_nothing_outside_the_checked_surface():
