@@ -6,6 +6,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -370,8 +371,9 @@ int pack_into(const uint8_t* host, csk_mxfp4& m) {
   HIP_TRY(hipMemcpyAsync(&bad, g_bad, sizeof bad, hipMemcpyDeviceToHost, g_stream));
   HIP_TRY(hipStreamSynchronize(g_stream));
   if (bad != ~0ull)
-    return fail(CSK_ERR_SCALE, "MXFP4 scale byte 255 on the non-zero block " + std::to_string(bad) +
-                                   ": its values (codes x 2^127) overflow fp32");
+    return fail(CSK_ERR_SCALE, "MXFP4 scale byte 255 on block " + std::to_string(bad) +
+                                   ", which holds a code of magnitude 1 or more: that value (code x 2^128) "
+                                   "overflows fp32 in the reference's decoding as well");
   return CSK_OK;
 }
 
@@ -628,7 +630,7 @@ int launch_f16_split(const float* x, int64_t rows, int64_t K, const int* gather_
 // y[P, N] <- W_down(expert of the position) x rows + b_down over two-term fp16 rows [P, K]:
 // the down projection of the experts, and any plain linear layer (one descriptor).
 int launch_f16_projection(int64_t E, int64_t T, int64_t P, int64_t K, int64_t N, const uint16_t* rows,
-                          const float* rscale, float* y, Workspace& ws) {
+                          const float* rscale, float* y, Workspace& ws, float wscale = 1.0f) {
   if (T <= 64) {
     ExpertF16Args a{};
     a.desc = ws.desc;
@@ -636,6 +638,7 @@ int launch_f16_projection(int64_t E, int64_t T, int64_t P, int64_t K, int64_t N,
     a.list_row = nullptr;
     a.B = reinterpret_cast<const u32x4*>(rows);
     a.rscale = rscale;
+    a.wscale[0] = a.wscale[1] = wscale;
     a.nkb = (int)f16_block_count(K);
     a.N = (int)N;
     a.ntile = (int)f16_tile_count(N);
@@ -649,6 +652,7 @@ int launch_f16_projection(int64_t E, int64_t T, int64_t P, int64_t K, int64_t N,
     ga.list_row = nullptr;
     ga.B = reinterpret_cast<const u32x4*>(rows);
     ga.rscale = rscale;
+    ga.wscale[0] = ga.wscale[1] = wscale;
     ga.nkb = (int)f16_block_count(K);
     ga.N = (int)N;
     ga.ntile = (int)f16_tile_count(N);
@@ -667,7 +671,8 @@ int launch_f16_projection(int64_t E, int64_t T, int64_t P, int64_t K, int64_t N,
 // [H, 2 F]), so every activation row is contracted twice over.
 int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int act_type,
                     const float* x, bool weight_before_ffn, int64_t gather_rows, Workspace& ws,
-                    bool timed = false, bool identity_rows = false, bool dup = false) {
+                    bool timed = false, bool identity_rows = false, bool dup = false,
+                    const float* wscales = nullptr /* gate, up, down; null: all 1 */) {
   const int64_t P = T * k;
   const int64_t KH = dup ? 2 * H : H, KF = dup ? 2 * F : F;
   int rc = g_f16.ensure((size_t)P, (size_t)F);
@@ -697,6 +702,8 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   const int64_t max_mtiles = P / 64 + std::min<int64_t>(E, P);
   auto gemm_grid = [&](int n_ntiles) { return dim3((unsigned)(cdiv(max_mtiles * n_ntiles, kF16Dies) * kF16Dies)); };
   a.rscale = g_f16.rs_x;
+  a.wscale[0] = wscales ? wscales[0] : 1.0f;
+  a.wscale[1] = wscales ? wscales[1] : 1.0f;
   a.nkb = (int)f16_block_count(KH);
   a.N = (int)F;
   a.ntile = (int)f16_tile_count(F);
@@ -706,6 +713,7 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
     expert_f16_kernel<0><<<grid, 256, 0, g_stream>>>(a);
   } else {
     ga.list_row = a.list_row, ga.B = a.B, ga.rscale = a.rscale, ga.nkb = a.nkb, ga.N = a.N;
+    ga.wscale[0] = a.wscale[0], ga.wscale[1] = a.wscale[1];
     ga.ntile = a.ntile, ga.out = a.out;
     ga.n_ntiles = (int)cdiv(F, 128);
     expert_f16_gemm_kernel<0><<<gemm_grid(ga.n_ntiles), 256, 0, g_stream>>>(ga);
@@ -713,7 +721,7 @@ int run_experts_f16(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F, int a
   if ((rc = check_launch("expert_f16_kernel<0>")) != CSK_OK) return rc;
   if (timed) mark(CSK_STAGE_DOWN);
   if ((rc = launch_f16_split(g_f16.actf, P, KF, nullptr, nullptr, ws.act, g_f16.rs_a, F)) != CSK_OK) return rc;
-  return launch_f16_projection(E, T, P, KF, H, ws.act, g_f16.rs_a, ws.y, ws);
+  return launch_f16_projection(E, T, P, KF, H, ws.act, g_f16.rs_a, ws.y, ws, wscales ? wscales[2] : 1.0f);
 }
 
 int check_dims(int64_t E, int64_t k, int64_t H, int64_t F) {
@@ -1170,6 +1178,7 @@ struct csk_f16 {
   int64_t rows = 0, K = 0;  // K: columns of the resident fp16 matrix
   int64_t Ksrc = 0;         // columns of the matrix the caller gave: K, or K / 2 for fp32 weights kept as [hi | lo]
   bool split() const { return K != Ksrc; }
+  float wscale = 1.0f;      // the resident halves hold w / wscale (a power of two; 1 unless the matrix came in as fp32)
 };
 
 namespace {
@@ -1524,19 +1533,34 @@ extern "C" int csk_f16_upload_f32(const float* w_host, int64_t rows, int64_t K, 
   if (rc == CSK_OK) rc = stage.upload(w_host, (size_t)rows * K * 4);
   if (rc == CSK_OK && !g_bad && counted_malloc((void**)&g_bad, sizeof(unsigned long long)) != hipSuccess)
     rc = fail(CSK_ERR_HIP, "hipMalloc failed");
-  unsigned long long bad = ~0ull;
   if (rc == CSK_OK) {
-    hipError_t e = hipMemsetAsync(g_bad, 0xFF, sizeof(unsigned long long), g_stream);
-    f32_split_pack_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(stage.as<float>(), m->w, rows, K,
-                                                                              ent, g_bad);
+    // largest magnitude first (g_bad's eight bytes serve as the 32-bit cell), then the split of w / wscale
+    const long n = (long)rows * K;
+    unsigned int top = 0u;
+    hipError_t e = hipMemsetAsync(g_bad, 0, sizeof(unsigned long long), g_stream);
+    f32_absmax_bits_kernel<<<dim3((unsigned)std::min<long>(cdiv(n, 256), 8L * std::max(g_cus, 1))), 256, 0, g_stream>>>(
+        stage.as<float>(), n, reinterpret_cast<unsigned int*>(g_bad));
     if (e == hipSuccess) e = hipGetLastError();
-    if (e == hipSuccess) e = hipMemcpyAsync(&bad, g_bad, sizeof bad, hipMemcpyDeviceToHost, g_stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(&top, g_bad, sizeof top, hipMemcpyDeviceToHost, g_stream);
     if (e == hipSuccess) e = hipStreamSynchronize(g_stream);
-    if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("csk_f16_upload_f32: ") + hipGetErrorString(e));
+    if (e != hipSuccess) {
+      rc = fail(CSK_ERR_HIP, std::string("csk_f16_upload_f32: ") + hipGetErrorString(e));
+    } else if (top >= 0x7f800000u) {
+      rc = fail(CSK_ERR_ARG, "csk_f16_upload_f32: the matrix holds a NaN or an infinity");
+    } else {
+      // wscale = 2^s with max|w| / 2^s in [2^14, 2^15); s kept where 2^s and 2^-s are normal numbers
+      const int eb = (int)(top >> 23);
+      const int sexp = top == 0u ? 0 : std::max(-126, std::min(126, eb - 127 - 14));
+      m->wscale = std::ldexp(1.0f, sexp);
+      f32_split_pack_kernel<<<dim3((unsigned)cdiv(ent, 256)), 256, 0, g_stream>>>(stage.as<float>(), m->w, rows, K, ent,
+                                                                                std::ldexp(1.0f, -sexp));
+      rc = check_launch("f32_split_pack_kernel");
+      if (rc == CSK_OK) {
+        e = hipStreamSynchronize(g_stream);  // the staging buffer is released on return
+        if (e != hipSuccess) rc = fail(CSK_ERR_HIP, std::string("csk_f16_upload_f32: ") + hipGetErrorString(e));
+      }
+    }
   }
-  if (rc == CSK_OK && bad != ~0ull)
-    rc = fail(CSK_ERR_ARG, "csk_f16_upload_f32: weight " + std::to_string(bad) +
-                               " is not finite or larger than 65504 in magnitude");
   if (rc != CSK_OK) {
     csk_f16_free(m);
     return rc;
@@ -2246,7 +2270,8 @@ extern "C" int csk_dense_ffn_f16(const float* hidden, int64_t T, int64_t H, int6
     if ((rc = dx.upload(hidden + t0 * H, (size_t)tn * H * 4)) != CSK_OK) return rc;
     dense_desc_kernel<<<1, 256, 0, g_stream>>>(ws.desc, dew.as<ExpertW>(), (int)tn, ws.tiles, ws.n_tiles);
     if ((rc = check_launch("dense_desc_kernel")) != CSK_OK) return rc;
-    rc = run_experts_f16(1, tn, 1, H, F, CSK_ACT_STANDARD_SWIGLU, dx.as<float>(), false, tn, ws, false, true, dup);
+    const float wscales[3] = {w_gate->wscale, w_up->wscale, w_down->wscale};
+    rc = run_experts_f16(1, tn, 1, H, F, CSK_ACT_STANDARD_SWIGLU, dx.as<float>(), false, tn, ws, false, true, dup, wscales);
     if (rc != CSK_OK) return rc;
     CSK_TRY(fetch(out + t0 * H, ws.y, (size_t)tn * H * 4));
     CSK_TRY(finish_fetches());
@@ -2278,7 +2303,7 @@ extern "C" int csk_matmul_transpose_f16(const float* a_host, int64_t M, int64_t 
     dense_desc_kernel<<<1, 256, 0, g_stream>>>(ws.desc, dew.as<ExpertW>(), (int)mn, ws.tiles, ws.n_tiles);
     if ((rc = check_launch("dense_desc_kernel")) != CSK_OK) return rc;
     if ((rc = launch_f16_split(da.as<float>(), mn, K2, nullptr, nullptr, ws.act, g_f16.rs_a, K)) != CSK_OK) return rc;
-    rc = launch_f16_projection(1, mn, mn, K2, N, ws.act, g_f16.rs_a, ws.y, ws);
+    rc = launch_f16_projection(1, mn, mn, K2, N, ws.act, g_f16.rs_a, ws.y, ws, w->wscale);
     if (rc != CSK_OK) return rc;
     CSK_TRY(fetch(out + m0 * N, ws.y, (size_t)mn * N * 4));
     CSK_TRY(finish_fetches());

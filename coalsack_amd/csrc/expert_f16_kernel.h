@@ -55,16 +55,29 @@ __global__ __launch_bounds__(256) void f16_pack_kernel(const uint16_t* __restric
   dst[idx] = u32x4{w[0], w[1], w[2], w[3]};
 }
 
-// Row-major fp32 [rows, K] -> tiles of the fp16 matrix [rows, 2 K] = [hi | lo], hi = fp16(w),
-// lo = fp16(w - hi): the two-term form of an fp32 weight (absolute error below 2^-25 for
-// |w| < 65504), contracted against activation rows that repeat themselves ([x | x], see
-// f16_split_rows_kernel), so that  x . w = x . hi + x . lo  comes out of the fp16 kernels
-// unchanged.  `bad` receives the lowest flat index of a weight whose magnitude is not finite
-// in fp16 (it must hold ~0 on entry).
+// Largest magnitude of an fp32 array, as the bit pattern of |w| (a NaN or an infinity
+// compares above every finite value); *out must hold 0 on entry.
+__global__ __launch_bounds__(256) void f32_absmax_bits_kernel(const float* __restrict__ src, long n,
+                                                              unsigned int* __restrict__ out) {
+  unsigned int m = 0u;
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256)
+    m = max(m, __float_as_uint(src[i]) & 0x7fffffffu);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = max(m, (unsigned int)__shfl_xor((int)m, o, 64));
+  if ((threadIdx.x & 63) == 0 && m != 0u) atomicMax(out, m);
+}
+
+// Row-major fp32 [rows, K] -> tiles of the fp16 matrix [rows, 2 K] = [hi | lo] of w' = w * inv,
+// hi = fp16(w'), lo = fp16(w' - hi): the two-term form of an fp32 weight, contracted against
+// activation rows that repeat themselves ([x | x], see f16_split_rows_kernel), so that
+// x . w' = x . hi + x . lo  comes out of the fp16 kernels unchanged.  inv is the power of two
+// that brings the matrix's largest magnitude into [2^14, 2^15) -- the kernels multiply their
+// sums by its reciprocal (wscale) -- so that hi and lo are normal fp16 numbers for every
+// weight down to 2^-18 of the largest (22 significant bits; below that the absolute error
+// is 2^-39 of the largest weight), whatever the matrix's overall magnitude.
 __global__ __launch_bounds__(256) void f32_split_pack_kernel(const float* __restrict__ src,
                                                              u32x4* __restrict__ dst, long rows, long K,
-                                                             long entries,
-                                                             unsigned long long* __restrict__ bad) {
+                                                             long entries, float inv) {
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= entries) return;
   const long nkb = f16_block_count(2 * K);
@@ -77,8 +90,7 @@ __global__ __launch_bounds__(256) void f32_split_pack_kernel(const float* __rest
     for (int j = 0; j < 8; ++j) {
       const long k = k0 + j;
       if (k >= 2 * K) continue;
-      const float v = src[row * K + (k < K ? k : k - K)];
-      if (!(fabsf(v) <= 65504.0f)) atomicMin(bad, (unsigned long long)(row * K + (k < K ? k : k - K)));
+      const float v = src[row * K + (k < K ? k : k - K)] * inv;
       const _Float16 h = (_Float16)v;
       const _Float16 r = k < K ? h : (_Float16)(v - (float)h);
       w[j >> 1] |= (uint32_t)__builtin_bit_cast(uint16_t, r) << (16 * (j & 1));
@@ -279,6 +291,7 @@ struct ExpertF16Args {
   const int* list_row;   // activation row of a packed position, or null: the position itself
   const u32x4* B;        // two-term fp16 activation rows
   const float* rscale;   // their scales
+  float wscale[2];       // power-of-two scale of the weights: gate and up (MODE 0), down (MODE 1, [0]); 1 for fp16 weights
   int nkb;               // ceil(K / 32)
   int N;                 // output features: F (gate/up) or H (down)
   int ntile;             // ceil(N / 16)
@@ -356,7 +369,8 @@ __global__ __launch_bounds__(256) void expert_f16_kernel(ExpertF16Args a) {
     const int pos_l = base + m0 + min(n16, cnt - 1);
     const long row = a.list_row ? a.list_row[pos_l] : pos_l;
     const CSK_GLOBAL u32x4* Brow = as_global(a.B) + row * a.nkb * 8 + g;
-    const float scale = a.rscale[row];
+    const float scale = a.rscale[row] * a.wscale[0];                          // row scale x weight scale: powers of two
+    const float scale1 = a.rscale[row] * a.wscale[MODE == 0 ? 1 : 0];
     floatx4 acc[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
 
     u32x4 qa[kF16Depth][2], qh[kF16Depth], ql[kF16Depth];
@@ -403,11 +417,11 @@ __global__ __launch_bounds__(256) void expert_f16_kernel(ExpertF16Args a) {
         if (MODE == 0) {
           const int f = 16 * p + 4 * g + i;
           if (f < a.N)
-            a.out[pos * a.N + f] = moe_activation(v[0][i] * scale + b0[f], v[1][i] * scale + b1[f], a.act_type);
+            a.out[pos * a.N + f] = moe_activation(v[0][i] * scale + b0[f], v[1][i] * scale1 + b1[f], a.act_type);
         } else {
           const int h0 = 16 * (2 * p) + 4 * g + i, h1 = h0 + 16;
           if (h0 < a.N) a.out[pos * a.N + h0] = v[0][i] * scale + b0[h0];
-          if (h1 < a.N) a.out[pos * a.N + h1] = v[1][i] * scale + b1[h1];
+          if (h1 < a.N) a.out[pos * a.N + h1] = v[1][i] * scale1 + b1[h1];
         }
       }
     }
@@ -433,6 +447,7 @@ struct ExpertF16GemmArgs {
   const int* list_row;  // activation row of a packed position, or null: the position itself
   const u32x4* B;       // two-term fp16 activation rows
   const float* rscale;
+  float wscale[2];      // as in ExpertF16Args
   int nkb, N, ntile, n_ntiles, act_type;
   float* out;
 };
@@ -574,11 +589,12 @@ __global__ __launch_bounds__(256, 3) void expert_f16_gemm_kernel(ExpertF16GemmAr
     for (int r = 0; r < 16; ++r) {
       const int tl = ms * 32 + (r & 3) + 8 * (r >> 2) + 4 * kg;
       if (tl >= mcount) continue;
-      const float sc_t = rs_sh[tl];
+      const float sc_t = rs_sh[tl] * a.wscale[0];
       float* o = a.out + (long)(base + tl) * a.N;
       if (MODE == 0) {
+        const float sc_u = rs_sh[tl] * a.wscale[1];
         if (rv[0])
-          o[rows[0]] = moe_activation(acc[ms][0][r] * sc_t + bias[0], acc[ms][1][r] * sc_t + bias[1], a.act_type);
+          o[rows[0]] = moe_activation(acc[ms][0][r] * sc_t + bias[0], acc[ms][1][r] * sc_u + bias[1], a.act_type);
       } else {
 #pragma unroll
         for (int s = 0; s < 2; ++s)

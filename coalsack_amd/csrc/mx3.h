@@ -40,13 +40,27 @@ typedef uint32_t u32x6 __attribute__((ext_vector_type(6)));
 __device__ __forceinline__ void mx3_quantize_block(float (&r)[32], u32x4 (&out)[kMx3ChunksPerBlock]) {
 #pragma unroll
   for (int t = 0; t < kMx3Terms; ++t) {
-    float m = 0.0f;
+    uint32_t eb;
+    if (t == 0) {
+      // the maximum of the magnitudes as integers: unlike a floating-point maximum it keeps a
+      // NaN (and an infinity), which then shows as exponent byte 255
+      uint32_t mb = 0u;
 #pragma unroll
-    for (int j = 0; j < 32; ++j) m = fmaxf(m, fabsf(r[j]));
-    const uint32_t eb = (__float_as_uint(m) >> 23) & 0xffu;
-    // block maximum / scale in [4, 8); blocks below 2^-124 are stored as zeros
-    const uint32_t s = eb < 3u ? 127u : min(eb - 2u, 252u);
-    const float sc = __uint_as_float(s << 23);  // 2^(s-127)
+      for (int j = 0; j < 32; ++j) mb = max(mb, __float_as_uint(r[j]) & 0x7fffffffu);
+      eb = mb >> 23;
+    } else {
+      float m = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 32; ++j) m = fmaxf(m, fabsf(r[j]));
+      eb = (__float_as_uint(m) >> 23) & 0xffu;
+    }
+    // block maximum / scale in [4, 8); blocks below 2^-124 are stored as zeros.  A block
+    // that holds a NaN or an infinity gets scale byte 255 on its first term -- the E8M0 NaN,
+    // which the matrix instruction turns into NaN products: every output of that row is then
+    // NaN, as in fp32 arithmetic, instead of a saturated finite value.
+    const bool nonfinite = t == 0 && eb == 255u;
+    const uint32_t s = nonfinite ? 255u : eb < 3u ? 127u : min(eb - 2u, 252u);
+    const float sc = __uint_as_float(min(s, 252u) << 23);  // 2^(s-127)
     f32x16 ev, od;
 #pragma unroll
     for (int j = 0; j < 16; ++j) {

@@ -47,19 +47,24 @@ __device__ __forceinline__ void entry_to_ref_block(uint4 q, uint8_t scale, uint8
   for (int j = 0; j < 16; ++j) blk[1 + j] = (uint8_t)(code[j] | (code[j + 16] << 4));
 }
 
-// True when every code of the block is +0 or -0 (codes 0 and 8): the block is zero
-// whatever its scale byte says.
-__device__ __forceinline__ bool entry_is_zero(const uint4& e) {
-  return ((e.x | e.y | e.z | e.w) & 0x77777777u) == 0u;
+// Every code of the entry is 0 or 0.5 in magnitude (E2M1 codes 0, 1, 8, 9).
+__device__ __forceinline__ bool entry_below_one(const uint4& e) {
+  return ((e.x | e.y | e.z | e.w) & 0x66666666u) == 0u;
+}
+// Such an entry with every magnitude doubled: code 1 (0.5) becomes code 2 (1.0), signs stay.
+__device__ __forceinline__ uint32_t double_small_codes(uint32_t w) {
+  return (w & 0x88888888u) | ((w & 0x11111111u) << 1);
 }
 
 // entries = ntile * nblk * 16
 // Scale bytes: every byte the reference decodes to a finite value is kept as it is
 // (gguf_dequant.h:419-433: 0 and 1 are 2^-128 and 2^-127 on the doubled code table; ggml
-// writes 0 for an all-zero block).  Byte 255 is 2^127 in the reference and "not a number" to
-// the matrix instruction: on a block of zeros it is stored as 254 (the block is zero either
-// way), on any other block the reference's own values overflow fp32 and `bad` receives the
-// lowest such block index (it must hold ~0 on entry).
+// writes 0 for an all-zero block).  Byte 255 is 2^127 on the doubled code table in the
+// reference and "not a number" to the matrix instruction.  Its finite values -- codes 0 and
+// +-0.5, i.e. 0 and +-2^127 -- are stored exactly as byte 254 with the codes doubled (+-0.5
+// becomes +-1); a block that holds any larger code decodes to an infinity in the reference
+// (2 x 2^127 and up overflow fp32) and `bad` receives the lowest such block index (it must
+// hold ~0 on entry).
 __global__ void pack_mxfp4_kernel(const uint8_t* __restrict__ src, uint4* __restrict__ q,
                                   uint8_t* __restrict__ s, int rows, int nblk, long entries,
                                   unsigned long long* __restrict__ bad) {
@@ -77,13 +82,17 @@ __global__ void pack_mxfp4_kernel(const uint8_t* __restrict__ src, uint4* __rest
     return;
   }
   const uint8_t* blk = src + (row * nblk + kb) * 17;
-  const uint4 e = ref_block_to_entry(blk);
-  q[i] = e;
+  uint4 e = ref_block_to_entry(blk);
   uint8_t sb = blk[0];
   if (sb == 255) {
-    if (entry_is_zero(e)) sb = 254;
-    else if (bad) atomicMin(bad, (unsigned long long)(row * nblk + kb));
+    if (entry_below_one(e)) {
+      e = make_uint4(double_small_codes(e.x), double_small_codes(e.y), double_small_codes(e.z), double_small_codes(e.w));
+      sb = 254;
+    } else if (bad) {
+      atomicMin(bad, (unsigned long long)(row * nblk + kb));
+    }
   }
+  q[i] = e;
   s[si] = sb;
 }
 

@@ -39,10 +39,30 @@ __device__ __forceinline__ float wave_max_all(float v) {
 // logits in question in exactly that order and selects again -- so the expert indices
 // and their slot order equal the reference's whenever the inputs are the same, not only
 // when no two logits are close.  Lane s < k returns slot s in (my_val, my_idx).
+//
+// The k experts returned are always distinct and below E, whatever the logits hold -- the
+// dispatch and the one-token launch (k token groups, known before the kernel runs) rely on
+// it.  Retired and out-of-range entries are -inf; the logits compete as max(logit, -FLT_MAX),
+// which turns a NaN or a -inf into the lowest finite key, so that such a logit is still a
+// candidate distinct from the retired ones (among equal keys the lowest index wins).  A token
+// whose logits hold a NaN or +inf, or nothing but -inf, has NaN routing weights in the
+// reference's softmax (moe_router_node.h:176-200: exp(inf - inf), or a NaN sum); which experts
+// its partial sort then returns is unspecified.  Here such a token gets NaN in every slot's value, hence NaN
+// weights, k distinct experts, and no close-call recomputation.
 __device__ __forceinline__ void select_topk(float (&v)[4], int lane, int E, int k, float& my_val,
                                             int& my_idx, float& vmax, bool& close_call, float tol,
                                             float& runner_up) {
   const float NEG = -__builtin_inff();
+  constexpr float kLowest = -3.402823466e+38f;
+  bool bad = false, finite = false;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const bool real = lane + 64 * j < E;
+    bad = bad || (real && !(v[j] <= -kLowest));           // NaN or +inf
+    finite = finite || (real && fabsf(v[j]) <= -kLowest);
+    if (real) v[j] = fmaxf(v[j], kLowest);
+  }
+  const bool poisoned = __any(bad) || !__any(finite);      // (every logit -inf: exp(-inf + inf))
   my_val = 0.0f, my_idx = 0, vmax = 0.0f;
   for (int s = 0; s <= k; ++s) {
     const float best = wave_max_all(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
@@ -74,8 +94,12 @@ __device__ __forceinline__ void select_topk(float (&v)[4], int lane, int E, int 
   const int mv = __float_as_int(my_val);
   const float below = __int_as_float(__builtin_amdgcn_update_dpp(mv, mv, 0x130, 0xf, 0xf, false));
   const bool close = lane < k && lane + 1 < E && (my_val - below) <= tol * fmaxf(1.0f, fabsf(my_val));
-  close_call = __any(close);
+  close_call = __any(close) && !poisoned;
   runner_up = __int_as_float(__builtin_amdgcn_readlane(mv, min(k, E - 1)));
+  if (poisoned) {
+    my_val = __builtin_nanf("");
+    vmax = my_val;
+  }
 }
 
 // Logits in the reference's order: a strictly sequential fp32 sum per logit, multiply and

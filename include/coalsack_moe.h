@@ -34,7 +34,7 @@ extern "C" {
 #define CSK_ERR_HIP 2          /* a HIP runtime call failed                      */
 #define CSK_ERR_RANGE 3        /* expert index outside [0, E)                    */
 #define CSK_ERR_ALL_EMPTY 4    /* merge: every expert tensor is empty            */
-#define CSK_ERR_SCALE 5        /* MXFP4 scale byte 255 on a non-zero block (overflows fp32) */
+#define CSK_ERR_SCALE 5        /* MXFP4 scale byte 255 on a block with a code of magnitude >= 1 (overflows fp32) */
 #define CSK_ERR_STATE 6        /* layer not fully populated                      */
 
 /* expert_mlp_node::activation_type (include/coalsack/nn/nn_ops/expert_mlp_node.h:27-30) */
@@ -115,8 +115,10 @@ int csk_mxfp4_upload(const uint8_t* blocks17_host, int64_t rows, int64_t K, csk_
 void csk_mxfp4_free(csk_mxfp4* m);
 /* Dequantise the resident copy on the GPU into host_out[rows*K]; bit-identical
  * to dequantize_block_mxfp4 (gguf_dequant.h:437-455) for every scale byte the upload
- * accepts: 0..254, and 255 on blocks of zeros (kept as 254: such a block is zero either way,
- * so csk_mxfp4_export returns it with scale byte 254).  Blocks with scale bytes 0 and 1
+ * accepts: 0..254, and 255 on blocks whose codes are all 0 or +-0.5 (the finite values of
+ * that byte, 0 and +-2^127; kept as byte 254 with the codes doubled, which is how
+ * csk_mxfp4_export and csk_layer_export return such a block; any larger code under byte 255
+ * is an infinity in the reference and is refused with CSK_ERR_SCALE).  Blocks with scale bytes 0 and 1
  * hold fp32 denormals (|w| <= 12 * 2^-127); the expert kernels contract them as zeros. */
 int csk_mxfp4_dequant(const csk_mxfp4* m, float* host_out);
 /* Recover the 17-byte blocks from the resident copy (round-trip check). */
@@ -143,12 +145,15 @@ int csk_f16_upload_ggml(int ggml_type, const void* data_host, int64_t rows, int6
 /* The same from a row-major fp32 matrix -- the FLOAT32 weights dense_ffn_node and
  * matmul_transpose_mixed_node also accept (dense_ffn_node.h:57-60, 101-114;
  * matmul_transpose_mixed_node.h:29-31, 91-101).  Kept as two fp16 terms side by side,
- * [rows, 2 K] = [fp16(w) | fp16(w - fp16(w))] (absolute error below 2^-25; |w| <= 65504), and
- * contracted against each activation row twice over, so the fp16 kernels serve both kinds.
- * Accepted by csk_dense_ffn_f16 and csk_matmul_transpose_f16. */
+ * [rows, 2 K] = [fp16(w') | fp16(w' - fp16(w'))] with w' = w / 2^s, one power of two per
+ * matrix that brings its largest magnitude into [2^14, 2^15) and that the kernels multiply
+ * back into their sums: 22 significant bits for every weight down to 2^-18 of the largest,
+ * whatever the magnitude of the matrix.  Contracted against each activation row twice
+ * over, so the fp16 kernels serve both kinds.  Any finite fp32 is accepted; a NaN or an
+ * infinity is refused.  Accepted by csk_dense_ffn_f16 and csk_matmul_transpose_f16. */
 int csk_f16_upload_f32(const float* w_host, int64_t rows, int64_t K, csk_f16** out);
-/* Recover the row-major halves from the resident copy (round-trip check); [rows, 2 K] for a
- * matrix that came in as fp32. */
+/* Recover the row-major halves from the resident copy (round-trip check); [rows, 2 K] (the
+ * two terms of w / 2^s) for a matrix that came in as fp32. */
 int csk_f16_export(const csk_f16* m, uint16_t* halves_host);
 
 /* ---- one MoE layer, weights resident ------------------------------------ */

@@ -331,11 +331,44 @@ def test_matmul_transpose_float32_weight_matches_oracle(lib, oracle, M, K, N):
         lib.matmul_transpose_f16(a[:, :K - 1] if K > 1 else a, w)
 
 
-def test_float32_weight_upload_refuses_what_two_halves_cannot_hold(lib):
+@pytest.mark.parametrize("scale", [1e-6, 1e5, 3e-30, 1e30])
+def test_float32_weights_of_any_magnitude(lib, oracle, scale):
+    """fp32 weights far outside the fp16 range (matmul_transpose_mixed_node.h:83-92 and
+    dense_ffn_node.h:102-113 take any fp32): the matrix travels as two fp16 terms of
+    w / 2^s, 2^s chosen per matrix, so tiny and huge weights keep the same relative accuracy
+    as weights of order one."""
+    rng = np.random.default_rng(int(abs(np.log10(scale))))
+    M, K, N = 9, 160, 96
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = (rng.standard_normal((N, K)) * scale).astype(np.float32)
+    got = lib.matmul_transpose_f16(a, w)
+    want = oracle.matmul_transpose_f32(a, w)
+    ref = a.astype(np.float64) @ w.astype(np.float64).T
+    assert np.abs(got - want).max() <= 1e-3 * np.abs(want).max()
+    assert np.abs(got - ref).max() <= 2e-5 * np.abs(ref).max()
+    if 1e-6 <= scale <= 1e5:
+        # dense FFN: gate and up of one magnitude, down of its inverse, so the three scales differ
+        T, H, F = 5, 64, 96
+        hidden = rng.standard_normal((T, H)).astype(np.float32)
+        w_gate = (rng.standard_normal((F, H)) * scale).astype(np.float32)
+        w_up = (rng.standard_normal((F, H)) * 0.1).astype(np.float32)
+        w_down = (rng.standard_normal((H, F)) / scale).astype(np.float32)
+        got = lib.dense_ffn_f16(hidden, w_gate, w_up, w_down, None, None, None)
+        want = oracle.dense_ffn_f32(hidden, w_gate, w_up, w_down, None, None, None)
+        x = hidden.astype(np.float64)
+        g = x @ w_gate.astype(np.float64).T
+        u = x @ w_up.astype(np.float64).T
+        with np.errstate(over="ignore"):
+            ref = (g / (1 + np.exp(-g)) * u) @ w_down.astype(np.float64).T
+        assert np.abs(got - want).max() <= 1e-3 * np.abs(want).max()
+        assert np.abs(got - ref).max() <= 2e-5 * np.abs(ref).max()
+
+
+def test_float32_weight_upload_refuses_non_finite_weights(lib):
     w = np.ones((4, 8), np.float32)
-    w[2, 3] = 1e6
-    with pytest.raises(capi.CskError, match="weight 19 is not finite or larger than 65504"):
-        lib.f16_upload_f32(w)
-    w[2, 3] = np.nan
-    with pytest.raises(capi.CskError, match="weight 19"):
-        lib.f16_upload_f32(w)
+    w[2, 3] = 1e6   # beyond fp16 by itself: fine, the matrix is scaled
+    lib.f16_free(lib.f16_upload_f32(w))
+    for bad in (np.nan, np.inf, -np.inf):
+        w[2, 3] = bad
+        with pytest.raises(capi.CskError, match="holds a NaN or an infinity"):
+            lib.f16_upload_f32(w)

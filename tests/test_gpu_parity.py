@@ -48,21 +48,28 @@ def test_dequant_every_scale_and_code(lib, oracle):
         lib.mxfp4_free(h)
 
 
-def test_scale_byte_255_only_on_zero_blocks(lib):
-    """2^127 times a non-zero code overflows fp32 in the reference itself: refused.  On a
-    block of zeros (codes 0 and 8) any scale byte is accepted; 255 is kept as 254."""
+def test_scale_byte_255_finite_values_exact_larger_codes_refused(lib, oracle):
+    """Scale byte 255 is 2^127 on the doubled code table (gguf_dequant.h:419-433): codes 0 and
+    +-0.5 decode to 0 and +-2^127, bit for bit as the oracle does; the resident copy keeps
+    them as byte 254 with the codes doubled, which is what the export returns.  Any larger
+    code overflows fp32 in the reference itself: refused."""
     blk = np.zeros(17, np.uint8)
     blk[0] = 255
-    blk[1:] = [0x00, 0x08, 0x80, 0x88] * 4
+    blk[1:] = [0x00, 0x08, 0x80, 0x88, 0x01, 0x10, 0x91, 0x19] * 2
+    want = oracle.dequant(blk, 32)
+    assert np.all(np.isfinite(want)) and np.abs(want).max() == 2.0 ** 127
     h = lib.mxfp4_upload(blk, 1, 32)
     try:
-        assert np.all(lib.mxfp4_dequant(h, 1, 32) == 0)
+        got = lib.mxfp4_dequant(h, 1, 32).reshape(-1)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
         back = lib.mxfp4_export(h, 1, 32)
-        assert back[0] == 254 and np.array_equal(back[1:], blk[1:])
+        assert back[0] == 254
+        assert np.array_equal(back[1:], [0x00, 0x08, 0x80, 0x88, 0x02, 0x20, 0xA2, 0x2A] * 2)
+        assert np.array_equal(oracle.dequant(back, 32).view(np.uint32), want.view(np.uint32))
     finally:
         lib.mxfp4_free(h)
-    blk[5] = 0x10
-    with pytest.raises(capi.CskError, match="overflow fp32") as ei:
+    blk[5] = 0x20
+    with pytest.raises(capi.CskError, match="overflows fp32") as ei:
         lib.mxfp4_upload(blk, 1, 32)
     assert ei.value.code == capi.ERR_SCALE
 
@@ -141,6 +148,34 @@ def test_router_matches_oracle(lib, oracle, T, H, E, k, bias, sigmoid):
     # weights inherit the difference between the two fp32 summation orders of the logits
     assert np.max(np.abs(got[same, :, 1] - want[same, :, 1])) <= ROUTING_WEIGHT_TOL
     assert np.all(got[..., 1] > 0) and np.allclose(got[..., 1].sum(axis=1), 1.0, atol=1e-5) or sigmoid
+
+
+@pytest.mark.parametrize("T,E,k", [(1, 8, 4), (3, 8, 8), (20, 32, 4), (100, 128, 4), (300, 7, 3)])
+def test_router_nonfinite_logits_still_select_k_distinct_experts(lib, oracle, T, E, k):
+    """Tokens whose logits are NaN, +inf or -inf: the k experts returned are distinct and in
+    range (the dispatch relies on it), the weights are NaN where the reference's softmax
+    gives NaN (moe_router_node.h:176-200), and the other tokens of the batch are untouched."""
+    H = 64
+    rng = np.random.default_rng(E * 100 + T)
+    h = rng.normal(0, 1, (T, H)).astype(np.float32)
+    g = rng.normal(0, 0.05, (E, H)).astype(np.float32)
+    g[:, 3] = np.abs(g[:, 3]) + 0.01          # column 3 positive: an infinity there drives every logit to it
+    b = rng.normal(0, 0.01, E).astype(np.float32)
+    clean = lib.moe_router(h, g, b, k)
+    kinds = {0: np.nan, T // 2: np.inf, T - 1: -np.inf}
+    for t, v in kinds.items():
+        h[t, 3] = v
+    got = lib.moe_router(h, g, b, k)
+    with np.errstate(all="ignore"):
+        want = oracle.router(h, g, b, k)
+    for t in range(T):
+        ids = got[t, :, 0].astype(int)
+        assert len(set(ids.tolist())) == k and ids.min() >= 0 and ids.max() < E, (t, ids)
+        if t in kinds:
+            assert np.all(np.isnan(want[t, :, 1])), "oracle weights finite?"
+            assert np.all(np.isnan(got[t, :, 1])), (t, got[t])
+        else:
+            assert np.array_equal(got[t], clean[t])
 
 
 @pytest.mark.parametrize("T,bias", [(1, True), (16, False), (300, True)])
@@ -441,6 +476,32 @@ def test_layer_config2_20b_decode_sweep(lib, oracle, T):
 def test_layer_decode_sweep_small_shape(lib, oracle, T):
     L = synth.LayerInputs(32, 4, 256, 192, seed=5)
     _check_layer(lib, oracle, L, T)
+
+
+@pytest.mark.parametrize("T", [1, 9, 150])
+def test_layer_nan_and_inf_tokens_propagate(lib, oracle, T):
+    """A NaN or an infinity in a token's hidden state comes out as a non-finite output row,
+    as in the reference's fp32 arithmetic (expert_mlp_node.h:651-732 has no clamp), in the
+    streaming and in the grouped-GEMM regime; the other tokens of the batch still match the
+    oracle.  (Which experts a token with NaN logits selects is unspecified in the reference
+    -- its partial sort compares NaNs -- so only finiteness is compared for those rows.)"""
+    L = synth.LayerInputs(8, 2, 128, 160, seed=9)
+    hidden = synth.hidden_states(T, L.H, seed=T + 3)
+    bad_nan, bad_inf = 0, (T - 1 if T > 1 else None)
+    hidden[bad_nan, 37] = np.nan
+    if bad_inf is not None:
+        hidden[bad_inf, 5] = np.inf
+    with build_layer(lib, L) as layer:
+        got = layer.forward(hidden, 0)
+    with np.errstate(all="ignore"):
+        want, _ = oracle_layer(oracle, L, hidden)
+    bad = [bad_nan] + ([bad_inf] if bad_inf is not None else [])
+    for t in bad:
+        assert not np.any(np.isfinite(want[t])), "oracle row finite?"
+        assert not np.any(np.isfinite(got[t])), (t, got[t][:8])
+    good = [t for t in range(T) if t not in bad]
+    if good:
+        assert_layer_close(got[good], want[good])
 
 
 @pytest.mark.parametrize("opts", [dict(act=1), dict(sigmoid=True), dict(weight_before_ffn=True),
