@@ -489,7 +489,7 @@ int launch_dispatch(const int* ids, const float* pairs, int64_t P, int64_t k, in
 
 // Weight-streaming kernel for small batches (every expert sees few tokens, the
 // layer is HBM-bound); grouped GEMM otherwise.
-template <int NMAT, int G>
+template <int NMAT, int G, bool ROUTE1 = false>
 int launch_stream(ExpertStreamArgs a, int64_t P, Workspace& ws) {
   a.groups = ws.groups;
   a.nv = ws.nv;
@@ -499,23 +499,27 @@ int launch_stream(ExpertStreamArgs a, int64_t P, Workspace& ws) {
   const int64_t cus = std::max(g_cus, 1);
   const int64_t nwg = (G == kStreamG && P * npair <= kStreamWgPerCu * cus) ? P * npair : kStreamWgPerCu * cus;  // (small P implies G == kStreamG)
   // activation rows as three FP6 terms (96 B per block, 96 blocks per row: zeros past K) + the reduction buffers
-  const size_t lds = (size_t)G * 96 * (kMx3ChunksPerBlock * 16) + (size_t)2 * 4 * ((G + 3) / 4) * 8 * 16 * sizeof(float);
+  size_t lds = (size_t)G * 96 * (kMx3ChunksPerBlock * 16) + (size_t)2 * 4 * ((G + 3) / 4) * 8 * 16 * sizeof(float);
+  if (ROUTE1) lds = std::max(lds, sizeof(CloseCallLds));  // a close call is recomputed where the rows go afterwards
   static bool lds_attr_set = false;  // per instantiation: dynamic LDS beyond the default limit is asked for once
   if (!lds_attr_set) {
-    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&expert_stream_kernel<NMAT == 2 ? 0 : 1, G>),
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(&expert_stream_kernel<NMAT == 2 ? 0 : 1, G, ROUTE1>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     lds_attr_set = true;
   }
-  launch_expert_kernel(NMAT == 2 ? 0 : 1, expert_stream_kernel<NMAT == 2 ? 0 : 1, G>, dim3((unsigned)nwg), dim3(256), lds, a);
+  launch_expert_kernel(NMAT == 2 ? 0 : 1, expert_stream_kernel<NMAT == 2 ? 0 : 1, G, ROUTE1>, dim3((unsigned)nwg), dim3(256), lds, a);
   return check_launch("expert_stream_kernel");
 }
 
 template <int NMAT>
 int launch_experts(ExpertStreamArgs a, const uint16_t* a_mx3, uint16_t* act_mx3, int64_t E, int64_t T, int64_t P,
                    Workspace& ws, bool stream) {
-  if (stream)
+  if (stream) {
+    if constexpr (NMAT == 2)
+      if (a.rin.logits) return launch_stream<NMAT, kStreamG, true>(a, P, ws);  // one token, routed by the kernel itself
     return stream_group_tokens(T) == kStreamG ? launch_stream<NMAT, kStreamG>(a, P, ws)
                                               : launch_stream<NMAT, kStreamGWide>(a, P, ws);
+  }
   ExpertGemmMxArgs ga{};
   ga.desc = a.desc;
   ga.mtiles = ws.tiles;
@@ -558,6 +562,8 @@ struct ExpertInput {
   const float* gather_w;
   const uint16_t* x_mx3;
   const int* mx3_list_row;
+  const RouteIn* rin = nullptr;    // both set: a one-token batch that the gate/up kernel routes itself
+  const RouteOut* rout = nullptr;
 };
 
 // Experts' MLPs over the dispatched tokens: ws.y[P,H] <- down(act(gate, up)).
@@ -580,8 +586,13 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   a.act_out = reinterpret_cast<float*>(ws.act);  // [P][F] fp32 (streaming) or three-term rows (GEMM), same bytes
   a.y_out = nullptr;
   if (timed) mark(CSK_STAGE_GATEUP);
+  if (in.rin && in.rout) {
+    if (!stream || T != 1) return fail(CSK_ERR_STATE, "in-kernel routing is for one token on the streaming path");
+    a.rin = *in.rin, a.rout = *in.rout;
+  }
   int rc = launch_experts<2>(a, in.x_mx3, ws.act, E, T, P, ws, stream);
   if (rc != CSK_OK) return rc;
+  a.rin = RouteIn{}, a.rout = RouteOut{};
   if (timed) mark(CSK_STAGE_DOWN);
   // down
   a.list_row = nullptr;
@@ -1655,6 +1666,9 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
   const int64_t P = T * L->k;
   const bool norm = (flags & CSK_FWD_RMSNORM) != 0;
   const float* xr = norm ? ws.xn : hidden;
+  bool route_in_kernel = false;
+  RouteIn rin_kept{};
+  RouteOut rout_kept{};
   if (phase == 2) {
     // routed already
   } else if (P <= 1024 && T <= 64) {
@@ -1676,7 +1690,12 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
                 (int)T, (int)L->E, (int)L->k, (int)L->H, L->sigmoid, stream_group_tokens(T)};
     RouteOut rout{ws.pairs, ws.ids, ws.pos, ws.counts, ws.offsets, ws.desc, ws.groups, ws.nv,
                   ws.tiles, ws.n_tiles, ws.list_tok, ws.list_w};
-    if (T <= kRouteTinyTokens && P <= kRouteTinyMaxP && !L->f16 && stream_path(T, L->H, L->F, L->E, L->k)) {
+    if (T == 1 && phase == 0 && L->E > 1 && !L->f16 && stream_path(T, L->H, L->F, L->E, L->k)) {
+      // one token: the gate/up kernel routes it itself (no launch here); phases keep the
+      // routing kernel, whose output they hand out before the experts run
+      route_in_kernel = true;
+      rin_kept = rin, rout_kept = rout;
+    } else if (T <= kRouteTinyTokens && P <= kRouteTinyMaxP && !L->f16 && stream_path(T, L->H, L->F, L->E, L->k)) {
       // a handful of tokens on the streaming kernels: each active expert is one token group
       route_tiny_kernel<<<dim3(1), 256, 0, g_stream>>>(rin, rout);
       if ((rc = check_launch("route_tiny_kernel")) != CSK_OK) return rc;
@@ -1730,6 +1749,7 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
   // grouped GEMM: rows written as three FP6 terms beforehand (per token, or gathered and
   // pre-scaled per dispatch position when the routing weight goes in front of the FFN)
   ExpertInput in{xr, ws.list_tok, L->wbf ? ws.list_w : nullptr, ws.xs, ws.list_tok};
+  if (route_in_kernel) in.rin = &rin_kept, in.rout = &rout_kept;
   if (L->wbf && !stream_path(T, L->H, L->F, L->E, L->k)) {
     if ((rc = launch_mx3(xr, ws.xg, P, L->H, ws.list_tok, ws.list_w)) != CSK_OK) return rc;
     in.x_mx3 = ws.xg;

@@ -16,6 +16,7 @@
 #pragma once
 #include "common.h"
 #include "mx3.h"
+#include "route_select.h"
 
 namespace csk {
 
@@ -36,6 +37,8 @@ struct ExpertStreamArgs {
   int act_type;
   float* act_out;        // gate/up: [P][N] fp32
   float* y_out;          // down: [P][N] fp32
+  RouteIn rin;           // ROUTE1 form only: what the token is routed from ...
+  RouteOut rout;         // ... and where workgroup 0 leaves the router's output and the lists
 };
 
 // exp and the reciprocal are the hardware's own approximations (v_exp_f32 on x log2 e,
@@ -89,8 +92,19 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t stream_plane_rsrc(const void* 
   return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(((uint64_t)hi << 32) | lo), 0, 0x7fffffff, 0x00020000);
 }
 
-template <int MODE, int G>
+//
+// ROUTE1 (gate/up of a one-token batch): there is no routing kernel in front.  Every
+// workgroup selects the token's k experts itself from the logits (select_topk on wave 0,
+// a close call recomputed by the whole workgroup, exactly as route_tiny_kernel does: all
+// workgroups compute the same thing from the same inputs) and takes the expert whose rank
+// among the selected ones is its team's number -- that rank is the expert's packed position,
+// as the dispatch would have numbered it.  Workgroup 0 also writes what the routing kernel
+// would have written (pairs, ids, positions, lists, counts, token groups) for the down
+// kernel, the combine and csk_layer_last_dispatch.  A launch and its dependent reads
+// (5.4 us) are replaced by about a microsecond in front of the first weight loads.
+template <int MODE, int G, bool ROUTE1 = false>
 __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs a) {
+  static_assert(!ROUTE1 || MODE == 0, "the gate/up kernel is the one that routes");
   constexpr int NS = 6;  // K steps per wave: 4 waves x 6 x 128 = 3072 elements
   constexpr int NV = 8;  // accumulator floats per lane per unit
   extern __shared__ __align__(16) unsigned char smem[];
@@ -115,6 +129,76 @@ __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs 
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
 
+  // ROUTE1: slot s of the token in lane s of every wave (all four waves select, from the same
+  // logits, so that nothing has to be handed from wave to wave)
+  int r_idx = 0;
+  float r_wt = 0.0f;
+  constexpr int kEwWords = kMaxExperts * (int)(sizeof(ExpertW) / 8), kEwPerThread = (kEwWords + 255) / 256;
+  __shared__ unsigned long long s_ew[ROUTE1 ? kEwWords : 1];  // the experts' weight pointers, staged beside the logits
+  if constexpr (ROUTE1) {
+    const RouteIn& r = a.rin;
+    const RouteOut& o = a.rout;
+    const int E = r.E, k = r.k;
+    // the recomputation's staging area lies where the activation rows go afterwards
+    CloseCallLds& cc = *reinterpret_cast<CloseCallLds*>(smem);
+    const float NEG = -__builtin_inff();
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = lane + 64 * j;
+      v[j] = e < E ? r.logits[e] : NEG;
+    }
+    unsigned long long ew_reg[kEwPerThread];
+#pragma unroll
+    for (int i = 0; i < kEwPerThread; ++i) {
+      const int w = threadIdx.x + i * 256;
+      ew_reg[i] = w < E * (int)(sizeof(ExpertW) / 8) ? reinterpret_cast<const unsigned long long*>(r.ew)[w] : 0ull;
+    }
+    float my_val, vmax, runner_up;  // lane s keeps slot s
+    bool close_call;
+    const float tol = close_call_tolerance(r.H);
+    select_topk(v, lane, E, k, my_val, r_idx, vmax, close_call, tol, runner_up);
+#pragma unroll
+    for (int i = 0; i < kEwPerThread; ++i) {
+      const int w = threadIdx.x + i * 256;
+      if (w < kEwWords) s_ew[w] = ew_reg[i];
+    }
+    if (close_call) {  // the same in every wave, and in every workgroup
+      const float thr = runner_up - 2.0f * tol * fmaxf(1.0f, fabsf(runner_up));
+      logits_reference_order_wg<256>(r.x, r.g, r.b, r.logits, E, r.H, thr, cc);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int e = lane + 64 * j;
+        v[j] = e < E ? cc.fixed[e] : NEG;
+      }
+      select_topk(v, lane, E, k, my_val, r_idx, vmax, close_call, 0.0f, runner_up);
+    }
+    r_wt = routing_weight(my_val, vmax, lane, k, r.sigmoid);
+    __syncthreads();  // the pointer table is in LDS; every thread is done with cc before the activation rows overwrite it
+    if (blockIdx.x == 0) {
+      // what the routing kernel would have written
+      __shared__ int w_ids[kMaxTopK];
+      if (wv == 0 && lane < k) w_ids[lane] = r_idx;
+      __syncthreads();
+      for (int e = threadIdx.x; e < E; e += 256) {
+        int c = 0;
+        for (int q = 0; q < k; ++q) c += w_ids[q] == e;
+        o.counts[e] = c;
+      }
+      if (wv == 0 && lane < k) {
+        int pos = 0;
+        for (int q = 0; q < k; ++q) pos += w_ids[q] < r_idx;  // the k experts are distinct
+        reinterpret_cast<float2*>(o.pairs)[lane] = make_float2((float)r_idx, r_wt);
+        o.ids[lane] = r_idx;
+        o.list_tok[pos] = 0;
+        o.list_w[pos] = r_wt;
+        o.pos_of_slot[lane] = pos;
+        write_stream_group(o.groups + pos, reinterpret_cast<const ExpertW*>(s_ew) + r_idx, r_idx, 1, pos);
+      }
+      if (threadIdx.x == 0) *o.nv = k;
+    }
+  }
+
   struct WSet {
     u32x4 q[NS][2];
     u32x2 sc[2];  // this wave's scale bytes of the two tiles, one byte per K step
@@ -125,18 +209,30 @@ __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs 
   for (int v = team; v < nvv; v += teams) {
     const int p_begin = tj, p_end = npair;
     const StreamGroup* gr = a.groups + v;
-    const int gcount = min(G, gr->left);
-    const int base = gr->base;
+    int r_e = 0;
+    float r_gw = 1.0f;
+    if constexpr (ROUTE1) {  // the selected expert with v selected experts below it: packed position v
+      const int k = a.rin.k;
+      int lower = 0;
+      for (int q = 0; q < k; ++q) lower += __builtin_amdgcn_readlane(r_idx, q) < r_idx;
+      const unsigned long long mine = __ballot(lane < k && lower == v);
+      const int sl = (int)__builtin_ctzll(mine | (1ull << 63));
+      r_e = __builtin_amdgcn_readlane(r_idx, sl);
+      r_gw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(r_wt), sl));
+    }
+    const ExpertW* gw_ptr = ROUTE1 ? reinterpret_cast<const ExpertW*>(s_ew) + r_e : &gr->w;
+    const int gcount = ROUTE1 ? 1 : min(G, gr->left);
+    const int base = ROUTE1 ? v : gr->base;
     // One buffer descriptor per weight plane: the unit's tile and the K step go into the
     // scalar offset of a load, the lane's place within the step (block g, row n) into its
     // vector offset, which never changes.
-    const auto q_rsrc0 = stream_plane_rsrc(MODE == 0 ? gr->w.q_gate : gr->w.q_down);
-    const auto q_rsrc1 = stream_plane_rsrc(MODE == 0 ? gr->w.q_up : gr->w.q_down);
+    const auto q_rsrc0 = stream_plane_rsrc(MODE == 0 ? gw_ptr->q_gate : gw_ptr->q_down);
+    const auto q_rsrc1 = stream_plane_rsrc(MODE == 0 ? gw_ptr->q_up : gw_ptr->q_down);
     const uint32_t qoff = (uint32_t)((g * 16 + n) * 16);
-    const CSK_GLOBAL u32x2* s0 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? gr->w.s_gate : gr->w.s_down)) + wv * 64 + lane;
-    const CSK_GLOBAL u32x2* s1 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? gr->w.s_up : gr->w.s_down)) + wv * 64 + lane;
-    const CSK_GLOBAL float* bp0 = as_global(MODE == 0 ? gr->w.b_gate : gr->w.b_down);
-    const CSK_GLOBAL float* bp1 = as_global(MODE == 0 ? gr->w.b_up : gr->w.b_down);
+    const CSK_GLOBAL u32x2* s0 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? gw_ptr->s_gate : gw_ptr->s_down)) + wv * 64 + lane;
+    const CSK_GLOBAL u32x2* s1 = as_global(reinterpret_cast<const u32x2*>(MODE == 0 ? gw_ptr->s_up : gw_ptr->s_down)) + wv * 64 + lane;
+    const CSK_GLOBAL float* bp0 = as_global(MODE == 0 ? gw_ptr->b_gate : gw_ptr->b_down);
+    const CSK_GLOBAL float* bp1 = as_global(MODE == 0 ? gw_ptr->b_up : gw_ptr->b_down);
 
     // tiles of a unit: (R, R) for gate/up, (2R, 2R+1) for down.
     // `idle`: a refill whose data nobody will use (past the workgroup's last unit).  It is
@@ -171,7 +267,7 @@ __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs 
     {
       const int rr = threadIdx.x / lrb, kb = threadIdx.x - rr * lrb;
       if ((int)threadIdx.x < nfill && kb < nblk) {
-        const int row = a.list_row ? a.list_row[base + rr] : base + rr;
+        const int row = ROUTE1 ? 0 : a.list_row ? a.list_row[base + rr] : base + rr;
         const float4* src = reinterpret_cast<const float4*>(a.X + ((size_t)row * nblk + kb) * 32);
 #pragma unroll
         for (int i = 0; i < 8; ++i) pre[i] = src[i];
@@ -199,7 +295,7 @@ __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs 
       } else {
         float r[32];
         if (idx != (int)threadIdx.x) {  // later blocks of this thread: fetched here
-          const int row = a.list_row ? a.list_row[base + rr] : base + rr;
+          const int row = ROUTE1 ? 0 : a.list_row ? a.list_row[base + rr] : base + rr;
           const float4* src = reinterpret_cast<const float4*>(a.X + ((size_t)row * nblk + kb) * 32);
 #pragma unroll
           for (int i = 0; i < 8; ++i) pre[i] = src[i];
@@ -207,7 +303,7 @@ __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs 
 #pragma unroll
         for (int i = 0; i < 8; ++i) r[4 * i] = pre[i].x, r[4 * i + 1] = pre[i].y, r[4 * i + 2] = pre[i].z, r[4 * i + 3] = pre[i].w;
         if (a.gather_w) {
-          const float gw = a.gather_w[base + rr];
+          const float gw = ROUTE1 ? r_gw : a.gather_w[base + rr];  // (the list of weights is being written by workgroup 0)
 #pragma unroll
           for (int i = 0; i < 32; ++i) r[i] = r[i] * gw;
         }

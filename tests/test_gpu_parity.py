@@ -515,6 +515,22 @@ def test_layer_variants(lib, oracle, opts):
     _check_layer(lib, oracle, L, 21, bias=bias, norm=norm, residual=residual, **opts)
 
 
+@pytest.mark.parametrize("opts", [dict(), dict(act=1), dict(sigmoid=True), dict(weight_before_ffn=True),
+                                  dict(bias=False), dict(norm=True, residual=True),
+                                  dict(weight_before_ffn=True, sigmoid=True, norm=True, residual=True)])
+@pytest.mark.parametrize("shape", [(8, 2, 128, 160), (128, 4, 256, 192), (5, 5, 64, 96), (200, 16, 96, 64)])
+def test_layer_one_token_variants(lib, oracle, opts, shape):
+    """One token: the gate/up kernel selects the experts itself (no routing launch in front);
+    every option of the layer, few and many experts, top_k = E and the largest top_k."""
+    opts = dict(opts)
+    bias = opts.pop("bias", True)
+    norm = opts.pop("norm", False)
+    residual = opts.pop("residual", False)
+    E, k, H, F = shape
+    L = synth.LayerInputs(E, k, H, F, seed=E + k, with_norm=True)
+    _check_layer(lib, oracle, L, 1, bias=bias, norm=norm, residual=residual, **opts)
+
+
 @pytest.mark.parametrize("opts", [dict(act=1), dict(sigmoid=True), dict(weight_before_ffn=True),
                                   dict(bias=False), dict(norm=True, residual=True),
                                   dict(weight_before_ffn=True, norm=True, residual=True)])
