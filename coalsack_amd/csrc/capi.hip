@@ -438,8 +438,11 @@ bool stream_path(int64_t T, int64_t H, int64_t F, int64_t E, int64_t k) {
   return T <= 64 || (T * k <= 10 * E && T * k <= kStreamMaxP);
 }
 
+// mx3_out: also rewrite the rows x as FP6 terms (the grouped GEMM's operand), riding on the
+// top-k launch.
 int launch_router(const float* x, const float* gate_w, const float* gate_b, int64_t T, int64_t E,
-                  int64_t H, int64_t k, int sigmoid, float* logits, float* pairs, int* ids) {
+                  int64_t H, int64_t k, int sigmoid, float* logits, float* pairs, int* ids,
+                  uint16_t* mx3_out = nullptr) {
   if (T == 0) return CSK_OK;
   const unsigned gx = (unsigned)cdiv(E, 4);
   int nsplit = 0;  // > 0: the logits kernel wrote partial logits behind the [T, E] final ones
@@ -465,8 +468,14 @@ int launch_router(const float* x, const float* gate_w, const float* gate_b, int6
   }
   int rc = check_launch("router_logits_kernel");
   if (rc != CSK_OK) return rc;
-  router_topk_kernel<<<dim3((unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
-      logits, pairs, ids, (int)T, (int)E, (int)k, sigmoid, x, gate_w, gate_b, (int)H, logits + T * E, nsplit);
+  Mx3Rider rider{};
+  int64_t riders = 0;
+  if (mx3_out) {
+    rider = Mx3Rider{x, reinterpret_cast<u32x4*>(mx3_out), (long)T, (int)(H / 32), (int)cdiv(T, 4)};
+    riders = cdiv(T * mx3_row_blocks((int)(H / 32)), 256);
+  }
+  router_topk_kernel<<<dim3((unsigned)(cdiv(T, 4) + riders)), 256, 0, g_stream>>>(
+      logits, pairs, ids, (int)T, (int)E, (int)k, sigmoid, x, gate_w, gate_b, (int)H, logits + T * E, nsplit, rider);
   return check_launch("router_topk_kernel");
 }
 
@@ -1704,7 +1713,7 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
       // workgroups, then the dispatch kernel -- a launch more, each much shorter
       router_topk_kernel<<<dim3((unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
           ws.logits, ws.pairs, ws.ids, (int)T, (int)L->E, (int)L->k, L->sigmoid, xr, L->gate_w,
-          L->has_gate_b ? L->gate_b : nullptr, (int)L->H, ws.logits + T * L->E, 0);
+          L->has_gate_b ? L->gate_b : nullptr, (int)L->H, ws.logits + T * L->E, 0, Mx3Rider{});
       if ((rc = check_launch("router_topk_kernel")) != CSK_OK) return rc;
       if ((rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, L->ew_dev, ws)) != CSK_OK) return rc;
     } else {
@@ -1722,13 +1731,11 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
       rc = launch_prep(hidden, L->norm_w, L->eps, ws.xn, T, L->H);
       if (rc != CSK_OK) return rc;
     }
-    if (!L->f16 && !stream && !L->wbf) {
-      rc = launch_mx3(xr, ws.xs, T, L->H, nullptr, nullptr);
-      if (rc != CSK_OK) return rc;
-    }
+    // the rows' FP6 form for the grouped GEMM is written by extra workgroups of the top-k launch
+    const bool ride = !L->f16 && !stream && !L->wbf;
     mark(CSK_STAGE_ROUTER);
     rc = launch_router(xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, T, L->E, L->H, L->k,
-                       L->sigmoid, ws.logits, ws.pairs, ws.ids);
+                       L->sigmoid, ws.logits, ws.pairs, ws.ids, ride ? ws.xs : nullptr);
     if (rc != CSK_OK) return rc;
     mark(CSK_STAGE_DISPATCH);
     rc = launch_dispatch(ws.ids, ws.pairs, P, L->k, L->E, L->ew_dev, ws);

@@ -82,12 +82,10 @@ __device__ __forceinline__ void mx3_quantize_block(float (&r)[32], u32x4 (&out)[
 //   x3[(row * mx3_row_blocks(nblk) + kb) * 6 + c] <- quantise(x[src(row)][32 kb .. 32 kb + 31] * w(row))
 // src(row) = gather_tok[row] and w(row) = gather_w[row] when given (rows gathered and
 // pre-scaled per dispatch position, expert_mlp_node.h:515-522), else row and 1.
-__global__ __launch_bounds__(256) void mx3_rows_kernel(const float* __restrict__ x,
-                                                       u32x4* __restrict__ x3, long rows, int nblk,
-                                                       const int* __restrict__ gather_tok,
-                                                       const float* __restrict__ gather_w) {
+__device__ __forceinline__ void mx3_rows_block(long b, const float* __restrict__ x, u32x4* __restrict__ x3,
+                                               long rows, int nblk, const int* __restrict__ gather_tok,
+                                               const float* __restrict__ gather_w) {
   const int rowblk = mx3_row_blocks(nblk);
-  const long b = (long)blockIdx.x * 256 + threadIdx.x;
   if (b >= rows * rowblk) return;
   const long row = b / rowblk;
   const int kb = (int)(b - row * rowblk);
@@ -117,5 +115,21 @@ __global__ __launch_bounds__(256) void mx3_rows_kernel(const float* __restrict__
 #pragma unroll
   for (int c = 0; c < kMx3ChunksPerBlock; ++c) x3[b * kMx3ChunksPerBlock + c] = out[c];
 }
+__global__ __launch_bounds__(256) void mx3_rows_kernel(const float* __restrict__ x,
+                                                       u32x4* __restrict__ x3, long rows, int nblk,
+                                                       const int* __restrict__ gather_tok,
+                                                       const float* __restrict__ gather_w) {
+  mx3_rows_block((long)blockIdx.x * 256 + threadIdx.x, x, x3, rows, nblk, gather_tok, gather_w);
+}
+
+// The same work as a rider of another kernel's launch: workgroups first_wg, first_wg + 1, ...
+// of that kernel's grid write the rows (x3 == nullptr: no such workgroups were launched).
+struct Mx3Rider {
+  const float* x;
+  u32x4* x3;
+  long rows;
+  int nblk;
+  int first_wg;
+};
 
 }  // namespace csk

@@ -399,10 +399,19 @@ __global__ __launch_bounds__(256) void router_topk_kernel(float* __restrict__ lo
                                                           const float* __restrict__ g,
                                                           const float* __restrict__ b, int H,
                                                           const float* __restrict__ partial,
-                                                          int nsplit) {
+                                                          int nsplit, Mx3Rider rider) {
   __shared__ CloseCallLds cc;
   __shared__ float cc_thr[4];
   __shared__ int cc_flag[4];
+  // Riders: workgroups past the tokens' rewrite the activation rows as FP6 terms for the
+  // grouped GEMM.  The two jobs share only their input; a token with a close call keeps
+  // one workgroup of this kernel busy for a chain of H dependent additions, during which
+  // the rest of the chip would have nothing to do.
+  if (rider.x3 && (int)blockIdx.x >= rider.first_wg) {
+    mx3_rows_block((long)(blockIdx.x - rider.first_wg) * 256 + threadIdx.x, rider.x, rider.x3, rider.rows, rider.nblk,
+                   nullptr, nullptr);
+    return;
+  }
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int t = blockIdx.x * 4 + wv;
   const bool live = t < T;  // waves past the end stay for the barriers below
