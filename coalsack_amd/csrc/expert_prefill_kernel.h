@@ -452,11 +452,11 @@ __device__ __forceinline__ void expert_gemm_mx_unit(const ExpertGemmMxArgs& a, c
   }
 }
 
-// Work unit = (M tile, N tile), numbered M-tile major.  Workgroups are handed to the
-// eight accelerator dies round-robin by linear id, and each die has its own L2: die x
-// takes the x-th contiguous eighth of the unit sequence, so that the workgroups resident
-// on one die at one time share a few activation panels and a few experts' weights, which
-// then come from that L2 instead of from memory.
+// Work unit = (M tile, N tile), numbered expert by expert (M-tile major for the down
+// projection).  Workgroups are handed to the eight accelerator dies round-robin by linear id,
+// and each die has its own L2: die x takes the x-th contiguous eighth of the unit sequence,
+// so that the workgroups resident on one die at one time share a few activation panels and
+// a few experts' weights, which then come from that L2 instead of from memory.
 template <int MODE, int NG>
 __global__ __launch_bounds__(64 * kMxWaves, 2) void expert_gemm_mx_kernel(ExpertGemmMxArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -465,9 +465,20 @@ __global__ __launch_bounds__(64 * kMxWaves, 2) void expert_gemm_mx_kernel(Expert
   const int slot = blockIdx.x / kDies;
   const int unit = (blockIdx.x % kDies) * per_die + slot;
   if (slot >= per_die || unit >= n_units) return;
-  const int mt = unit / a.n_ntiles, nt = unit - mt * a.n_ntiles;
+  const int mt = unit / a.n_ntiles;
+  int nt = unit - mt * a.n_ntiles;
   const WorkDesc* wd = a.desc + a.mtiles[2 * mt];
-  const int m0 = a.mtiles[2 * mt + 1];
+  int m0 = a.mtiles[2 * mt + 1];
+  if (MODE == 0) {
+    // Within an expert's block of the sequence the gate/up units run N tile by N tile, the
+    // expert's M tiles side by side: the workgroups resident together then read the same
+    // weight rows at about the same time (20b shape, 2048 tokens: 525 -> 506 us per layer;
+    // the down projection is no faster that way and keeps the M-tile-major order).
+    const int tiles_e = (wd->Te + kGemmBM - 1) / kGemmBM;
+    const int r = unit - (mt - m0 / kGemmBM) * a.n_ntiles;  // position within the expert's block
+    nt = r / tiles_e;
+    m0 = (r - nt * tiles_e) * kGemmBM;
+  }
   const int mcount = min(kGemmBM, wd->Te - m0);
   if (mcount <= 32)
     expert_gemm_mx_unit<MODE, NG, 1>(a, wd, m0, mcount, nt, smem);
