@@ -517,21 +517,26 @@ __global__ __launch_bounds__(256, 3) void expert_f16_gemm_kernel(ExpertF16GemmAr
 
   u32x4 wq[2][4];  // [row group][16-wide K slice of the step]
   u32x4 aq[4];
+  // Every load of the loop is unconditional (addresses are clamped, never branched around):
+  // with a branch around a load the compiler's wait-count pass gives up at the join and
+  // drains the whole queue at the head of every step.  A block past K (odd block count: the
+  // second half of the last step) re-reads the last block of the weights and meets a panel
+  // chunk of zeros.
   auto load_w = [&](int s, int sl, int j) {
-    const int kb = 2 * j + (sl >> 1);
-    // a block past K (odd block count) contributes nothing
-    wq[s][sl] = kb < nkb ? W[s][(long)kb * 64 + 32 * (sl & 1)] : u32x4{0u, 0u, 0u, 0u};
+    const int kb = min(2 * j + (sl >> 1), nkb - 1);
+    wq[s][sl] = W[s][(long)kb * 64 + 32 * (sl & 1)];
   };
   auto load_a = [&](int j) {
     const int kbs = min(2 * j + sblk, nkb - 1);
 #pragma unroll
     for (int i = 0; i < 4; ++i) aq[i] = Arow[i][(long)kbs * 8];
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf, int j) {
+    const bool past = 2 * j + sblk >= nkb;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int tok = st + 16 * i;
-      panel[buf][tok * 16 + (sc ^ (tok & 15))] = aq[i];
+      panel[buf][tok * 16 + (sc ^ (tok & 15))] = past ? u32x4{0u, 0u, 0u, 0u} : aq[i];
     }
   };
 #pragma unroll
@@ -539,39 +544,60 @@ __global__ __launch_bounds__(256, 3) void expert_f16_gemm_kernel(ExpertF16GemmAr
 #pragma unroll
     for (int sl = 0; sl < 4; ++sl) load_w(s, sl, 0);
   load_a(0);
-  stash(0);
+  stash(0, 0);
   __syncthreads();
-  for (int j = 0; j < nsteps; ++j) {
+  // One step = 64 of K: four 16-wide slices, each 2 row groups x 2 token halves x 2 terms of
+  // matrix instructions.  The panel fragments of a token half are read from LDS while the
+  // matrix instructions of the other half issue (the same four fragment registers in
+  // rotation); a slice's weight registers are reloaded for the next step as soon as its
+  // matrix instructions have issued; the next step's panel rows are requested at the head
+  // of the step and stored to the other LDS buffer at its end, behind a wait that leaves the
+  // weight loads in flight.
+  auto step = [&](int j, auto more_t) {
+    constexpr bool more = decltype(more_t)::value;
     const int buf = j & 1;
-    const bool more = j + 1 < nsteps;
     if (more) load_a(j + 1);
-#pragma unroll
-    for (int sl = 0; sl < 4; ++sl) {
+    half8 hi[2], lo[2];
+    auto read_half = [&](int sl, int ms) {
       // logical chunk of this lane's 8 halves: block sl / 2, [hi | lo], quarter 2 (sl % 2) + kg
       const int c_hi = (sl >> 1) * 8 + 2 * (sl & 1) + kg, c_lo = c_hi + 4;
-      half8 hi[2], lo[2];
+      const int tok = ms * 32 + n32;
+      hi[ms] = __builtin_bit_cast(half8, panel[buf][tok * 16 + (c_hi ^ n16)]);
+      lo[ms] = __builtin_bit_cast(half8, panel[buf][tok * 16 + (c_lo ^ n16)]);
+    };
+    read_half(0, 0);
 #pragma unroll
-      for (int ms = 0; ms < 2; ++ms) {
-        const int tok = ms * 32 + n32;
-        hi[ms] = __builtin_bit_cast(half8, panel[buf][tok * 16 + (c_hi ^ n16)]);
-        lo[ms] = __builtin_bit_cast(half8, panel[buf][tok * 16 + (c_lo ^ n16)]);
-      }
+    for (int sl = 0; sl < 4; ++sl) {
+      read_half(sl, 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         const half8 w = __builtin_bit_cast(half8, wq[s][sl]);
-#pragma unroll
-        for (int ms = 0; ms < 2; ++ms) {
-          acc[ms][s] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi[ms], w, acc[ms][s], 0, 0, 0);
-          acc[ms][s] = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo[ms], w, acc[ms][s], 0, 0, 0);
-        }
-        // the slice's registers are free as soon as its matrix instructions have issued:
-        // the next step's weights go straight back into them (one register set in rotation)
-        if (more) load_w(s, sl, j + 1);
+        acc[0][s] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi[0], w, acc[0][s], 0, 0, 0);
+        acc[0][s] = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo[0], w, acc[0][s], 0, 0, 0);
       }
+      __builtin_amdgcn_sched_barrier(0);
+      if (sl + 1 < 4) read_half(sl + 1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const half8 w = __builtin_bit_cast(half8, wq[s][sl]);
+        acc[1][s] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi[1], w, acc[1][s], 0, 0, 0);
+        acc[1][s] = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo[1], w, acc[1][s], 0, 0, 0);
+      }
+      // the slice's registers are free as soon as its matrix instructions have issued:
+      // the next step's weights go straight back into them (one register set in rotation)
+      if (more) {
+        load_w(0, sl, j + 1);
+        load_w(1, sl, j + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    if (more) stash(buf ^ 1);
+    if (more) stash(buf ^ 1, j + 1);
     __syncthreads();
-  }
+  };
+  for (int j = 0; j + 1 < nsteps; ++j) step(j, std::true_type{});
+  step(nsteps - 1, std::false_type{});
 
   // accumulator register r is token (r % 4) + 8 (r / 4) + 4 kg of its 32-token half
   const CSK_GLOBAL float* b0 = as_global(MODE == 0 ? wd->w.b_gate : wd->w.b_down);
