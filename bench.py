@@ -284,7 +284,9 @@ def layer_roofline(res, shape, T, workload):
                     algorithmic_flops=fl)
     else:
         roof = dict(bound="hbm",
-                    kernel=("expert_f16_kernel<0>" if f16 else "expert_stream_kernel<0,*>") + " (gate/up + SwiGLU)",
+                    kernel=("expert_f16_kernel<0>" if f16 else "expert_stream_kernel<0,*>") +
+                    (" (top-k routing of the one token + gate/up + SwiGLU: no routing launch in front)"
+                     if (T == 1 and not f16) else " (gate/up + SwiGLU)"),
                     achieved=res["gateup_gbs"], peak=HBM_PEAK_GBS, unit="GB/s", traffic=None,
                     algorithmic_bytes=res["gateup_bytes"])
     # HBM traffic of that kernel from a recorded counter run of this workload, where there is one
