@@ -412,6 +412,9 @@ __device__ __forceinline__ void expert_gemm_mx_unit(const ExpertGemmMxArgs& a, c
             const float v = moe_activation(acc[ms][gi][r], acc[ms][NG / 2 + gi][r], kAct);
             tile[tl * G::kEpiRow + 32 * gi + n32] = rv ? v : 0.0f;
           }
+          // one pair of accumulator tiles at a time: left to itself the scheduler copies several
+          // tiles out of the accumulation registers ahead of their use and spills one of them
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     };
