@@ -571,6 +571,7 @@ struct ExpertInput {
   const float* gather_w;
   const uint16_t* x_mx3;
   const int* mx3_list_row;
+  const uint16_t* x_mx3_tokens = nullptr;  // streaming path: the token rows already as FP6 terms (written by the routing prologue)
   const RouteIn* rin = nullptr;    // both set: a one-token batch that the gate/up kernel routes itself
   const RouteOut* rout = nullptr;
 };
@@ -589,6 +590,8 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   a.list_row = stream ? in.list_row : in.mx3_list_row;
   a.gather_w = in.gather_w;
   a.X = in.x;
+  a.X3 = stream ? reinterpret_cast<const u32x4*>(in.x_mx3_tokens) : nullptr;
+  a.zeros = g_zero;
   a.nblk = (int)(H / 32);
   a.N = (int)F;
   a.ntile = (int)cdiv(F, 16);
@@ -606,6 +609,7 @@ int run_experts(int64_t E, int64_t T, int64_t k, int64_t H, int64_t F,
   // down
   a.list_row = nullptr;
   a.gather_w = nullptr;
+  a.X3 = nullptr;
   a.X = reinterpret_cast<const float*>(ws.act);
   a.nblk = (int)(F / 32);
   a.N = (int)H;
@@ -1675,7 +1679,7 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
   const int64_t P = T * L->k;
   const bool norm = (flags & CSK_FWD_RMSNORM) != 0;
   const float* xr = norm ? ws.xn : hidden;
-  bool route_in_kernel = false;
+  bool route_in_kernel = false, rows_mx3_ready = false;
   RouteIn rin_kept{};
   RouteOut rout_kept{};
   if (phase == 2) {
@@ -1684,15 +1688,19 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
     // small batch: prologue + logits in one launch, top-k + dispatch in another
     mark(CSK_STAGE_PREP);
     mark(CSK_STAGE_ROUTER);
+    // the streaming kernels copy their token rows as FP6 terms, written once per token by the
+    // prologue workgroups of this launch (not when the routing weight multiplies the rows first)
+    u32x4* rows_mx3 = (!L->f16 && !L->wbf && stream_path(T, L->H, L->F, L->E, L->k)) ? reinterpret_cast<u32x4*>(ws.xs) : nullptr;
+    rows_mx3_ready = rows_mx3 != nullptr;
     // a workgroup takes one expert (latency) as long as all of them are resident at once, four beyond
     if (cdiv(T, 4) * (L->E + 4) <= 4 * std::max(g_cus, 1) + 64)  // four of these workgroups fit a compute unit
       router_prep_logits_kernel<1><<<dim3((unsigned)(L->E + 4), (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
           hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, L->gate_w,
-          L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
+          L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H, rows_mx3);
     else
       router_prep_logits_kernel<4><<<dim3((unsigned)(cdiv(L->E, 4) + 4), (unsigned)cdiv(T, 4)), 256, 0, g_stream>>>(
           hidden, norm ? L->norm_w : nullptr, L->eps, ws.xn, L->gate_w,
-          L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H);
+          L->has_gate_b ? L->gate_b : nullptr, ws.logits, (int)T, (int)L->E, (int)L->H, rows_mx3);
     if ((rc = check_launch("router_prep_logits_kernel")) != CSK_OK) return rc;
     mark(CSK_STAGE_DISPATCH);
     RouteIn rin{ws.logits, xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, L->ew_dev,
@@ -1732,7 +1740,8 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
       if (rc != CSK_OK) return rc;
     }
     // the rows' FP6 form for the grouped GEMM is written by extra workgroups of the top-k launch
-    const bool ride = !L->f16 && !stream && !L->wbf;
+    const bool ride = !L->f16 && !L->wbf;  // (the streaming kernels copy the rows in this form, too)
+    rows_mx3_ready = ride && stream;
     mark(CSK_STAGE_ROUTER);
     rc = launch_router(xr, L->gate_w, L->has_gate_b ? L->gate_b : nullptr, T, L->E, L->H, L->k,
                        L->sigmoid, ws.logits, ws.pairs, ws.ids, ride ? ws.xs : nullptr);
@@ -1757,6 +1766,7 @@ int forward_pass(csk_layer* L, const float* hidden, int64_t T, float* out, int f
   // pre-scaled per dispatch position when the routing weight goes in front of the FFN)
   ExpertInput in{xr, ws.list_tok, L->wbf ? ws.list_w : nullptr, ws.xs, ws.list_tok};
   if (route_in_kernel) in.rin = &rin_kept, in.rout = &rout_kept;
+  if (rows_mx3_ready) in.x_mx3_tokens = ws.xs;
   if (L->wbf && !stream_path(T, L->H, L->F, L->E, L->k)) {
     if ((rc = launch_mx3(xr, ws.xg, P, L->H, ws.list_tok, ws.list_w)) != CSK_OK) return rc;
     in.x_mx3 = ws.xg;

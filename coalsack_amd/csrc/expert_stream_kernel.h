@@ -31,6 +31,8 @@ struct ExpertStreamArgs {
   const int* list_row;   // packed position -> row of X; null: row = packed position
   const float* gather_w; // packed position -> factor applied to its row (weight_before_ffn); null: 1
   const float* X;        // [rows][32 nblk] fp32 activation rows
+  const u32x4* X3;       // the same rows already as three FP6 terms, [rows][mx3_row_blocks(nblk)][6] (mx3.h), or null
+  const float* zeros;    // at least 16 bytes of zeros (with X3)
   int nblk;              // K / 32
   int ntile;             // ceil(N / 16)
   int N;                 // output features (F for gate/up, H for down)
@@ -265,8 +267,19 @@ __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs 
     // A thread's first block of activations is requested first (loads return in order: asked
     // for after the weights it would arrive behind them), then the first unit's weights ...
     const int nfill = gcount * lrb;
+    // Rows that arrive as FP6 terms already (written once per token by the routing prologue)
+    // are only copied into LDS, behind the first unit's weights (below).
+    const bool copy_rows = MODE == 0 && a.X3 != nullptr && a.gather_w == nullptr;
+    int copy_row[G];  // the rows' numbers, read before the weights are requested
+    if (copy_rows) {
+#pragma unroll
+      for (int rr = 0; rr < G; ++rr) {
+        const int p = base + min(rr, gcount - 1);
+        copy_row[rr] = ROUTE1 ? 0 : a.list_row ? a.list_row[p] : p;
+      }
+    }
     float4 pre[8];
-    {
+    if (!copy_rows) {
       const int rr = threadIdx.x / lrb, kb = threadIdx.x - rr * lrb;
       if ((int)threadIdx.x < nfill && kb < nblk) {
         const int row = ROUTE1 ? 0 : a.list_row ? a.list_row[base + rr] : base + rr;
@@ -284,8 +297,39 @@ __global__ __launch_bounds__(256, 2) void expert_stream_kernel(ExpertStreamArgs 
     // quantised into LDS, one thread per 32-value block (every wave is past its last read
     // of the previous group: it has crossed that unit's barrier).  Rows may be gathered
     // through list_row and scaled by the routing weight (weight_before_ffn).
+    if (MODE == 0 && copy_rows) {
+      // The LDS image of a row is its blocks in order, [lrb][6 chunks of 16 bytes]; the row in
+      // memory has mx3_row_blocks(nblk) of them, the rest are zeros (any scale byte will do
+      // for a block of zero codes: they come from the library's page of zeros).  Copied by
+      // global_load_lds -- nothing of it lives in a register; instruction i of wave wv fills
+      // the 64 chunks from (4 i + wv) * 64 on -- and waited for explicitly: the compiler does
+      // not count these loads, so none of them may be in flight past the wait below.
+      const int rowblk = mx3_row_blocks(nblk);
+      constexpr int kRowChunks = lrb * kMx3ChunksPerBlock;
+      constexpr int kCopyInstr = (G * kRowChunks + 255) / 256;
+      const int total = gcount * kRowChunks;
+      const uint32_t lds_as = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 #pragma unroll 1
-    for (int idx = threadIdx.x; idx < nfill; idx += 256) {
+      for (int i = 0; i < kCopyInstr; ++i) {
+        const int ch0 = (4 * i + wv) * 64;
+        const int ch = ch0 + lane;
+        if (ch < total) {
+          const int rr = ch / kRowChunks, q = ch - rr * kRowChunks;
+          int row = copy_row[0];
+#pragma unroll
+          for (int x = 1; x < G; ++x) row = rr == x ? copy_row[x] : row;
+          const u32x4* src = q < rowblk * kMx3ChunksPerBlock ? a.X3 + (size_t)row * rowblk * kMx3ChunksPerBlock + q
+                                                            : reinterpret_cast<const u32x4*>(a.zeros);
+          asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                       :
+                       : "v"(src), "s"(__builtin_amdgcn_readfirstlane((int)(lds_as + (uint32_t)ch0 * 16u)))
+                       : "memory");
+        }
+      }
+      __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): the copies (and the first weights) have landed
+    }
+#pragma unroll 1
+    for (int idx = threadIdx.x; idx < (copy_rows ? 0 : nfill); idx += 256) {
       const int rr = idx / lrb, kb = idx - rr * lrb;
       u32x4 out[kMx3ChunksPerBlock];
       if (kb >= nblk) {

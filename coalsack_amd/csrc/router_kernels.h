@@ -163,14 +163,15 @@ template <int EPW>
 __global__ __launch_bounds__(256) void router_prep_logits_kernel(
     const float* __restrict__ hidden, const float* __restrict__ norm_w, float eps,
     float* __restrict__ xn, const float* __restrict__ g,
-    const float* __restrict__ b, float* __restrict__ logits, int T, int E, int H) {
+    const float* __restrict__ b, float* __restrict__ logits, int T, int E, int H,
+    u32x4* __restrict__ x3) {
   __shared__ float part[4][4];
   __shared__ float dots[EPW][4][4];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int n_ewg = (E + EPW - 1) / EPW;  // workgroups that compute logits
   if ((int)blockIdx.x >= n_ewg) {  // ---- prologue of token t (one of four per token tile)
     const int t = (blockIdx.x - n_ewg) + 4 * blockIdx.y;
-    if (blockIdx.x - n_ewg >= 4 || t >= T || !norm_w) return;  // without a norm the rows are used as they are
+    if (blockIdx.x - n_ewg >= 4 || t >= T || (!norm_w && !x3)) return;  // without a norm the rows are used as they are
     // four columns per thread, the row's loads all in flight at once and kept in registers
     // between the two passes (rows longer than 4096 take further rounds of the same)
     const float4* x4 = reinterpret_cast<const float4*>(hidden + (size_t)t * H);
@@ -229,6 +230,40 @@ __global__ __launch_bounds__(256) void router_prep_logits_kernel(
             reinterpret_cast<float4*>(xn + (size_t)t * H)[c] = v;
           }
         }
+      }
+    }
+    if (x3) {
+      // The row the experts will contract, as three FP6 terms (mx3.h), one thread per 32-value
+      // block: the weight-streaming kernels copy it into LDS instead of each of their
+      // workgroups quantising the rows of its token group again (a team of fifteen workgroups
+      // used to do the same 1.4 us of vector arithmetic per block and thread fifteen times).
+      // The values are formed from the inputs with the operations of the loop above, so they
+      // are the bits of xn.  H is a multiple of 32 here.
+      const int nblk = H >> 5, rowblk = mx3_row_blocks(nblk);
+      for (int kb = threadIdx.x; kb < rowblk; kb += 256) {
+        u32x4 out[kMx3ChunksPerBlock];
+        if (kb >= nblk) {
+#pragma unroll
+          for (int tt = 0; tt < kMx3Terms; ++tt) {
+            out[2 * tt] = u32x4{0u, 0u, 0u, 0u};
+            out[2 * tt + 1] = u32x4{0u, 0u, 127u, 0u};
+          }
+        } else {
+          float r[32];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            float4 v = x4[kb * 8 + i];
+            if (norm_w) {
+              const float4 w = nw4[kb * 8 + i];
+              v.x = (v.x / den) * w.x, v.y = (v.y / den) * w.y, v.z = (v.z / den) * w.z, v.w = (v.w / den) * w.w;
+            }
+            r[4 * i] = v.x, r[4 * i + 1] = v.y, r[4 * i + 2] = v.z, r[4 * i + 3] = v.w;
+          }
+          mx3_quantize_block(r, out);
+        }
+        u32x4* dst = x3 + ((size_t)t * rowblk + kb) * kMx3ChunksPerBlock;
+#pragma unroll
+        for (int c = 0; c < kMx3ChunksPerBlock; ++c) dst[c] = out[c];
       }
     }
     return;
